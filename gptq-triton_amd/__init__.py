@@ -1,0 +1,17 @@
+"""MI355X-native 4-bit GPTQ inference hot path.
+
+Same module API as the reference package (src/gptq_triton/__init__.py:10-13):
+QuantLinear / make_quant / triton_matmul4, QuantLlamaMLP / make_fused_mlp /
+triton_llama_mlp_4, QuantLlamaAttention / make_quant_attn, load_quant,
+autotune_warmup - computed by hand-written gfx950 kernels behind a C ABI.
+"""
+from . import fused_mlp, quant_linear
+from .fused_attention import (LlamaConfigLite, QuantLlamaAttention, RotaryTable, make_quant_attn, qkv_rotary)
+from .fused_mlp import QuantLlamaMLP, llama_mlp_4, make_fused_mlp, triton_llama_mlp_4
+from .quant_linear import (QuantLinear, dequantize, make_quant, matmul4, prepare_act_order, triton_matmul4)
+
+__all__ = [
+    "QuantLinear", "make_quant", "matmul4", "triton_matmul4", "dequantize", "prepare_act_order",
+    "QuantLlamaMLP", "make_fused_mlp", "llama_mlp_4", "triton_llama_mlp_4",
+    "QuantLlamaAttention", "make_quant_attn", "qkv_rotary", "RotaryTable", "LlamaConfigLite",
+]

@@ -1,0 +1,101 @@
+"""ctypes binding of csrc/libgptq4.so (the C ABI declared in include/gptq4.h).
+
+The HIP library is the only compute path: if it is missing, load() raises, and every
+operator that needs it raises with it.  There is no CPU fallback.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_char_p, c_float, c_int, c_size_t, c_void_p
+from pathlib import Path
+
+import torch
+
+LIB_PATH = Path(__file__).resolve().parent / "csrc" / "libgptq4.so"
+ABI_VERSION = 1
+WS_COUNTER_BYTES = 16384
+OP_MATMUL, OP_MLP_GATEUP, OP_QKV_ROTARY = 0, 1, 2
+
+# every symbol include/gptq4.h declares: (restype, argtypes)
+SIGNATURES = {
+    "gptq4_abi_version": (c_int, []),
+    "gptq4_strerror": (c_char_p, [c_int]),
+    "gptq4_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
+    "gptq4_dequant": (c_int, [c_void_p] * 5 + [c_int, c_int, c_int, c_void_p]),
+    "gptq4_actorder_sort_rows": (c_int, [c_void_p] * 3 + [c_int, c_int, c_void_p]),
+    "gptq4_matmul": (c_int, [c_void_p] * 7 + [c_int] * 4 + [c_void_p, c_size_t, c_void_p]),
+    "gptq4_mlp_gateup": (c_int, [c_void_p] * 9 + [c_int] * 4 + [c_void_p, c_size_t, c_void_p]),
+    "gptq4_rope_table": (c_int, [c_void_p, c_void_p, c_int, c_int, c_float, c_void_p]),
+    "gptq4_qkv_rotary": (c_int, [c_void_p] * 8 + [c_int] + [c_void_p] * 3 + [c_int] * 8 + [c_void_p, c_size_t, c_void_p]),
+    "gptq4_set_splitk": (None, [c_int]),
+}
+
+
+class LibraryMissing(RuntimeError):
+    pass
+
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Open the in-tree shared object and bind every entry point."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not LIB_PATH.exists():
+        raise LibraryMissing(
+            f"{LIB_PATH} is not built; run `python -c 'import __graft_entry__ as g; g.build()'` "
+            "or `python gptq-triton_amd/build.py` (needs hipcc)")
+    lib = ctypes.CDLL(str(LIB_PATH))
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    got = lib.gptq4_abi_version()
+    if got != ABI_VERSION:
+        raise LibraryMissing(f"{LIB_PATH} has ABI version {got}, expected {ABI_VERSION}; rebuild it")
+    _lib = lib
+    return lib
+
+
+class Gptq4Error(RuntimeError):
+    def __init__(self, code: int, where: str):
+        self.code = code
+        msg = load().gptq4_strerror(code).decode()
+        super().__init__(f"{where}: {msg} (code {code})")
+
+
+def check(code: int, where: str) -> None:
+    if code != 0:
+        raise Gptq4Error(code, where)
+
+
+def ptr(t: torch.Tensor | None):
+    return None if t is None else t.data_ptr()
+
+
+def current_stream(device: torch.device):
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+# One workspace per (device, stream): split-K partials + arrival counters.  The counter
+# region must start zeroed; the kernels restore it to zero.
+_workspaces: dict = {}
+_WS_BYTES = WS_COUNTER_BYTES + 16 * 16 * 2 * 32768 * 4  # splitk 16, M 16, 2 matrices, 32768 columns
+
+
+def workspace(device: torch.device, need: int):
+    key = (device.index if device.index is not None else torch.cuda.current_device(),
+           torch.cuda.current_stream(device).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < need:
+        ws = torch.zeros(max(need, _WS_BYTES), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def require_cuda(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must live on the GPU: the HIP library is the only compute path "
+                           f"(got device {t.device})")

@@ -1,0 +1,211 @@
+// C ABI of the library (declared in include/gptq4.h): argument validation on the
+// host, then one kernel launch on the caller's stream.  No allocation, no
+// synchronisation, no exceptions.
+#include "../../include/gptq4.h"
+
+#include "gptq4_internal.h"
+
+namespace {
+
+inline bool misaligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) != 0; }
+
+// groupsize: -1 -> K.  Accepts what the reference accepts (quant_linear.py:244-257).
+int check_dims(int K, int N, int *groupsize) {
+    if (K <= 0 || N <= 0 || (K % 128) != 0 || (N % 256) != 0) return -GPTQ4_E_SHAPE;
+    int g = *groupsize;
+    if (g == -1) g = K;
+    if (g <= 0 || (g % 128) != 0 || (K % g) != 0) return -GPTQ4_E_GROUPSIZE;
+    *groupsize = g;
+    return 0;
+}
+
+size_t partial_bytes(int splitk, int M, int ncols_total) {
+    return (size_t)splitk * (size_t)M * (size_t)ncols_total * sizeof(float);
+}
+
+// Fill the split-K fields of `a`; `ncols_total` = columns summed over all tiles
+// (N, or 2*I for the gate/up pair).
+int setup_skinny(MatmulArgs &a, int tile_cols, int ncols_total, void *workspace, size_t workspace_bytes) {
+    a.tiles = a.N / tile_cols;
+    if (a.tiles > SKINNY_MAX_TILES) return -GPTQ4_E_SHAPE;
+    a.splitk = skinny_pick_splitk(a.tiles, a.K / 128);
+    if (workspace == nullptr || workspace_bytes < GPTQ4_WS_COUNTER_BYTES) return -GPTQ4_E_WORKSPACE;
+    if (a.splitk > 1 &&
+        workspace_bytes < GPTQ4_WS_COUNTER_BYTES + partial_bytes(a.splitk, a.M, ncols_total))
+        return -GPTQ4_E_WORKSPACE;
+    a.counters = reinterpret_cast<int *>(workspace);
+    a.partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_COUNTER_BYTES);
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int gptq4_abi_version(void) { return GPTQ4_ABI_VERSION; }
+
+const char *gptq4_strerror(int code) {
+    if (code == 0) return "success";
+    if (code > 0) return hipGetErrorString((hipError_t)code);
+    switch (-code) {
+        case GPTQ4_E_NULL:
+            return "a required pointer is NULL";
+        case GPTQ4_E_SHAPE:
+            return "unsupported shape (need K % 128 == 0, N % 256 == 0, M >= 1, head_dim == 128)";
+        case GPTQ4_E_GROUPSIZE:
+            return "groupsize must be -1, K, or a multiple of 128 dividing K";
+        case GPTQ4_E_WORKSPACE:
+            return "workspace is NULL or too small (see gptq4_workspace_bytes)";
+        case GPTQ4_E_ALIGN:
+            return "a pointer is not 16-byte aligned";
+        default:
+            return "unknown gptq4 error";
+    }
+}
+
+void gptq4_set_splitk(int splitk) { g_forced_splitk = splitk < 0 ? 0 : splitk; }
+
+size_t gptq4_workspace_bytes(int op, int M, int K, int N) {
+    (void)K;
+    size_t bytes = GPTQ4_WS_COUNTER_BYTES;
+    if (M >= 1 && M <= SKINNY_MAX_M && N > 0) {
+        const int cols = (op == GPTQ4_OP_MLP_GATEUP) ? 2 * N : N;
+        bytes += partial_bytes(SKINNY_MAX_SPLITK, M, cols);
+    }
+    return bytes;
+}
+
+int gptq4_dequant(const int32_t *qweight, const int32_t *qzeros, const void *scales, const int32_t *g_idx,
+                  void *W_out, int K, int N, int groupsize, void *stream) {
+    if (!qweight || !qzeros || !scales || !W_out) return -GPTQ4_E_NULL;
+    if (K <= 0 || N <= 0 || (K % 8) != 0 || (N % 8) != 0) return -GPTQ4_E_SHAPE;
+    if (groupsize == -1) groupsize = K;
+    if (groupsize <= 0 || (groupsize % 8) != 0) return -GPTQ4_E_GROUPSIZE;
+    return launch_dequant(reinterpret_cast<const uint32_t *>(qweight), reinterpret_cast<const uint32_t *>(qzeros),
+                          reinterpret_cast<const half_t *>(scales), g_idx, reinterpret_cast<half_t *>(W_out), K,
+                          N, groupsize, reinterpret_cast<hipStream_t>(stream));
+}
+
+int gptq4_actorder_sort_rows(const int32_t *qweight, const int32_t *perm, int32_t *qweight_out, int K, int N,
+                             void *stream) {
+    if (!qweight || !perm || !qweight_out) return -GPTQ4_E_NULL;
+    if (K <= 0 || N <= 0 || (K % 8) != 0) return -GPTQ4_E_SHAPE;
+    return launch_sort_rows(reinterpret_cast<const uint32_t *>(qweight), perm,
+                            reinterpret_cast<uint32_t *>(qweight_out), K, N, reinterpret_cast<hipStream_t>(stream));
+}
+
+int gptq4_matmul(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
+                 const int32_t *perm, const void *bias, void *y, int M, int K, int N, int groupsize,
+                 void *workspace, size_t workspace_bytes, void *stream) {
+    if (!x || !qweight || !qzeros || !scales || !y) return -GPTQ4_E_NULL;
+    if (M < 1) return -GPTQ4_E_SHAPE;
+    int rc = check_dims(K, N, &groupsize);
+    if (rc) return rc;
+    if (misaligned16(x) || misaligned16(qweight) || misaligned16(scales) || misaligned16(y) ||
+        (perm && misaligned16(perm)) || (bias && misaligned16(bias)))
+        return -GPTQ4_E_ALIGN;
+    MatmulArgs a = {};
+    a.x = reinterpret_cast<const half_t *>(x);
+    a.w[0] = QMat{reinterpret_cast<const uint32_t *>(qweight), reinterpret_cast<const uint32_t *>(qzeros),
+                  reinterpret_cast<const half_t *>(scales)};
+    a.perm = perm;
+    a.bias = reinterpret_cast<const half_t *>(bias);
+    a.y = reinterpret_cast<half_t *>(y);
+    a.M = M;
+    a.K = K;
+    a.N = N;
+    a.groupsize = groupsize;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (M <= SKINNY_MAX_M) {
+        rc = setup_skinny(a, 64, N, workspace, workspace_bytes);
+        if (rc) return rc;
+        return launch_skinny(EPI_PLAIN, a, s);
+    }
+    return launch_gemm(EPI_PLAIN, a, s);
+}
+
+int gptq4_mlp_gateup(const void *x, const int32_t *gate_qweight, const int32_t *gate_qzeros,
+                     const void *gate_scales, const int32_t *up_qweight, const int32_t *up_qzeros,
+                     const void *up_scales, const int32_t *perm, void *h, int M, int K, int I, int groupsize,
+                     void *workspace, size_t workspace_bytes, void *stream) {
+    if (!x || !gate_qweight || !gate_qzeros || !gate_scales || !up_qweight || !up_qzeros || !up_scales || !h)
+        return -GPTQ4_E_NULL;
+    if (M < 1) return -GPTQ4_E_SHAPE;
+    int rc = check_dims(K, I, &groupsize);
+    if (rc) return rc;
+    if (misaligned16(x) || misaligned16(gate_qweight) || misaligned16(up_qweight) || misaligned16(gate_scales) ||
+        misaligned16(up_scales) || misaligned16(h) || (perm && misaligned16(perm)))
+        return -GPTQ4_E_ALIGN;
+    MatmulArgs a = {};
+    a.x = reinterpret_cast<const half_t *>(x);
+    a.w[0] = QMat{reinterpret_cast<const uint32_t *>(gate_qweight), reinterpret_cast<const uint32_t *>(gate_qzeros),
+                  reinterpret_cast<const half_t *>(gate_scales)};
+    a.w[1] = QMat{reinterpret_cast<const uint32_t *>(up_qweight), reinterpret_cast<const uint32_t *>(up_qzeros),
+                  reinterpret_cast<const half_t *>(up_scales)};
+    a.perm = perm;
+    a.y = reinterpret_cast<half_t *>(h);
+    a.M = M;
+    a.K = K;
+    a.N = I;
+    a.groupsize = groupsize;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (M <= SKINNY_MAX_M) {
+        rc = setup_skinny(a, 64, 2 * I, workspace, workspace_bytes);
+        if (rc) return rc;
+        return launch_skinny(EPI_SILU_MUL, a, s);
+    }
+    return launch_gemm(EPI_SILU_MUL, a, s);
+}
+
+int gptq4_rope_table(float *cos_out, float *sin_out, int max_pos, int D, float base, void *stream) {
+    if (!cos_out || !sin_out) return -GPTQ4_E_NULL;
+    if (max_pos < 1 || D < 2 || (D % 2) != 0 || !(base > 0.f)) return -GPTQ4_E_SHAPE;
+    return launch_rope_table(cos_out, sin_out, max_pos, D, base, reinterpret_cast<hipStream_t>(stream));
+}
+
+int gptq4_qkv_rotary(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
+                     const int32_t *perm, const int32_t *position_ids, const float *cos_table,
+                     const float *sin_table, int max_pos, void *q, void *k, void *v, int B, int S, int H, int D,
+                     int K, int groupsize, int kv_capacity, int kv_offset, void *workspace,
+                     size_t workspace_bytes, void *stream) {
+    if (!x || !qweight || !qzeros || !scales || !position_ids || !cos_table || !sin_table || !q || !k || !v)
+        return -GPTQ4_E_NULL;
+    if (B < 1 || S < 1 || H < 1 || D != 128 || max_pos < 1) return -GPTQ4_E_SHAPE;
+    if (kv_offset < 0 || kv_capacity < kv_offset + S) return -GPTQ4_E_SHAPE;
+    if ((long)B * S > 0x7fffffffL) return -GPTQ4_E_SHAPE;
+    const int N = 3 * H * D;
+    int rc = check_dims(K, N, &groupsize);
+    if (rc) return rc;
+    if (misaligned16(x) || misaligned16(qweight) || misaligned16(scales) || misaligned16(q) || misaligned16(k) ||
+        misaligned16(v) || misaligned16(cos_table) || misaligned16(sin_table) || (perm && misaligned16(perm)))
+        return -GPTQ4_E_ALIGN;
+    MatmulArgs a = {};
+    a.x = reinterpret_cast<const half_t *>(x);
+    a.w[0] = QMat{reinterpret_cast<const uint32_t *>(qweight), reinterpret_cast<const uint32_t *>(qzeros),
+                  reinterpret_cast<const half_t *>(scales)};
+    a.perm = perm;
+    a.M = B * S;
+    a.K = K;
+    a.N = N;
+    a.groupsize = groupsize;
+    a.rope.position_ids = position_ids;
+    a.rope.cos_table = cos_table;
+    a.rope.sin_table = sin_table;
+    a.rope.q = reinterpret_cast<half_t *>(q);
+    a.rope.k = reinterpret_cast<half_t *>(k);
+    a.rope.v = reinterpret_cast<half_t *>(v);
+    a.rope.S = S;
+    a.rope.H = H;
+    a.rope.kv_capacity = kv_capacity;
+    a.rope.kv_offset = kv_offset;
+    a.rope.max_pos = max_pos;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (a.M <= SKINNY_MAX_M) {
+        rc = setup_skinny(a, 128, N, workspace, workspace_bytes);
+        if (rc) return rc;
+        return launch_skinny(EPI_ROPE, a, s);
+    }
+    return launch_gemm(EPI_ROPE, a, s);
+}
+
+}  // extern "C"

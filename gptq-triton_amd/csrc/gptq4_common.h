@@ -1,0 +1,122 @@
+// Shared device helpers for the gfx950 4-bit GPTQ kernels.
+//
+// Weight decode (README.md:93 of the reference, `w = (w - z - 1) * s`):
+//   W[k,n] = fp16( float(q - (z + 1)) * float(s) )
+// is produced here entirely in packed fp16 with ONE rounding:
+//   (w & 0x000F000F) | 0x64006400  is the fp16 pair (1024 + q_t, 1024 + q_{t+4});
+//   adding -(1024 + z + 1) is exact (small integers), the multiply by s rounds once.
+// For the odd nibbles the mask 0x00F000F0 gives 1024 + 16*q; fma(v, 1/16, -(64+z+1))
+// is again an exact small integer.  One 32-bit word therefore decodes to four fp16
+// pairs holding rows (0,4) (1,5) (2,6) (3,7) of its 8-row block - "pair order".
+// Matrix-core B operands are consumed in pair order; the activation operand is put
+// in the same order (pair_order_a) so the sum over k is unchanged.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+typedef _Float16 half_t;
+typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
+typedef float f4_t __attribute__((ext_vector_type(4)));
+typedef float f16_t __attribute__((ext_vector_type(16)));
+
+union U32H2 {
+    uint32_t u;
+    h2_t h;
+};
+
+__device__ __forceinline__ h2_t as_h2(uint32_t u) {
+    U32H2 c;
+    c.u = u;
+    return c.h;
+}
+__device__ __forceinline__ uint32_t as_u32(h2_t h) {
+    U32H2 c;
+    c.h = h;
+    return c.u;
+}
+__device__ __forceinline__ h2_t splat_h2(float v) {
+    half_t x = (half_t)v;
+    h2_t r = {x, x};
+    return r;
+}
+
+// Per-column decode constants (both halves of each pair hold the same value).
+struct ColDecode {
+    h2_t neg_lo;  // -(1024 + z + 1)
+    h2_t neg_hi;  // -(64 + z + 1)
+    h2_t scale;   // s
+};
+
+__device__ __forceinline__ ColDecode make_col_decode(uint32_t stored_zero, half_t s) {
+    ColDecode c;
+    c.neg_lo = splat_h2(-(float)(1025u + stored_zero));
+    c.neg_hi = splat_h2(-(float)(65u + stored_zero));
+    h2_t sc = {s, s};
+    c.scale = sc;
+    return c;
+}
+
+// Decode one packed word into 4 fp16 pairs in pair order: out[j] = (row j, row j+4).
+__device__ __forceinline__ void decode_word(uint32_t w, const ColDecode &c, h2_t out[4]) {
+    const h2_t sixteenth = {(half_t)0.0625f, (half_t)0.0625f};
+    const uint32_t w8 = w >> 8;
+    const h2_t lo0 = as_h2((w & 0x000F000Fu) | 0x64006400u);
+    const h2_t hi0 = as_h2((w & 0x00F000F0u) | 0x64006400u);
+    const h2_t lo1 = as_h2((w8 & 0x000F000Fu) | 0x64006400u);
+    const h2_t hi1 = as_h2((w8 & 0x00F000F0u) | 0x64006400u);
+    out[0] = (lo0 + c.neg_lo) * c.scale;
+    out[1] = __builtin_elementwise_fma(hi0, sixteenth, c.neg_hi) * c.scale;
+    out[2] = (lo1 + c.neg_lo) * c.scale;
+    out[3] = __builtin_elementwise_fma(hi1, sixteenth, c.neg_hi) * c.scale;
+}
+
+__device__ __forceinline__ h8_t decode_word_h8(uint32_t w, const ColDecode &c) {
+    h2_t p[4];
+    decode_word(w, c, p);
+    h8_t r = {p[0].x, p[0].y, p[1].x, p[1].y, p[2].x, p[2].y, p[3].x, p[3].y};
+    return r;
+}
+
+// 8 consecutive activations a0..a7 (natural order, as a uint4) -> pair order
+// (a0,a4,a1,a5,a2,a6,a3,a7).
+__device__ __forceinline__ h8_t pair_order_a(uint4 v) {
+    union {
+        uint32_t u[4];
+        h8_t h;
+    } r;
+    r.u[0] = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);  // (a0, a4)
+    r.u[1] = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);  // (a1, a5)
+    r.u[2] = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);  // (a2, a6)
+    r.u[3] = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);  // (a3, a7)
+    return r.h;
+}
+
+__device__ __forceinline__ uint4 pair_order_u4(uint4 v) {
+    uint4 r;
+    r.x = __builtin_amdgcn_perm(v.z, v.x, 0x05040100u);
+    r.y = __builtin_amdgcn_perm(v.z, v.x, 0x07060302u);
+    r.z = __builtin_amdgcn_perm(v.w, v.y, 0x05040100u);
+    r.w = __builtin_amdgcn_perm(v.w, v.y, 0x07060302u);
+    return r;
+}
+
+__device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + __expf(-x)); }
+
+// Epilogue selectors shared by the small-M and the tiled kernels.
+enum { EPI_PLAIN = 0, EPI_SILU_MUL = 1, EPI_ROPE = 2 };
+
+struct RopeArgs {
+    const int32_t *position_ids;  // [B*S]
+    const float *cos_table;       // [max_pos, 64]
+    const float *sin_table;
+    half_t *q;
+    half_t *k;
+    half_t *v;
+    int S;
+    int H;
+    int kv_capacity;
+    int kv_offset;
+    int max_pos;  // rows of the tables; positions are clamped into [0, max_pos)
+};

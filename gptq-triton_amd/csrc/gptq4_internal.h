@@ -1,0 +1,44 @@
+// Host-side contracts between the C ABI (gptq4_api.hip) and the kernel launchers.
+#pragma once
+
+#include "gptq4_common.h"
+
+// One quantised projection as the kernels see it.
+struct QMat {
+    const uint32_t *qweight;  // [K/8, N]
+    const uint32_t *qzeros;   // [G, N/8]
+    const half_t *scales;     // [G, N]
+};
+
+struct MatmulArgs {
+    const half_t *x;  // [M, K]
+    QMat w[2];        // w[1] only for EPI_SILU_MUL (w[0] = gate, w[1] = up)
+    const int32_t *perm;
+    const half_t *bias;
+    half_t *y;  // [M, N] (EPI_PLAIN, EPI_SILU_MUL)
+    int M, K, N;
+    int groupsize;  // normalised: K when the caller passed -1
+    RopeArgs rope;  // EPI_ROPE only
+    float *partials;
+    int *counters;
+    int splitk;
+    int tiles;
+};
+
+// Small-M (M <= 16) split-K matrix-core GEMV.  Returns hipError_t.
+int launch_skinny(int epi, MatmulArgs a, hipStream_t stream);
+// Tiled matrix-core GEMM for any M.  Returns hipError_t.
+int launch_gemm(int epi, const MatmulArgs &a, hipStream_t stream);
+
+int launch_dequant(const uint32_t *qweight, const uint32_t *qzeros, const half_t *scales,
+                   const int32_t *g_idx, half_t *out, int K, int N, int groupsize,
+                   hipStream_t stream);
+int launch_sort_rows(const uint32_t *qweight, const int32_t *perm, uint32_t *out, int K, int N,
+                     hipStream_t stream);
+int launch_rope_table(float *cos_out, float *sin_out, int max_pos, int D, float base,
+                      hipStream_t stream);
+
+// Split-K policy shared by the launcher and the workspace-size query.
+enum { SKINNY_MAX_M = 16, SKINNY_MAX_SPLITK = 16, SKINNY_MAX_TILES = 4096 };
+int skinny_pick_splitk(int tiles, int k_batches);
+extern int g_forced_splitk;

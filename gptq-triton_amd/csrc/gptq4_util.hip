@@ -1,0 +1,104 @@
+// Format kernels: weight materialisation (bit-exact decode), act-order row sort,
+// rotary table.  None of them is on the per-token path.
+#include "gptq4_internal.h"
+
+namespace {
+
+// One thread per packed word: 8 rows of one column.  Uses the same decode_word as the
+// matmul kernels, so a bit-exact check of this kernel checks their decode too.
+__global__ __launch_bounds__(256) void gptq4_dequant_kernel(const uint32_t *__restrict__ qweight,
+                                                            const uint32_t *__restrict__ qzeros,
+                                                            const half_t *__restrict__ scales,
+                                                            const int32_t *__restrict__ g_idx,
+                                                            half_t *__restrict__ out, int K, int N,
+                                                            int groupsize) {
+    const int n = blockIdx.x * blockDim.x + threadIdx.x;
+    const int r = blockIdx.y;
+    if (n >= N) return;
+    const uint32_t w = qweight[(size_t)r * N + n];
+    const int zshift = (n & 7) * 4;
+    half_t vals[8];
+    if (g_idx == nullptr) {
+        const int g = (8 * r) / groupsize;
+        const uint32_t z = (qzeros[(size_t)g * (N >> 3) + (n >> 3)] >> zshift) & 0xFu;
+        const ColDecode c = make_col_decode(z, scales[(size_t)g * N + n]);
+        h2_t p[4];
+        decode_word(w, c, p);
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+            vals[jj] = p[jj].x;
+            vals[jj + 4] = p[jj].y;
+        }
+    } else {
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const int g = g_idx[8 * r + t];
+            const uint32_t z = (qzeros[(size_t)g * (N >> 3) + (n >> 3)] >> zshift) & 0xFu;
+            const ColDecode c = make_col_decode(z, scales[(size_t)g * N + n]);
+            h2_t p[4];
+            decode_word(w, c, p);
+            vals[t] = (t < 4) ? p[t & 3].x : p[t & 3].y;
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < 8; ++t) out[(size_t)(8 * r + t) * N + n] = vals[t];
+}
+
+// out nibble-row j = in nibble-row perm[j]
+__global__ __launch_bounds__(256) void gptq4_sort_rows_kernel(const uint32_t *__restrict__ qweight,
+                                                              const int32_t *__restrict__ perm,
+                                                              uint32_t *__restrict__ out, int K, int N) {
+    const int n = blockIdx.x * blockDim.x + threadIdx.x;
+    const int r = blockIdx.y;
+    if (n >= N) return;
+    uint32_t w = 0;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        const int src = perm[8 * r + t];
+        const uint32_t sw = qweight[(size_t)(src >> 3) * N + n];
+        w |= ((sw >> ((src & 7) * 4)) & 0xFu) << (4 * t);
+    }
+    out[(size_t)r * N + n] = w;
+}
+
+__global__ __launch_bounds__(256) void gptq4_rope_table_kernel(float *__restrict__ cos_out,
+                                                               float *__restrict__ sin_out, int max_pos,
+                                                               int half_dim, float base) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= max_pos * half_dim) return;
+    const int pos = idx / half_dim;
+    const int i = idx - pos * half_dim;
+    // inv_freq = float32 nearest to base^(-2i/D) (evaluated in double, rounded once);
+    // angle = float(pos) * inv_freq as a float32 product
+    const double expo = (double)(2 * i) / (double)(2 * half_dim);
+    const float inv_freq = (float)(1.0 / pow((double)base, expo));
+    const float theta = (float)pos * inv_freq;
+    // evaluate in double on the float32 angle: exact-to-rounding table values
+    cos_out[idx] = (float)cos((double)theta);
+    sin_out[idx] = (float)sin((double)theta);
+}
+
+}  // namespace
+
+int launch_dequant(const uint32_t *qweight, const uint32_t *qzeros, const half_t *scales,
+                   const int32_t *g_idx, half_t *out, int K, int N, int groupsize, hipStream_t stream) {
+    dim3 grid((unsigned)((N + 255) / 256), (unsigned)(K / 8)), block(256);
+    hipLaunchKernelGGL(gptq4_dequant_kernel, grid, block, 0, stream, qweight, qzeros, scales, g_idx, out, K,
+                       N, groupsize);
+    return (int)hipGetLastError();
+}
+
+int launch_sort_rows(const uint32_t *qweight, const int32_t *perm, uint32_t *out, int K, int N,
+                     hipStream_t stream) {
+    dim3 grid((unsigned)((N + 255) / 256), (unsigned)(K / 8)), block(256);
+    hipLaunchKernelGGL(gptq4_sort_rows_kernel, grid, block, 0, stream, qweight, perm, out, K, N);
+    return (int)hipGetLastError();
+}
+
+int launch_rope_table(float *cos_out, float *sin_out, int max_pos, int D, float base, hipStream_t stream) {
+    const int total = max_pos * (D / 2);
+    dim3 grid((unsigned)((total + 255) / 256)), block(256);
+    hipLaunchKernelGGL(gptq4_rope_table_kernel, grid, block, 0, stream, cos_out, sin_out, max_pos, D / 2,
+                       base);
+    return (int)hipGetLastError();
+}

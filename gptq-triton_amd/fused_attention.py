@@ -1,0 +1,228 @@
+"""Fused QKV projection + rotary embedding on the HIP kernels, and the attention module
+built on it.
+
+Mirrors src/gptq_triton/fused_attention.py of the reference: `make_quant_attn` (:10-45,
+q/k/v packed tensors concatenated along N in the order q, k, v) and
+`QuantLlamaAttention` (:48-153, same constructor, forward signature, return triple and
+ValueErrors).  Where the reference runs one matmul, a split, three view/transposes and
+the third-party rotary (:91-102), this module makes ONE call, `gptq4_qkv_rotary`, which
+writes rotated Q, rotated K and V directly in [B, H, S, D].
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import Optional, Tuple
+
+import torch
+import torch.nn as nn
+
+from . import _lib
+from .quant_linear import QuantLinear, _check_device_tensors, _check_matmul_args
+
+
+@dataclass
+class LlamaConfigLite:
+    """The fields of a LLaMA config this path reads."""
+    hidden_size: int = 4096
+    num_attention_heads: int = 32
+    max_position_embeddings: int = 2048
+    rope_theta: float = 10000.0
+    intermediate_size: int = 11008
+    num_hidden_layers: int = 32
+    vocab_size: int = 32000
+    rms_norm_eps: float = 1e-6
+
+
+class RotaryTable:
+    """cos/sin float32 [max_pos, D/2] on the device, made by gptq4_rope_table:
+    angle = float32(p) * float32(base^(-2i/D)).  Stands in for the rotary_emb module
+    the reference takes from its model (fused_attention.py:98-101)."""
+
+    def __init__(self, head_dim: int, max_pos: int = 2048, base: float = 10000.0):
+        self.head_dim, self.max_pos, self.base = head_dim, max_pos, float(base)
+        self._tables = {}
+
+    def get(self, device: torch.device, need_pos: int):
+        key = device.index if device.index is not None else torch.cuda.current_device()
+        tab = self._tables.get(key)
+        if tab is None or tab[0].shape[0] < need_pos:
+            n = max(self.max_pos, need_pos)
+            cos = torch.empty((n, self.head_dim // 2), dtype=torch.float32, device=device)
+            sin = torch.empty_like(cos)
+            rc = _lib.load().gptq4_rope_table(cos.data_ptr(), sin.data_ptr(), n, self.head_dim, self.base,
+                                              _lib.current_stream(device))
+            _lib.check(rc, "gptq4_rope_table")
+            tab = (cos, sin)
+            self._tables[key] = tab
+        return tab
+
+
+def qkv_rotary(groupsize: int, hidden_states: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor,
+               qzeros: torch.Tensor, position_ids: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
+               num_heads: int, head_dim: int = 128, perm: Optional[torch.Tensor] = None,
+               kv_out: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, kv_offset: int = 0):
+    """hidden_states fp16 [B, S, K]; packed weights with N = 3*H*D in q, k, v order.
+    Returns (q, k, v): q [B,H,S,D] rotated; k, v [B,H,S,D], or - when `kv_out` gives
+    preallocated [B,H,cap,D] buffers - those buffers with rows kv_offset..kv_offset+S
+    filled.  position_ids int [B, S] index the cos/sin tables."""
+    k_in, n = _check_matmul_args(hidden_states, qweight, groupsize)
+    _check_device_tensors(hidden_states, qweight, scales, qzeros, perm, cos, sin)
+    if hidden_states.dim() != 3:
+        raise ValueError(f"hidden_states must be [B, S, hidden], got {tuple(hidden_states.shape)}")
+    bsz, q_len, _ = hidden_states.shape
+    if n != 3 * num_heads * head_dim:
+        raise ValueError(f"packed QKV has {n} columns, expected 3*{num_heads}*{head_dim}")
+    dev = hidden_states.device
+    pos = position_ids.to(device=dev, dtype=torch.int32).expand(bsz, q_len).contiguous()
+    q = torch.empty((bsz, num_heads, q_len, head_dim), dtype=torch.float16, device=dev)
+    if kv_out is None:
+        kk = torch.empty_like(q)
+        vv = torch.empty_like(q)
+        cap, off = q_len, 0
+    else:
+        kk, vv = kv_out
+        cap, off = kk.shape[2], kv_offset
+        if kk.shape != vv.shape or kk.shape[0] != bsz or kk.shape[1] != num_heads or kk.shape[3] != head_dim \
+                or not kk.is_contiguous() or not vv.is_contiguous() or off + q_len > cap:
+            raise ValueError("kv_out buffers must be contiguous [B, H, capacity, D] with room for the new rows")
+    if bsz * q_len == 0:
+        return q, kk, vv
+    lib = _lib.load()
+    need = lib.gptq4_workspace_bytes(_lib.OP_QKV_ROTARY, bsz * q_len, k_in, n)
+    ws = _lib.workspace(dev, need)
+    rc = lib.gptq4_qkv_rotary(hidden_states.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(),
+                              _lib.ptr(perm), pos.data_ptr(), cos.data_ptr(), sin.data_ptr(), cos.shape[0],
+                              q.data_ptr(), kk.data_ptr(), vv.data_ptr(), bsz, q_len, num_heads, head_dim, k_in,
+                              groupsize, cap, off, ws.data_ptr(), ws.numel(), _lib.current_stream(dev))
+    _lib.check(rc, "gptq4_qkv_rotary")
+    return q, kk, vv
+
+
+def _fuse_qkv(q_proj: QuantLinear, k_proj: QuantLinear, v_proj: QuantLinear) -> QuantLinear:
+    gq, gk, gv = (getattr(p, 'g_idx', None) for p in (q_proj, k_proj, v_proj))
+    have = [g is not None for g in (gq, gk, gv)]
+    if any(have) and not (all(have) and torch.equal(gq.cpu(), gk.cpu()) and torch.equal(gq.cpu(), gv.cpu())):
+        raise NotImplementedError("q_proj, k_proj and v_proj must share one g_idx to be fused")
+    layer = QuantLinear(q_proj.bits, q_proj.groupsize, q_proj.infeatures,
+                        q_proj.outfeatures + k_proj.outfeatures + v_proj.outfeatures, bias=False,
+                        act_order=all(have))
+    layer.qweight = torch.cat([q_proj.qweight, k_proj.qweight, v_proj.qweight], dim=1)
+    layer.qzeros = torch.cat([q_proj.qzeros, k_proj.qzeros, v_proj.qzeros], dim=1)
+    layer.scales = torch.cat([q_proj.scales, k_proj.scales, v_proj.scales], dim=1)
+    layer.bias = None
+    if all(have):
+        layer.g_idx = gq
+    return layer
+
+
+def _is_llama_attention(m: nn.Module) -> bool:
+    if isinstance(m, QuantLlamaAttention):
+        return False
+    return all(isinstance(getattr(m, n, None), QuantLinear) for n in ('q_proj', 'k_proj', 'v_proj', 'o_proj'))
+
+
+def make_quant_attn(model: nn.Module):
+    """Replace every LLaMA attention block (q_proj/k_proj/v_proj/o_proj QuantLinears) by a
+    QuantLlamaAttention with the three projections fused (fused_attention.py:10-45)."""
+    for name, m in list(model.named_modules()):
+        if not _is_llama_attention(m):
+            continue
+        qkv = _fuse_qkv(m.q_proj, m.k_proj, m.v_proj)
+        attn = QuantLlamaAttention(m.config, qkv, m.o_proj, getattr(m, 'rotary_emb', None))
+        parent_name, _, child = name.rpartition('.')
+        parent = model.get_submodule(parent_name) if parent_name else model
+        if not name:
+            raise ValueError("the model itself is an attention block; wrap it in a parent module")
+        setattr(parent, child, attn)
+
+
+class QuantLlamaAttention(nn.Module):
+    """LLaMA self-attention with the q, k, v projections and the rotary embedding fused
+    into one kernel call.  Signature and return values follow the reference module."""
+
+    def __init__(self, config, qkv_proj: QuantLinear, o_proj: QuantLinear, rotary_emb=None):
+        super().__init__()
+        self.config = config
+        self.hidden_size = config.hidden_size
+        self.num_heads = config.num_attention_heads
+        self.head_dim = self.hidden_size // self.num_heads
+        self.max_position_embeddings = config.max_position_embeddings
+        if (self.head_dim * self.num_heads) != self.hidden_size:
+            raise ValueError(
+                f"hidden_size must be divisible by num_heads (got `hidden_size`: {self.hidden_size}"
+                f" and `num_heads`: {self.num_heads}).")
+        self.qkv_proj = qkv_proj
+        self.o_proj = o_proj
+        # kept for interface compatibility; the kernel reads its own table, which follows
+        # the same closed form (base from config.rope_theta, default 10000)
+        self.rotary_emb = rotary_emb
+        self.rope = RotaryTable(self.head_dim, self.max_position_embeddings,
+                                float(getattr(config, 'rope_theta', 10000.0)))
+
+    def project_qkv(self, hidden_states: torch.Tensor, position_ids: torch.Tensor,
+                    kv_out=None, kv_offset: int = 0):
+        need = kv_offset + hidden_states.shape[1]
+        cos, sin = self.rope.get(hidden_states.device, max(need, self.max_position_embeddings))
+        qweight, perm = self.qkv_proj.kernel_weights()
+        return qkv_rotary(self.qkv_proj.groupsize, hidden_states, qweight, self.qkv_proj.scales,
+                          self.qkv_proj.qzeros, position_ids, cos, sin, self.num_heads, self.head_dim,
+                          perm=perm, kv_out=kv_out, kv_offset=kv_offset)
+
+    def forward(
+        self,
+        hidden_states: torch.Tensor,
+        attention_mask: Optional[torch.Tensor] = None,
+        position_ids: Optional[torch.LongTensor] = None,
+        past_key_value: Optional[Tuple[torch.Tensor]] = None,
+        output_attentions: bool = False,
+        use_cache: bool = False,
+    ) -> Tuple[torch.Tensor, Optional[torch.Tensor], Optional[Tuple[torch.Tensor]]]:
+        """Input shape: Batch x Time x Channel"""
+        bsz, q_len, _ = hidden_states.size()
+        past_len = 0 if past_key_value is None else past_key_value[0].shape[-2]
+        kv_seq_len = past_len + q_len
+        if position_ids is None:
+            position_ids = torch.arange(past_len, kv_seq_len, device=hidden_states.device).unsqueeze(0)
+
+        if past_key_value is None:
+            query_states, key_states, value_states = self.project_qkv(hidden_states, position_ids)
+        else:
+            # new K/V rows are written by the kernel behind the copied past: no separate cat
+            shape = (bsz, self.num_heads, kv_seq_len, self.head_dim)
+            key_states = torch.empty(shape, dtype=torch.float16, device=hidden_states.device)
+            value_states = torch.empty(shape, dtype=torch.float16, device=hidden_states.device)
+            key_states[:, :, :past_len].copy_(past_key_value[0])
+            value_states[:, :, :past_len].copy_(past_key_value[1])
+            query_states, _, _ = self.project_qkv(hidden_states, position_ids,
+                                                  kv_out=(key_states, value_states), kv_offset=past_len)
+        past_key_value = (key_states, value_states) if use_cache else None
+
+        if attention_mask is not None and attention_mask.size() != (bsz, 1, q_len, kv_seq_len):
+            raise ValueError(
+                f"Attention mask should be of size {(bsz, 1, q_len, kv_seq_len)}, but is {attention_mask.size()}")
+
+        attn_weights = None
+        if output_attentions:
+            # explicit path, as the reference computes it (fused_attention.py:119-137)
+            attn_weights = torch.matmul(query_states, key_states.transpose(2, 3)) / math.sqrt(self.head_dim)
+            if attn_weights.size() != (bsz, self.num_heads, q_len, kv_seq_len):
+                raise ValueError(
+                    f"Attention weights should be of size {(bsz * self.num_heads, q_len, kv_seq_len)}, but is"
+                    f" {attn_weights.size()}")
+            if attention_mask is not None:
+                attn_weights = attn_weights + attention_mask
+                attn_weights = torch.clamp_min(attn_weights, torch.finfo(attn_weights.dtype).min)
+            attn_weights = nn.functional.softmax(attn_weights, dim=-1, dtype=torch.float32).to(query_states.dtype)
+            attn_output = torch.matmul(attn_weights, value_states)
+        else:
+            attn_output = nn.functional.scaled_dot_product_attention(
+                query_states, key_states, value_states, attn_mask=attention_mask)
+
+        if attn_output.size() != (bsz, self.num_heads, q_len, self.head_dim):
+            raise ValueError(
+                f"`attn_output` should be of size {(bsz, self.num_heads, q_len, self.head_dim)}, but is"
+                f" {attn_output.size()}")
+        attn_output = attn_output.transpose(1, 2).reshape(bsz, q_len, self.hidden_size)
+        attn_output = self.o_proj(attn_output)
+        return attn_output, attn_weights, past_key_value

@@ -1,0 +1,119 @@
+"""Fused LLaMA MLP on the HIP kernels: h = silu(x @ Wgate) * (x @ Wup) in one launch
+(`gptq4_mlp_gateup`), then down_proj as an ordinary QuantLinear.
+
+Mirrors src/gptq_triton/fused_mlp.py of the reference: `QuantLlamaMLP` (:52-79, note
+the constructor order gate, down, up), `make_fused_mlp` (:13-27) and the functional
+`triton_llama_mlp_4` (:241-302; kept as an alias of `llama_mlp_4`).
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+import torch.nn as nn
+
+from . import _lib
+from .quant_linear import QuantLinear, _check_device_tensors, _check_matmul_args
+
+
+def llama_mlp_4(groupsize: int, a: torch.Tensor,
+                gate_qweight: torch.Tensor, gate_scales: torch.Tensor, gate_qzeros: torch.Tensor,
+                up_qweight: torch.Tensor, up_scales: torch.Tensor, up_qzeros: torch.Tensor,
+                perm: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """silu(gate(a)) * up(a).  A (..., K) fp16; *_qweight (K//8, N) int32; *_scales (G, N)
+    fp16; *_qzeros (G, N//8) int32.  Returns (..., N) fp16.  SiLU and the product are
+    taken on the fp32 accumulators and rounded once."""
+    assert (gate_qweight.shape == up_qweight.shape and gate_scales.shape == up_scales.shape
+            and gate_qzeros.shape == up_qzeros.shape), "All weights must have the same shape"
+    k, n = _check_matmul_args(a, gate_qweight, groupsize)
+    _check_device_tensors(a, gate_qweight, gate_scales, gate_qzeros, up_qweight, up_scales, up_qzeros, perm)
+    lib = _lib.load()
+    x = a.view(-1, k)
+    m = x.shape[0]
+    c = torch.empty((m, n), device=a.device, dtype=torch.float16)
+    if m == 0:
+        return c.view(a.shape[:-1] + (n,))
+    need = lib.gptq4_workspace_bytes(_lib.OP_MLP_GATEUP, m, k, n)
+    ws = _lib.workspace(a.device, need)
+    rc = lib.gptq4_mlp_gateup(x.data_ptr(), gate_qweight.data_ptr(), gate_qzeros.data_ptr(), gate_scales.data_ptr(),
+                              up_qweight.data_ptr(), up_qzeros.data_ptr(), up_scales.data_ptr(), _lib.ptr(perm),
+                              c.data_ptr(), m, k, n, groupsize, ws.data_ptr(), ws.numel(),
+                              _lib.current_stream(a.device))
+    _lib.check(rc, "gptq4_mlp_gateup")
+    return c.view(a.shape[:-1] + (n,))
+
+
+triton_llama_mlp_4 = llama_mlp_4
+
+
+class QuantLlamaMLP(nn.Module):
+    """forward(x) = down_proj(silu(gate(x)) * up(x)).  Holds the six gate/up tensors as its
+    own buffers under the reference's names and keeps down_proj as a submodule
+    (fused_mlp.py:52-79)."""
+
+    def __init__(self, gate_proj: QuantLinear, down_proj: QuantLinear, up_proj: QuantLinear):
+        super().__init__()
+        assert gate_proj.groupsize == up_proj.groupsize
+        self.register_buffer('gate_proj_qweight', gate_proj.qweight)
+        self.register_buffer('gate_proj_scales', gate_proj.scales)
+        self.register_buffer('gate_proj_qzeros', gate_proj.qzeros)
+        self.register_buffer('up_proj_qweight', up_proj.qweight)
+        self.register_buffer('up_proj_scales', up_proj.scales)
+        self.register_buffer('up_proj_qzeros', up_proj.qzeros)
+        self.groupsize = gate_proj.groupsize
+        self.infeatures = gate_proj.infeatures
+        self.outfeatures = down_proj.outfeatures
+        self.down_proj = down_proj
+        # act-order: the gate and up rows must be sorted by ONE permutation because the
+        # kernel streams x once for both (they share their input, hence their g_idx)
+        g_gate, g_up = getattr(gate_proj, 'g_idx', None), getattr(up_proj, 'g_idx', None)
+        if (g_gate is None) != (g_up is None) or (g_gate is not None and not torch.equal(g_gate.cpu(), g_up.cpu())):
+            raise NotImplementedError("gate_proj and up_proj must share one g_idx to be fused")
+        if g_gate is not None:
+            self.register_buffer('g_idx', g_gate)
+        else:
+            self.g_idx = None
+        self._sorted = None
+
+    def _kernel_weights(self):
+        if self.g_idx is None:
+            return self.gate_proj_qweight, self.up_proj_qweight, None
+        key = (self.gate_proj_qweight.data_ptr(), self.up_proj_qweight.data_ptr(), self.g_idx.data_ptr())
+        if self._sorted is None or self._sorted[0] != key:
+            from .quant_linear import prepare_act_order
+            gq, perm = prepare_act_order(self.gate_proj_qweight, self.g_idx, self.groupsize)
+            uq, _ = prepare_act_order(self.up_proj_qweight, self.g_idx, self.groupsize)
+            self._sorted = (key, gq, uq, perm)
+        return self._sorted[1], self._sorted[2], self._sorted[3]
+
+    def gate_up(self, x: torch.Tensor) -> torch.Tensor:
+        gq, uq, perm = self._kernel_weights()
+        return llama_mlp_4(self.groupsize, x, gq, self.gate_proj_scales, self.gate_proj_qzeros,
+                           uq, self.up_proj_scales, self.up_proj_qzeros, perm)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.down_proj(self.gate_up(x))
+
+
+def _is_llama_mlp(m: nn.Module) -> bool:
+    """An MLP block with three quantised projections named as in LLaMA."""
+    if isinstance(m, QuantLlamaMLP):
+        return False
+    return all(isinstance(getattr(m, n, None), QuantLinear) for n in ('gate_proj', 'down_proj', 'up_proj'))
+
+
+def make_fused_mlp(m: nn.Module, parent_name: str = ''):
+    """Replace every LLaMA MLP block under `m` by a QuantLlamaMLP; returns `m` itself, or
+    its replacement when `m` is such a block (fused_mlp.py:13-27)."""
+    if _is_llama_mlp(m):
+        return QuantLlamaMLP(m.gate_proj, m.down_proj, m.up_proj)
+    for name, child in list(m.named_children()):
+        new = make_fused_mlp(child, parent_name=f"{parent_name}.{name}")
+        if new is not child:
+            setattr(m, name, new)
+    return m
+
+
+def autotune_warmup(model):
+    """Nothing to tune (see quant_linear.autotune_warmup); reference: fused_mlp.py:30-49."""
+    return iter(())

@@ -1,0 +1,181 @@
+"""4-bit weight-only linear layer on the HIP kernels.
+
+Mirrors the reference's operator interface for this path (src/gptq_triton/quant_linear.py):
+`QuantLinear` (:49-77), `make_quant` (:13-32), the functional `triton_matmul4`
+(:228-283; kept as an alias of `matmul4`).  Same buffer names, shapes, dtypes and the
+same host-side argument errors; the compute is `gptq4_matmul` of the C ABI.
+
+Extension the reference does not have: an optional `g_idx` buffer (act-order).  Rows are
+re-laid-out once, at first use, so each group's rows are contiguous (see
+`prepare_act_order`); the checkpoint tensors themselves are never modified.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+import torch.nn as nn
+
+from . import _lib
+
+
+def _check_matmul_args(a: torch.Tensor, qweight: torch.Tensor, groupsize: int):
+    # the reference's host-side contract (quant_linear.py:244-257)
+    assert a.shape[-1] == qweight.shape[0] * 8, "A must be a multiple of 8 in the last dimension"
+    assert a.is_contiguous(), "A must be contiguous"
+    k = a.shape[-1]
+    n = qweight.shape[1]
+    assert k % 128 == 0, "K must be a multiple of 16, 32, 64, and 128"
+    assert n % 256 == 0, "N must be a multiple of 16, 32, 64, 128, and 256"
+    assert groupsize % 128 == 0, "groupsize must be a multiple of 32, 64, and 128"
+    return k, n
+
+
+def _check_device_tensors(a, *tensors):
+    _lib.require_cuda(a, "activations")
+    if a.dtype != torch.float16:
+        raise TypeError(f"activations must be float16, got {a.dtype}")
+    for t in tensors:
+        if t is not None and t.device != a.device:
+            raise RuntimeError(f"tensor on {t.device} but activations on {a.device}")
+        if t is not None and not t.is_contiguous():
+            raise RuntimeError("quantised tensors must be contiguous")
+
+
+def matmul4(groupsize: int, a: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor,
+            qzeros: torch.Tensor, bias: Optional[torch.Tensor] = None,
+            perm: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """C = A x dequant(qweight, qzeros, scales) + bias.
+
+    A (..., K) fp16 contiguous; qweight (K//8, N) int32; scales (G, N) fp16; qzeros
+    (G, N//8) int32; bias (N) fp16.  Returns (..., N) fp16.  `groupsize` is the number
+    of input features per group (K when there is one group).  `perm` is the row
+    permutation from `prepare_act_order` (qweight must then be the sorted copy).
+    """
+    k, n = _check_matmul_args(a, qweight, groupsize)
+    _check_device_tensors(a, qweight, scales, qzeros, bias, perm)
+    lib = _lib.load()
+    x = a.view(-1, k)
+    m = x.shape[0]
+    c = torch.empty((m, n), device=a.device, dtype=torch.float16)
+    if m == 0:
+        return c.view(a.shape[:-1] + (n,))
+    need = lib.gptq4_workspace_bytes(_lib.OP_MATMUL, m, k, n)
+    ws = _lib.workspace(a.device, need)
+    rc = lib.gptq4_matmul(x.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(),
+                          _lib.ptr(perm), _lib.ptr(bias), c.data_ptr(), m, k, n, groupsize,
+                          ws.data_ptr(), ws.numel(), _lib.current_stream(a.device))
+    _lib.check(rc, "gptq4_matmul")
+    return c.view(a.shape[:-1] + (n,))
+
+
+# the reference's name for the same functional
+triton_matmul4 = matmul4
+
+
+def dequantize(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor, groupsize: int,
+               g_idx: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp16 [K, N] weight, bit-exact to fp16(float(q - (z + 1)) * float(s))."""
+    _lib.require_cuda(qweight, "qweight")
+    lib = _lib.load()
+    k, n = qweight.shape[0] * 8, qweight.shape[1]
+    out = torch.empty((k, n), device=qweight.device, dtype=torch.float16)
+    rc = lib.gptq4_dequant(qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(), _lib.ptr(g_idx),
+                           out.data_ptr(), k, n, groupsize, _lib.current_stream(qweight.device))
+    _lib.check(rc, "gptq4_dequant")
+    return out
+
+
+def prepare_act_order(qweight: torch.Tensor, g_idx: torch.Tensor, groupsize: int):
+    """Load-time re-layout for act-order checkpoints.
+
+    Returns (qweight_sorted, perm): perm = stable argsort of g_idx, qweight_sorted's
+    nibble row j is qweight's row perm[j].  Sorted row j then belongs to group
+    j // groupsize, which requires every group to own exactly `groupsize` rows (true
+    for g_idx made by permuting arange(K) // groupsize).
+    """
+    _lib.require_cuda(qweight, "qweight")
+    k, n = qweight.shape[0] * 8, qweight.shape[1]
+    gs = k if groupsize == -1 else groupsize
+    g = g_idx.to(torch.int64)
+    counts = torch.bincount(g, minlength=math.ceil(k / gs))
+    if g.numel() != k or bool((counts != gs).any()):
+        raise NotImplementedError("act-order g_idx must assign exactly `groupsize` rows to every group")
+    perm = torch.argsort(g, stable=True).to(torch.int32).contiguous()
+    out = torch.empty_like(qweight)
+    lib = _lib.load()
+    rc = lib.gptq4_actorder_sort_rows(qweight.data_ptr(), perm.data_ptr(), out.data_ptr(), k, n,
+                                      _lib.current_stream(qweight.device))
+    _lib.check(rc, "gptq4_actorder_sort_rows")
+    return out, perm
+
+
+class QuantLinear(nn.Module):
+    """Drop-in for the reference module (quant_linear.py:49-77): same constructor, buffer
+    names and shapes.  `act_order=True` additionally registers `g_idx` int32[K]."""
+
+    def __init__(self, bits: int, groupsize: int, infeatures: int, outfeatures: int, bias: bool,
+                 act_order: bool = False):
+        super().__init__()
+        if bits not in [4]:
+            raise NotImplementedError("Only 4 bits are supported.")
+        groupsize = infeatures if groupsize == -1 else groupsize
+        self.infeatures = infeatures
+        self.outfeatures = outfeatures
+        self.bits = bits
+        self.groupsize = groupsize
+        features_per_int = 32 // bits
+        assert outfeatures % features_per_int == 0, "outfeatures must be a multiple of features_per_int"
+        groups = math.ceil(infeatures / groupsize)
+        self.register_buffer('qweight', torch.empty((infeatures // features_per_int, outfeatures), dtype=torch.int32))
+        self.register_buffer('qzeros', torch.empty((groups, outfeatures // features_per_int), dtype=torch.int32))
+        self.register_buffer('scales', torch.empty((groups, outfeatures), dtype=torch.float16))
+        if bias:
+            self.register_buffer('bias', torch.empty(outfeatures, dtype=torch.float16))
+        else:
+            self.register_parameter('bias', None)
+        if act_order:
+            self.register_buffer('g_idx', (torch.arange(infeatures) // groupsize).to(torch.int32))
+        else:
+            self.g_idx = None
+        self._sorted = None  # (key, qweight_sorted, perm), built at first use
+
+    def _act_order(self):
+        key = (self.qweight.data_ptr(), self.g_idx.data_ptr(), self.qweight.device)
+        if self._sorted is None or self._sorted[0] != key:
+            qs, perm = prepare_act_order(self.qweight, self.g_idx, self.groupsize)
+            self._sorted = (key, qs, perm)
+        return self._sorted[1], self._sorted[2]
+
+    def kernel_weights(self):
+        """(qweight, perm) as the kernels consume them."""
+        if self.g_idx is None:
+            return self.qweight, None
+        return self._act_order()
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        qweight, perm = self.kernel_weights()
+        return matmul4(self.groupsize, x, qweight, self.scales, self.qzeros, self.bias, perm)
+
+    def dequantize(self) -> torch.Tensor:
+        return dequantize(self.qweight, self.qzeros, self.scales, self.groupsize, self.g_idx)
+
+
+def make_quant(model: nn.Module, bits: int, groupsize: int, act_order: bool = False):
+    """Swap every nn.Linear for a QuantLinear, except the module named exactly
+    'lm_head' (quant_linear.py:13-32)."""
+    for name, m in list(model.named_modules()):
+        if not isinstance(m, nn.Linear) or name == 'lm_head':
+            continue
+        parent_name, _, child = name.rpartition('.')
+        parent = model.get_submodule(parent_name) if parent_name else model
+        setattr(parent, child, QuantLinear(bits, groupsize, m.in_features, m.out_features,
+                                           m.bias is not None, act_order=act_order))
+
+
+def autotune_warmup(model):
+    """The reference tunes Triton configs per shape here (quant_linear.py:35-46).  The HIP
+    kernels pick their launch shape statically, so there is nothing to tune: yields no
+    warm-up work and keeps the call site valid."""
+    return iter(())

@@ -1,0 +1,130 @@
+/*
+ * gptq4.h - C ABI of the MI355X (gfx950) 4-bit GPTQ inference kernels.
+ *
+ * The reference (fpgaminer/GPTQ-triton) has no FFI: its hot path is two Triton JIT
+ * kernels launched from Python.  Each entry point below replaces one such launch
+ * site; the citation names it (paths relative to the reference checkout).
+ *
+ * Conventions
+ *  - Every pointer is a DEVICE pointer owned by the caller.  The library never
+ *    allocates or frees memory and never synchronises the device or the stream.
+ *  - Work is enqueued on `stream` (a hipStream_t passed as void*; NULL = default
+ *    stream).  Calls are stream-ordered and may be issued back to back.
+ *  - Return value: 0 on success; a negative GPTQ4_E_* code when an argument is
+ *    rejected on the host (nothing was launched); a positive value is a hipError_t
+ *    reported by the launch.  Nothing throws, nothing exits.
+ *  - Tensor layouts are the reference checkpoint layouts, row-major contiguous:
+ *      qweight int32 [K/8, N]  bits [4t,4t+4) of word (r,n) = nibble of row k=8r+t
+ *      qzeros  int32 [G, N/8]  bits [4t,4t+4) of word (g,c) = stored zero of col 8c+t
+ *      scales  fp16  [G, N]
+ *    with G = K / groupsize (groupsize == K, or -1, means one group).  A weight
+ *    decodes as  w = fp16( float(q - (z + 1)) * float(s) )  - exactly one rounding.
+ *  - `groupsize` must be -1, K, or a multiple of 128 that divides K; K % 128 == 0;
+ *    N % 256 == 0 (what the reference accepts: quant_linear.py:244-257).
+ *  - `perm` (nullable) is the act-order row permutation made by
+ *    gptq4_actorder_sort_rows(): logical weight row j multiplies x[:, perm[j]] and
+ *    belongs to group j / groupsize.
+ *  - `workspace` holds split-K partial sums and arrival counters.  Size it with
+ *    gptq4_workspace_bytes(); its first GPTQ4_WS_COUNTER_BYTES bytes must be zero
+ *    before the FIRST call that uses it (each call leaves them zero again).  One
+ *    workspace may be shared by all calls on one stream; calls that run
+ *    concurrently on different streams need a workspace each.
+ */
+#ifndef GPTQ4_H
+#define GPTQ4_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GPTQ4_ABI_VERSION 1
+
+/* host-side argument errors (returned negated: -GPTQ4_E_SHAPE ...) */
+#define GPTQ4_E_NULL 1       /* a required pointer is NULL                       */
+#define GPTQ4_E_SHAPE 2      /* K, N, M, B, S, H or D outside what is supported  */
+#define GPTQ4_E_GROUPSIZE 3  /* groupsize does not divide K / not a multiple of 128 */
+#define GPTQ4_E_WORKSPACE 4  /* workspace NULL or smaller than required          */
+#define GPTQ4_E_ALIGN 5      /* a pointer is not 16-byte aligned                 */
+
+#define GPTQ4_WS_COUNTER_BYTES 16384
+
+/* operation selector for gptq4_workspace_bytes */
+#define GPTQ4_OP_MATMUL 0
+#define GPTQ4_OP_MLP_GATEUP 1
+#define GPTQ4_OP_QKV_ROTARY 2
+
+int gptq4_abi_version(void);
+const char *gptq4_strerror(int code);
+
+/* Bytes of workspace an operation needs for M rows and N output columns
+ * (N = I for MLP_GATEUP, N = 3*H*D for QKV_ROTARY).  No reference counterpart: the
+ * Triton kernels own a whole K loop per output tile; split-K across workgroups is
+ * what fills 256 CUs on GEMV-sized problems. */
+size_t gptq4_workspace_bytes(int op, int M, int K, int N);
+
+/* W_out fp16 [K, N] = dequantised weight, bit-exact to the formula above.
+ * Replaces the in-kernel decode of matmul4_kernel (quant_linear.py:177-188,211-212)
+ * as a stand-alone materialisation; g_idx (nullable) is int32 [K], the group of each
+ * row in the ORIGINAL checkpoint row order (quantize.py:253 is the default). */
+int gptq4_dequant(const int32_t *qweight, const int32_t *qzeros, const void *scales,
+                  const int32_t *g_idx, void *W_out, int K, int N, int groupsize,
+                  void *stream);
+
+/* Load-time act-order re-layout: qweight_out row j = qweight row perm[j] (nibble rows,
+ * K of them).  With perm = stable argsort(g_idx) the rows of each group become
+ * contiguous so the matmul kernels can index groups as j / groupsize.  The reference
+ * has no act-order kernel path (quantize.py:41-42 rejects act-order with groups). */
+int gptq4_actorder_sort_rows(const int32_t *qweight, const int32_t *perm,
+                             int32_t *qweight_out, int K, int N, void *stream);
+
+/* y fp16 [M, N] = x fp16 [M, K] @ dequant(qweight, qzeros, scales) (+ bias fp16 [N]).
+ * fp16 operands, fp32 accumulation, one rounding to fp16, then an fp16 bias add.
+ * Replaces triton_matmul4 / matmul4_kernel (quant_linear.py:125-283). */
+int gptq4_matmul(const void *x, const int32_t *qweight, const int32_t *qzeros,
+                 const void *scales, const int32_t *perm, const void *bias, void *y,
+                 int M, int K, int N, int groupsize, void *workspace,
+                 size_t workspace_bytes, void *stream);
+
+/* h fp16 [M, I] = silu(x @ Wgate) * (x @ Wup); SiLU and the product are taken on the
+ * fp32 accumulators, one rounding to fp16.
+ * Replaces triton_llama_mlp_4 / llama_mlp_fused_4_kernel (fused_mlp.py:109-302). */
+int gptq4_mlp_gateup(const void *x, const int32_t *gate_qweight, const int32_t *gate_qzeros,
+                     const void *gate_scales, const int32_t *up_qweight,
+                     const int32_t *up_qzeros, const void *up_scales, const int32_t *perm,
+                     void *h, int M, int K, int I, int groupsize, void *workspace,
+                     size_t workspace_bytes, void *stream);
+
+/* cos, sin float32 [max_pos, D/2]:  angle = float(p) * (1 / base^(2i/D)).
+ * Stands in for the rotary_emb module the reference receives from its model
+ * (fused_attention.py:98-101). */
+int gptq4_rope_table(float *cos_out, float *sin_out, int max_pos, int D, float base,
+                     void *stream);
+
+/* Fused QKV projection + rotary embedding.  x fp16 [B*S, K]; packed weights have
+ * N = 3*H*D columns in the order q, k, v.  position_ids int32 [B*S] index the
+ * cos/sin tables ([max_pos, D/2] float32).  Outputs (fp16):
+ *   q [B, H, S, D]                      rotated
+ *   k [B, H, kv_capacity, D] rows kv_offset + s, rotated
+ *   v [B, H, kv_capacity, D] rows kv_offset + s, as projected
+ * kv_capacity = S and kv_offset = 0 give the reference's three [B,H,S,D] tensors;
+ * other values write straight into a preallocated KV cache.
+ * Replaces qkv_proj + split + view/transpose + apply_rotary_pos_emb
+ * (fused_attention.py:91-102).  D must be 128. */
+int gptq4_qkv_rotary(const void *x, const int32_t *qweight, const int32_t *qzeros,
+                     const void *scales, const int32_t *perm, const int32_t *position_ids,
+                     const float *cos_table, const float *sin_table, int max_pos,
+                     void *q, void *k, void *v, int B, int S, int H, int D, int K,
+                     int groupsize, int kv_capacity, int kv_offset, void *workspace,
+                     size_t workspace_bytes, void *stream);
+
+/* Host-side launch tuning for measurements: split-K factor of the small-M kernels
+ * (0 = automatic).  Process-wide; not thread-safe against concurrent launches. */
+void gptq4_set_splitk(int splitk);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GPTQ4_H */
