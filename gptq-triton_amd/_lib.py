@@ -27,7 +27,7 @@ SIGNATURES = {
     "gptq4_mlp_gateup": (c_int, [c_void_p] * 9 + [c_int] * 4 + [c_void_p, c_size_t, c_void_p]),
     "gptq4_rope_table": (c_int, [c_void_p, c_void_p, c_int, c_int, c_float, c_void_p]),
     "gptq4_qkv_rotary": (c_int, [c_void_p] * 8 + [c_int] + [c_void_p] * 3 + [c_int] * 8 + [c_void_p, c_size_t, c_void_p]),
-    "gptq4_set_splitk": (None, [c_int]),
+    "gptq4_set_tuning": (None, [c_int, c_int, c_int]),
 }
 
 

@@ -23,15 +23,18 @@ size_t partial_bytes(int splitk, int M, int ncols_total) {
     return (size_t)splitk * (size_t)M * (size_t)ncols_total * sizeof(float);
 }
 
-// Fill the split-K fields of `a`; `ncols_total` = columns summed over all tiles
-// (N, or 2*I for the gate/up pair).
-int setup_skinny(MatmulArgs &a, int tile_cols, int ncols_total, void *workspace, size_t workspace_bytes) {
-    a.tiles = a.N / tile_cols;
+// Fill the split-K fields of `a` from the launch plan; `nmat` = matrices summed per
+// tile (2 for the gate/up pair).
+int setup_skinny(MatmulArgs &a, const SkinnyPlan &pl, int nmat, void *workspace, size_t workspace_bytes) {
+    a.tiles = pl.tiles;
+    a.splitk = pl.splitk;
+    const int nbatches = a.K / 128, slots = pl.splitk * 4;
+    a.slot_q = nbatches / slots;
+    a.slot_rem = nbatches % slots;
+    a.batches_per_group = a.groupsize / 128;
     if (a.tiles > SKINNY_MAX_TILES) return -GPTQ4_E_SHAPE;
-    a.splitk = skinny_pick_splitk(a.tiles, a.K / 128);
     if (workspace == nullptr || workspace_bytes < GPTQ4_WS_COUNTER_BYTES) return -GPTQ4_E_WORKSPACE;
-    if (a.splitk > 1 &&
-        workspace_bytes < GPTQ4_WS_COUNTER_BYTES + partial_bytes(a.splitk, a.M, ncols_total))
+    if (a.splitk > 1 && workspace_bytes < GPTQ4_WS_COUNTER_BYTES + partial_bytes(a.splitk, a.M, nmat * a.N))
         return -GPTQ4_E_WORKSPACE;
     a.counters = reinterpret_cast<int *>(workspace);
     a.partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_COUNTER_BYTES);
@@ -63,7 +66,11 @@ const char *gptq4_strerror(int code) {
     }
 }
 
-void gptq4_set_splitk(int splitk) { g_forced_splitk = splitk < 0 ? 0 : splitk; }
+void gptq4_set_tuning(int words, int depth, int splitk) {
+    g_skinny_tuning.words = (words == 1 || words == 2 || words == 4) ? words : 0;
+    g_skinny_tuning.depth = (depth >= 1 && depth <= 4) ? depth : 0;
+    g_skinny_tuning.splitk = splitk > 0 ? splitk : 0;
+}
 
 size_t gptq4_workspace_bytes(int op, int M, int K, int N) {
     (void)K;
@@ -117,9 +124,10 @@ int gptq4_matmul(const void *x, const int32_t *qweight, const int32_t *qzeros, c
     a.groupsize = groupsize;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     if (M <= SKINNY_MAX_M) {
-        rc = setup_skinny(a, 64, N, workspace, workspace_bytes);
+        const SkinnyPlan pl = skinny_plan(EPI_PLAIN, N, K);
+        rc = setup_skinny(a, pl, 1, workspace, workspace_bytes);
         if (rc) return rc;
-        return launch_skinny(EPI_PLAIN, a, s);
+        return launch_skinny(EPI_PLAIN, a, pl, s);
     }
     return launch_gemm(EPI_PLAIN, a, s);
 }
@@ -150,9 +158,10 @@ int gptq4_mlp_gateup(const void *x, const int32_t *gate_qweight, const int32_t *
     a.groupsize = groupsize;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     if (M <= SKINNY_MAX_M) {
-        rc = setup_skinny(a, 64, 2 * I, workspace, workspace_bytes);
+        const SkinnyPlan pl = skinny_plan(EPI_SILU_MUL, I, K);
+        rc = setup_skinny(a, pl, 2, workspace, workspace_bytes);
         if (rc) return rc;
-        return launch_skinny(EPI_SILU_MUL, a, s);
+        return launch_skinny(EPI_SILU_MUL, a, pl, s);
     }
     return launch_gemm(EPI_SILU_MUL, a, s);
 }
@@ -201,9 +210,10 @@ int gptq4_qkv_rotary(const void *x, const int32_t *qweight, const int32_t *qzero
     a.rope.max_pos = max_pos;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     if (a.M <= SKINNY_MAX_M) {
-        rc = setup_skinny(a, 128, N, workspace, workspace_bytes);
+        const SkinnyPlan pl = skinny_plan(EPI_ROPE, N, K);
+        rc = setup_skinny(a, pl, 1, workspace, workspace_bytes);
         if (rc) return rc;
-        return launch_skinny(EPI_ROPE, a, s);
+        return launch_skinny(EPI_ROPE, a, pl, s);
     }
     return launch_gemm(EPI_ROPE, a, s);
 }

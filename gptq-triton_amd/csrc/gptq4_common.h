@@ -21,26 +21,8 @@ typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
 typedef float f4_t __attribute__((ext_vector_type(4)));
 typedef float f16_t __attribute__((ext_vector_type(16)));
 
-union U32H2 {
-    uint32_t u;
-    h2_t h;
-};
-
-__device__ __forceinline__ h2_t as_h2(uint32_t u) {
-    U32H2 c;
-    c.u = u;
-    return c.h;
-}
-__device__ __forceinline__ uint32_t as_u32(h2_t h) {
-    U32H2 c;
-    c.h = h;
-    return c.u;
-}
-__device__ __forceinline__ h2_t splat_h2(float v) {
-    half_t x = (half_t)v;
-    h2_t r = {x, x};
-    return r;
-}
+__device__ __forceinline__ h2_t as_h2(uint32_t u) { return __builtin_bit_cast(h2_t, u); }
+__device__ __forceinline__ uint32_t as_u32(h2_t h) { return __builtin_bit_cast(uint32_t, h); }
 
 // Per-column decode constants (both halves of each pair hold the same value).
 struct ColDecode {
@@ -49,23 +31,36 @@ struct ColDecode {
     h2_t scale;   // s
 };
 
-__device__ __forceinline__ ColDecode make_col_decode(uint32_t stored_zero, half_t s) {
+// Built with integer ops only.  fp16 bit patterns: for v in [1024, 2048) the pattern
+// is 0x6400 + (v - 1024), so -(1025 + z) is 0xE401 + z; for v in [64, 128) it is
+// 0x5400 + 16 * (v - 64), so -(65 + z) is 0xD410 + 16 * z.  `scale_bits` holds the
+// fp16 scale in its low 16 bits.
+__device__ __forceinline__ ColDecode make_col_decode(uint32_t stored_zero, uint32_t scale_bits) {
     ColDecode c;
-    c.neg_lo = splat_h2(-(float)(1025u + stored_zero));
-    c.neg_hi = splat_h2(-(float)(65u + stored_zero));
-    h2_t sc = {s, s};
-    c.scale = sc;
+    c.neg_lo = as_h2((0xE401u + stored_zero) * 0x10001u);
+    c.neg_hi = as_h2((0xD410u + (stored_zero << 4)) * 0x10001u);
+    c.scale = as_h2((scale_bits & 0xFFFFu) * 0x10001u);
     return c;
+}
+
+// (a & mask) | orv in one VALU op.  v_and_or_b32 is VOP3 and gfx950 lets a VOP3 read a
+// single scalar operand and no literal, so the mask travels in an SGPR and the fp16
+// magic 0x64006400 in a VGPR; written as asm because the compiler emits v_and + v_or.
+__device__ __forceinline__ uint32_t and_or_b32(uint32_t a, uint32_t mask, uint32_t orv) {
+    uint32_t r;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "s"(mask), "v"(orv));
+    return r;
 }
 
 // Decode one packed word into 4 fp16 pairs in pair order: out[j] = (row j, row j+4).
 __device__ __forceinline__ void decode_word(uint32_t w, const ColDecode &c, h2_t out[4]) {
     const h2_t sixteenth = {(half_t)0.0625f, (half_t)0.0625f};
+    const uint32_t magic = 0x64006400u;
     const uint32_t w8 = w >> 8;
-    const h2_t lo0 = as_h2((w & 0x000F000Fu) | 0x64006400u);
-    const h2_t hi0 = as_h2((w & 0x00F000F0u) | 0x64006400u);
-    const h2_t lo1 = as_h2((w8 & 0x000F000Fu) | 0x64006400u);
-    const h2_t hi1 = as_h2((w8 & 0x00F000F0u) | 0x64006400u);
+    const h2_t lo0 = as_h2(and_or_b32(w, 0x000F000Fu, magic));
+    const h2_t hi0 = as_h2(and_or_b32(w, 0x00F000F0u, magic));
+    const h2_t lo1 = as_h2(and_or_b32(w8, 0x000F000Fu, magic));
+    const h2_t hi1 = as_h2(and_or_b32(w8, 0x00F000F0u, magic));
     out[0] = (lo0 + c.neg_lo) * c.scale;
     out[1] = __builtin_elementwise_fma(hi0, sixteenth, c.neg_hi) * c.scale;
     out[2] = (lo1 + c.neg_lo) * c.scale;

@@ -32,7 +32,7 @@ __global__ __launch_bounds__(256) void gptq4_gemm_kernel(MatmulArgs p) {
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave & 1;
     const int wn = wave >> 1;
     const int l32 = lane & 31;
@@ -132,11 +132,10 @@ __global__ __launch_bounds__(256) void gptq4_gemm_kernel(MatmulArgs p) {
         if (g != grp_decoded) {
             grp_decoded = g;
             const uint32_t z4 = raw_z >> ((l32 & 1) * 16);
-            const h2_t s01 = as_h2(raw_s.x), s23 = as_h2(raw_s.y);
-            cd[0] = make_col_decode(z4 & 0xFu, s01.x);
-            cd[1] = make_col_decode((z4 >> 4) & 0xFu, s01.y);
-            cd[2] = make_col_decode((z4 >> 8) & 0xFu, s23.x);
-            cd[3] = make_col_decode((z4 >> 12) & 0xFu, s23.y);
+            cd[0] = make_col_decode(z4 & 0xFu, raw_s.x);
+            cd[1] = make_col_decode((z4 >> 4) & 0xFu, raw_s.x >> 16);
+            cd[2] = make_col_decode((z4 >> 8) & 0xFu, raw_s.y);
+            cd[3] = make_col_decode((z4 >> 12) & 0xFu, raw_s.y >> 16);
         }
         __syncthreads();
         if (kt + 1 < nk) {

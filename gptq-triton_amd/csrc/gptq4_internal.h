@@ -13,20 +13,36 @@ struct QMat {
 struct MatmulArgs {
     const half_t *x;  // [M, K]
     QMat w[2];        // w[1] only for EPI_SILU_MUL (w[0] = gate, w[1] = up)
-    const int32_t *perm;
-    const half_t *bias;
-    half_t *y;  // [M, N] (EPI_PLAIN, EPI_SILU_MUL)
-    int M, K, N;
-    int groupsize;  // normalised: K when the caller passed -1
-    RopeArgs rope;  // EPI_ROPE only
     float *partials;
     int *counters;
+    half_t *y;  // [M, N] (EPI_PLAIN, EPI_SILU_MUL)
+    const half_t *bias;
+    const int32_t *perm;
+    int M, K, N;
+    int groupsize;  // normalised: K when the caller passed -1
     int splitk;
     int tiles;
+    // small-M kernel: K batches (128 k each) dealt to splitk * 4 wave slots - slot i
+    // gets slot_q batches, the first slot_rem slots one more
+    int slot_q, slot_rem;
+    int batches_per_group;  // groupsize / 128
+    RopeArgs rope;          // EPI_ROPE only
 };
 
+// Launch shape of the small-M kernel.
+struct SkinnyPlan {
+    int words;   // packed words per lane and load: strip width = 16 * words columns
+    int depth;   // batches of loads kept in flight per wave
+    int splitk;  // workgroups sharing one tile
+    int tiles;
+};
+struct SkinnyTuning {
+    int words, depth, splitk;  // 0 = automatic
+};
+extern SkinnyTuning g_skinny_tuning;
+SkinnyPlan skinny_plan(int epi, int N, int K);
 // Small-M (M <= 16) split-K matrix-core GEMV.  Returns hipError_t.
-int launch_skinny(int epi, MatmulArgs a, hipStream_t stream);
+int launch_skinny(int epi, const MatmulArgs &a, const SkinnyPlan &plan, hipStream_t stream);
 // Tiled matrix-core GEMM for any M.  Returns hipError_t.
 int launch_gemm(int epi, const MatmulArgs &a, hipStream_t stream);
 
@@ -38,7 +54,4 @@ int launch_sort_rows(const uint32_t *qweight, const int32_t *perm, uint32_t *out
 int launch_rope_table(float *cos_out, float *sin_out, int max_pos, int D, float base,
                       hipStream_t stream);
 
-// Split-K policy shared by the launcher and the workspace-size query.
 enum { SKINNY_MAX_M = 16, SKINNY_MAX_SPLITK = 16, SKINNY_MAX_TILES = 4096 };
-int skinny_pick_splitk(int tiles, int k_batches);
-extern int g_forced_splitk;

@@ -1,69 +1,118 @@
 // Small-M (1..16 rows) dequant-fused matmul for gfx950: the decode GEMV / skinny GEMM.
 //
-// Memory-bound by design: the packed weights are streamed from HBM exactly once with
-// 128-bit loads, decoded in registers and fed to v_mfma_f32_16x16x32_f16 (the 16-row
-// matrix-core tile holds all of x even at M = 16; at M = 1 the unused rows cost
-// nothing because the matrix pipe is otherwise idle and the decode, not the MFMA, is
-// the VALU work).
+// Memory-bound by design: the packed weights are streamed from HBM exactly once,
+// decoded in registers and fed to v_mfma_f32_16x16x32_f16 (the 16-row matrix-core tile
+// holds all of x even at M = 16; at M = 1 the unused rows cost nothing because the
+// matrix pipe is otherwise idle - the decode is the VALU work either way).
 //
 // Work decomposition
-//   strip  = 64 output columns.  A wave-wide 128-bit load covers 4 qweight rows
-//            (= 32 values of k, one MFMA K step) x 64 columns: lane l reads row
-//            l/16 and columns 4*(l%16) .. +3.  Word t of the lane is the complete B
-//            operand of MFMA t, whose 16 columns are {4j + t}: no transposition
-//            between the checkpoint layout and the matrix-core register layout.
-//   batch  = 128 values of k (4 K steps): the unit of K distribution.
-//   tile   = the strips one workgroup owns: 1 strip (plain), the same strip of the
-//            gate and up matrices (SiLU*mul), or the 2 strips of one 128-wide head
-//            (rotary: column d and its partner d + 64 meet in one workgroup).
-//   The 4 waves of a workgroup take disjoint contiguous batch ranges and are summed
-//   through LDS; `splitk` workgroups share a tile and are summed, in fixed order, by
-//   the workgroup that arrives last (arrival counter in global memory), which also
-//   runs the epilogue.  Results are therefore deterministic.
-//   blockIdx -> (tile, split) keeps all splits of a tile on one XCD (blockIdx % 8),
-//   so the partial sums it re-reads are in that XCD's L2.
+//   K step = 32 values of k = 4 qweight rows.  Lane l of a wave reads row l/16 and
+//            W adjacent columns W*(l%16) .. +W-1 (W = 1, 2 or 4 words = 4/8/16-byte
+//            loads).  Word t of the lane is the complete B operand of MFMA t, whose
+//            16 columns are {W*j + t}: no transposition between the checkpoint layout
+//            and the matrix-core register layout.
+//   strip  = 16*W output columns.
+//   batch  = 128 values of k (4 K steps): the unit of K distribution; a quantisation
+//            group is a whole number of batches.
+//   tile   = what one workgroup owns: 1 strip (plain), the same strip of the gate and
+//            of the up matrix (SiLU*mul), or a strip of head columns d and the strip
+//            d + 64 of the same head (rotary: partners meet in one workgroup).
+//   The 4 waves of a workgroup take disjoint contiguous batch ranges, keep DEPTH
+//   batches of loads in flight, and are summed through LDS.  With splitk > 1, that many
+//   workgroups share a tile; each publishes its partial sums and the one that arrives
+//   last (arrival counter) adds them in fixed order and runs the epilogue, so results
+//   are deterministic.
+//   blockIdx -> (tile, split): all splits of a tile, and tiles that share a 128-byte
+//   line of a qweight row, land on one XCD (blockIdx % 8) and hence one L2.
 #include "gptq4_internal.h"
+
+// Development aid, compiled out of the product build: per-workgroup cycle stamps at
+// the phase boundaries of the kernel, written 32 MiB into the workspace (size it so).
+#ifdef GPTQ4_PHASE_TIMERS
+#define PHASE_STAMP(i)                                                                     \
+    do {                                                                                   \
+        if (threadIdx.x == 0)                                                              \
+            reinterpret_cast<unsigned long long *>(reinterpret_cast<char *>(p.counters) + (32 << 20))[blockIdx.x * 8 + (i)] = \
+                __builtin_readcyclecounter();                                              \
+    } while (0)
+#else
+#define PHASE_STAMP(i)
+#endif
 
 namespace {
 
-template <int NV>
+template <int W>
+struct WordVec;
+template <>
+struct WordVec<1> {
+    typedef uint32_t type;
+};
+template <>
+struct WordVec<2> {
+    typedef uint2 type;
+};
+template <>
+struct WordVec<4> {
+    typedef uint4 type;
+};
+
+__device__ __forceinline__ uint32_t word_of(uint32_t v, int) { return v; }
+__device__ __forceinline__ uint32_t word_of(uint2 v, int t) { return t == 0 ? v.x : v.y; }
+__device__ __forceinline__ uint32_t word_of(uint4 v, int t) { return t == 0 ? v.x : (t == 1 ? v.y : (t == 2 ? v.z : v.w)); }
+
+template <int NV, int W>
 struct Batch {
-    uint4 w[NV][4];   // packed weights: [loaded strip][K step]
-    uint4 a[4];       // activations for row lane%16, natural k order, per K step
-    uint2 raw_s[NV];  // 4 fp16 scales of the lane's columns
+    typename WordVec<W>::type w[NV][4];  // packed weights: [loaded strip][K step]
+    uint4 a[4];                          // activations of row lane%16, natural k order, per K step
+    uint2 raw_s[NV];                     // W fp16 scales of the lane's columns (low halves first)
     uint32_t raw_z[NV];
     int group;
 };
 
-template <int EPI>
+template <int EPI, int W, int DEPTH, bool PERM>
 __global__ __launch_bounds__(256) void gptq4_skinny_kernel(MatmulArgs p) {
-    constexpr int NV = (EPI == EPI_PLAIN) ? 1 : 2;       // strips loaded per K step
-    constexpr int NSTRIP = (EPI == EPI_ROPE) ? 2 : 1;    // distinct column strips per tile
-    constexpr int TILE_COLS = 64 * NV;                    // columns of the LDS tile
+    constexpr int NV = (EPI == EPI_PLAIN) ? 1 : 2;  // strips loaded per K step
+    constexpr int SW = 16 * W;                      // strip width in columns
+    constexpr int TILE_COLS = SW * NV;              // columns of the LDS tile
+    constexpr int Q = SW / 16;                      // output elements per thread and row block
+    constexpr int LINE_TILES = (SW >= 32) ? 1 : 32 / SW;  // tiles sharing a 128-byte row segment
 
     __shared__ float red[4][SKINNY_MAX_M][TILE_COLS];
     __shared__ int s_is_last;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    // the wave index is uniform: keep it (and everything derived from it - batch range,
+    // group index, row base addresses) in scalar registers
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lrow = lane >> 4;  // k-block inside a K step; also output row group
     const int lcol = lane & 15;
 
+    // grid: x = 8 * (tiles per XCD, rounded up), y = split.  grid.x is a multiple of 8,
+    // so blockIdx.x % 8 is the XCD for every y.  No runtime divisions here: the host
+    // precomputes how the K batches are dealt to the splitk * 4 wave slots.
     const int xcd = blockIdx.x & 7;
     const int j = blockIdx.x >> 3;
-    const int split = j % p.splitk;
-    const int tile = (j / p.splitk) * 8 + xcd;
+    const int split = blockIdx.y;
+    const int sub = j % LINE_TILES;
+    const int tile = ((j / LINE_TILES) * 8 + xcd) * LINE_TILES + sub;
     if (tile >= p.tiles) return;
 
+    PHASE_STAMP(0);
     const int M = p.M, K = p.K, N = p.N;
-    const int nbatches = K >> 7;
-    const int slots = p.splitk * 4;
     const int slot = split * 4 + wave;
-    const int b0 = (int)(((long)slot * nbatches) / slots);
-    const int b1 = (int)(((long)(slot + 1) * nbatches) / slots);
-    const int n0 = tile * 64 * NSTRIP;
-    const int gs = p.groupsize;
+    const int b0 = slot * p.slot_q + min(slot, p.slot_rem);
+    const int b1 = b0 + p.slot_q + (slot < p.slot_rem ? 1 : 0);
+    const int bpg = p.batches_per_group;
+
+    // first column of the tile's strip(s)
+    int n0;
+    if (EPI == EPI_ROPE) {
+        constexpr int per_head = 64 / SW;
+        n0 = (tile / per_head) * 128 + (tile % per_head) * SW;
+    } else {
+        n0 = tile * SW;
+    }
 
     const uint32_t *qw[NV];
     const uint32_t *qz[NV];
@@ -72,71 +121,85 @@ __global__ __launch_bounds__(256) void gptq4_skinny_kernel(MatmulArgs p) {
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
         const int m = (EPI == EPI_SILU_MUL) ? v : 0;
-        ncol[v] = n0 + ((EPI == EPI_ROPE) ? 64 * v : 0) + 4 * lcol;
+        ncol[v] = n0 + ((EPI == EPI_ROPE) ? 64 * v : 0) + W * lcol;
         qw[v] = p.w[m].qweight + ncol[v];
         qz[v] = p.w[m].qzeros;
         sc[v] = p.w[m].scales;
     }
 
-    f4_t acc[NV][4];
+    // Lanes of rows >= M read row M-1 instead of branching: A row m only feeds output row
+    // m, and output rows >= M are never stored.
+    const half_t *xrow = p.x + (size_t)(lcol < M ? lcol : M - 1) * K;
+
+    f4_t acc[NV][W];
 #pragma unroll
     for (int v = 0; v < NV; ++v)
 #pragma unroll
-        for (int t = 0; t < 4; ++t) acc[v][t] = (f4_t){0.f, 0.f, 0.f, 0.f};
+        for (int t = 0; t < W; ++t) acc[v][t] = (f4_t){0.f, 0.f, 0.f, 0.f};
 
-    ColDecode cd[NV][4];
+    ColDecode cd[NV][W];
     int cur_group = -1;
+    // group of the next batch to be loaded (loads are issued in increasing batch order)
+    int ld_group = (bpg >= (K >> 7)) ? 0 : b0 / bpg;
+    int ld_left = (bpg >= (K >> 7)) ? 0x7fffffff : bpg - (b0 - ld_group * bpg);
 
-    auto load_batch = [&](Batch<NV> &B, int b, int prev_group) {
+    typedef typename WordVec<W>::type wvec_t;
+    typedef Batch<NV, W> batch_t;
+
+    auto load_batch = [&](batch_t &B, int b) {
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             const uint32_t *base = qw[v] + (size_t)(b * 16 + lrow) * N;
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                B.w[v][i] = *reinterpret_cast<const uint4 *>(base + (size_t)(4 * i) * N);
+            for (int i = 0; i < 4; ++i) B.w[v][i] = *reinterpret_cast<const wvec_t *>(base + (size_t)(4 * i) * N);
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int k = b * 128 + 32 * i + 8 * lrow;
-            uint4 a = make_uint4(0u, 0u, 0u, 0u);
-            if (lcol < M) {
-                const half_t *xr = p.x + (size_t)lcol * K;
-                if (p.perm == nullptr) {
-                    a = *reinterpret_cast<const uint4 *>(xr + k);
-                } else {
-                    const int4 i0 = *reinterpret_cast<const int4 *>(p.perm + k);
-                    const int4 i1 = *reinterpret_cast<const int4 *>(p.perm + k + 4);
-                    const uint16_t *xs = reinterpret_cast<const uint16_t *>(xr);
-                    a.x = (uint32_t)xs[i0.x] | ((uint32_t)xs[i0.y] << 16);
-                    a.y = (uint32_t)xs[i0.z] | ((uint32_t)xs[i0.w] << 16);
-                    a.z = (uint32_t)xs[i1.x] | ((uint32_t)xs[i1.y] << 16);
-                    a.w = (uint32_t)xs[i1.z] | ((uint32_t)xs[i1.w] << 16);
-                }
+            uint4 a;
+            if (!PERM) {
+                a = *reinterpret_cast<const uint4 *>(xrow + k);
+            } else {
+                const int4 i0 = *reinterpret_cast<const int4 *>(p.perm + k);
+                const int4 i1 = *reinterpret_cast<const int4 *>(p.perm + k + 4);
+                const uint16_t *xs = reinterpret_cast<const uint16_t *>(xrow);
+                a.x = (uint32_t)xs[i0.x] | ((uint32_t)xs[i0.y] << 16);
+                a.y = (uint32_t)xs[i0.z] | ((uint32_t)xs[i0.w] << 16);
+                a.z = (uint32_t)xs[i1.x] | ((uint32_t)xs[i1.y] << 16);
+                a.w = (uint32_t)xs[i1.z] | ((uint32_t)xs[i1.w] << 16);
             }
             B.a[i] = a;
         }
-        B.group = (b * 128) / gs;
-        if (B.group != prev_group) {
+        B.group = ld_group;
+        if (--ld_left == 0) {
+            ld_left = bpg;
+            ++ld_group;
+        }
 #pragma unroll
-            for (int v = 0; v < NV; ++v) {
-                B.raw_s[v] = *reinterpret_cast<const uint2 *>(sc[v] + (size_t)B.group * N + ncol[v]);
-                B.raw_z[v] = qz[v][(size_t)B.group * (N >> 3) + (ncol[v] >> 3)];
-            }
+        for (int v = 0; v < NV; ++v) {
+            const half_t *sp = sc[v] + (size_t)B.group * N + ncol[v];
+            if (W == 1)
+                B.raw_s[v] = make_uint2(*reinterpret_cast<const uint16_t *>(sp), 0u);
+            else if (W == 2)
+                B.raw_s[v] = make_uint2(*reinterpret_cast<const uint32_t *>(sp), 0u);
+            else
+                B.raw_s[v] = *reinterpret_cast<const uint2 *>(sp);
+            B.raw_z[v] = qz[v][(size_t)B.group * (N >> 3) + (ncol[v] >> 3)];
         }
     };
 
-    auto compute_batch = [&](const Batch<NV> &B) {
+    auto compute_batch = [&](const batch_t &B) {
         if (B.group != cur_group) {
             cur_group = B.group;
 #pragma unroll
             for (int v = 0; v < NV; ++v) {
-                // the lane's 4 columns are nibbles (4*lcol % 8) .. +3 of the zero word
-                const uint32_t z4 = B.raw_z[v] >> ((lcol & 1) * 16);
-                const h2_t s01 = as_h2(B.raw_s[v].x), s23 = as_h2(B.raw_s[v].y);
-                cd[v][0] = make_col_decode(z4 & 0xFu, s01.x);
-                cd[v][1] = make_col_decode((z4 >> 4) & 0xFu, s01.y);
-                cd[v][2] = make_col_decode((z4 >> 8) & 0xFu, s23.x);
-                cd[v][3] = make_col_decode((z4 >> 12) & 0xFu, s23.y);
+                // the lane's W columns are nibbles (ncol % 8) .. +W-1 of the zero word
+                const uint32_t zs = B.raw_z[v] >> (((W * lcol) & 7) * 4);
+#pragma unroll
+                for (int t = 0; t < W; ++t) {
+                    const uint32_t sw = (t >> 1) ? B.raw_s[v].y : B.raw_s[v].x;
+                    cd[v][t] = make_col_decode((zs >> (4 * t)) & 0xFu, sw >> (16 * (t & 1)));
+                }
             }
         }
 #pragma unroll
@@ -144,99 +207,128 @@ __global__ __launch_bounds__(256) void gptq4_skinny_kernel(MatmulArgs p) {
             const h8_t a = pair_order_a(B.a[i]);
 #pragma unroll
             for (int v = 0; v < NV; ++v) {
-                const uint32_t ww[4] = {B.w[v][i].x, B.w[v][i].y, B.w[v][i].z, B.w[v][i].w};
 #pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    const h8_t bf = decode_word_h8(ww[t], cd[v][t]);
+                for (int t = 0; t < W; ++t) {
+                    const h8_t bf = decode_word_h8(word_of(B.w[v][i], t), cd[v][t]);
                     acc[v][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, bf, acc[v][t], 0, 0, 0);
                 }
             }
         }
     };
 
-    if (b0 < b1) {
-        Batch<NV> cur, nxt;
-        load_batch(cur, b0, -1);
-        for (int b = b0; b < b1; ++b) {
-            if (b + 1 < b1) load_batch(nxt, b + 1, cur.group);
-            compute_batch(cur);
-            if (b + 1 < b1) {
-                // when the group did not change, the decode constants stay valid and
-                // nxt.raw_* were not loaded
-                cur = nxt;
+    // software pipeline: DEPTH batches of loads in flight per wave
+    {
+        batch_t ring[DEPTH];
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d)
+            if (b0 + d < b1) load_batch(ring[d], b0 + d);
+#ifdef GPTQ4_PHASE_TIMERS
+        PHASE_STAMP(7);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        PHASE_STAMP(5);
+#endif
+        for (int b = b0; b < b1; b += DEPTH) {
+#pragma unroll
+            for (int d = 0; d < DEPTH; ++d) {
+                if (b + d < b1) {
+                    compute_batch(ring[d]);
+                    if (b + d + DEPTH < b1) load_batch(ring[d], b + d + DEPTH);
+                }
             }
         }
     }
 
-    // ---- sum the 4 waves through LDS: lane holds rows 4*lrow+i, columns 4*lcol+t
+    PHASE_STAMP(1);
+    // ---- sum the 4 waves through LDS: lane holds rows 4*lrow+i, columns W*lcol+t
 #pragma unroll
     for (int v = 0; v < NV; ++v)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int row = 4 * lrow + i;
             if (row < M) {
-                const float4 q4 = make_float4(acc[v][0][i], acc[v][1][i], acc[v][2][i], acc[v][3][i]);
-                *reinterpret_cast<float4 *>(&red[wave][row][v * 64 + 4 * lcol]) = q4;
+#pragma unroll
+                for (int t = 0; t < W; ++t) red[wave][row][v * SW + W * lcol + t] = acc[v][t][i];
             }
         }
     __syncthreads();
 
-    // thread owns elements (row = 4*q + tid/64, c = tid%64), each with NV values
-    const int c = tid & 63;
-    const int rbase = tid >> 6;
-    float val[4][NV];
+    // thread owns elements (row = (256/SW)*q + tid/SW, c = tid%SW), each with NV values
+    constexpr int ROWS_PER_PASS = 256 / SW;
+    const int c = tid % SW;
+    const int rbase = tid / SW;
+    float val[Q][NV];
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        const int row = 4 * q + rbase;
+    for (int q = 0; q < Q; ++q) {
+        const int row = ROWS_PER_PASS * q + rbase;
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             float s = 0.f;
-            if (row < M) s = ((red[0][row][v * 64 + c] + red[1][row][v * 64 + c]) + red[2][row][v * 64 + c]) + red[3][row][v * 64 + c];
+            if (row < M)
+                s = ((red[0][row][v * SW + c] + red[1][row][v * SW + c]) + red[2][row][v * SW + c]) + red[3][row][v * SW + c];
             val[q][v] = s;
         }
     }
 
+    PHASE_STAMP(2);
     if (p.splitk > 1) {
+        // Cross-workgroup exchange without cache maintenance: partial sums are written
+        // and read with agent-scope (sc1) relaxed atomics, which are coherent across the
+        // XCDs' L2s by themselves.  A release/acquire fence would add an L2 write-back
+        // and invalidate per workgroup, which serialises the whole grid.  Ordering is
+        // by completion: every wave waits until its stores are acknowledged
+        // (s_waitcnt vmcnt(0)) before the barrier that precedes the arrival count.
         const size_t tile_elems = (size_t)M * TILE_COLS;
         float *mine = p.partials + ((size_t)tile * p.splitk + split) * tile_elems;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int row = 4 * q + rbase;
+        for (int q = 0; q < Q; ++q) {
+            const int row = ROWS_PER_PASS * q + rbase;
             if (row < M) {
 #pragma unroll
-                for (int v = 0; v < NV; ++v) mine[(size_t)row * TILE_COLS + v * 64 + c] = val[q][v];
+                for (int v = 0; v < NV; ++v)
+                    __hip_atomic_store(&mine[(size_t)row * TILE_COLS + v * SW + c], val[q][v], __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
             }
         }
-        __threadfence();
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        PHASE_STAMP(3);
         __syncthreads();
         if (tid == 0) {
-            const int old = atomicAdd(&p.counters[tile], 1);
+            const int old = __hip_atomic_fetch_add(&p.counters[tile], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             s_is_last = (old == p.splitk - 1);
         }
         __syncthreads();
+        PHASE_STAMP(4);
         if (!s_is_last) return;
-        __threadfence();
         const float *all = p.partials + (size_t)tile * p.splitk * tile_elems;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int row = 4 * q + rbase;
+        for (int q = 0; q < Q; ++q) {
+            const int row = ROWS_PER_PASS * q + rbase;
             if (row < M) {
 #pragma unroll
                 for (int v = 0; v < NV; ++v) {
+                    // all loads in flight at once, then a fixed-order sum
+                    const float *src = all + (size_t)row * TILE_COLS + v * SW + c;
+                    float part[SKINNY_MAX_SPLITK];
+#pragma unroll
+                    for (int sp = 0; sp < SKINNY_MAX_SPLITK; ++sp)
+                        part[sp] = (sp < p.splitk) ? __hip_atomic_load(src + (size_t)sp * tile_elems, __ATOMIC_RELAXED,
+                                                                       __HIP_MEMORY_SCOPE_AGENT)
+                                                   : 0.f;
                     float s = 0.f;
-                    for (int sp = 0; sp < p.splitk; ++sp)
-                        s += all[(size_t)sp * tile_elems + (size_t)row * TILE_COLS + v * 64 + c];
+#pragma unroll
+                    for (int sp = 0; sp < SKINNY_MAX_SPLITK; ++sp) s += part[sp];
                     val[q][v] = s;
                 }
             }
         }
-        if (tid == 0) p.counters[tile] = 0;
+        PHASE_STAMP(5);
+        if (tid == 0) __hip_atomic_store(&p.counters[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 
     // ---- epilogue
 #pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        const int row = 4 * q + rbase;
+    for (int q = 0; q < Q; ++q) {
+        const int row = ROWS_PER_PASS * q + rbase;
         if (row >= M) continue;
         if (EPI == EPI_PLAIN) {
             const int n = n0 + c;
@@ -247,17 +339,19 @@ __global__ __launch_bounds__(256) void gptq4_skinny_kernel(MatmulArgs p) {
             const int n = n0 + c;
             p.y[(size_t)row * N + n] = (half_t)(silu_f32(val[q][0]) * val[q][NV - 1]);
         } else {
-            // tile = one 128-wide head of q, k or v; c = d < 64, partner d + 64
+            // columns n0 + c (d < 64) and n0 + 64 + c (its partner) of one head of q, k or v
             const RopeArgs &r = p.rope;
-            const int which = tile / r.H;
-            const int head = tile - which * r.H;
+            const int head_col = n0 >> 7;
+            const int d = (n0 & 127) + c;
+            const int which = head_col / r.H;
+            const int head = head_col - which * r.H;
             const int bb = row / r.S;
             const int ss = row - bb * r.S;
             float o1 = val[q][0], o2 = val[q][NV - 1];
             if (which < 2) {
                 const int pos = min(max(r.position_ids[row], 0), r.max_pos - 1);
-                const float cs = r.cos_table[(size_t)pos * 64 + c];
-                const float sn = r.sin_table[(size_t)pos * 64 + c];
+                const float cs = r.cos_table[(size_t)pos * 64 + d];
+                const float sn = r.sin_table[(size_t)pos * 64 + d];
                 const float x1 = o1, x2 = o2;
                 o1 = x1 * cs - x2 * sn;
                 o2 = x2 * cs + x1 * sn;
@@ -271,44 +365,76 @@ __global__ __launch_bounds__(256) void gptq4_skinny_kernel(MatmulArgs p) {
                 dst = (which == 1) ? r.k : r.v;
                 off = ((size_t)(bb * r.H + head) * r.kv_capacity + r.kv_offset + ss) * 128;
             }
-            dst[off + c] = (half_t)o1;
-            dst[off + 64 + c] = (half_t)o2;
+            dst[off + d] = (half_t)o1;
+            dst[off + 64 + d] = (half_t)o2;
         }
+    }
+    PHASE_STAMP(6);
+}
+
+template <int EPI, int W, int DEPTH>
+int launch_variant(const MatmulArgs &a, hipStream_t stream) {
+    constexpr int SW = 16 * W;
+    constexpr int LINE_TILES = (SW >= 32) ? 1 : 32 / SW;
+    const int per_xcd = 8 * LINE_TILES;
+    const int groups = (a.tiles + per_xcd - 1) / per_xcd;
+    dim3 grid((unsigned)(groups * per_xcd), (unsigned)a.splitk), block(256);
+    if (a.perm == nullptr)
+        hipLaunchKernelGGL((gptq4_skinny_kernel<EPI, W, DEPTH, false>), grid, block, 0, stream, a);
+    else
+        hipLaunchKernelGGL((gptq4_skinny_kernel<EPI, W, DEPTH, true>), grid, block, 0, stream, a);
+    return (int)hipGetLastError();
+}
+
+template <int EPI>
+int launch_epi(const MatmulArgs &a, int words, int depth, hipStream_t stream) {
+    const int key = words * 10 + depth;
+    switch (key) {
+        case 11: return launch_variant<EPI, 1, 1>(a, stream);
+        case 12: return launch_variant<EPI, 1, 2>(a, stream);
+        case 14: return launch_variant<EPI, 1, 4>(a, stream);
+        case 21: return launch_variant<EPI, 2, 1>(a, stream);
+        case 22: return launch_variant<EPI, 2, 2>(a, stream);
+        case 24: return launch_variant<EPI, 2, 4>(a, stream);
+        case 41: return launch_variant<EPI, 4, 1>(a, stream);
+        case 42: return launch_variant<EPI, 4, 2>(a, stream);
+        default: return launch_variant<EPI, 4, 3>(a, stream);
     }
 }
 
 }  // namespace
 
-int g_forced_splitk = 0;
+SkinnyTuning g_skinny_tuning = {0, 0, 0};
 
-int skinny_pick_splitk(int tiles, int k_batches) {
+// Launch shape for a small-M problem, from sweeps on MI355X: 8-byte loads (32-column
+// strips, full 128-byte lines per row) beat 16-byte loads because they give twice the
+// tiles; two batches in flight per wave, one for the gate/up pair (register budget);
+// split K until there are ~1024 workgroups (4 per CU) but keep >= 2 batches per wave.
+SkinnyPlan skinny_plan(int epi, int N, int K) {
+    SkinnyPlan pl;
+    pl.words = g_skinny_tuning.words > 0 ? g_skinny_tuning.words : 2;
+    pl.depth = g_skinny_tuning.depth > 0 ? g_skinny_tuning.depth : (epi == EPI_SILU_MUL ? 1 : 2);
+    const int sw = 16 * pl.words;
+    pl.tiles = (epi == EPI_ROPE) ? (N / 128) * (64 / sw) : N / sw;
+    const int k_batches = K / 128;
     int s;
-    if (g_forced_splitk > 0) {
-        s = g_forced_splitk;
+    if (g_skinny_tuning.splitk > 0) {
+        s = g_skinny_tuning.splitk;
+        if (s > k_batches / 4) s = k_batches / 4;  // at least one batch per wave
     } else {
-        // aim for ~1024 workgroups (4 per CU) so every CU has loads in flight
-        s = (1024 + tiles - 1) / tiles;
+        s = (1024 + pl.tiles - 1) / pl.tiles;
+        if (s > k_batches / 8) s = k_batches / 8;
     }
-    const int by_k = k_batches / 4;  // at least one batch per wave
-    if (s > by_k) s = by_k;
     if (s > SKINNY_MAX_SPLITK) s = SKINNY_MAX_SPLITK;
     if (s < 1) s = 1;
-    return s;
+    pl.splitk = s;
+    return pl;
 }
 
-int launch_skinny(int epi, MatmulArgs a, hipStream_t stream) {
-    const int groups = ((a.tiles + 7) / 8) * 8;
-    dim3 grid((unsigned)(groups * a.splitk)), block(256);
+int launch_skinny(int epi, const MatmulArgs &a, const SkinnyPlan &pl, hipStream_t stream) {
     switch (epi) {
-        case EPI_PLAIN:
-            hipLaunchKernelGGL(gptq4_skinny_kernel<EPI_PLAIN>, grid, block, 0, stream, a);
-            break;
-        case EPI_SILU_MUL:
-            hipLaunchKernelGGL(gptq4_skinny_kernel<EPI_SILU_MUL>, grid, block, 0, stream, a);
-            break;
-        default:
-            hipLaunchKernelGGL(gptq4_skinny_kernel<EPI_ROPE>, grid, block, 0, stream, a);
-            break;
+        case EPI_PLAIN: return launch_epi<EPI_PLAIN>(a, pl.words, pl.depth, stream);
+        case EPI_SILU_MUL: return launch_epi<EPI_SILU_MUL>(a, pl.words, pl.depth, stream);
+        default: return launch_epi<EPI_ROPE>(a, pl.words, pl.depth, stream);
     }
-    return (int)hipGetLastError();
 }

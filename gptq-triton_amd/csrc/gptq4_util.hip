@@ -21,7 +21,7 @@ __global__ __launch_bounds__(256) void gptq4_dequant_kernel(const uint32_t *__re
     if (g_idx == nullptr) {
         const int g = (8 * r) / groupsize;
         const uint32_t z = (qzeros[(size_t)g * (N >> 3) + (n >> 3)] >> zshift) & 0xFu;
-        const ColDecode c = make_col_decode(z, scales[(size_t)g * N + n]);
+        const ColDecode c = make_col_decode(z, reinterpret_cast<const uint16_t *>(scales)[(size_t)g * N + n]);
         h2_t p[4];
         decode_word(w, c, p);
 #pragma unroll
@@ -34,7 +34,7 @@ __global__ __launch_bounds__(256) void gptq4_dequant_kernel(const uint32_t *__re
         for (int t = 0; t < 8; ++t) {
             const int g = g_idx[8 * r + t];
             const uint32_t z = (qzeros[(size_t)g * (N >> 3) + (n >> 3)] >> zshift) & 0xFu;
-            const ColDecode c = make_col_decode(z, scales[(size_t)g * N + n]);
+            const ColDecode c = make_col_decode(z, reinterpret_cast<const uint16_t *>(scales)[(size_t)g * N + n]);
             h2_t p[4];
             decode_word(w, c, p);
             vals[t] = (t < 4) ? p[t & 3].x : p[t & 3].y;

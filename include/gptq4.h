@@ -120,9 +120,12 @@ int gptq4_qkv_rotary(const void *x, const int32_t *qweight, const int32_t *qzero
                      int groupsize, int kv_capacity, int kv_offset, void *workspace,
                      size_t workspace_bytes, void *stream);
 
-/* Host-side launch tuning for measurements: split-K factor of the small-M kernels
- * (0 = automatic).  Process-wide; not thread-safe against concurrent launches. */
-void gptq4_set_splitk(int splitk);
+/* Host-side launch tuning of the small-M kernels, for measurements: words per lane and
+ * load (1, 2 or 4: strips of 16, 32 or 64 columns), batches of loads in flight per
+ * wave (1..4) and the split-K factor; 0 = automatic for each.  Process-wide; not
+ * thread-safe against concurrent launches.  No reference counterpart (the reference
+ * tunes through Triton's autotuner, custom_autotune.py:12-172). */
+void gptq4_set_tuning(int words, int depth, int splitk);
 
 #ifdef __cplusplus
 }

@@ -168,12 +168,12 @@ def test_splitk_variants_agree_and_counters_reset(splitk):
     lib = _lib.load()
     ref = O.quant_matmul_ref(x, L["qweight"], L["qzeros"], L["scales"], g)
     try:
-        lib.gptq4_set_splitk(splitk)
+        lib.gptq4_set_tuning(0, 0, splitk)
         xd = torch.from_numpy(x).cuda()
         y1 = gptq().matmul4(g, xd, D["qweight"], D["scales"], D["qzeros"])
         y2 = gptq().matmul4(g, xd, D["qweight"], D["scales"], D["qzeros"])
     finally:
-        lib.gptq4_set_splitk(0)
+        lib.gptq4_set_tuning(0, 0, 0)
     assert torch.equal(y1, y2), "split-K result must be deterministic"
     assert_close(y1.cpu().numpy(), ref, f"splitk={splitk}")
     ws = _lib.workspace(xd.device, 0)
