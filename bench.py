@@ -56,6 +56,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the per-operator / prefill extras")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="for rocprofv3 --pmc runs: a 256 MiB device copy (calibration) followed by plain launches of "
+                         "each decode operator on distinct weights; prints no JSON")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures the single-GPU hot path: run with --gpus 1 (nothing here uses a second GPU)",
@@ -136,6 +139,24 @@ def main():
     x1 = torch.randn((1, 1, HIDDEN), device=dev, generator=gen).half()
     pos1 = torch.tensor([[2047]], device=dev, dtype=torch.int32)
 
+    if args.traffic_probe:
+        # counters are read per dispatch, so no graph here; the copy kernel moves a known
+        # 256 MiB in and 256 MiB out and calibrates FETCH_SIZE / WRITE_SIZE
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(generator=gen)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        for L in layers:
+            qkv_op(x1, L, pos1)
+        for L in layers:
+            o_op(x1, L)
+        hs = [gateup_op(x1, L) for L in layers]
+        for h, L in zip(hs, layers):
+            down_op(h, L)
+        torch.cuda.synchronize()
+        log("traffic probe done")
+        return
+
     def decode_step():
         outs = []
         for L in layers:
@@ -174,7 +195,10 @@ def main():
     gu_bytes = 2 * weight_bytes(HIDDEN, INTER, GROUPSIZE) + HIDDEN * 2 + INTER * 2
     gu_gbs = gu_bytes / gu_us / 1e3
     roofline = {"bound": "hbm", "achieved": round(gu_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(gu_gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                "frac": round(gu_gbs / HBM_PEAK_GBS, 4),
+                # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+                # `bench.py --traffic-probe`, scaled by a 256 MiB copy (x2.000 / x1.000)
+                "traffic": 51_190_000 + 330_000,
                 "kernel": "gptq4_skinny_kernel<SILU_MUL> (gate/up GEMV, M=1, K=4096, I=11008, g=128)",
                 "bytes_per_launch": gu_bytes, "avg_launch_us": round(gu_us, 2)}
     log(f"gate/up GEMV: {gu_us:.2f} us/launch, {gu_gbs:.0f} GB/s = {100 * gu_gbs / HBM_PEAK_GBS:.1f}% of HBM peak")
