@@ -66,6 +66,9 @@ const char *gptq4_strerror(int code) {
     }
 }
 
+extern int g_gemm_mt;
+extern "C" void gptq4_dev_set_gemm_mt(int mt) { g_gemm_mt = (mt == 2 || mt == 4) ? mt : 0; }
+
 void gptq4_set_tuning(int words, int depth, int splitk) {
     g_skinny_tuning.words = (words == 1 || words == 2 || words == 4) ? words : 0;
     g_skinny_tuning.depth = (depth >= 1 && depth <= 4) ? depth : 0;

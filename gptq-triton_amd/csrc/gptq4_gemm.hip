@@ -3,18 +3,28 @@
 // v_mfma_f32_32x32x16_f16 with fp32 accumulation.  The checkpoint layout already IS
 // the matrix-core B layout: one packed word = 8 consecutive k of one column = one
 // lane's B operand for a 16-deep K step.  So the weights never touch LDS: every lane
-// loads 128 bits (4 adjacent columns x 8 k) straight from global memory, decodes the
-// 4 words in registers and uses word t as the B operand of column tile t, whose 32
-// columns are {4j + t}.  Each decoded operand is reused by all M tiles of the wave.
-// Only the activations go through LDS (stored in pair order, rows padded to 144 B).
+// loads 2 adjacent words (8 bytes; a wave covers 2 qweight rows x 64 columns = one K
+// step) straight from global memory, decodes them in registers and uses word t as the
+// B operand of column tile t, whose 32 columns are {2j + t}.
 //
-// Workgroup = 4 waves as 2 (M) x 2 (N).  Wave tile = (32*MT) rows x 128 columns.
-//   plain / rotary : workgroup tile (64*MT) x 256; a wave's 128 columns are one head,
-//                    so the rotary partner d +- 64 is lane ^ 16 of the same register.
-//   SiLU*mul       : the two N waves take the SAME 128 columns of the gate and of the
-//                    up matrix; the up accumulators are handed over through LDS.
+// The decode is VALU work (13 ops per word) that has to hide under the MFMAs, and each
+// decoded operand is reused only by the row tiles of its own wave.  The wave tile is
+// therefore tall and narrow: (32*MT) rows x 64 columns, MT = 4 by default - 8 MFMAs
+// per pair of decoded words, 128 accumulator registers, two waves per SIMD.  The
+// decode of K step s+1 is written between the MFMAs of step s; the packed words of a
+// step are refilled in place with the same step of the next K tile; every load in the
+// loop is unconditional (clamped indices) so the waits are exact vmcnt(N).
+// Only the activations go through LDS (stored in pair order, rows padded to 144 B,
+// double buffered, one barrier per K tile of 64).
+//
+// Workgroup = 4 waves as 2 (M) x 2 (N): tile (64*MT) x 128.
+//   plain   : the two N waves take adjacent 64-column halves.
+//   rotary  : the 128 columns are one head; column d and its partner d + 64 sit in the
+//             two N waves at the same lane and register, and are swapped through LDS.
+//   SiLU*mul: the two N waves take the SAME 64 columns of the gate and of the up
+//             matrix (tile (64*MT) x 64 of the output); up is handed over through LDS.
 // blockIdx is remapped so each XCD (blockIdx % 8) owns a contiguous range of tiles:
-// the M tiles that share a weight panel then share one L2.
+// the row tiles that share a weight panel then share one L2.
 #include "gptq4_internal.h"
 
 namespace {
@@ -22,13 +32,14 @@ namespace {
 constexpr int BK = 64;
 constexpr int LDS_ROW = BK + 8;  // halves; 144-byte rows keep 128-bit reads conflict-free
 
-template <int EPI, int MT>
-__global__ __launch_bounds__(256) void gptq4_gemm_kernel(MatmulArgs p) {
+template <int EPI, int MT, bool PERM>
+__global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
     constexpr int BM = 64 * MT;
-    constexpr int BN = (EPI == EPI_SILU_MUL) ? 128 : 256;
+    constexpr int BN = (EPI == EPI_SILU_MUL) ? 64 : 128;
     constexpr int A_UNITS = BM * (BK / 8) / 256;  // 16-byte units each thread stages per K tile
 
     __shared__ __attribute__((aligned(16))) half_t As[2][BM][LDS_ROW];
+    static_assert(sizeof(As) >= 4 * 32 * 64 * sizeof(float), "epilogue exchange buffer does not fit");
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -41,7 +52,7 @@ __global__ __launch_bounds__(256) void gptq4_gemm_kernel(MatmulArgs p) {
     const int M = p.M, K = p.K, N = p.N;
     const int tiles_m = (M + BM - 1) / BM;
 
-    // XCD-contiguous logical tile index
+    // XCD-contiguous logical tile index, row tiles fastest
     const int total = gridDim.x;
     const int per = total >> 3, rem = total & 7;
     const int xcd = blockIdx.x & 7;
@@ -52,96 +63,105 @@ __global__ __launch_bounds__(256) void gptq4_gemm_kernel(MatmulArgs p) {
     const int n0 = tile_n * BN;
 
     const int mat = (EPI == EPI_SILU_MUL) ? wn : 0;
-    const int nw0 = n0 + ((EPI == EPI_SILU_MUL) ? 0 : wn * 128);  // first column of the wave
-    const int ncol = nw0 + 4 * l32;                                // lane's 4 columns
-    const uint32_t *qw = p.w[mat].qweight + ncol;
-    const uint32_t *qz = p.w[mat].qzeros;
-    const half_t *sc = p.w[mat].scales;
-    const int gs = p.groupsize;
+    const int nw0 = n0 + ((EPI == EPI_SILU_MUL) ? 0 : wn * 64);  // first column of the wave
+    const int ncol = nw0 + 2 * l32;                               // lane's 2 columns
+    const uint32_t *bptr = p.w[mat].qweight + (size_t)lhi * N + ncol;  // row lhi of K tile 0
+    const uint32_t *qz = p.w[mat].qzeros + (ncol >> 3);
+    const half_t *sc = p.w[mat].scales + ncol;
+    const int tiles_per_group = p.groupsize / BK;
+    const int last_group = K / p.groupsize - 1;
 
-    f16_t acc[MT][4];
+    f16_t acc[MT][2];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+        for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[mt][t][i] = 0.f;
 
+    // Activation staging: each thread owns A_UNITS 16-byte units (row, 8 k) of the tile.
+    // Rows beyond M read row M-1 instead of branching: A row m only feeds output row m and
+    // rows >= M are never stored.  Addresses: one uniform base (scalar registers) plus a
+    // small per-lane element offset.
+    const half_t *a_base = p.x + (size_t)m0 * K;
+    uint32_t a_off[A_UNITS];
+    const int a_row = tid >> 3, a_ku = tid & 7;  // unit u of this thread: row a_row + 32*u, k-unit a_ku
+#pragma unroll
+    for (int u = 0; u < A_UNITS; ++u) {
+        const int row = min(a_row + 32 * u, M - 1 - m0);
+        a_off[u] = (uint32_t)row * (uint32_t)K + 8u * a_ku;
+    }
+    half_t *const a_lds = &As[0][a_row][8 * a_ku];
+
     uint4 a_stage[A_UNITS];
-    uint4 b_cur[4], b_nxt[4];
-    uint2 raw_s = make_uint2(0u, 0u);
-    uint32_t raw_z = 0;
-    int grp_loaded = -1, grp_decoded = -1;
-    ColDecode cd[4];
+    uint2 bw[4];  // packed B words of the 4 K steps; refilled in place for the next K tile
+    uint32_t raw_s, raw_z;
+    ColDecode cd[2];
 
     auto load_a = [&](int kt) {
 #pragma unroll
         for (int u = 0; u < A_UNITS; ++u) {
-            const int unit = tid + 256 * u;
-            const int row = unit >> 3, ku = unit & 7;
-            const int gm = m0 + row;
-            const int k = kt * BK + 8 * ku;
-            uint4 a = make_uint4(0u, 0u, 0u, 0u);
-            if (gm < M) {
-                const half_t *xr = p.x + (size_t)gm * K;
-                if (p.perm == nullptr) {
-                    a = *reinterpret_cast<const uint4 *>(xr + k);
-                } else {
-                    const int4 i0 = *reinterpret_cast<const int4 *>(p.perm + k);
-                    const int4 i1 = *reinterpret_cast<const int4 *>(p.perm + k + 4);
-                    const uint16_t *xs = reinterpret_cast<const uint16_t *>(xr);
-                    a.x = (uint32_t)xs[i0.x] | ((uint32_t)xs[i0.y] << 16);
-                    a.y = (uint32_t)xs[i0.z] | ((uint32_t)xs[i0.w] << 16);
-                    a.z = (uint32_t)xs[i1.x] | ((uint32_t)xs[i1.y] << 16);
-                    a.w = (uint32_t)xs[i1.z] | ((uint32_t)xs[i1.w] << 16);
-                }
+            if (!PERM) {
+                a_stage[u] = *reinterpret_cast<const uint4 *>(a_base + a_off[u] + kt * BK);
+            } else {
+                const int k = kt * BK + 8 * a_ku;
+                const int4 i0 = *reinterpret_cast<const int4 *>(p.perm + k);
+                const int4 i1 = *reinterpret_cast<const int4 *>(p.perm + k + 4);
+                const uint16_t *xs = reinterpret_cast<const uint16_t *>(a_base + (a_off[u] - 8u * a_ku));
+                uint4 a;
+                a.x = (uint32_t)xs[i0.x] | ((uint32_t)xs[i0.y] << 16);
+                a.y = (uint32_t)xs[i0.z] | ((uint32_t)xs[i0.w] << 16);
+                a.z = (uint32_t)xs[i1.x] | ((uint32_t)xs[i1.y] << 16);
+                a.w = (uint32_t)xs[i1.z] | ((uint32_t)xs[i1.w] << 16);
+                a_stage[u] = a;
             }
-            a_stage[u] = a;
         }
     };
     auto store_a = [&](int buf) {
 #pragma unroll
-        for (int u = 0; u < A_UNITS; ++u) {
-            const int unit = tid + 256 * u;
-            const int row = unit >> 3, ku = unit & 7;
-            *reinterpret_cast<uint4 *>(&As[buf][row][8 * ku]) = pair_order_u4(a_stage[u]);
-        }
+        for (int u = 0; u < A_UNITS; ++u)
+            *reinterpret_cast<uint4 *>(a_lds + buf * (BM * LDS_ROW) + u * (32 * LDS_ROW)) = pair_order_u4(a_stage[u]);
     };
-    auto load_b = [&](uint4 (&b)[4], int kt) {
-        const uint32_t *base = qw + (size_t)(kt * (BK / 8) + lhi) * N;
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) b[ks] = *reinterpret_cast<const uint4 *>(base + (size_t)(2 * ks) * N);
-        const int g = (kt * BK) / gs;
-        if (g != grp_loaded) {
-            grp_loaded = g;
-            raw_s = *reinterpret_cast<const uint2 *>(sc + (size_t)g * N + ncol);
-            raw_z = qz[(size_t)g * (N >> 3) + (ncol >> 3)];
-        }
+    auto load_b_step = [&](int kt, int ks) {
+        bw[ks] = *reinterpret_cast<const uint2 *>(bptr + ((size_t)kt * (BK / 8) + 2 * ks) * N);
+    };
+    auto load_group = [&](int g) {
+        raw_s = *reinterpret_cast<const uint32_t *>(sc + (size_t)g * N);
+        raw_z = qz[(size_t)g * (N >> 3)];
+    };
+    // Decode constants from the raw scale / zero words.  Recomputed for every K tile from
+    // that tile's own group (a few integer ops) rather than only at group boundaries:
+    // with no branch around the loads that feed them, every wait in the loop is exact.
+    auto make_cd = [&]() {
+        const uint32_t z2 = raw_z >> (((2 * l32) & 7) * 4);
+        cd[0] = make_col_decode(z2 & 0xFu, raw_s);
+        cd[1] = make_col_decode((z2 >> 4) & 0xFu, raw_s >> 16);
     };
 
     const int nk = K / BK;
     load_a(0);
-    load_b(b_cur, 0);
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) load_b_step(0, ks);
+    load_group(0);
+    make_cd();
+    int group = 0, left_in_group = tiles_per_group;  // K tiles left in the current group, this one included
+
+    // B operands of the K step about to be multiplied.  They are decoded one step ahead,
+    // in place, right after the MFMAs that consumed the previous contents were issued, so
+    // the decode (VALU) of step s+1 runs under the MFMAs of step s.
+    h8_t bf[2];
+    bf[0] = decode_word_h8(bw[0].x, cd[0]);
+    bf[1] = decode_word_h8(bw[0].y, cd[1]);
+    load_b_step(min(1, nk - 1), 0);
 
     for (int kt = 0; kt < nk; ++kt) {
         const int buf = kt & 1;
         store_a(buf);
-        // decode constants of the group this K tile belongs to (raw_* were fetched
-        // together with b_cur)
-        const int g = (kt * BK) / gs;
-        if (g != grp_decoded) {
-            grp_decoded = g;
-            const uint32_t z4 = raw_z >> ((l32 & 1) * 16);
-            cd[0] = make_col_decode(z4 & 0xFu, raw_s.x);
-            cd[1] = make_col_decode((z4 >> 4) & 0xFu, raw_s.x >> 16);
-            cd[2] = make_col_decode((z4 >> 8) & 0xFu, raw_s.y);
-            cd[3] = make_col_decode((z4 >> 12) & 0xFu, raw_s.y >> 16);
-        }
         __syncthreads();
-        if (kt + 1 < nk) {
-            load_a(kt + 1);
-            load_b(b_nxt, kt + 1);
-        }
+        const int kn = min(kt + 1, nk - 1), kn2 = min(kt + 2, nk - 1);
+        const bool new_group = (left_in_group == 1);
+        load_a(kn);
+        load_group(min(group + (new_group ? 1 : 0), last_group));
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
             h8_t af[MT];
@@ -150,103 +170,112 @@ __global__ __launch_bounds__(256) void gptq4_gemm_kernel(MatmulArgs p) {
                 const int row = wm * (32 * MT) + mt * 32 + l32;
                 af[mt] = *reinterpret_cast<const h8_t *>(&As[buf][row][8 * (2 * ks + lhi)]);
             }
-            const uint32_t ww[4] = {b_cur[ks].x, b_cur[ks].y, b_cur[ks].z, b_cur[ks].w};
+            if (ks == 3) make_cd();  // constants of the next K tile; this tile's decodes are all done
+            const uint2 nw = bw[(ks + 1) & 3];  // words of the next step (step 0 of the next tile when ks == 3)
+            // refill: step ks+1 of the next tile (step 0 of tile kt+2 when ks == 3)
+            if (ks < 3)
+                load_b_step(kn, ks + 1);
+            else
+                load_b_step(kn2, 0);
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                const h8_t bf = decode_word_h8(ww[t], cd[t]);
+            for (int mt = 0; mt < MT; ++mt) acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt], bf[0], acc[mt][0], 0, 0, 0);
+            bf[0] = decode_word_h8(nw.x, cd[0]);
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt)
-                    acc[mt][t] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt], bf, acc[mt][t], 0, 0, 0);
-            }
+            for (int mt = 0; mt < MT; ++mt) acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt], bf[1], acc[mt][1], 0, 0, 0);
+            bf[1] = decode_word_h8(nw.y, cd[1]);
         }
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) b_cur[ks] = b_nxt[ks];
+        if (new_group) {
+            ++group;
+            left_in_group = tiles_per_group;
+        } else {
+            --left_in_group;
+        }
     }
 
     // ---- epilogue.  acc[mt][t][i]: row = 32*mt + 8*(i/4) + 4*lhi + i%4 of the wave,
-    //      column = 4*l32 + t of the wave.
+    //      column = 2*l32 + t of the wave.
     const int wrow0 = m0 + wm * (32 * MT);
+    // exchange buffer: [wave][t*16 + i][lane], reusing the activation tiles
+    float *const ex = reinterpret_cast<float *>(&As[0][0][0]);
     if (EPI == EPI_PLAIN) {
-        h2_t bias01 = {(half_t)0.f, (half_t)0.f}, bias23 = bias01;
-        if (p.bias != nullptr) {
-            const uint2 braw = *reinterpret_cast<const uint2 *>(p.bias + ncol);
-            bias01 = as_h2(braw.x);
-            bias23 = as_h2(braw.y);
-        }
+        h2_t bias2 = {(half_t)0.f, (half_t)0.f};
+        if (p.bias != nullptr) bias2 = as_h2(*reinterpret_cast<const uint32_t *>(p.bias + ncol));
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const int row = wrow0 + mt * 32 + 8 * (i >> 2) + 4 * lhi + (i & 3);
                 if (row < M) {
-                    h2_t o01 = {(half_t)acc[mt][0][i], (half_t)acc[mt][1][i]};
-                    h2_t o23 = {(half_t)acc[mt][2][i], (half_t)acc[mt][3][i]};
-                    if (p.bias != nullptr) {
-                        o01 = o01 + bias01;
-                        o23 = o23 + bias23;
-                    }
-                    *reinterpret_cast<uint2 *>(p.y + (size_t)row * N + ncol) = make_uint2(as_u32(o01), as_u32(o23));
+                    h2_t o = {(half_t)acc[mt][0][i], (half_t)acc[mt][1][i]};
+                    if (p.bias != nullptr) o = o + bias2;
+                    *reinterpret_cast<uint32_t *>(p.y + (size_t)row * N + ncol) = as_u32(o);
                 }
             }
     } else if (EPI == EPI_SILU_MUL) {
         // hand the up accumulators (wn == 1) to the gate wave (wn == 0) with the same wm
-        float *ex = reinterpret_cast<float *>(&As[0][0][0]) + wm * (64 * 64);
-        static_assert(sizeof(As) >= 2 * 64 * 64 * sizeof(float), "exchange buffer does not fit");
+        float *const mine = ex + wm * (32 * 64);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             __syncthreads();
             if (wn == 1) {
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
+                for (int t = 0; t < 2; ++t)
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) ex[(t * 16 + i) * 64 + lane] = acc[mt][t][i];
+                    for (int i = 0; i < 16; ++i) mine[(t * 16 + i) * 64 + lane] = acc[mt][t][i];
             }
             __syncthreads();
             if (wn == 0) {
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const int row = wrow0 + mt * 32 + 8 * (i >> 2) + 4 * lhi + (i & 3);
-                    float o[4];
-#pragma unroll
-                    for (int t = 0; t < 4; ++t) o[t] = silu_f32(acc[mt][t][i]) * ex[(t * 16 + i) * 64 + lane];
+                    const float o0 = silu_f32(acc[mt][0][i]) * mine[(0 * 16 + i) * 64 + lane];
+                    const float o1 = silu_f32(acc[mt][1][i]) * mine[(1 * 16 + i) * 64 + lane];
                     if (row < M) {
-                        const h2_t o01 = {(half_t)o[0], (half_t)o[1]};
-                        const h2_t o23 = {(half_t)o[2], (half_t)o[3]};
-                        *reinterpret_cast<uint2 *>(p.y + (size_t)row * N + ncol) = make_uint2(as_u32(o01), as_u32(o23));
+                        const h2_t o = {(half_t)o0, (half_t)o1};
+                        *reinterpret_cast<uint32_t *>(p.y + (size_t)row * N + ncol) = as_u32(o);
                     }
                 }
             }
         }
     } else {
+        // the workgroup's 128 columns are one head of q, k or v; this wave holds d in
+        // [64*wn, 64*wn + 64), the partner d +- 64 is the same lane and register of the
+        // other N wave
         const RopeArgs &r = p.rope;
-        const int head_col = nw0 >> 7;  // 128-wide head index over q | k | v
+        const int head_col = n0 >> 7;
         const int which = head_col / r.H;
         const int head = head_col - which * r.H;
-        const int c0 = 4 * (lane & 15);  // column of the cos/sin row shared by d and d +- 64
-        const bool upper = (lane & 16) != 0;
+        float *const mine = ex + wave * (32 * 64);
+        const float *const theirs = ex + (wave ^ 2) * (32 * 64);
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
+        for (int mt = 0; mt < MT; ++mt) {
+            if (which < 2) {
+                __syncthreads();
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) mine[(t * 16 + i) * 64 + lane] = acc[mt][t][i];
+                __syncthreads();
+            }
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const int row = wrow0 + mt * 32 + 8 * (i >> 2) + 4 * lhi + (i & 3);
-                float o[4];
-#pragma unroll
-                for (int t = 0; t < 4; ++t) o[t] = acc[mt][t][i];
+                float o0 = acc[mt][0][i], o1 = acc[mt][1][i];
                 if (which < 2) {
-                    float partner[4];
-#pragma unroll
-                    for (int t = 0; t < 4; ++t) partner[t] = __shfl_xor(o[t], 16, 64);
-                    float4 cs = make_float4(1.f, 1.f, 1.f, 1.f), sn = make_float4(0.f, 0.f, 0.f, 0.f);
+                    const float p0 = theirs[(0 * 16 + i) * 64 + lane], p1 = theirs[(1 * 16 + i) * 64 + lane];
+                    float2 cs = make_float2(1.f, 1.f), sn = make_float2(0.f, 0.f);
                     if (row < M) {
                         const int pos = min(max(r.position_ids[row], 0), r.max_pos - 1);
-                        cs = *reinterpret_cast<const float4 *>(r.cos_table + (size_t)pos * 64 + c0);
-                        sn = *reinterpret_cast<const float4 *>(r.sin_table + (size_t)pos * 64 + c0);
+                        cs = *reinterpret_cast<const float2 *>(r.cos_table + (size_t)pos * 64 + 2 * l32);
+                        sn = *reinterpret_cast<const float2 *>(r.sin_table + (size_t)pos * 64 + 2 * l32);
                     }
-                    const float cc[4] = {cs.x, cs.y, cs.z, cs.w};
-                    const float ss[4] = {sn.x, sn.y, sn.z, sn.w};
-#pragma unroll
-                    for (int t = 0; t < 4; ++t)
-                        o[t] = upper ? (o[t] * cc[t] + partner[t] * ss[t]) : (o[t] * cc[t] - partner[t] * ss[t]);
+                    if (wn == 0) {
+                        o0 = o0 * cs.x - p0 * sn.x;
+                        o1 = o1 * cs.y - p1 * sn.y;
+                    } else {
+                        o0 = o0 * cs.x + p0 * sn.x;
+                        o1 = o1 * cs.y + p1 * sn.y;
+                    }
                 }
                 if (row < M) {
                     const int bb = row / r.S;
@@ -260,32 +289,47 @@ __global__ __launch_bounds__(256) void gptq4_gemm_kernel(MatmulArgs p) {
                         dst = (which == 1) ? r.k : r.v;
                         off = ((size_t)(bb * r.H + head) * r.kv_capacity + r.kv_offset + srow) * 128;
                     }
-                    const h2_t o01 = {(half_t)o[0], (half_t)o[1]};
-                    const h2_t o23 = {(half_t)o[2], (half_t)o[3]};
-                    *reinterpret_cast<uint2 *>(dst + off + 4 * l32) = make_uint2(as_u32(o01), as_u32(o23));
+                    const h2_t o = {(half_t)o0, (half_t)o1};
+                    *reinterpret_cast<uint32_t *>(dst + off + 64 * wn + 2 * l32) = as_u32(o);
                 }
             }
+        }
     }
 }
 
 template <int EPI, int MT>
 int launch_one(const MatmulArgs &a, hipStream_t stream) {
     constexpr int BM = 64 * MT;
-    constexpr int BN = (EPI == EPI_SILU_MUL) ? 128 : 256;
+    constexpr int BN = (EPI == EPI_SILU_MUL) ? 64 : 128;
     const int tiles = ((a.M + BM - 1) / BM) * (a.N / BN);
-    hipLaunchKernelGGL((gptq4_gemm_kernel<EPI, MT>), dim3((unsigned)tiles), dim3(256), 0, stream, a);
+    if (a.perm == nullptr)
+        hipLaunchKernelGGL((gptq4_gemm_kernel<EPI, MT, false>), dim3((unsigned)tiles), dim3(256), 0, stream, a);
+    else
+        hipLaunchKernelGGL((gptq4_gemm_kernel<EPI, MT, true>), dim3((unsigned)tiles), dim3(256), 0, stream, a);
     return (int)hipGetLastError();
+}
+
+template <int EPI>
+int launch_epi(const MatmulArgs &a, int mt, hipStream_t stream) {
+    return mt == 4 ? launch_one<EPI, 4>(a, stream) : launch_one<EPI, 2>(a, stream);
 }
 
 }  // namespace
 
+int g_gemm_mt = 0;  // measurement hook: force the row-tile count (2 or 4); 0 = automatic
+
 int launch_gemm(int epi, const MatmulArgs &a, hipStream_t stream) {
+    // 256-row tiles (MT = 4) once there are enough of them to fill the chip twice over;
+    // otherwise 128-row tiles for more workgroups
+    int mt = g_gemm_mt;
+    if (mt == 0) {
+        const int bn = (epi == EPI_SILU_MUL) ? 64 : 128;
+        const long tiles4 = (long)((a.M + 255) / 256) * (a.N / bn);
+        mt = (a.M > 128 && tiles4 >= 512) ? 4 : 2;
+    }
     switch (epi) {
-        case EPI_PLAIN:
-            return launch_one<EPI_PLAIN, 2>(a, stream);
-        case EPI_SILU_MUL:
-            return launch_one<EPI_SILU_MUL, 2>(a, stream);
-        default:
-            return launch_one<EPI_ROPE, 2>(a, stream);
+        case EPI_PLAIN: return launch_epi<EPI_PLAIN>(a, mt, stream);
+        case EPI_SILU_MUL: return launch_epi<EPI_SILU_MUL>(a, mt, stream);
+        default: return launch_epi<EPI_ROPE>(a, mt, stream);
     }
 }
