@@ -41,6 +41,22 @@ int setup_skinny(MatmulArgs &a, const SkinnyPlan &pl, int nmat, void *workspace,
     return 0;
 }
 
+// Fill the split-K fields of `a` for the tiled kernel.
+int setup_gemm(MatmulArgs &a, const GemmPlan &pl, void *workspace, size_t workspace_bytes) {
+    a.tiles = pl.tiles;
+    a.splitk = pl.splitk;
+    const int nk = a.K / 64;
+    a.slot_q = nk / pl.splitk;
+    a.slot_rem = nk % pl.splitk;
+    if (pl.splitk > 1) {
+        if (workspace == nullptr || workspace_bytes < GPTQ4_WS_COUNTER_BYTES + gemm_partial_bytes(pl))
+            return -GPTQ4_E_WORKSPACE;
+        a.counters = reinterpret_cast<int *>(workspace);
+        a.partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_COUNTER_BYTES);
+    }
+    return 0;
+}
+
 }  // namespace
 
 extern "C" {
@@ -66,8 +82,10 @@ const char *gptq4_strerror(int code) {
     }
 }
 
-extern int g_gemm_mt;
-extern "C" void gptq4_dev_set_gemm_mt(int mt) { g_gemm_mt = (mt == 2 || mt == 4) ? mt : 0; }
+void gptq4_set_gemm_tuning(int mt, int splitk) {
+    g_gemm_tuning.mt = (mt == 2 || mt == 4) ? mt : 0;
+    g_gemm_tuning.splitk = splitk > 0 ? splitk : 0;
+}
 
 void gptq4_set_tuning(int words, int depth, int splitk) {
     g_skinny_tuning.words = (words == 1 || words == 2 || words == 4) ? words : 0;
@@ -76,11 +94,14 @@ void gptq4_set_tuning(int words, int depth, int splitk) {
 }
 
 size_t gptq4_workspace_bytes(int op, int M, int K, int N) {
-    (void)K;
     size_t bytes = GPTQ4_WS_COUNTER_BYTES;
-    if (M >= 1 && M <= SKINNY_MAX_M && N > 0) {
+    if (M < 1 || N <= 0 || K <= 0) return bytes;
+    if (M <= SKINNY_MAX_M) {
         const int cols = (op == GPTQ4_OP_MLP_GATEUP) ? 2 * N : N;
         bytes += partial_bytes(SKINNY_MAX_SPLITK, M, cols);
+    } else if ((K % 64) == 0) {
+        const int epi = (op == GPTQ4_OP_MLP_GATEUP) ? EPI_SILU_MUL : (op == GPTQ4_OP_QKV_ROTARY ? EPI_ROPE : EPI_PLAIN);
+        bytes += gemm_partial_bytes(gemm_plan(epi, M, N, K));  // for the current (automatic or forced) plan
     }
     return bytes;
 }
@@ -132,7 +153,12 @@ int gptq4_matmul(const void *x, const int32_t *qweight, const int32_t *qzeros, c
         if (rc) return rc;
         return launch_skinny(EPI_PLAIN, a, pl, s);
     }
-    return launch_gemm(EPI_PLAIN, a, s);
+    {
+        const GemmPlan pl = gemm_plan(EPI_PLAIN, M, N, K);
+        rc = setup_gemm(a, pl, workspace, workspace_bytes);
+        if (rc) return rc;
+        return launch_gemm(EPI_PLAIN, a, pl, s);
+    }
 }
 
 int gptq4_mlp_gateup(const void *x, const int32_t *gate_qweight, const int32_t *gate_qzeros,
@@ -166,7 +192,12 @@ int gptq4_mlp_gateup(const void *x, const int32_t *gate_qweight, const int32_t *
         if (rc) return rc;
         return launch_skinny(EPI_SILU_MUL, a, pl, s);
     }
-    return launch_gemm(EPI_SILU_MUL, a, s);
+    {
+        const GemmPlan pl = gemm_plan(EPI_SILU_MUL, M, I, K);
+        rc = setup_gemm(a, pl, workspace, workspace_bytes);
+        if (rc) return rc;
+        return launch_gemm(EPI_SILU_MUL, a, pl, s);
+    }
 }
 
 int gptq4_rope_table(float *cos_out, float *sin_out, int max_pos, int D, float base, void *stream) {
@@ -218,7 +249,12 @@ int gptq4_qkv_rotary(const void *x, const int32_t *qweight, const int32_t *qzero
         if (rc) return rc;
         return launch_skinny(EPI_ROPE, a, pl, s);
     }
-    return launch_gemm(EPI_ROPE, a, s);
+    {
+        const GemmPlan pl = gemm_plan(EPI_ROPE, a.M, N, K);
+        rc = setup_gemm(a, pl, workspace, workspace_bytes);
+        if (rc) return rc;
+        return launch_gemm(EPI_ROPE, a, pl, s);
+    }
 }
 
 }  // extern "C"

@@ -138,13 +138,18 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
         cd[1] = make_col_decode((z2 >> 4) & 0xFu, raw_s >> 16);
     };
 
-    const int nk = K / BK;
-    load_a(0);
+    // K tiles [k_begin, nk) of this split (host-side quotient / remainder, no division here
+    // except the one that finds the first group)
+    const int split = blockIdx.y;
+    const int k_begin = split * p.slot_q + min(split, p.slot_rem);
+    const int nk = k_begin + p.slot_q + (split < p.slot_rem ? 1 : 0);
+    int group = (p.splitk > 1) ? k_begin / tiles_per_group : 0;
+    int left_in_group = tiles_per_group - (k_begin - group * tiles_per_group);  // K tiles left in the group
+    load_a(k_begin);
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) load_b_step(0, ks);
-    load_group(0);
+    for (int ks = 0; ks < 4; ++ks) load_b_step(k_begin, ks);
+    load_group(group);
     make_cd();
-    int group = 0, left_in_group = tiles_per_group;  // K tiles left in the current group, this one included
 
     // B operands of the K step about to be multiplied.  They are decoded one step ahead,
     // in place, right after the MFMAs that consumed the previous contents were issued, so
@@ -152,9 +157,9 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
     h8_t bf[2];
     bf[0] = decode_word_h8(bw[0].x, cd[0]);
     bf[1] = decode_word_h8(bw[0].y, cd[1]);
-    load_b_step(min(1, nk - 1), 0);
+    load_b_step(min(k_begin + 1, nk - 1), 0);
 
-    for (int kt = 0; kt < nk; ++kt) {
+    for (int kt = k_begin; kt < nk; ++kt) {
         const int buf = kt & 1;
         store_a(buf);
         __syncthreads();
@@ -190,6 +195,50 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
         } else {
             --left_in_group;
         }
+    }
+
+    if (p.splitk > 1) {
+        // Split-K for problems with too few tiles to fill the chip: every split publishes its
+        // fp32 accumulators (agent-scope atomics, no cache maintenance - see the small-M
+        // kernel), the last one to arrive sums them in split order and runs the epilogue.
+        __shared__ int s_is_last;
+        constexpr int NREG = MT * 32;
+        const int tile = logical;
+        float *const mine = p.partials + ((size_t)tile * p.splitk + split) * (NREG * 256) + tid;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+                    __hip_atomic_store(mine + ((mt * 2 + t) * 16 + i) * 256, acc[mt][t][i], __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) {
+            const int old = __hip_atomic_fetch_add(&p.counters[tile], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s_is_last = (old == p.splitk - 1);
+        }
+        __syncthreads();
+        if (!s_is_last) return;
+        const float *const all = p.partials + (size_t)tile * p.splitk * (NREG * 256) + tid;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) acc[mt][t][i] = 0.f;
+        for (int sp = 0; sp < p.splitk; ++sp) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i)
+                        acc[mt][t][i] += __hip_atomic_load(all + ((size_t)sp * NREG + (mt * 2 + t) * 16 + i) * 256,
+                                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (tid == 0) __hip_atomic_store(&p.counters[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 
     // ---- epilogue.  acc[mt][t][i]: row = 32*mt + 8*(i/4) + 4*lhi + i%4 of the wave,
@@ -298,38 +347,56 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
 }
 
 template <int EPI, int MT>
-int launch_one(const MatmulArgs &a, hipStream_t stream) {
-    constexpr int BM = 64 * MT;
-    constexpr int BN = (EPI == EPI_SILU_MUL) ? 64 : 128;
-    const int tiles = ((a.M + BM - 1) / BM) * (a.N / BN);
+int launch_one(const MatmulArgs &a, int tiles, hipStream_t stream) {
+    dim3 grid((unsigned)tiles, (unsigned)a.splitk), block(256);
     if (a.perm == nullptr)
-        hipLaunchKernelGGL((gptq4_gemm_kernel<EPI, MT, false>), dim3((unsigned)tiles), dim3(256), 0, stream, a);
+        hipLaunchKernelGGL((gptq4_gemm_kernel<EPI, MT, false>), grid, block, 0, stream, a);
     else
-        hipLaunchKernelGGL((gptq4_gemm_kernel<EPI, MT, true>), dim3((unsigned)tiles), dim3(256), 0, stream, a);
+        hipLaunchKernelGGL((gptq4_gemm_kernel<EPI, MT, true>), grid, block, 0, stream, a);
     return (int)hipGetLastError();
 }
 
 template <int EPI>
-int launch_epi(const MatmulArgs &a, int mt, hipStream_t stream) {
-    return mt == 4 ? launch_one<EPI, 4>(a, stream) : launch_one<EPI, 2>(a, stream);
+int launch_epi(const MatmulArgs &a, const GemmPlan &pl, hipStream_t stream) {
+    return pl.mt == 4 ? launch_one<EPI, 4>(a, pl.tiles, stream) : launch_one<EPI, 2>(a, pl.tiles, stream);
 }
 
 }  // namespace
 
-int g_gemm_mt = 0;  // measurement hook: force the row-tile count (2 or 4); 0 = automatic
+GemmTuning g_gemm_tuning = {0, 0};
 
-int launch_gemm(int epi, const MatmulArgs &a, hipStream_t stream) {
-    // 256-row tiles (MT = 4) once there are enough of them to fill the chip twice over;
-    // otherwise 128-row tiles for more workgroups
-    int mt = g_gemm_mt;
-    if (mt == 0) {
-        const int bn = (epi == EPI_SILU_MUL) ? 64 : 128;
-        const long tiles4 = (long)((a.M + 255) / 256) * (a.N / bn);
-        mt = (a.M > 128 && tiles4 >= 512) ? 4 : 2;
+// Tile height and split-K factor of the tiled kernel.  256-row tiles (MT = 4) once there
+// are enough of them to fill the chip twice over, otherwise 128-row tiles; K is split
+// only when even those leave most CUs idle (the M = 17..255 range on narrow layers).
+GemmPlan gemm_plan(int epi, int M, int N, int K) {
+    GemmPlan pl;
+    const int bn = (epi == EPI_SILU_MUL) ? 64 : 128;
+    const long tiles4 = (long)((M + 255) / 256) * (N / bn);
+    pl.mt = g_gemm_tuning.mt ? g_gemm_tuning.mt : ((M > 128 && tiles4 >= 512) ? 4 : 2);
+    pl.tiles = ((M + 64 * pl.mt - 1) / (64 * pl.mt)) * (N / bn);
+    const int nk = K / 64;
+    int s = 1;
+    if (g_gemm_tuning.splitk > 0) {
+        s = g_gemm_tuning.splitk;
+    } else if (pl.tiles < 192) {
+        s = 512 / pl.tiles;   // aim for ~2 workgroups per CU
+        if (s > nk / 8) s = nk / 8;   // keep at least 8 K tiles (512 k) per split
     }
+    if (s > GEMM_MAX_SPLITK) s = GEMM_MAX_SPLITK;
+    if (s > nk) s = nk;
+    if (s < 1 || pl.tiles > SKINNY_MAX_TILES) s = 1;
+    pl.splitk = s;
+    return pl;
+}
+
+size_t gemm_partial_bytes(const GemmPlan &pl) {
+    return pl.splitk > 1 ? (size_t)pl.tiles * pl.splitk * (pl.mt * 32 * 256) * sizeof(float) : 0;
+}
+
+int launch_gemm(int epi, const MatmulArgs &a, const GemmPlan &pl, hipStream_t stream) {
     switch (epi) {
-        case EPI_PLAIN: return launch_epi<EPI_PLAIN>(a, mt, stream);
-        case EPI_SILU_MUL: return launch_epi<EPI_SILU_MUL>(a, mt, stream);
-        default: return launch_epi<EPI_ROPE>(a, mt, stream);
+        case EPI_PLAIN: return launch_epi<EPI_PLAIN>(a, pl, stream);
+        case EPI_SILU_MUL: return launch_epi<EPI_SILU_MUL>(a, pl, stream);
+        default: return launch_epi<EPI_ROPE>(a, pl, stream);
     }
 }

@@ -23,7 +23,8 @@ struct MatmulArgs {
     int splitk;
     int tiles;
     // small-M kernel: K batches (128 k each) dealt to splitk * 4 wave slots - slot i
-    // gets slot_q batches, the first slot_rem slots one more
+    // gets slot_q batches, the first slot_rem slots one more.  Tiled kernel: K tiles
+    // (64 k each) dealt to splitk splits the same way.
     int slot_q, slot_rem;
     int batches_per_group;  // groupsize / 128
     RopeArgs rope;          // EPI_ROPE only
@@ -43,8 +44,20 @@ extern SkinnyTuning g_skinny_tuning;
 SkinnyPlan skinny_plan(int epi, int N, int K);
 // Small-M (M <= 16) split-K matrix-core GEMV.  Returns hipError_t.
 int launch_skinny(int epi, const MatmulArgs &a, const SkinnyPlan &plan, hipStream_t stream);
+// Launch shape of the tiled kernel.
+struct GemmPlan {
+    int mt;      // row tiles per wave: workgroup tile = (64 * mt) rows
+    int splitk;  // workgroups sharing one tile along K
+    int tiles;
+};
+struct GemmTuning {
+    int mt, splitk;  // 0 = automatic
+};
+extern GemmTuning g_gemm_tuning;
+GemmPlan gemm_plan(int epi, int M, int N, int K);
+size_t gemm_partial_bytes(const GemmPlan &plan);
 // Tiled matrix-core GEMM for any M.  Returns hipError_t.
-int launch_gemm(int epi, const MatmulArgs &a, hipStream_t stream);
+int launch_gemm(int epi, const MatmulArgs &a, const GemmPlan &plan, hipStream_t stream);
 
 int launch_dequant(const uint32_t *qweight, const uint32_t *qzeros, const half_t *scales,
                    const int32_t *g_idx, half_t *out, int K, int N, int groupsize,
@@ -54,4 +67,4 @@ int launch_sort_rows(const uint32_t *qweight, const int32_t *perm, uint32_t *out
 int launch_rope_table(float *cos_out, float *sin_out, int max_pos, int D, float base,
                       hipStream_t stream);
 
-enum { SKINNY_MAX_M = 16, SKINNY_MAX_SPLITK = 16, SKINNY_MAX_TILES = 4096 };
+enum { SKINNY_MAX_M = 16, SKINNY_MAX_SPLITK = 16, SKINNY_MAX_TILES = 4096, GEMM_MAX_SPLITK = 16 };

@@ -127,6 +127,10 @@ int gptq4_qkv_rotary(const void *x, const int32_t *qweight, const int32_t *qzero
  * tunes through Triton's autotuner, custom_autotune.py:12-172). */
 void gptq4_set_tuning(int words, int depth, int splitk);
 
+/* Same for the tiled (M > 16) kernel: rows per workgroup tile = 64 * mt (mt = 2 or 4) and
+ * the split-K factor; 0 = automatic. */
+void gptq4_set_gemm_tuning(int mt, int splitk);
+
 #ifdef __cplusplus
 }
 #endif
