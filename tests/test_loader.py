@@ -1,0 +1,165 @@
+"""Checkpoint format: packer, save/load round trip, model surgery by load_quant (CPU), and
+the loaded model on the GPU against a float32 CPU reference decoder."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+import gptq_triton_amd as G
+from gptq_triton_amd.llama import LlamaForCausalLM
+from oracle import gptq_oracle as O
+
+
+def tiny_config(**kw):
+    cfg = G.LlamaConfigLite(hidden_size=256, num_attention_heads=2, max_position_embeddings=512,
+                            intermediate_size=768, num_hidden_layers=2, vocab_size=320)
+    for k, v in kw.items():
+        setattr(cfg, k, v)
+    return cfg
+
+
+def make_checkpoint(path, groupsize, safetensors=True, seed=0, act_order=False):
+    """Random fp16 model -> RTN-quantised, packed, saved in the reference layout."""
+    torch.manual_seed(seed)
+    cfg = tiny_config()
+    model = LlamaForCausalLM(cfg).half()
+    for p in model.parameters():
+        p.requires_grad_(False)
+    model.model.embed_tokens.weight.normal_(0, 1.0)
+    for n, m in model.named_modules():
+        if isinstance(m, nn.Linear):
+            m.weight.normal_(0, 0.05)
+    floats = {n: m.weight.clone() for n, m in model.named_modules() if isinstance(m, nn.Linear) and n != "lm_head"}
+    G.make_quant(model, 4, groupsize, act_order=act_order)
+    gen = torch.Generator().manual_seed(seed + 1)
+    shared = {}
+    for n, m in model.named_modules():
+        if isinstance(m, G.QuantLinear):
+            deq, scale, zero = G.quantize_rtn(floats[n], groupsize)
+            G.pack_linear(m, deq, scale, zero)
+            if act_order:
+                # q/k/v (and gate/up) share their input, hence one g_idx per group of projections
+                key = (n.rsplit(".", 1)[0], m.infeatures, n.endswith(("o_proj", "down_proj")))
+                if key not in shared:
+                    shared[key] = torch.randperm(m.infeatures, generator=gen)
+                perm = shared[key]
+                # scatter the rows so that row r of the new layout is old row perm[r]
+                q = torch.from_numpy(O.unpack_qweight(m.qweight.numpy()))[perm]
+                m.qweight = torch.from_numpy(O.pack_qweight(q.numpy()))
+                m.g_idx = (perm // m.groupsize).to(torch.int32)
+    G.save_quant(model, path, 4, groupsize, safetensors=safetensors)
+    return cfg
+
+
+def test_packer_layout_and_round_trip():
+    torch.manual_seed(3)
+    w = torch.randn(256, 512) * 0.1          # [out, in]
+    for gs in (-1, 128):
+        deq, scale, zero = G.quantize_rtn(w, gs)
+        ql = G.QuantLinear(4, gs, 512, 256, bias=False)
+        G.pack_linear(ql, deq, scale, zero)
+        # integer weights recomputed independently, then the oracle's unpackers
+        g = 512 if gs == -1 else gs
+        q_expect = torch.round(w.reshape(256, 512 // g, g) / scale[..., None]).add(zero[..., None]).clamp(0, 15)
+        q_expect = q_expect.reshape(256, 512).t().numpy().astype(np.uint8)
+        assert (O.unpack_qweight(ql.qweight.numpy()) == q_expect).all()
+        assert (O.unpack_qzeros(ql.qzeros.numpy()) == (zero.t().numpy() - 1).astype(np.uint8)).all()
+        assert ql.qweight.dtype == torch.int32 and ql.qweight.shape == (64, 256)
+        # decoding gives back the grid values up to the fp16 rounding of scale and weight
+        W = O.dequant_fp16(ql.qweight.numpy(), ql.qzeros.numpy(), ql.scales.numpy(), gs)
+        assert np.abs(W.astype(np.float32) - deq.t().numpy()).max() < 2e-3
+        # quantisation error itself is at most half a step
+        assert (deq - w).abs().max() <= scale.max() / 2 + 1e-6
+    # the first eight input rows of column 0 are the eight nibbles of word (0, 0), LSB first
+    ql = G.QuantLinear(4, -1, 128, 256, bias=False)
+    wq = torch.zeros(256, 128)
+    wq[0, :8] = torch.arange(8).float()
+    G.pack_linear(ql, wq, torch.ones(256, 1), torch.ones(256, 1))      # scale 1, zero 1: q = w + 1
+    assert int(ql.qweight[0, 0]) & 0xFFFFFFFF == 0x87654321
+    assert int(ql.qzeros[0, 0]) == 0                                    # stored zero = true zero - 1
+    with pytest.raises(ValueError):
+        G.pack_linear(ql, wq + 100, torch.ones(256, 1), torch.ones(256, 1))
+
+
+@pytest.mark.parametrize("groupsize,safetensors", [(-1, True), (128, True), (128, False)])
+def test_load_quant_surgery_on_cpu(tmp_path, groupsize, safetensors):
+    cfg = make_checkpoint(tmp_path, groupsize, safetensors)
+    assert os.path.exists(tmp_path / ("model.safetensors" if safetensors else "model.pt"))
+    assert json.load(open(tmp_path / "quant_config.json")) == {"wbits": 4, "groupsize": groupsize}
+    model = G.load_quant(str(tmp_path), warmup_autotune=False, device=None)
+    attn = model.model.layers[1].self_attn
+    assert isinstance(attn, G.QuantLlamaAttention)
+    assert attn.qkv_proj.qweight.shape == (256 // 8, 3 * 256) and isinstance(attn.o_proj, G.QuantLinear)
+    mlp = model.model.layers[0].mlp
+    # the reference fuses the MLP by default only without grouping (__init__.py:76-77)
+    assert isinstance(mlp, G.QuantLlamaMLP) == (groupsize == -1)
+    assert isinstance(model.lm_head, nn.Linear) and model.lm_head.weight.dtype == torch.float16
+    assert model.seqlen == 2048
+    fused = G.load_quant(str(tmp_path), warmup_autotune=False, device=None, fuse_mlp=True)
+    assert isinstance(fused.model.layers[0].mlp, G.QuantLlamaMLP)
+    # fused QKV tensors are the three projections side by side, q then k then v
+    from safetensors.torch import load_file
+    state = load_file(str(tmp_path / "model.safetensors")) if safetensors else torch.load(tmp_path / "model.pt", weights_only=True)
+    cat = torch.cat([state[f"model.layers.1.self_attn.{n}_proj.qweight"] for n in "qkv"], dim=1)
+    assert torch.equal(attn.qkv_proj.qweight, cat)
+
+
+def test_load_quant_errors(tmp_path):
+    make_checkpoint(tmp_path, -1)
+    with pytest.raises(ValueError, match="device"):
+        G.load_quant(str(tmp_path), warmup_autotune=True, device=None)
+    os.remove(tmp_path / "model.safetensors")
+    with pytest.raises(FileNotFoundError):
+        G.load_quant(str(tmp_path), warmup_autotune=False, device=None)
+
+
+def test_all_zero_bias_is_dropped(tmp_path):
+    cfg = make_checkpoint(tmp_path, -1)
+    from safetensors.torch import load_file, save_file
+    state = load_file(str(tmp_path / "model.safetensors"))
+    state["model.layers.0.self_attn.o_proj.bias"] = torch.zeros(256, dtype=torch.float16)
+    save_file(state, str(tmp_path / "model.safetensors"))
+    # a checkpoint with a bias tensor needs a bias buffer: build the skeleton by hand as the loader does
+    model = G.load_quant(str(tmp_path), warmup_autotune=False, device=None)
+    assert model.model.layers[0].self_attn.o_proj.bias is None
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("groupsize,act_order", [(-1, False), (128, False), (128, True)])
+def test_loaded_model_matches_cpu_reference(tmp_path, groupsize, act_order):
+    from oracle import decoder_ref
+    from safetensors.torch import load_file
+    cfg = make_checkpoint(tmp_path, groupsize, act_order=act_order, seed=7)
+    state = load_file(str(tmp_path / "model.safetensors"))
+    model = G.load_quant(str(tmp_path), device="cuda", fuse_mlp=True)
+    torch.manual_seed(1)
+    ids = torch.randint(0, cfg.vocab_size, (2, 40))
+    ref = decoder_ref.forward(state, cfg, groupsize, ids)
+    logits, _ = model(ids.cuda())
+    got = logits.float().cpu()
+    # fp16 activations through 2 layers against a float32 reference
+    err = (got - ref).abs()
+    assert err.max() < 0.05 * ref.abs().max() and err.mean() < 0.01 * ref.abs().mean() + 1e-3
+    assert (got.argmax(-1) == ref.argmax(-1)).float().mean() > 0.9
+
+    # incremental decoding with the KV cache equals the full forward
+    full, _ = model(ids.cuda())
+    part, past = model(ids[:, :30].cuda(), use_cache=True)
+    steps = [part]
+    for t in range(30, 40):
+        lg, past = model(ids[:, t:t + 1].cuda(), past_key_values=past, use_cache=True)
+        steps.append(lg)
+    inc = torch.cat(steps, dim=1)
+    assert (inc.float() - full.float()).abs().max() < 0.03 * full.float().abs().max()
+
+    # greedy generation with the preallocated cache follows the argmax of the full forward
+    out = model.generate_greedy(ids[:, :8].cuda(), 6)
+    assert out.shape == (2, 14) and torch.equal(out[:, :8].cpu(), ids[:, :8])
+    cur = ids[:, :8].cuda()
+    for _ in range(6):
+        lg, _ = model(cur)
+        cur = torch.cat([cur, lg[:, -1:].argmax(-1)], dim=1)
+    assert (out == cur).float().mean() > 0.9
