@@ -28,7 +28,7 @@ size_t partial_bytes(int splitk, int M, int ncols_total) {
 int setup_skinny(MatmulArgs &a, const SkinnyPlan &pl, int nmat, void *workspace, size_t workspace_bytes) {
     a.tiles = pl.tiles;
     a.splitk = pl.splitk;
-    const int nbatches = a.K / 128, slots = pl.splitk * 4;
+    const int nbatches = a.K / 128, slots = pl.splitk * pl.waves;
     a.slot_q = nbatches / slots;
     a.slot_rem = nbatches % slots;
     a.batches_per_group = a.groupsize / 128;
@@ -86,6 +86,8 @@ void gptq4_set_gemm_tuning(int mt, int splitk) {
     g_gemm_tuning.mt = (mt == 2 || mt == 4) ? mt : 0;
     g_gemm_tuning.splitk = splitk > 0 ? splitk : 0;
 }
+
+extern "C" void gptq4_dev_set_waves(int waves) { g_skinny_tuning.waves = (waves == 4 || waves == 8 || waves == 16) ? waves : 0; }
 
 void gptq4_set_tuning(int words, int depth, int splitk) {
     g_skinny_tuning.words = (words == 1 || words == 2 || words == 4) ? words : 0;

@@ -306,24 +306,35 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
                     for (int i = 0; i < 16; ++i) mine[(t * 16 + i) * 64 + lane] = acc[mt][t][i];
                 __syncthreads();
             }
+            // positions and table rows of the 16 rows this lane holds: all loads are
+            // unconditional (rows beyond M read row M-1) and issued together, so their
+            // latencies overlap instead of forming 16 dependent chains
+            float2 cs[16], sn[16];
+            if (which < 2) {
+                int pos[16];
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int row = min(wrow0 + mt * 32 + 8 * (i >> 2) + 4 * lhi + (i & 3), M - 1);
+                    pos[i] = min(max(r.position_ids[row], 0), r.max_pos - 1);
+                }
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    cs[i] = *reinterpret_cast<const float2 *>(r.cos_table + (size_t)pos[i] * 64 + 2 * l32);
+                    sn[i] = *reinterpret_cast<const float2 *>(r.sin_table + (size_t)pos[i] * 64 + 2 * l32);
+                }
+            }
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const int row = wrow0 + mt * 32 + 8 * (i >> 2) + 4 * lhi + (i & 3);
                 float o0 = acc[mt][0][i], o1 = acc[mt][1][i];
                 if (which < 2) {
                     const float p0 = theirs[(0 * 16 + i) * 64 + lane], p1 = theirs[(1 * 16 + i) * 64 + lane];
-                    float2 cs = make_float2(1.f, 1.f), sn = make_float2(0.f, 0.f);
-                    if (row < M) {
-                        const int pos = min(max(r.position_ids[row], 0), r.max_pos - 1);
-                        cs = *reinterpret_cast<const float2 *>(r.cos_table + (size_t)pos * 64 + 2 * l32);
-                        sn = *reinterpret_cast<const float2 *>(r.sin_table + (size_t)pos * 64 + 2 * l32);
-                    }
                     if (wn == 0) {
-                        o0 = o0 * cs.x - p0 * sn.x;
-                        o1 = o1 * cs.y - p1 * sn.y;
+                        o0 = o0 * cs[i].x - p0 * sn[i].x;
+                        o1 = o1 * cs[i].y - p1 * sn[i].y;
                     } else {
-                        o0 = o0 * cs.x + p0 * sn.x;
-                        o1 = o1 * cs.y + p1 * sn.y;
+                        o0 = o0 * cs[i].x + p0 * sn[i].x;
+                        o1 = o1 * cs[i].y + p1 * sn[i].y;
                     }
                 }
                 if (row < M) {
@@ -378,9 +389,9 @@ GemmPlan gemm_plan(int epi, int M, int N, int K) {
     int s = 1;
     if (g_gemm_tuning.splitk > 0) {
         s = g_gemm_tuning.splitk;
-    } else if (pl.tiles < 192) {
-        s = 512 / pl.tiles;   // aim for ~2 workgroups per CU
-        if (s > nk / 8) s = nk / 8;   // keep at least 8 K tiles (512 k) per split
+    } else if (pl.tiles < 384) {
+        s = (512 + pl.tiles / 2) / pl.tiles;  // aim for ~2 workgroups per CU
+        if (s > nk / 8) s = nk / 8;            // keep at least 8 K tiles (512 k) per split
     }
     if (s > GEMM_MAX_SPLITK) s = GEMM_MAX_SPLITK;
     if (s > nk) s = nk;

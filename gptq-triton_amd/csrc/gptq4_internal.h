@@ -35,10 +35,11 @@ struct SkinnyPlan {
     int words;   // packed words per lane and load: strip width = 16 * words columns
     int depth;   // batches of loads kept in flight per wave
     int splitk;  // workgroups sharing one tile
+    int waves;   // waves per workgroup (4, 8 or 16), each with its own K range
     int tiles;
 };
 struct SkinnyTuning {
-    int words, depth, splitk;  // 0 = automatic
+    int words, depth, splitk, waves;  // 0 = automatic
 };
 extern SkinnyTuning g_skinny_tuning;
 SkinnyPlan skinny_plan(int epi, int N, int K);

@@ -69,15 +69,15 @@ struct Batch {
     int group;
 };
 
-template <int EPI, int W, int DEPTH, bool PERM>
-__global__ __launch_bounds__(256) void gptq4_skinny_kernel(MatmulArgs p) {
+template <int EPI, int W, int DEPTH, bool PERM, int NW>
+__global__ __launch_bounds__(64 * NW) void gptq4_skinny_kernel(MatmulArgs p) {
     constexpr int NV = (EPI == EPI_PLAIN) ? 1 : 2;  // strips loaded per K step
     constexpr int SW = 16 * W;                      // strip width in columns
     constexpr int TILE_COLS = SW * NV;              // columns of the LDS tile
     constexpr int Q = SW / 16;                      // output elements per thread and row block
     constexpr int LINE_TILES = (SW >= 32) ? 1 : 32 / SW;  // tiles sharing a 128-byte row segment
 
-    __shared__ float red[4][SKINNY_MAX_M][TILE_COLS];
+    __shared__ float red[NW][SKINNY_MAX_M][TILE_COLS];
     __shared__ int s_is_last;
 
     const int tid = threadIdx.x;
@@ -100,7 +100,7 @@ __global__ __launch_bounds__(256) void gptq4_skinny_kernel(MatmulArgs p) {
 
     PHASE_STAMP(0);
     const int M = p.M, K = p.K, N = p.N;
-    const int slot = split * 4 + wave;
+    const int slot = split * NW + wave;
     const int b0 = slot * p.slot_q + min(slot, p.slot_rem);
     const int b1 = b0 + p.slot_q + (slot < p.slot_rem ? 1 : 0);
     const int bpg = p.batches_per_group;
@@ -252,7 +252,10 @@ __global__ __launch_bounds__(256) void gptq4_skinny_kernel(MatmulArgs p) {
         }
     __syncthreads();
 
-    // thread owns elements (row = (256/SW)*q + tid/SW, c = tid%SW), each with NV values
+    // the first 256 threads finish the tile: thread owns elements (row = (256/SW)*q + tid/SW,
+    // c = tid%SW), each with NV values
+    // (the other waves stay for the barriers below but own no rows)
+    const int Mf = (NW > 4 && tid >= 256) ? 0 : M;
     constexpr int ROWS_PER_PASS = 256 / SW;
     const int c = tid % SW;
     const int rbase = tid / SW;
@@ -263,8 +266,10 @@ __global__ __launch_bounds__(256) void gptq4_skinny_kernel(MatmulArgs p) {
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             float s = 0.f;
-            if (row < M)
-                s = ((red[0][row][v * SW + c] + red[1][row][v * SW + c]) + red[2][row][v * SW + c]) + red[3][row][v * SW + c];
+            if (row < Mf) {
+#pragma unroll
+                for (int w = 0; w < NW; ++w) s += red[w][row][v * SW + c];
+            }
             val[q][v] = s;
         }
     }
@@ -282,7 +287,7 @@ __global__ __launch_bounds__(256) void gptq4_skinny_kernel(MatmulArgs p) {
 #pragma unroll
         for (int q = 0; q < Q; ++q) {
             const int row = ROWS_PER_PASS * q + rbase;
-            if (row < M) {
+            if (row < Mf) {
 #pragma unroll
                 for (int v = 0; v < NV; ++v)
                     __hip_atomic_store(&mine[(size_t)row * TILE_COLS + v * SW + c], val[q][v], __ATOMIC_RELAXED,
@@ -303,7 +308,7 @@ __global__ __launch_bounds__(256) void gptq4_skinny_kernel(MatmulArgs p) {
 #pragma unroll
         for (int q = 0; q < Q; ++q) {
             const int row = ROWS_PER_PASS * q + rbase;
-            if (row < M) {
+            if (row < Mf) {
 #pragma unroll
                 for (int v = 0; v < NV; ++v) {
                     // all loads in flight at once, then a fixed-order sum
@@ -329,7 +334,7 @@ __global__ __launch_bounds__(256) void gptq4_skinny_kernel(MatmulArgs p) {
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
         const int row = ROWS_PER_PASS * q + rbase;
-        if (row >= M) continue;
+        if (row >= Mf) continue;
         if (EPI == EPI_PLAIN) {
             const int n = n0 + c;
             half_t o = (half_t)val[q][0];
@@ -372,39 +377,44 @@ __global__ __launch_bounds__(256) void gptq4_skinny_kernel(MatmulArgs p) {
     PHASE_STAMP(6);
 }
 
-template <int EPI, int W, int DEPTH>
+template <int EPI, int W, int DEPTH, int NW>
 int launch_variant(const MatmulArgs &a, hipStream_t stream) {
     constexpr int SW = 16 * W;
     constexpr int LINE_TILES = (SW >= 32) ? 1 : 32 / SW;
     const int per_xcd = 8 * LINE_TILES;
     const int groups = (a.tiles + per_xcd - 1) / per_xcd;
-    dim3 grid((unsigned)(groups * per_xcd), (unsigned)a.splitk), block(256);
+    dim3 grid((unsigned)(groups * per_xcd), (unsigned)a.splitk), block(64 * NW);
     if (a.perm == nullptr)
-        hipLaunchKernelGGL((gptq4_skinny_kernel<EPI, W, DEPTH, false>), grid, block, 0, stream, a);
+        hipLaunchKernelGGL((gptq4_skinny_kernel<EPI, W, DEPTH, false, NW>), grid, block, 0, stream, a);
     else
-        hipLaunchKernelGGL((gptq4_skinny_kernel<EPI, W, DEPTH, true>), grid, block, 0, stream, a);
+        hipLaunchKernelGGL((gptq4_skinny_kernel<EPI, W, DEPTH, true, NW>), grid, block, 0, stream, a);
     return (int)hipGetLastError();
 }
 
 template <int EPI>
-int launch_epi(const MatmulArgs &a, int words, int depth, hipStream_t stream) {
-    const int key = words * 10 + depth;
+int launch_epi(const MatmulArgs &a, const SkinnyPlan &pl, hipStream_t stream) {
+    const int key = pl.waves * 100 + pl.words * 10 + pl.depth;
     switch (key) {
-        case 11: return launch_variant<EPI, 1, 1>(a, stream);
-        case 12: return launch_variant<EPI, 1, 2>(a, stream);
-        case 14: return launch_variant<EPI, 1, 4>(a, stream);
-        case 21: return launch_variant<EPI, 2, 1>(a, stream);
-        case 22: return launch_variant<EPI, 2, 2>(a, stream);
-        case 24: return launch_variant<EPI, 2, 4>(a, stream);
-        case 41: return launch_variant<EPI, 4, 1>(a, stream);
-        case 42: return launch_variant<EPI, 4, 2>(a, stream);
-        default: return launch_variant<EPI, 4, 3>(a, stream);
+        case 412: return launch_variant<EPI, 1, 2, 4>(a, stream);
+        case 414: return launch_variant<EPI, 1, 4, 4>(a, stream);
+        case 421: return launch_variant<EPI, 2, 1, 4>(a, stream);
+        case 422: return launch_variant<EPI, 2, 2, 4>(a, stream);
+        case 424: return launch_variant<EPI, 2, 4, 4>(a, stream);
+        case 441: return launch_variant<EPI, 4, 1, 4>(a, stream);
+        case 442: return launch_variant<EPI, 4, 2, 4>(a, stream);
+        case 821: return launch_variant<EPI, 2, 1, 8>(a, stream);
+        case 822: return launch_variant<EPI, 2, 2, 8>(a, stream);
+        case 841: return launch_variant<EPI, 4, 1, 8>(a, stream);
+        case 842: return launch_variant<EPI, 4, 2, 8>(a, stream);
+        case 1621: return launch_variant<EPI, 2, 1, 16>(a, stream);
+        case 1622: return launch_variant<EPI, 2, 2, 16>(a, stream);
+        default: return launch_variant<EPI, 2, 2, 4>(a, stream);
     }
 }
 
 }  // namespace
 
-SkinnyTuning g_skinny_tuning = {0, 0, 0};
+SkinnyTuning g_skinny_tuning = {0, 0, 0, 0};
 
 // Launch shape for a small-M problem, from sweeps on MI355X: 8-byte loads (32-column
 // strips, full 128-byte lines per row) beat 16-byte loads because they give twice the
@@ -414,16 +424,17 @@ SkinnyPlan skinny_plan(int epi, int N, int K) {
     SkinnyPlan pl;
     pl.words = g_skinny_tuning.words > 0 ? g_skinny_tuning.words : 2;
     pl.depth = g_skinny_tuning.depth > 0 ? g_skinny_tuning.depth : (epi == EPI_SILU_MUL ? 1 : 2);
+    pl.waves = g_skinny_tuning.waves > 0 ? g_skinny_tuning.waves : 4;
     const int sw = 16 * pl.words;
     pl.tiles = (epi == EPI_ROPE) ? (N / 128) * (64 / sw) : N / sw;
     const int k_batches = K / 128;
     int s;
     if (g_skinny_tuning.splitk > 0) {
         s = g_skinny_tuning.splitk;
-        if (s > k_batches / 4) s = k_batches / 4;  // at least one batch per wave
+        if (s > k_batches / pl.waves) s = k_batches / pl.waves;  // at least one batch per wave
     } else {
         s = (1024 + pl.tiles - 1) / pl.tiles;
-        if (s > k_batches / 8) s = k_batches / 8;
+        if (s > k_batches / (2 * pl.waves)) s = k_batches / (2 * pl.waves);
     }
     if (s > SKINNY_MAX_SPLITK) s = SKINNY_MAX_SPLITK;
     if (s < 1) s = 1;
@@ -433,8 +444,8 @@ SkinnyPlan skinny_plan(int epi, int N, int K) {
 
 int launch_skinny(int epi, const MatmulArgs &a, const SkinnyPlan &pl, hipStream_t stream) {
     switch (epi) {
-        case EPI_PLAIN: return launch_epi<EPI_PLAIN>(a, pl.words, pl.depth, stream);
-        case EPI_SILU_MUL: return launch_epi<EPI_SILU_MUL>(a, pl.words, pl.depth, stream);
-        default: return launch_epi<EPI_ROPE>(a, pl.words, pl.depth, stream);
+        case EPI_PLAIN: return launch_epi<EPI_PLAIN>(a, pl, stream);
+        case EPI_SILU_MUL: return launch_epi<EPI_SILU_MUL>(a, pl, stream);
+        default: return launch_epi<EPI_ROPE>(a, pl, stream);
     }
 }
