@@ -13,7 +13,7 @@ import torch
 
 LIB_PATH = Path(__file__).resolve().parent / "csrc" / "libgptq4.so"
 ABI_VERSION = 1
-WS_COUNTER_BYTES = 16384
+WS_COUNTER_BYTES = 524288
 OP_MATMUL, OP_MLP_GATEUP, OP_QKV_ROTARY = 0, 1, 2
 
 # every symbol include/gptq4.h declares: (restype, argtypes)

@@ -41,6 +41,37 @@ int setup_skinny(MatmulArgs &a, const SkinnyPlan &pl, int nmat, void *workspace,
     return 0;
 }
 
+// M <= 16: the streaming kernel when it has a variant for the plan and its x slice fits
+// in LDS, the register-operand kernel otherwise.
+int run_small(int epi, MatmulArgs &a, int nmat, void *workspace, size_t workspace_bytes, hipStream_t s) {
+    if (a.M <= GEMV_MAX_M) {
+        const GemvPlan pl = gemv_plan(epi, a.M, a.N, a.K);
+        if (pl.ok) {
+            if (workspace == nullptr || workspace_bytes < GPTQ4_WS_COUNTER_BYTES + gemv_partial_bytes(pl, a.M, epi))
+                return -GPTQ4_E_WORKSPACE;
+            a.counters = reinterpret_cast<int *>(workspace);
+            a.partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_COUNTER_BYTES);
+            return launch_gemv(epi, a, pl, s);
+        }
+    }
+    if (g_stream_enabled) {
+        const SkinnyPlan pl = stream_plan(epi, a.M, a.N, a.K);
+        if (pl.splitk > 0) {
+            int rc = setup_skinny(a, pl, nmat, workspace, workspace_bytes);
+            if (rc) return rc;
+            const unsigned bpg = (unsigned)a.batches_per_group;
+            a.group_magic = bpg > 1 ? (uint32_t)(0x100000000ull / bpg + 1) : 0u;
+            a.m_shift = 0;
+            while ((1 << a.m_shift) < a.M) ++a.m_shift;
+            return launch_stream(epi, a, pl, s);
+        }
+    }
+    const SkinnyPlan pl = skinny_plan(epi, a.N, a.K);
+    int rc = setup_skinny(a, pl, nmat, workspace, workspace_bytes);
+    if (rc) return rc;
+    return launch_skinny(epi, a, pl, s);
+}
+
 // Fill the split-K fields of `a` for the tiled kernel.
 int setup_gemm(MatmulArgs &a, const GemmPlan &pl, void *workspace, size_t workspace_bytes) {
     a.tiles = pl.tiles;
@@ -88,6 +119,10 @@ void gptq4_set_gemm_tuning(int mt, int splitk) {
 }
 
 extern "C" void gptq4_dev_set_waves(int waves) { g_skinny_tuning.waves = (waves == 4 || waves == 8 || waves == 16) ? waves : 0; }
+extern "C" void gptq4_dev_set_stream(int on) { g_stream_enabled = on; }
+extern "C" void gptq4_dev_set_gemv(int enabled, int words, int depth, int waves, int waves_per_cu) {
+    g_gemv_tuning = GemvTuning{words, depth, waves, waves_per_cu, enabled};
+}
 
 void gptq4_set_tuning(int words, int depth, int splitk) {
     g_skinny_tuning.words = (words == 1 || words == 2 || words == 4) ? words : 0;
@@ -100,7 +135,13 @@ size_t gptq4_workspace_bytes(int op, int M, int K, int N) {
     if (M < 1 || N <= 0 || K <= 0) return bytes;
     if (M <= SKINNY_MAX_M) {
         const int cols = (op == GPTQ4_OP_MLP_GATEUP) ? 2 * N : N;
-        bytes += partial_bytes(SKINNY_MAX_SPLITK, M, cols);
+        size_t need = partial_bytes(SKINNY_MAX_SPLITK, M, cols);
+        if (M <= GEMV_MAX_M && (K % 128) == 0 && (N % 256) == 0) {
+            const int epi = (op == GPTQ4_OP_MLP_GATEUP) ? EPI_SILU_MUL : (op == GPTQ4_OP_QKV_ROTARY ? EPI_ROPE : EPI_PLAIN);
+            const GemvPlan pl = gemv_plan(epi, M, N, K);
+            if (pl.ok && gemv_partial_bytes(pl, M, epi) > need) need = gemv_partial_bytes(pl, M, epi);
+        }
+        bytes += need;
     } else if ((K % 64) == 0) {
         const int epi = (op == GPTQ4_OP_MLP_GATEUP) ? EPI_SILU_MUL : (op == GPTQ4_OP_QKV_ROTARY ? EPI_ROPE : EPI_PLAIN);
         bytes += gemm_partial_bytes(gemm_plan(epi, M, N, K));  // for the current (automatic or forced) plan
@@ -150,10 +191,7 @@ int gptq4_matmul(const void *x, const int32_t *qweight, const int32_t *qzeros, c
     a.groupsize = groupsize;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     if (M <= SKINNY_MAX_M) {
-        const SkinnyPlan pl = skinny_plan(EPI_PLAIN, N, K);
-        rc = setup_skinny(a, pl, 1, workspace, workspace_bytes);
-        if (rc) return rc;
-        return launch_skinny(EPI_PLAIN, a, pl, s);
+        return run_small(EPI_PLAIN, a, 1, workspace, workspace_bytes, s);
     }
     {
         const GemmPlan pl = gemm_plan(EPI_PLAIN, M, N, K);
@@ -189,10 +227,7 @@ int gptq4_mlp_gateup(const void *x, const int32_t *gate_qweight, const int32_t *
     a.groupsize = groupsize;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     if (M <= SKINNY_MAX_M) {
-        const SkinnyPlan pl = skinny_plan(EPI_SILU_MUL, I, K);
-        rc = setup_skinny(a, pl, 2, workspace, workspace_bytes);
-        if (rc) return rc;
-        return launch_skinny(EPI_SILU_MUL, a, pl, s);
+        return run_small(EPI_SILU_MUL, a, 2, workspace, workspace_bytes, s);
     }
     {
         const GemmPlan pl = gemm_plan(EPI_SILU_MUL, M, I, K);
@@ -246,10 +281,7 @@ int gptq4_qkv_rotary(const void *x, const int32_t *qweight, const int32_t *qzero
     a.rope.max_pos = max_pos;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     if (a.M <= SKINNY_MAX_M) {
-        const SkinnyPlan pl = skinny_plan(EPI_ROPE, N, K);
-        rc = setup_skinny(a, pl, 1, workspace, workspace_bytes);
-        if (rc) return rc;
-        return launch_skinny(EPI_ROPE, a, pl, s);
+        return run_small(EPI_ROPE, a, 1, workspace, workspace_bytes, s);
     }
     {
         const GemmPlan pl = gemm_plan(EPI_ROPE, a.M, N, K);

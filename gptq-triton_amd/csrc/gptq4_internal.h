@@ -27,6 +27,19 @@ struct MatmulArgs {
     // (64 k each) dealt to splitk splits the same way.
     int slot_q, slot_rem;
     int batches_per_group;  // groupsize / 128
+    int groups;             // K / groupsize
+    // streaming small-M kernel: batch -> group is umulhi(batch, group_magic) (exact for
+    // batch * batches_per_group < 2^32; unused when batches_per_group == 1), and x rows
+    // are dealt to threads in blocks of (threads >> m_shift), 1 << m_shift >= M
+    uint32_t group_magic;
+    int m_shift;
+    // balanced GEMV: units = tiles * nb are dealt to waves, slot_q each and one more for
+    // the first slot_rem; reciprocals (floor(2^32 / d) + 1) of nb, slot_q, slot_q + 1
+    int nb;
+    uint32_t nb_magic, q_magic, q1_magic;
+    int lds_wave_chunks;  // 16-byte chunks of LDS per wave
+    int x_chunks_max;     // chunks of the largest x slice: (slot_q + 1) << (4 + m_shift)
+    int max_contrib;      // partial-sum slots per tile
     RopeArgs rope;          // EPI_ROPE only
 };
 
@@ -45,6 +58,30 @@ extern SkinnyTuning g_skinny_tuning;
 SkinnyPlan skinny_plan(int epi, int N, int K);
 // Small-M (M <= 16) split-K matrix-core GEMV.  Returns hipError_t.
 int launch_skinny(int epi, const MatmulArgs &a, const SkinnyPlan &plan, hipStream_t stream);
+// Streaming small-M kernel (x staged in LDS, scale/zero applied to the accumulator).
+extern int g_stream_enabled;
+SkinnyPlan stream_plan(int epi, int M, int N, int K);
+bool stream_has_variant(const SkinnyPlan &plan);
+size_t stream_lds_bytes(int epi, int M, int K, const SkinnyPlan &plan);
+int launch_stream(int epi, const MatmulArgs &a, const SkinnyPlan &plan, hipStream_t stream);
+// Balanced decode GEMV (M <= GEMV_MAX_M): (tile, batch) units dealt evenly to waves.
+struct GemvPlan {
+    int words, depth, waves;  // words per lane and load, units in flight, waves per workgroup
+    int tiles, nb;            // column tiles, 128-k batches per tile
+    int workgroups;
+    int q, r;                 // units per wave, waves with one more
+    int m_shift, lds_wave_chunks, max_contrib;
+    size_t lds_bytes;
+    bool ok;                  // false: use another kernel
+};
+struct GemvTuning {
+    int words, depth, waves, waves_per_cu;  // 0 = automatic
+    int enabled;
+};
+extern GemvTuning g_gemv_tuning;
+GemvPlan gemv_plan(int epi, int M, int N, int K);
+size_t gemv_partial_bytes(const GemvPlan &plan, int M, int epi);
+int launch_gemv(int epi, MatmulArgs &a, const GemvPlan &plan, hipStream_t stream);
 // Launch shape of the tiled kernel.
 struct GemmPlan {
     int mt;      // row tiles per wave: workgroup tile = (64 * mt) rows
@@ -68,4 +105,7 @@ int launch_sort_rows(const uint32_t *qweight, const int32_t *perm, uint32_t *out
 int launch_rope_table(float *cos_out, float *sin_out, int max_pos, int D, float base,
                       hipStream_t stream);
 
-enum { SKINNY_MAX_M = 16, SKINNY_MAX_SPLITK = 16, SKINNY_MAX_TILES = 4096, GEMM_MAX_SPLITK = 16 };
+// arrival counters sit one per 128-byte line: atomics on one line are served one after
+// the other by the memory side
+enum { COUNTER_STRIDE = 32 };
+enum { GEMV_MAX_M = 4, SKINNY_MAX_M = 16, SKINNY_MAX_SPLITK = 16, SKINNY_MAX_TILES = 4096, GEMM_MAX_SPLITK = 16 };

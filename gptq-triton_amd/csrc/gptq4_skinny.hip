@@ -32,8 +32,8 @@
 #define PHASE_STAMP(i)                                                                     \
     do {                                                                                   \
         if (threadIdx.x == 0)                                                              \
-            reinterpret_cast<unsigned long long *>(reinterpret_cast<char *>(p.counters) + (32 << 20))[blockIdx.x * 8 + (i)] = \
-                __builtin_readcyclecounter();                                              \
+            reinterpret_cast<unsigned long long *>(reinterpret_cast<char *>(p.counters) + (32 << 20))[(blockIdx.y * gridDim.x + blockIdx.x) * 8 + (i)] = \
+                wall_clock64();                                                            \
     } while (0)
 #else
 #define PHASE_STAMP(i)
@@ -298,7 +298,7 @@ __global__ __launch_bounds__(64 * NW) void gptq4_skinny_kernel(MatmulArgs p) {
         PHASE_STAMP(3);
         __syncthreads();
         if (tid == 0) {
-            const int old = __hip_atomic_fetch_add(&p.counters[tile], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const int old = __hip_atomic_fetch_add(&p.counters[tile * COUNTER_STRIDE], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             s_is_last = (old == p.splitk - 1);
         }
         __syncthreads();
@@ -327,7 +327,7 @@ __global__ __launch_bounds__(64 * NW) void gptq4_skinny_kernel(MatmulArgs p) {
             }
         }
         PHASE_STAMP(5);
-        if (tid == 0) __hip_atomic_store(&p.counters[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (tid == 0) __hip_atomic_store(&p.counters[tile * COUNTER_STRIDE], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 
     // ---- epilogue

@@ -49,7 +49,7 @@ extern "C" {
 #define GPTQ4_E_WORKSPACE 4  /* workspace NULL or smaller than required          */
 #define GPTQ4_E_ALIGN 5      /* a pointer is not 16-byte aligned                 */
 
-#define GPTQ4_WS_COUNTER_BYTES 16384
+#define GPTQ4_WS_COUNTER_BYTES 524288
 
 /* operation selector for gptq4_workspace_bytes */
 #define GPTQ4_OP_MATMUL 0
