@@ -29,6 +29,7 @@ SIGNATURES = {
     "gptq4_qkv_rotary": (c_int, [c_void_p] * 8 + [c_int] + [c_void_p] * 3 + [c_int] * 8 + [c_void_p, c_size_t, c_void_p]),
     "gptq4_set_tuning": (None, [c_int, c_int, c_int]),
     "gptq4_set_gemm_tuning": (None, [c_int, c_int]),
+    "gptq4_set_gemv_tuning": (None, [c_int, c_int, c_int, c_int]),
 }
 
 

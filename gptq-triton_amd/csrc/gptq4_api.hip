@@ -41,8 +41,8 @@ int setup_skinny(MatmulArgs &a, const SkinnyPlan &pl, int nmat, void *workspace,
     return 0;
 }
 
-// M <= 16: the streaming kernel when it has a variant for the plan and its x slice fits
-// in LDS, the register-operand kernel otherwise.
+// M <= 16: the balanced GEMV where its plan says so (by default the one-row gate/up pair),
+// the split-K kernel otherwise.
 int run_small(int epi, MatmulArgs &a, int nmat, void *workspace, size_t workspace_bytes, hipStream_t s) {
     if (a.M <= GEMV_MAX_M) {
         const GemvPlan pl = gemv_plan(epi, a.M, a.N, a.K);
@@ -52,18 +52,6 @@ int run_small(int epi, MatmulArgs &a, int nmat, void *workspace, size_t workspac
             a.counters = reinterpret_cast<int *>(workspace);
             a.partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_COUNTER_BYTES);
             return launch_gemv(epi, a, pl, s);
-        }
-    }
-    if (g_stream_enabled) {
-        const SkinnyPlan pl = stream_plan(epi, a.M, a.N, a.K);
-        if (pl.splitk > 0) {
-            int rc = setup_skinny(a, pl, nmat, workspace, workspace_bytes);
-            if (rc) return rc;
-            const unsigned bpg = (unsigned)a.batches_per_group;
-            a.group_magic = bpg > 1 ? (uint32_t)(0x100000000ull / bpg + 1) : 0u;
-            a.m_shift = 0;
-            while ((1 << a.m_shift) < a.M) ++a.m_shift;
-            return launch_stream(epi, a, pl, s);
         }
     }
     const SkinnyPlan pl = skinny_plan(epi, a.N, a.K);
@@ -118,13 +106,16 @@ void gptq4_set_gemm_tuning(int mt, int splitk) {
     g_gemm_tuning.splitk = splitk > 0 ? splitk : 0;
 }
 
-extern "C" void gptq4_dev_set_waves(int waves) { g_skinny_tuning.waves = (waves == 4 || waves == 8 || waves == 16) ? waves : 0; }
-extern "C" void gptq4_dev_set_stream(int on) { g_stream_enabled = on; }
-extern "C" void gptq4_dev_set_gemv(int enabled, int words, int depth, int waves, int waves_per_cu) {
-    g_gemv_tuning = GemvTuning{words, depth, waves, waves_per_cu, enabled};
+void gptq4_set_gemv_tuning(int mode, int depth, int waves, int waves_per_cu) {
+    g_gemv_tuning.mode = (mode >= 0 && mode <= 2) ? mode : 1;
+    g_gemv_tuning.depth = (depth == 2 || depth == 3) ? depth : 0;
+    g_gemv_tuning.waves = (waves == 4 || waves == 8 || waves == 16) ? waves : 0;
+    g_gemv_tuning.waves_per_cu = (waves_per_cu >= 4 && waves_per_cu <= 32) ? waves_per_cu : 0;
 }
+static_assert(GPTQ4_WS_COUNTER_BYTES == SKINNY_MAX_TILES * COUNTER_STRIDE * 4, "one counter line per tile");
 
 void gptq4_set_tuning(int words, int depth, int splitk) {
+    g_skinny_tuning.waves = 0;
     g_skinny_tuning.words = (words == 1 || words == 2 || words == 4) ? words : 0;
     g_skinny_tuning.depth = (depth >= 1 && depth <= 4) ? depth : 0;
     g_skinny_tuning.splitk = splitk > 0 ? splitk : 0;

@@ -61,21 +61,10 @@ __device__ __forceinline__ void decode_word(uint32_t w, const ColDecode &c, h2_t
     const h2_t hi0 = as_h2(and_or_b32(w, 0x00F000F0u, magic));
     const h2_t lo1 = as_h2(and_or_b32(w8, 0x000F000Fu, magic));
     const h2_t hi1 = as_h2(and_or_b32(w8, 0x00F000F0u, magic));
-#if defined(GPTQ4_EXP) && GPTQ4_EXP == 1
-    out[0] = (lo0 + c.neg_lo);
-    out[1] = __builtin_elementwise_fma(hi0, sixteenth, c.neg_hi);
-    out[2] = (lo1 + c.neg_lo);
-    out[3] = __builtin_elementwise_fma(hi1, sixteenth, c.neg_hi);
-#elif defined(GPTQ4_EXP) && GPTQ4_EXP == 2
-    out[0] = lo0; out[1] = hi0; out[2] = lo1; out[3] = hi1;
-#elif defined(GPTQ4_EXP) && GPTQ4_EXP == 3
-    out[0] = as_h2(w); out[1] = as_h2(w8); out[2] = as_h2(w); out[3] = as_h2(w8);
-#else
     out[0] = (lo0 + c.neg_lo) * c.scale;
     out[1] = __builtin_elementwise_fma(hi0, sixteenth, c.neg_hi) * c.scale;
     out[2] = (lo1 + c.neg_lo) * c.scale;
     out[3] = __builtin_elementwise_fma(hi1, sixteenth, c.neg_hi) * c.scale;
-#endif
 }
 
 __device__ __forceinline__ h8_t decode_word_h8(uint32_t w, const ColDecode &c) {

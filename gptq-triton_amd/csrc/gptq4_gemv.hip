@@ -402,17 +402,16 @@ uint32_t magic_of(int d) { return d > 1 ? (uint32_t)(0x100000000ull / (unsigned)
 
 }  // namespace
 
-GemvTuning g_gemv_tuning = {0, 0, 0, 0, 1};
+GemvTuning g_gemv_tuning = {1, 0, 0, 0};
 
 // Launch shape: the grid holds `waves_per_cu` waves per CU on all 256 CUs (or fewer
 // waves when there are fewer units than that), each wave owning q or q+1 units.
 GemvPlan gemv_plan(int epi, int M, int N, int K) {
     GemvPlan pl = {};
-    pl.words = 2;
     pl.depth = g_gemv_tuning.depth > 0 ? g_gemv_tuning.depth : 2;
-    pl.waves = g_gemv_tuning.waves > 0 ? g_gemv_tuning.waves : 8;
+    pl.waves = g_gemv_tuning.waves > 0 ? g_gemv_tuning.waves : 4;
     const int waves_per_cu = g_gemv_tuning.waves_per_cu > 0 ? g_gemv_tuning.waves_per_cu : 8;
-    const int sw = 16 * pl.words;
+    const int sw = 32;
     pl.tiles = (epi == EPI_ROPE) ? (N / 128) * (64 / sw) : N / sw;
     pl.nb = K / 128;
     const long units = (long)pl.tiles * pl.nb;
@@ -422,7 +421,12 @@ GemvPlan gemv_plan(int epi, int M, int N, int K) {
     total_waves = (long)pl.workgroups * pl.waves;
     pl.q = (int)(units / total_waves);
     pl.r = (int)(units % total_waves);
-    pl.ok = g_gemv_tuning.enabled && M >= 1 && M <= GEMV_MAX_M && pl.tiles <= SKINNY_MAX_TILES && pl.q + 1 <= pl.nb &&
+    // measured on MI355X at LLaMA-7B shapes: ahead of the split-K kernel for the one-row
+    // gate/up pair (344 tiles, the shape that divides worst by 256 CUs: 16.0 against
+    // 17.0 us), level with it for the one-row plain projections and behind it for more
+    // rows and for the rotary epilogue
+    const bool wanted = g_gemv_tuning.mode == 2 || (g_gemv_tuning.mode == 1 && M == 1 && epi == EPI_SILU_MUL);
+    pl.ok = wanted && M >= 1 && M <= GEMV_MAX_M && pl.tiles <= SKINNY_MAX_TILES && pl.q + 1 <= pl.nb &&
             units < (1L << 24) && (long)K * N < (1L << 32) && (long)M * K < (1L << 30);
     int mshift = 0;
     while ((1 << mshift) < M) ++mshift;
@@ -445,7 +449,7 @@ GemvPlan gemv_plan(int epi, int M, int N, int K) {
 }
 
 size_t gemv_partial_bytes(const GemvPlan &pl, int M, int epi) {
-    const int tile_cols = 16 * pl.words * (epi == EPI_PLAIN ? 1 : 2);
+    const int tile_cols = 32 * (epi == EPI_PLAIN ? 1 : 2);
     return (size_t)pl.tiles * pl.max_contrib * M * tile_cols * sizeof(float);
 }
 

@@ -28,13 +28,12 @@ struct MatmulArgs {
     int slot_q, slot_rem;
     int batches_per_group;  // groupsize / 128
     int groups;             // K / groupsize
-    // streaming small-M kernel: batch -> group is umulhi(batch, group_magic) (exact for
-    // batch * batches_per_group < 2^32; unused when batches_per_group == 1), and x rows
-    // are dealt to threads in blocks of (threads >> m_shift), 1 << m_shift >= M
+    // balanced GEMV: units = tiles * nb are dealt to waves, slot_q each and one more for
+    // the first slot_rem.  Divisions run through host-made reciprocals floor(2^32 / d) + 1:
+    // of batches_per_group (batch -> group), nb, slot_q and slot_q + 1.  The x slice of a
+    // wave has 1 << m_shift >= M rows per unit.
     uint32_t group_magic;
     int m_shift;
-    // balanced GEMV: units = tiles * nb are dealt to waves, slot_q each and one more for
-    // the first slot_rem; reciprocals (floor(2^32 / d) + 1) of nb, slot_q, slot_q + 1
     int nb;
     uint32_t nb_magic, q_magic, q1_magic;
     int lds_wave_chunks;  // 16-byte chunks of LDS per wave
@@ -58,15 +57,9 @@ extern SkinnyTuning g_skinny_tuning;
 SkinnyPlan skinny_plan(int epi, int N, int K);
 // Small-M (M <= 16) split-K matrix-core GEMV.  Returns hipError_t.
 int launch_skinny(int epi, const MatmulArgs &a, const SkinnyPlan &plan, hipStream_t stream);
-// Streaming small-M kernel (x staged in LDS, scale/zero applied to the accumulator).
-extern int g_stream_enabled;
-SkinnyPlan stream_plan(int epi, int M, int N, int K);
-bool stream_has_variant(const SkinnyPlan &plan);
-size_t stream_lds_bytes(int epi, int M, int K, const SkinnyPlan &plan);
-int launch_stream(int epi, const MatmulArgs &a, const SkinnyPlan &plan, hipStream_t stream);
 // Balanced decode GEMV (M <= GEMV_MAX_M): (tile, batch) units dealt evenly to waves.
 struct GemvPlan {
-    int words, depth, waves;  // words per lane and load, units in flight, waves per workgroup
+    int depth, waves;         // units in flight per wave, waves per workgroup
     int tiles, nb;            // column tiles, 128-k batches per tile
     int workgroups;
     int q, r;                 // units per wave, waves with one more
@@ -75,8 +68,8 @@ struct GemvPlan {
     bool ok;                  // false: use another kernel
 };
 struct GemvTuning {
-    int words, depth, waves, waves_per_cu;  // 0 = automatic
-    int enabled;
+    int mode;                        // 0 never, 1 where it is the faster kernel, 2 wherever it can run
+    int depth, waves, waves_per_cu;  // 0 = automatic
 };
 extern GemvTuning g_gemv_tuning;
 GemvPlan gemv_plan(int epi, int M, int N, int K);

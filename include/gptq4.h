@@ -131,6 +131,12 @@ void gptq4_set_tuning(int words, int depth, int splitk);
  * the split-K factor; 0 = automatic. */
 void gptq4_set_gemm_tuning(int mt, int splitk);
 
+/* Same for the balanced decode GEMV (M <= 4): mode 0 = never use it, 1 = where it is the
+ * faster kernel (one row, SiLU*mul epilogue), 2 = wherever it can run; units in
+ * flight per wave (2, 3), waves per workgroup (4, 8, 16), waves per CU (4..32), 0 =
+ * automatic. */
+void gptq4_set_gemv_tuning(int mode, int depth, int waves, int waves_per_cu);
+
 #ifdef __cplusplus
 }
 #endif
