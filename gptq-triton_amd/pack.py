@@ -8,7 +8,9 @@ is the true zero minus one.  `quantize_rtn` is the published round-to-nearest mi
 quantiser (the GPTQ paper's baseline, what the reference's `dumbquant` applies,
 quantize.py:294-329): per output channel and group, scale = (max - min) / 15 with the
 range widened to include 0, zero = round(-min / scale).
-CPU-side, load-time code; not on the inference path.
+CPU-side, load-time code; not on the inference path.  The bit layout is pinned by round trips
+through the unpackers; the rounding of the computed quotients is parity unpinned (the
+reference holds no vectors for it).
 """
 from __future__ import annotations
 
