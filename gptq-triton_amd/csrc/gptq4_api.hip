@@ -242,7 +242,8 @@ int gptq4_qkv_rotary(const void *x, const int32_t *qweight, const int32_t *qzero
     if (!x || !qweight || !qzeros || !scales || !position_ids || !cos_table || !sin_table || !q || !k || !v)
         return -GPTQ4_E_NULL;
     if (B < 1 || S < 1 || H < 1 || D != 128 || max_pos < 1) return -GPTQ4_E_SHAPE;
-    if (kv_offset < 0 || kv_capacity < kv_offset + S) return -GPTQ4_E_SHAPE;
+    if (kv_offset < GPTQ4_KV_AT_POSITION || kv_capacity < 1 || (kv_offset >= 0 && kv_capacity < kv_offset + S))
+        return -GPTQ4_E_SHAPE;
     if ((long)B * S > 0x7fffffffL) return -GPTQ4_E_SHAPE;
     const int N = 3 * H * D;
     int rc = check_dims(K, N, &groupsize);

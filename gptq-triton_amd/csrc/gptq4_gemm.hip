@@ -347,7 +347,9 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
                         off = ((size_t)(bb * r.H + head) * r.S + srow) * 128;
                     } else {
                         dst = (which == 1) ? r.k : r.v;
-                        off = ((size_t)(bb * r.H + head) * r.kv_capacity + r.kv_offset + srow) * 128;
+                        // kv_offset < 0: the cache row is the token's position
+                        const int crow = r.kv_offset >= 0 ? r.kv_offset + srow : min(max(r.position_ids[row], 0), r.kv_capacity - 1);
+                        off = ((size_t)(bb * r.H + head) * r.kv_capacity + crow) * 128;
                     }
                     const h2_t o = {(half_t)o0, (half_t)o1};
                     *reinterpret_cast<uint32_t *>(dst + off + 64 * wn + 2 * l32) = as_u32(o);

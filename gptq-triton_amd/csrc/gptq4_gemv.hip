@@ -364,7 +364,9 @@ __global__ __launch_bounds__(64 * NW) void gptq4_gemv_kernel(MatmulArgs p) {
                         off = ((size_t)(bb * ra.H + head) * ra.S + ss) * 128;
                     } else {
                         dst = (which == 1) ? ra.k : ra.v;
-                        off = ((size_t)(bb * ra.H + head) * ra.kv_capacity + ra.kv_offset + ss) * 128;
+                        // kv_offset < 0: the cache row is the token's position
+                        const int crow = ra.kv_offset >= 0 ? ra.kv_offset + ss : min(max(ra.position_ids[row], 0), ra.kv_capacity - 1);
+                        off = ((size_t)(bb * ra.H + head) * ra.kv_capacity + crow) * 128;
                     }
                     dst[off + dd] = (half_t)o1;
                     dst[off + 64 + dd] = (half_t)o2;

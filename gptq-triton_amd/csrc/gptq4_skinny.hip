@@ -368,7 +368,9 @@ __global__ __launch_bounds__(64 * NW) void gptq4_skinny_kernel(MatmulArgs p) {
                 off = ((size_t)(bb * r.H + head) * r.S + ss) * 128;
             } else {
                 dst = (which == 1) ? r.k : r.v;
-                off = ((size_t)(bb * r.H + head) * r.kv_capacity + r.kv_offset + ss) * 128;
+                // kv_offset < 0: the cache row is the token's position
+                const int crow = r.kv_offset >= 0 ? r.kv_offset + ss : min(max(r.position_ids[row], 0), r.kv_capacity - 1);
+                off = ((size_t)(bb * r.H + head) * r.kv_capacity + crow) * 128;
             }
             dst[off + d] = (half_t)o1;
             dst[off + 64 + d] = (half_t)o2;

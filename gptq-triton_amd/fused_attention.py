@@ -58,6 +58,9 @@ class RotaryTable:
         return tab
 
 
+KV_AT_POSITION = -1  # GPTQ4_KV_AT_POSITION of the C ABI
+
+
 def qkv_rotary(groupsize: int, hidden_states: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor,
                qzeros: torch.Tensor, position_ids: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
                num_heads: int, head_dim: int = 128, perm: Optional[torch.Tensor] = None,
@@ -65,7 +68,9 @@ def qkv_rotary(groupsize: int, hidden_states: torch.Tensor, qweight: torch.Tenso
     """hidden_states fp16 [B, S, K]; packed weights with N = 3*H*D in q, k, v order.
     Returns (q, k, v): q [B,H,S,D] rotated; k, v [B,H,S,D], or - when `kv_out` gives
     preallocated [B,H,cap,D] buffers - those buffers with rows kv_offset..kv_offset+S
-    filled.  position_ids int [B, S] index the cos/sin tables."""
+    filled (kv_offset = KV_AT_POSITION: row position_ids[b, s] for token (b, s), so that a
+    decode step has no host-side scalar that changes from token to token).
+    position_ids int [B, S] index the cos/sin tables."""
     k_in, n = _check_matmul_args(hidden_states, qweight, groupsize)
     _check_device_tensors(hidden_states, qweight, scales, qzeros, perm, cos, sin)
     if hidden_states.dim() != 3:
@@ -74,7 +79,9 @@ def qkv_rotary(groupsize: int, hidden_states: torch.Tensor, qweight: torch.Tenso
     if n != 3 * num_heads * head_dim:
         raise ValueError(f"packed QKV has {n} columns, expected 3*{num_heads}*{head_dim}")
     dev = hidden_states.device
-    pos = position_ids.to(device=dev, dtype=torch.int32).expand(bsz, q_len).contiguous()
+    pos = position_ids
+    if pos.dtype != torch.int32 or pos.device != dev or tuple(pos.shape) != (bsz, q_len) or not pos.is_contiguous():
+        pos = position_ids.to(device=dev, dtype=torch.int32).expand(bsz, q_len).contiguous()
     q = torch.empty((bsz, num_heads, q_len, head_dim), dtype=torch.float16, device=dev)
     if kv_out is None:
         kk = torch.empty_like(q)
@@ -84,7 +91,7 @@ def qkv_rotary(groupsize: int, hidden_states: torch.Tensor, qweight: torch.Tenso
         kk, vv = kv_out
         cap, off = kk.shape[2], kv_offset
         if kk.shape != vv.shape or kk.shape[0] != bsz or kk.shape[1] != num_heads or kk.shape[3] != head_dim \
-                or not kk.is_contiguous() or not vv.is_contiguous() or off + q_len > cap:
+                or not kk.is_contiguous() or not vv.is_contiguous() or off < KV_AT_POSITION or off + q_len > cap:
             raise ValueError("kv_out buffers must be contiguous [B, H, capacity, D] with room for the new rows")
     if bsz * q_len == 0:
         return q, kk, vv
@@ -162,7 +169,7 @@ class QuantLlamaAttention(nn.Module):
 
     def project_qkv(self, hidden_states: torch.Tensor, position_ids: torch.Tensor,
                     kv_out=None, kv_offset: int = 0):
-        need = kv_offset + hidden_states.shape[1]
+        need = max(kv_offset, 0) + hidden_states.shape[1]
         cos, sin = self.rope.get(hidden_states.device, max(need, self.max_position_embeddings))
         qweight, perm = self.qkv_proj.kernel_weights()
         return qkv_rotary(self.qkv_proj.groupsize, hidden_states, qweight, self.qkv_proj.scales,

@@ -140,33 +140,114 @@ class LlamaForCausalLM(nn.Module):
         return self.lm_head(h), (presents if use_cache else None)
 
     @torch.no_grad()
-    def generate_greedy(self, input_ids: torch.Tensor, max_new_tokens: int) -> torch.Tensor:
+    def generate_greedy(self, input_ids: torch.Tensor, max_new_tokens: int, use_graph: bool = False) -> torch.Tensor:
         """Prefill + greedy decode with a preallocated KV cache: the fused QKV kernel writes
-        rotated K and V straight into the cache (no cat, no copies)."""
+        rotated K and V straight into the cache (no cat, no copies).  use_graph replays one
+        captured HIP graph per decode token instead of launching the step's kernels one by
+        one."""
         bsz, prompt = input_ids.shape
-        dev = input_ids.device
-        cfg = self.config
+        dec = GreedyDecoder(self, bsz, prompt + max_new_tokens)
+        first = dec.prefill(input_ids)
+        rest = dec.decode(max_new_tokens - 1, use_graph=use_graph) if max_new_tokens > 1 else first[:, :0]
+        return torch.cat([input_ids, first, rest], dim=1)
+
+
+class GreedyDecoder:
+    """Greedy generation state for one batch: KV caches of fixed capacity plus the static
+    token / position buffers a decode step reads and writes.  Nothing in a decode step
+    depends on a host-side value that changes from token to token (the QKV kernel places
+    K and V by position id, attention runs over the whole cache under a mask derived from
+    the position), so the step can be captured once as a HIP graph and replayed."""
+
+    def __init__(self, model: LlamaForCausalLM, bsz: int, capacity: int):
+        cfg = model.config
+        self.model, self.bsz, self.capacity = model, bsz, capacity
+        dev = model.lm_head.weight.device
         heads, hd = cfg.num_attention_heads, cfg.hidden_size // cfg.num_attention_heads
-        cap = prompt + max_new_tokens
-        caches = [(torch.empty((bsz, heads, cap, hd), dtype=torch.float16, device=dev),
-                   torch.empty((bsz, heads, cap, hd), dtype=torch.float16, device=dev)) for _ in self.model.layers]
-        out = [input_ids]
-        tokens, cur = input_ids, 0
-        for step in range(max_new_tokens):
-            q_len = tokens.shape[1]
-            position_ids = torch.arange(cur, cur + q_len, device=dev).unsqueeze(0)
-            mask = causal_mask(q_len, cur + q_len, dev)
-            h = self.model.embed_tokens(tokens)
-            for layer, (kc, vc) in zip(self.model.layers, caches):
-                x = layer.input_layernorm(h)
-                attn = layer.self_attn
-                q, _, _ = attn.project_qkv(x, position_ids, kv_out=(kc, vc), kv_offset=cur)
-                o = torch.nn.functional.scaled_dot_product_attention(q, kc[:, :, :cur + q_len], vc[:, :, :cur + q_len],
-                                                                     attn_mask=mask)
-                h = h + attn.o_proj(o.transpose(1, 2).reshape(bsz, q_len, cfg.hidden_size))
-                h = h + layer.mlp(layer.post_attention_layernorm(h))
-            logits = self.lm_head(self.model.norm(h[:, -1:, :]))
-            tokens = logits.argmax(-1)
-            out.append(tokens)
-            cur += q_len
-        return torch.cat(out, dim=1)
+        self.caches = [(torch.zeros((bsz, heads, capacity, hd), dtype=torch.float16, device=dev),
+                        torch.zeros((bsz, heads, capacity, hd), dtype=torch.float16, device=dev))
+                       for _ in model.model.layers]
+        self.tokens = torch.zeros((bsz, 1), dtype=torch.long, device=dev)
+        self.position = torch.zeros((bsz, 1), dtype=torch.int32, device=dev)
+        self.slots = torch.arange(capacity, device=dev, dtype=torch.int32)[None, None, None, :]
+        self.graph = None
+
+    def _layers(self, h, position_ids, kv_offset, attend):
+        cfg = self.model.config
+        bsz, q_len, _ = h.shape
+        for layer, (kc, vc) in zip(self.model.model.layers, self.caches):
+            attn = layer.self_attn
+            q, _, _ = attn.project_qkv(layer.input_layernorm(h), position_ids, kv_out=(kc, vc), kv_offset=kv_offset)
+            o = attend(q, kc, vc)
+            h = h + attn.o_proj(o.transpose(1, 2).reshape(bsz, q_len, cfg.hidden_size))
+            h = h + layer.mlp(layer.post_attention_layernorm(h))
+        return self.model.lm_head(self.model.model.norm(h[:, -1:, :])).argmax(-1)
+
+    @torch.no_grad()
+    def prefill(self, input_ids: torch.Tensor) -> torch.Tensor:
+        """Run the prompt (positions 0..S-1), fill the caches, return the first new token [B, 1]."""
+        bsz, prompt = input_ids.shape
+        if bsz != self.bsz or prompt >= self.capacity:
+            raise ValueError("prompt does not fit this decoder's batch size / capacity")
+        dev = input_ids.device
+        position_ids = torch.arange(prompt, device=dev, dtype=torch.int32).unsqueeze(0).expand(bsz, prompt).contiguous()
+        sdpa = torch.nn.functional.scaled_dot_product_attention
+
+        def attend(q, kc, vc):
+            return sdpa(q, kc[:, :, :prompt], vc[:, :, :prompt], is_causal=prompt > 1)
+
+        nxt = self._layers(self.model.model.embed_tokens(input_ids), position_ids, 0, attend)
+        self.tokens.copy_(nxt)
+        self.position.fill_(prompt)
+        return nxt
+
+    def _step(self):
+        """One decode token from the static buffers: reads tokens/position, writes them back."""
+        from .fused_attention import KV_AT_POSITION
+        mask = torch.zeros((self.bsz, 1, 1, self.capacity), dtype=torch.float16, device=self.tokens.device)
+        mask.masked_fill_(self.slots > self.position[:, None, None, :], torch.finfo(torch.float16).min)
+        sdpa = torch.nn.functional.scaled_dot_product_attention
+
+        def attend(q, kc, vc):
+            return sdpa(q, kc, vc, attn_mask=mask)
+
+        nxt = self._layers(self.model.model.embed_tokens(self.tokens), self.position, KV_AT_POSITION, attend)
+        self.tokens.copy_(nxt)
+        self.position.add_(1)
+
+    @torch.no_grad()
+    def decode(self, steps: int, use_graph: bool = False) -> torch.Tensor:
+        """`steps` more greedy tokens after prefill -> [B, steps]."""
+        out = torch.empty((self.bsz, steps), dtype=torch.long, device=self.tokens.device)
+        if int(self.position.max()) + steps > self.capacity:
+            raise ValueError("decode would run past the cache capacity")
+        if use_graph and self.graph is None and steps > 0:
+            self._capture()
+        for i in range(steps):
+            if use_graph:
+                self.graph.replay()
+            else:
+                self._step()
+            out[:, i:i + 1].copy_(self.tokens)
+        return out
+
+    def _capture(self):
+        """Capture _step as a graph.  The warm-up steps run on the capture stream first, so
+        workspaces and tables exist before capture; their effect on tokens, position and the
+        cache rows they wrote is undone (the rows lie beyond the current position and are
+        rewritten before any later step attends to them)."""
+        tokens0, position0 = self.tokens.clone(), self.position.clone()
+        side = torch.cuda.Stream(device=self.tokens.device)
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            self._step()
+            self.tokens.copy_(tokens0)
+            self.position.copy_(position0)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph, stream=side):
+            self._step()
+        self.tokens.copy_(tokens0)
+        self.position.copy_(position0)
+        torch.cuda.synchronize()

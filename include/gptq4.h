@@ -50,6 +50,7 @@ extern "C" {
 #define GPTQ4_E_ALIGN 5      /* a pointer is not 16-byte aligned                 */
 
 #define GPTQ4_WS_COUNTER_BYTES 524288
+#define GPTQ4_KV_AT_POSITION (-1)
 
 /* operation selector for gptq4_workspace_bytes */
 #define GPTQ4_OP_MATMUL 0
@@ -110,7 +111,10 @@ int gptq4_rope_table(float *cos_out, float *sin_out, int max_pos, int D, float b
  *   k [B, H, kv_capacity, D] rows kv_offset + s, rotated
  *   v [B, H, kv_capacity, D] rows kv_offset + s, as projected
  * kv_capacity = S and kv_offset = 0 give the reference's three [B,H,S,D] tensors;
- * other values write straight into a preallocated KV cache.
+ * other values write straight into a preallocated KV cache.  kv_offset =
+ * GPTQ4_KV_AT_POSITION writes token (b, s) to cache row position_ids[b*S + s] (clamped
+ * into [0, kv_capacity)): no argument changes from one decode step to the next, so a
+ * captured HIP graph of the step can be replayed.
  * Replaces qkv_proj + split + view/transpose + apply_rotary_pos_emb
  * (fused_attention.py:91-102).  D must be 128. */
 int gptq4_qkv_rotary(const void *x, const int32_t *qweight, const int32_t *qzeros,

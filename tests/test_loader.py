@@ -163,3 +163,57 @@ def test_loaded_model_matches_cpu_reference(tmp_path, groupsize, act_order):
         lg, _ = model(cur)
         cur = torch.cat([cur, lg[:, -1:].argmax(-1)], dim=1)
     assert (out == cur).float().mean() > 0.9
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("groupsize,act_order,bsz", [(128, False, 1), (128, True, 3), (-1, False, 2)])
+def test_graph_replayed_decode_equals_eager_decode(tmp_path, groupsize, act_order, bsz):
+    """The captured decode step (K/V placed by position id, attention over the whole cache
+    under a position mask) gives the tokens of the step launched kernel by kernel, on
+    every replay."""
+    cfg = make_checkpoint(tmp_path, groupsize, act_order=act_order, seed=11)
+    model = G.load_quant(str(tmp_path), device="cuda", fuse_mlp=True)
+    torch.manual_seed(3)
+    ids = torch.randint(0, cfg.vocab_size, (bsz, 9)).cuda()
+    eager = model.generate_greedy(ids, 12)
+    graph = model.generate_greedy(ids, 12, use_graph=True)
+    assert eager.shape == (bsz, 21)
+    assert torch.equal(eager, graph)
+    # a decoder can be prefilled again and its graph replayed with other contents
+    from gptq_triton_amd.llama import GreedyDecoder
+    dec = GreedyDecoder(model, bsz, 32)
+    for seed in (4, 5):
+        torch.manual_seed(seed)
+        ids2 = torch.randint(0, cfg.vocab_size, (bsz, 7)).cuda()
+        first = dec.prefill(ids2)
+        rest = dec.decode(10, use_graph=True)
+        want = model.generate_greedy(ids2, 11)
+        assert torch.equal(torch.cat([ids2, first, rest], dim=1), want)
+
+
+@pytest.mark.gpu
+def test_qkv_rotary_places_kv_by_position():
+    import numpy as np
+    from conftest import to_dev
+    from oracle import gptq_oracle as O
+    from gptq_triton_amd.fused_attention import KV_AT_POSITION
+    H, Dh, hidden, g, cap = 8, 128, 1024, 128, 24
+    L = O.make_layer(hidden, 3 * hidden, g, seed=300)
+    D = to_dev(L)
+    cos, sin = G.RotaryTable(Dh, 2048).get(torch.device("cuda"), 2048)
+    for s in (1, 5, 20):   # 20 rows of 2 sequences: the tiled kernel
+        x = O.make_x(2 * s, hidden, seed=301 + s).reshape(2, s, hidden)
+        pos = np.stack([np.arange(s) + 2, np.arange(s)[::-1].copy() + 1]).astype(np.int32)
+        kc = torch.full((2, H, cap, Dh), 7.0, dtype=torch.float16, device="cuda")
+        vc = torch.full((2, H, cap, Dh), 7.0, dtype=torch.float16, device="cuda")
+        xd, pd = torch.from_numpy(x).cuda(), torch.from_numpy(pos).cuda()
+        q, _, _ = G.qkv_rotary(g, xd, D["qweight"], D["scales"], D["qzeros"], pd, cos, sin, H, Dh,
+                               kv_out=(kc, vc), kv_offset=KV_AT_POSITION)
+        q0, k0, v0 = G.qkv_rotary(g, xd, D["qweight"], D["scales"], D["qzeros"], pd, cos, sin, H, Dh)
+        assert torch.equal(q, q0)
+        for b in range(2):
+            rows = torch.from_numpy(pos[b].astype(np.int64)).cuda()
+            assert torch.equal(kc[b][:, rows], k0[b]) and torch.equal(vc[b][:, rows], v0[b])
+            untouched = torch.ones(cap, dtype=torch.bool)
+            untouched[pos[b]] = False
+            assert bool((kc[b][:, untouched] == 7.0).all()) and bool((vc[b][:, untouched] == 7.0).all())
