@@ -19,7 +19,14 @@ Also reported on the same line:
                 on the host cores for 1 of the 32 layers, extrapolated to a token
   extra         per-operator decode timings and prefill TFLOP/s (M = 128 / 512 / 2048)
 
-Usage: python bench.py [--gpus 1] [--steps K] [--warmup W]
+Other workloads (--workload llama7b | llama13b | llama30b): a full random-init decoder of
+that shape (embedding, RMSNorm, fused QKV + rotary into a preallocated KV cache, torch
+SDPA, o_proj, fused MLP, fp16 lm_head, greedy argmax) - one timed prefill of --prompt
+tokens, then --new-tokens greedy tokens with one HIP-graph replay per token; value =
+decode tokens/s over the batch, prefill TFLOP/s and the eager (kernel-by-kernel) decode
+rate in `extra`.
+
+Usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]
 """
 from __future__ import annotations
 
@@ -49,6 +56,128 @@ def weight_bytes(k, n, g):
     return k * n // 2 + groups * n // 2 + groups * n * 2
 
 
+DECODERS = {
+    # layers, hidden, intermediate, heads, groupsize, act-order
+    "llama7b": (32, 4096, 11008, 32, 128, False),
+    "llama13b": (40, 5120, 13824, 40, 128, True),
+    "llama30b": (60, 6656, 17920, 52, 512, False),
+}
+
+
+def run_decoder(args):
+    """Full-decoder workload: prefill + graph-replayed greedy decode on a random-init model."""
+    import torch
+
+    torch.set_grad_enabled(False)
+
+    import gptq_triton_amd as G
+    from gptq_triton_amd import _lib
+    from gptq_triton_amd.fused_attention import LlamaConfigLite
+    from gptq_triton_amd.llama import GreedyDecoder, LlamaForCausalLM, LlamaRMSNorm
+
+    _lib.load()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    layers, hidden, inter, heads, groupsize, act_order = DECODERS[args.workload]
+    bsz, prompt, new = args.batch, args.prompt, args.new_tokens
+    cfg = LlamaConfigLite()
+    cfg.hidden_size, cfg.intermediate_size, cfg.num_attention_heads, cfg.num_hidden_layers = hidden, inter, heads, layers
+    cfg.vocab_size, cfg.max_position_embeddings = 32000, max(2048, prompt + new)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1234)
+
+    log(f"building a random-init {args.workload} decoder ({layers} layers, groupsize {groupsize}, act-order {act_order}) ...")
+    dtype0 = torch.get_default_dtype()
+    torch.set_default_dtype(torch.half)
+    try:
+        with torch.device("meta"):
+            model = LlamaForCausalLM(cfg)
+    finally:
+        torch.set_default_dtype(dtype0)
+    with torch.device("meta"):
+        G.make_quant(model, 4, groupsize, act_order=act_order)
+    model = model.to_empty(device=dev)
+    qbytes = 0
+    for layer in model.model.layers:
+        # projections that share an input share its act-order permutation
+        perms = {}
+        for group, names in (("attn_in", ("self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj")),
+                             ("attn_out", ("self_attn.o_proj",)), ("mlp_in", ("mlp.gate_proj", "mlp.up_proj")),
+                             ("mlp_out", ("mlp.down_proj",))):
+            for name in names:
+                q = layer.get_submodule(name)
+                q.qweight.copy_(torch.randint(-2**31, 2**31 - 1, q.qweight.shape, dtype=torch.int32, device=dev, generator=gen))
+                q.qzeros.copy_(torch.randint(-2**31, 2**31 - 1, q.qzeros.shape, dtype=torch.int32, device=dev, generator=gen))
+                # scales sized so that activations stay O(1) through the depth of the stack
+                q.scales.copy_(((0.2 + 0.3 * torch.rand(q.scales.shape, device=dev, generator=gen)) / (4.6 * q.infeatures ** 0.5)).half())
+                qbytes += q.qweight.numel() * 4 + q.qzeros.numel() * 4 + q.scales.numel() * 2
+                if act_order:
+                    if group not in perms:
+                        g = q.infeatures // (q.infeatures if groupsize == -1 else groupsize)
+                        base = torch.arange(q.infeatures, device=dev) // (q.infeatures // g)
+                        perms[group] = base[torch.randperm(q.infeatures, device=dev, generator=gen)].int()
+                    q.g_idx.copy_(perms[group])
+    for m in model.modules():
+        if isinstance(m, LlamaRMSNorm):
+            m.weight.fill_(1.0)
+    model.model.embed_tokens.weight.copy_(torch.randn(model.model.embed_tokens.weight.shape, device=dev, generator=gen) * 0.5)
+    model.lm_head.weight.copy_(torch.randn(model.lm_head.weight.shape, device=dev, generator=gen) * 0.02)
+    G.make_quant_attn(model)
+    G.make_fused_mlp(model)
+
+    ids = torch.randint(0, cfg.vocab_size, (bsz, prompt), device=dev, generator=gen)
+    dec = GreedyDecoder(model, bsz, prompt + new)
+    log("warm-up prefill ...")
+    dec.prefill(ids)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    dec.prefill(ids)
+    torch.cuda.synchronize()
+    prefill_s = time.perf_counter() - t0
+    per_token_kn = layers * (hidden * 3 * hidden + hidden * hidden + 2 * hidden * inter + inter * hidden)
+    prefill_tf = 2.0 * bsz * prompt * per_token_kn / prefill_s / 1e12
+    log(f"prefill: {prefill_s * 1e3:.1f} ms for {bsz} x {prompt} tokens = {prefill_tf:.0f} TFLOP/s in the quantised linears")
+
+    eager_steps = min(8, new - 1)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    dec.decode(eager_steps)
+    torch.cuda.synchronize()
+    eager_s = (time.perf_counter() - t0) / max(eager_steps, 1)
+    dec.decode(2, use_graph=True)  # captures the step
+    steps = new - 1 - eager_steps - 2
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    toks = dec.decode(steps, use_graph=True)
+    torch.cuda.synchronize()
+    step_s = (time.perf_counter() - t0) / steps
+    kv_bytes = 2 * layers * bsz * heads * (prompt + new) * 128 * 2
+    step_bytes = qbytes + model.lm_head.weight.numel() * 2 + kv_bytes
+    gbs = step_bytes / step_s / 1e9
+    log(f"decode: {step_s * 1e3:.3f} ms/step graph-replayed ({bsz / step_s:.1f} tok/s), {eager_s * 1e3:.3f} ms/step eager; "
+        f"{step_bytes / 1e9:.2f} GB per step -> {gbs:.0f} GB/s")
+    result = {
+        "metric": f"{args.workload}-shape 4-bit greedy decode tok/s (full decoder)", "value": round(bsz / step_s, 2),
+        "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": eager_steps + 2, "ms_per_step": round(step_s * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp16", "data": "synthetic",
+        "config": {"workload": f"random-init {args.workload}-shape decoder, batch {bsz}, {prompt}-token prompt prefill then "
+                               f"{new} greedy tokens, 4-bit groupsize {groupsize}{' act-order' if act_order else ''}, "
+                               "fp16 lm_head, one HIP-graph replay per token",
+                   "layers": layers, "hidden": hidden, "intermediate": inter, "heads": heads, "batch": bsz,
+                   "prompt": prompt, "new_tokens": new},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "whole decode step: packed weights + fp16 lm_head + the full-capacity KV cache, read once",
+                     "bytes_per_launch": step_bytes, "avg_launch_us": round(step_s * 1e6, 1)},
+        "cpu_baseline": None,
+        "extra": {"prefill_ms": round(prefill_s * 1e3, 2), "prefill_linear_TFLOPs": round(prefill_tf, 1),
+                  "prefill_frac_of_fp16_mfma_peak": round(prefill_tf / MFMA_FP16_PEAK_TFLOPS, 4),
+                  "eager_decode_ms_per_step": round(eager_s * 1e3, 3), "last_tokens": toks[0, -4:].tolist()},
+    }
+    print(json.dumps(result), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -59,11 +188,20 @@ def main():
     ap.add_argument("--traffic-probe", action="store_true",
                     help="for rocprofv3 --pmc runs: a 256 MiB device copy (calibration) followed by plain launches of "
                          "each decode operator on distinct weights; prints no JSON")
+    ap.add_argument("--workload", default="linears7b", choices=["linears7b"] + sorted(DECODERS),
+                    help="linears7b (default): the quantised-linear hot path of one 7B decode token; llamaNNb: a full "
+                         "random-init decoder of that shape, prefill + greedy decode")
+    ap.add_argument("--batch", type=int, default=1)
+    ap.add_argument("--prompt", type=int, default=2048)
+    ap.add_argument("--new-tokens", type=int, default=128)
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures the single-GPU hot path: run with --gpus 1 (nothing here uses a second GPU)",
               file=sys.stderr)
         sys.exit(2)
+
+    if args.workload != "linears7b":
+        return run_decoder(args)
 
     import torch
 

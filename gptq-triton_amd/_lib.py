@@ -14,7 +14,7 @@ import torch
 LIB_PATH = Path(__file__).resolve().parent / "csrc" / "libgptq4.so"
 ABI_VERSION = 1
 WS_COUNTER_BYTES = 524288
-OP_MATMUL, OP_MLP_GATEUP, OP_QKV_ROTARY = 0, 1, 2
+OP_MATMUL, OP_MLP_GATEUP, OP_QKV_ROTARY, OP_DECODE_ATTENTION = 0, 1, 2, 3
 
 # every symbol include/gptq4.h declares: (restype, argtypes)
 SIGNATURES = {
@@ -27,6 +27,8 @@ SIGNATURES = {
     "gptq4_mlp_gateup": (c_int, [c_void_p] * 9 + [c_int] * 4 + [c_void_p, c_size_t, c_void_p]),
     "gptq4_rope_table": (c_int, [c_void_p, c_void_p, c_int, c_int, c_float, c_void_p]),
     "gptq4_qkv_rotary": (c_int, [c_void_p] * 8 + [c_int] + [c_void_p] * 3 + [c_int] * 8 + [c_void_p, c_size_t, c_void_p]),
+    "gptq4_rmsnorm": (c_int, [c_void_p] * 3 + [c_int, c_int, c_float, c_void_p]),
+    "gptq4_decode_attention": (c_int, [c_void_p] * 5 + [c_int] * 4 + [c_float, c_void_p, c_size_t, c_void_p]),
     "gptq4_set_tuning": (None, [c_int, c_int, c_int]),
     "gptq4_set_gemm_tuning": (None, [c_int, c_int]),
     "gptq4_set_gemv_tuning": (None, [c_int, c_int, c_int, c_int]),

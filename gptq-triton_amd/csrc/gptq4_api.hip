@@ -123,6 +123,7 @@ void gptq4_set_tuning(int words, int depth, int splitk) {
 
 size_t gptq4_workspace_bytes(int op, int M, int K, int N) {
     size_t bytes = GPTQ4_WS_COUNTER_BYTES;
+    if (op == GPTQ4_OP_DECODE_ATTENTION) return (M < 1 || K < 1) ? bytes : bytes + attn_decode_partial_bytes(M, K);
     if (M < 1 || N <= 0 || K <= 0) return bytes;
     if (M <= SKINNY_MAX_M) {
         const int cols = (op == GPTQ4_OP_MLP_GATEUP) ? 2 * N : N;
@@ -281,6 +282,28 @@ int gptq4_qkv_rotary(const void *x, const int32_t *qweight, const int32_t *qzero
         if (rc) return rc;
         return launch_gemm(EPI_ROPE, a, pl, s);
     }
+}
+
+int gptq4_rmsnorm(const void *x, const void *weight, void *y, int M, int H, float eps, void *stream) {
+    if (!x || !weight || !y) return -GPTQ4_E_NULL;
+    if (M < 1 || H < 8 || (H % 8) != 0 || !(eps >= 0.f)) return -GPTQ4_E_SHAPE;
+    if (misaligned16(x) || misaligned16(weight) || misaligned16(y)) return -GPTQ4_E_ALIGN;
+    return launch_rmsnorm(reinterpret_cast<const half_t *>(x), reinterpret_cast<const half_t *>(weight),
+                          reinterpret_cast<half_t *>(y), M, H, eps, reinterpret_cast<hipStream_t>(stream));
+}
+
+int gptq4_decode_attention(const void *q, const void *k_cache, const void *v_cache, const int32_t *positions, void *out,
+                           int B, int H, int D, int kv_capacity, float scale, void *workspace, size_t workspace_bytes,
+                           void *stream) {
+    if (!q || !k_cache || !v_cache || !positions || !out) return -GPTQ4_E_NULL;
+    if (B < 1 || H < 1 || D != 128 || kv_capacity < 1 || (long)B * H > 65535) return -GPTQ4_E_SHAPE;
+    if (misaligned16(q) || misaligned16(k_cache) || misaligned16(v_cache) || misaligned16(out)) return -GPTQ4_E_ALIGN;
+    if (workspace == nullptr || workspace_bytes < GPTQ4_WS_COUNTER_BYTES + attn_decode_partial_bytes(B * H, kv_capacity))
+        return -GPTQ4_E_WORKSPACE;
+    float *partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_COUNTER_BYTES);
+    return launch_attn_decode(reinterpret_cast<const half_t *>(q), reinterpret_cast<const half_t *>(k_cache),
+                              reinterpret_cast<const half_t *>(v_cache), positions, reinterpret_cast<half_t *>(out), B, H,
+                              kv_capacity, scale, partials, reinterpret_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

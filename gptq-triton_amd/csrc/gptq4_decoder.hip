@@ -1,0 +1,194 @@
+// The two non-matmul operators a decode step runs between the quantised linears, so that a
+// whole step is a short chain of HIP launches: RMSNorm and single-query attention over a
+// preallocated KV cache.  Both are HBM/L2-bound elementwise-and-reduce kernels.
+#include "gptq4_internal.h"
+
+namespace {
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+
+// y[row] = weight * fp16( x[row] * rsqrt(mean(x[row]^2) + eps) ): statistics and the
+// normalisation in fp32, rounded to fp16, then an fp16 multiply by the weight - the
+// rounding order of the LLaMA RMSNorm module.  One workgroup per row, H % 8 == 0.
+__global__ __launch_bounds__(256) void gptq4_rmsnorm_kernel(const half_t *__restrict__ x, const half_t *__restrict__ w,
+                                                            half_t *__restrict__ y, int H, float eps) {
+    __shared__ float part[4];
+    const int tid = threadIdx.x;
+    const uint4 *xr = reinterpret_cast<const uint4 *>(x + (size_t)blockIdx.x * H);
+    const uint4 *wr = reinterpret_cast<const uint4 *>(w);
+    uint4 *yr = reinterpret_cast<uint4 *>(y + (size_t)blockIdx.x * H);
+    const int chunks = H >> 3;
+    float ss = 0.f;
+    for (int c = tid; c < chunks; c += 256) {
+        const uint4 v = xr[c];
+        const h2_t p[4] = {as_h2(v.x), as_h2(v.y), as_h2(v.z), as_h2(v.w)};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ss += (float)p[i].x * (float)p[i].x + (float)p[i].y * (float)p[i].y;
+    }
+    ss = wave_sum(ss);
+    if ((tid & 63) == 0) part[tid >> 6] = ss;
+    __syncthreads();
+    const float inv = rsqrtf((part[0] + part[1] + part[2] + part[3]) / (float)H + eps);
+    for (int c = tid; c < chunks; c += 256) {
+        const uint4 v = xr[c], g = wr[c];
+        const uint32_t vi[4] = {v.x, v.y, v.z, v.w}, gi[4] = {g.x, g.y, g.z, g.w};
+        uint32_t o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const h2_t p = as_h2(vi[i]);
+            const h2_t n = {(half_t)((float)p.x * inv), (half_t)((float)p.y * inv)};
+            o[i] = as_u32(as_h2(gi[i]) * n);
+        }
+        yr[c] = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+}
+
+// Single-query attention, split over the cache length.  Workgroup (split, b*H + h) takes
+// rows [split*chunk, ...) of the valid prefix 0..positions[b]; 16 lanes share a row (8
+// head dimensions each, one 16-byte load of K and of V per lane), 16 rows per pass,
+// running (max, sum, weighted V) per thread in fp32; the 16 row slots are merged through
+// LDS and the partial [max, sum, acc[128]] goes to the workspace.
+constexpr int ATT_PART = 130;  // floats per partial: max, sum, 128 accumulators
+
+__global__ __launch_bounds__(256) void gptq4_attn_partial_kernel(const half_t *__restrict__ q, const half_t *__restrict__ kc,
+                                                                 const half_t *__restrict__ vc, const int *__restrict__ positions,
+                                                                 float *__restrict__ part, int H, int capacity, int chunk,
+                                                                 float scale) {
+    __shared__ float s_m[16], s_l[16];
+    __shared__ float s_acc[16][128];
+    const int tid = threadIdx.x;
+    const int slot = tid >> 4, sub = tid & 15;
+    const int bh = blockIdx.y, split = blockIdx.x, nsplit = gridDim.x;
+    const int b = bh / H;
+    const int len = min(max(positions[b], 0), capacity - 1) + 1;
+    const int r0 = split * chunk, r1 = min(r0 + chunk, len);
+
+    float qf[8];
+    {
+        const uint4 v = *reinterpret_cast<const uint4 *>(q + (size_t)bh * 128 + 8 * sub);
+        const h2_t p[4] = {as_h2(v.x), as_h2(v.y), as_h2(v.z), as_h2(v.w)};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            qf[2 * i] = (float)p[i].x * scale;
+            qf[2 * i + 1] = (float)p[i].y * scale;
+        }
+    }
+    const half_t *kb = kc + (size_t)bh * capacity * 128 + 8 * sub;
+    const half_t *vb = vc + (size_t)bh * capacity * 128 + 8 * sub;
+    float m = -INFINITY, l = 0.f, acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+
+    constexpr int U = 4;  // rows in flight per thread
+    for (int r = r0 + slot; r < r1; r += 16 * U) {
+        uint4 kv[U], vv[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int rr = min(r + 16 * u, r1 - 1);  // clamped: the load is always valid
+            kv[u] = *reinterpret_cast<const uint4 *>(kb + (size_t)rr * 128);
+            vv[u] = *reinterpret_cast<const uint4 *>(vb + (size_t)rr * 128);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const h2_t kp[4] = {as_h2(kv[u].x), as_h2(kv[u].y), as_h2(kv[u].z), as_h2(kv[u].w)};
+            float s = 0.f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s += qf[2 * i] * (float)kp[i].x + qf[2 * i + 1] * (float)kp[i].y;
+            s += __shfl_xor(s, 1);
+            s += __shfl_xor(s, 2);
+            s += __shfl_xor(s, 4);
+            s += __shfl_xor(s, 8);
+            if (r + 16 * u < r1) {  // uniform over the 16 lanes of a row
+                const float mn = fmaxf(m, s);
+                const float corr = __expf(m - mn), pw = __expf(s - mn);
+                const h2_t vp[4] = {as_h2(vv[u].x), as_h2(vv[u].y), as_h2(vv[u].z), as_h2(vv[u].w)};
+                l = l * corr + pw;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    acc[2 * i] = acc[2 * i] * corr + pw * (float)vp[i].x;
+                    acc[2 * i + 1] = acc[2 * i + 1] * corr + pw * (float)vp[i].y;
+                }
+                m = mn;
+            }
+        }
+    }
+    if (sub == 0) {
+        s_m[slot] = m;
+        s_l[slot] = l;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s_acc[slot][8 * sub + i] = acc[i];
+    __syncthreads();
+    if (tid < 128) {
+        float mw = -INFINITY;
+#pragma unroll
+        for (int s = 0; s < 16; ++s) mw = fmaxf(mw, s_m[s]);
+        float lw = 0.f, a = 0.f;
+#pragma unroll
+        for (int s = 0; s < 16; ++s) {
+            const float f = (s_m[s] == -INFINITY) ? 0.f : __expf(s_m[s] - mw);
+            lw += s_l[s] * f;
+            a += s_acc[s][tid] * f;
+        }
+        float *dst = part + ((size_t)bh * nsplit + split) * ATT_PART;
+        if (tid == 0) {
+            dst[0] = mw;
+            dst[1] = lw;
+        }
+        dst[2 + tid] = a;
+    }
+}
+
+// out[b, h*128 + d] = sum over splits of acc * exp(max_s - max) / sum of sums likewise.
+__global__ __launch_bounds__(128) void gptq4_attn_combine_kernel(const float *__restrict__ part, half_t *__restrict__ out, int nsplit) {
+    const int bh = blockIdx.x, d = threadIdx.x;
+    const float *src = part + (size_t)bh * nsplit * ATT_PART;
+    float mw = -INFINITY;
+    for (int s = 0; s < nsplit; ++s) mw = fmaxf(mw, src[s * ATT_PART]);
+    float lw = 0.f, a = 0.f;
+    for (int s = 0; s < nsplit; ++s) {
+        const float ms = src[s * ATT_PART];
+        const float f = (ms == -INFINITY) ? 0.f : __expf(ms - mw);
+        lw += src[s * ATT_PART + 1] * f;
+        a += src[s * ATT_PART + 2 + d] * f;
+    }
+    out[(size_t)bh * 128 + d] = (half_t)(a / lw);
+}
+
+}  // namespace
+
+int launch_rmsnorm(const half_t *x, const half_t *w, half_t *y, int M, int H, float eps, hipStream_t stream) {
+    hipLaunchKernelGGL(gptq4_rmsnorm_kernel, dim3((unsigned)M), dim3(256), 0, stream, x, w, y, H, eps);
+    return (int)hipGetLastError();
+}
+
+// Rows per split: enough workgroups to cover the chip (~2 per CU), at least 64 rows each.
+int attn_decode_splits(int BH, int capacity) {
+    int nsplit = (512 + BH - 1) / BH;
+    const int max_split = (capacity + 63) / 64;
+    if (nsplit > max_split) nsplit = max_split;
+    if (nsplit < 1) nsplit = 1;
+    return nsplit;
+}
+
+size_t attn_decode_partial_bytes(int BH, int capacity) {
+    return (size_t)BH * attn_decode_splits(BH, capacity) * ATT_PART * sizeof(float);
+}
+
+int launch_attn_decode(const half_t *q, const half_t *kc, const half_t *vc, const int *positions, half_t *out, int B,
+                       int H, int capacity, float scale, float *partials, hipStream_t stream) {
+    const int BH = B * H;
+    const int nsplit = attn_decode_splits(BH, capacity);
+    int chunk = (capacity + nsplit - 1) / nsplit;
+    chunk = (chunk + 15) & ~15;
+    hipLaunchKernelGGL(gptq4_attn_partial_kernel, dim3((unsigned)nsplit, (unsigned)BH), dim3(256), 0, stream, q, kc, vc,
+                       positions, partials, H, capacity, chunk, scale);
+    int rc = (int)hipGetLastError();
+    if (rc) return rc;
+    hipLaunchKernelGGL(gptq4_attn_combine_kernel, dim3((unsigned)BH), dim3(128), 0, stream, partials, out, nsplit);
+    return (int)hipGetLastError();
+}

@@ -1,0 +1,61 @@
+"""The two non-matmul operators of a decode step, as HIP kernels behind the C ABI: RMSNorm
+and single-query attention over a preallocated KV cache.  The reference runs both as torch
+ops of the HF model it patches (LlamaRMSNorm; fused_attention.py:118-148); here they exist
+so that a whole decode step is a short chain of HIP launches that a graph can replay."""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import _lib
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """y = weight * fp16(x * rsqrt(mean(x^2, -1) + eps)) for fp16 x [..., H] on the GPU."""
+    _lib.require_cuda(x, "x")
+    _lib.require_cuda(weight, "weight")
+    if x.dtype != torch.float16 or weight.dtype != torch.float16:
+        raise TypeError("rms_norm takes fp16 tensors")
+    h = x.shape[-1]
+    if weight.shape != (h,) or h % 8 != 0:
+        raise ValueError(f"weight must be [{h}] and the hidden size a multiple of 8")
+    x2 = x.reshape(-1, h)
+    if not x2.is_contiguous():
+        x2 = x2.contiguous()
+    y = torch.empty_like(x2)
+    if x2.shape[0] == 0:
+        return y.reshape(x.shape)
+    rc = _lib.load().gptq4_rmsnorm(x2.data_ptr(), weight.data_ptr(), y.data_ptr(), x2.shape[0], h, float(eps),
+                                   _lib.current_stream(x.device))
+    _lib.check(rc, "gptq4_rmsnorm")
+    return y.reshape(x.shape)
+
+
+def decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+    """q fp16 [B, H, 1, 128]; caches fp16 [B, H, capacity, 128]; positions int32 [B] or [B, 1]:
+    sequence b attends to cache rows 0..positions[b].  Returns fp16 [B, 1, H*128]."""
+    for t, name in ((q, "q"), (k_cache, "k_cache"), (v_cache, "v_cache"), (positions, "positions")):
+        _lib.require_cuda(t, name)
+    bsz, heads, q_len, hd = q.shape
+    if q_len != 1 or hd != 128:
+        raise ValueError("decode_attention takes one query token per sequence and head_dim 128")
+    if k_cache.shape != v_cache.shape or k_cache.shape[:2] != (bsz, heads) or k_cache.shape[3] != hd \
+            or not (q.is_contiguous() and k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise ValueError("caches must be contiguous [B, H, capacity, 128] tensors matching q")
+    if q.dtype != torch.float16 or k_cache.dtype != torch.float16 or v_cache.dtype != torch.float16:
+        raise TypeError("decode_attention takes fp16 tensors")
+    pos = positions.reshape(-1)
+    if pos.dtype != torch.int32 or pos.numel() != bsz or not pos.is_contiguous():
+        pos = pos.to(torch.int32).contiguous()
+        if pos.numel() != bsz:
+            raise ValueError("one position per sequence")
+    cap = k_cache.shape[2]
+    out = torch.empty((bsz, 1, heads * hd), dtype=torch.float16, device=q.device)
+    lib = _lib.load()
+    ws = _lib.workspace(q.device, lib.gptq4_workspace_bytes(_lib.OP_DECODE_ATTENTION, bsz * heads, cap, 0))
+    rc = lib.gptq4_decode_attention(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), pos.data_ptr(), out.data_ptr(),
+                                    bsz, heads, hd, cap, 1.0 / math.sqrt(hd), ws.data_ptr(), ws.numel(),
+                                    _lib.current_stream(q.device))
+    _lib.check(rc, "gptq4_decode_attention")
+    return out

@@ -17,6 +17,7 @@ from typing import List, Optional, Tuple
 import torch
 import torch.nn as nn
 
+from .decoder_ops import decode_attention, rms_norm
 from .fused_attention import LlamaConfigLite
 
 
@@ -41,6 +42,8 @@ class LlamaRMSNorm(nn.Module):
         self.variance_epsilon = eps
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if x.is_cuda and x.dtype == torch.float16:
+            return rms_norm(x, self.weight, self.variance_epsilon)  # one HIP launch
         xf = x.float()
         xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.variance_epsilon)
         return self.weight * xf.to(x.dtype)
@@ -156,8 +159,8 @@ class GreedyDecoder:
     """Greedy generation state for one batch: KV caches of fixed capacity plus the static
     token / position buffers a decode step reads and writes.  Nothing in a decode step
     depends on a host-side value that changes from token to token (the QKV kernel places
-    K and V by position id, attention runs over the whole cache under a mask derived from
-    the position), so the step can be captured once as a HIP graph and replayed."""
+    K and V by position id, the attention kernel reads how far to attend from the position
+    buffer), so the step can be captured once as a HIP graph and replayed."""
 
     def __init__(self, model: LlamaForCausalLM, bsz: int, capacity: int):
         cfg = model.config
@@ -169,17 +172,13 @@ class GreedyDecoder:
                        for _ in model.model.layers]
         self.tokens = torch.zeros((bsz, 1), dtype=torch.long, device=dev)
         self.position = torch.zeros((bsz, 1), dtype=torch.int32, device=dev)
-        self.slots = torch.arange(capacity, device=dev, dtype=torch.int32)[None, None, None, :]
         self.graph = None
 
     def _layers(self, h, position_ids, kv_offset, attend):
-        cfg = self.model.config
-        bsz, q_len, _ = h.shape
         for layer, (kc, vc) in zip(self.model.model.layers, self.caches):
             attn = layer.self_attn
             q, _, _ = attn.project_qkv(layer.input_layernorm(h), position_ids, kv_out=(kc, vc), kv_offset=kv_offset)
-            o = attend(q, kc, vc)
-            h = h + attn.o_proj(o.transpose(1, 2).reshape(bsz, q_len, cfg.hidden_size))
+            h = h + attn.o_proj(attend(q, kc, vc))  # attend -> [B, q_len, hidden]
             h = h + layer.mlp(layer.post_attention_layernorm(h))
         return self.model.lm_head(self.model.model.norm(h[:, -1:, :])).argmax(-1)
 
@@ -194,7 +193,8 @@ class GreedyDecoder:
         sdpa = torch.nn.functional.scaled_dot_product_attention
 
         def attend(q, kc, vc):
-            return sdpa(q, kc[:, :, :prompt], vc[:, :, :prompt], is_causal=prompt > 1)
+            o = sdpa(q, kc[:, :, :prompt], vc[:, :, :prompt], is_causal=prompt > 1)
+            return o.transpose(1, 2).reshape(bsz, prompt, self.model.config.hidden_size)
 
         nxt = self._layers(self.model.model.embed_tokens(input_ids), position_ids, 0, attend)
         self.tokens.copy_(nxt)
@@ -204,12 +204,9 @@ class GreedyDecoder:
     def _step(self):
         """One decode token from the static buffers: reads tokens/position, writes them back."""
         from .fused_attention import KV_AT_POSITION
-        mask = torch.zeros((self.bsz, 1, 1, self.capacity), dtype=torch.float16, device=self.tokens.device)
-        mask.masked_fill_(self.slots > self.position[:, None, None, :], torch.finfo(torch.float16).min)
-        sdpa = torch.nn.functional.scaled_dot_product_attention
 
-        def attend(q, kc, vc):
-            return sdpa(q, kc, vc, attn_mask=mask)
+        def attend(q, kc, vc):  # rows 0..position of the cache, one HIP launch pair
+            return decode_attention(q, kc, vc, self.position)
 
         nxt = self._layers(self.model.model.embed_tokens(self.tokens), self.position, KV_AT_POSITION, attend)
         self.tokens.copy_(nxt)

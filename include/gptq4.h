@@ -56,6 +56,7 @@ extern "C" {
 #define GPTQ4_OP_MATMUL 0
 #define GPTQ4_OP_MLP_GATEUP 1
 #define GPTQ4_OP_QKV_ROTARY 2
+#define GPTQ4_OP_DECODE_ATTENTION 3 /* M = B * H, K = kv_capacity, N unused */
 
 int gptq4_abi_version(void);
 const char *gptq4_strerror(int code);
@@ -123,6 +124,23 @@ int gptq4_qkv_rotary(const void *x, const int32_t *qweight, const int32_t *qzero
                      void *q, void *k, void *v, int B, int S, int H, int D, int K,
                      int groupsize, int kv_capacity, int kv_offset, void *workspace,
                      size_t workspace_bytes, void *stream);
+
+/* RMSNorm over the last dimension: y = weight * fp16(x * rsqrt(mean(x^2) + eps)), x and y
+ * fp16 [M, H], weight fp16 [H], H a multiple of 8; statistics in fp32.  Stands in for the
+ * LlamaRMSNorm modules of the model the reference builds and runs between its fused blocks
+ * (src/gptq_triton/__init__.py:32-47; the quantised linears are the only modules it swaps). */
+int gptq4_rmsnorm(const void *x, const void *weight, void *y, int M, int H, float eps, void *stream);
+
+/* Attention of ONE query token per sequence over a preallocated KV cache: for each (b, h)
+ * softmax(q . K[0..positions[b]]^T * scale) . V[0..positions[b]], in fp32, written as fp16
+ * out [B, H*D] (the layout o_proj consumes).  q fp16 [B, H, 1, D]; k_cache, v_cache fp16
+ * [B, H, kv_capacity, D]; positions int32 [B] (clamped into [0, kv_capacity)); D must be
+ * 128.  Replaces the attention core of QuantLlamaAttention.forward for q_len == 1
+ * (fused_attention.py:118-148: scores, mask, fp32 softmax, weighted sum, transpose). */
+int gptq4_decode_attention(const void *q, const void *k_cache, const void *v_cache,
+                           const int32_t *positions, void *out, int B, int H, int D,
+                           int kv_capacity, float scale, void *workspace,
+                           size_t workspace_bytes, void *stream);
 
 /* Host-side launch tuning of the small-M kernels, for measurements: words per lane and
  * load (1, 2 or 4: strips of 16, 32 or 64 columns), batches of loads in flight per

@@ -323,3 +323,35 @@ def within_tolerance(y, y_ref, rtol=1e-2, atol=2e-3):
     err = np.abs(y - r)
     lim = atol + rtol * np.abs(r)
     return bool((err <= lim).all()), float(err.max(initial=0.0)), float((err - lim).max(initial=-np.inf))
+
+
+# ------------------------------------------------------------------ decoder-side operators
+def rmsnorm_ref(x: np.ndarray, weight: np.ndarray, eps: float) -> np.ndarray:
+    """LLaMA RMSNorm with the module's rounding order: statistics and normalisation in wide
+    precision, ONE rounding to fp16, then an fp16 multiply by the weight.  The reference
+    runs transformers' LlamaRMSNorm between its fused blocks (the model it patches,
+    src/gptq_triton/__init__.py:32-47).  Pinned by: constant rows (y = weight * sign), scale
+    invariance for eps = 0, unit-norm rows."""
+    xf = np.asarray(x, dtype=np.float64)
+    n = (xf / np.sqrt((xf * xf).mean(-1, keepdims=True) + eps)).astype(np.float16)
+    return (np.asarray(weight, dtype=np.float16) * n).astype(np.float16)
+
+
+def decode_attention_ref(q: np.ndarray, k_cache: np.ndarray, v_cache: np.ndarray, positions) -> np.ndarray:
+    """One query token per sequence over a KV cache, in float64: for (b, h)
+    softmax(q . K[:p+1]^T / sqrt(D)) . V[:p+1] with p = positions[b]; returns [B, 1, H*D]
+    (src/gptq_triton/fused_attention.py:118-148 for q_len == 1: scores, fp32 softmax,
+    weighted sum, transpose + reshape).  Pinned by: p = 0 gives V[0]; equal keys give the
+    mean of V; one key far ahead gives its V row."""
+    q = np.asarray(q, dtype=np.float64)
+    bsz, heads, _, hd = q.shape
+    out = np.zeros((bsz, 1, heads * hd))
+    for b in range(bsz):
+        p = int(np.asarray(positions).reshape(-1)[b])
+        for h in range(heads):
+            k = np.asarray(k_cache[b, h, :p + 1], dtype=np.float64)
+            v = np.asarray(v_cache[b, h, :p + 1], dtype=np.float64)
+            s = k @ q[b, h, 0] / np.sqrt(hd)
+            w = np.exp(s - s.max())
+            out[b, 0, h * hd:(h + 1) * hd] = (w / w.sum()) @ v
+    return out

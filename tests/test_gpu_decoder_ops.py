@@ -1,0 +1,69 @@
+"""GPU parity of the decoder-side kernels (RMSNorm, single-query attention over the KV
+cache) against the oracle, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import bits
+from oracle import gptq_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def gptq():
+    import gptq_triton_amd
+    return gptq_triton_amd
+
+
+@pytest.mark.parametrize("m,h", [(1, 4096), (3, 5120), (17, 6656), (2048, 4096), (5, 64), (2, 8200)])
+def test_rmsnorm(m, h):
+    rng = np.random.default_rng(m + h)
+    x = (rng.standard_normal((m, h)) * rng.uniform(0.01, 30.0, size=(m, 1))).astype(np.float16)
+    w = (1.0 + 0.1 * rng.standard_normal(h)).astype(np.float16)
+    y = gptq().rms_norm(torch.from_numpy(x).cuda(), torch.from_numpy(w).cuda(), 1e-6).cpu().numpy()
+    ref = O.rmsnorm_ref(x, w, 1e-6)
+    # fp32 statistics against float64: the normalised value can round one fp16 step apart
+    diff = np.abs(y.astype(np.float64) - ref.astype(np.float64))
+    assert (diff <= 2 * np.spacing(np.abs(ref)).astype(np.float64)).all()
+    assert (bits(y) == bits(ref)).mean() > 0.98
+
+
+def test_rmsnorm_keeps_batch_dims_and_rejects_host_tensors():
+    x = torch.randn(2, 3, 256).half()
+    w = torch.ones(256).half()
+    with pytest.raises(RuntimeError):
+        gptq().rms_norm(x, w, 1e-6)
+    y = gptq().rms_norm(x.cuda(), w.cuda(), 1e-6)
+    assert y.shape == (2, 3, 256)
+    assert np.array_equal(y.cpu().numpy(), O.rmsnorm_ref(x.numpy(), w.numpy(), 1e-6)) or \
+        (np.abs(y.cpu().numpy().astype(np.float32) - O.rmsnorm_ref(x.numpy(), w.numpy(), 1e-6).astype(np.float32)) < 4e-3).all()
+
+
+@pytest.mark.parametrize("bsz,heads,cap,positions", [(1, 32, 2176, [2047]), (2, 8, 40, [0, 39]), (3, 5, 300, [1, 150, 299]),
+                                                     (8, 52, 515, [3, 100, 200, 300, 400, 500, 514, 64]), (1, 2, 16, [15])])
+def test_decode_attention(bsz, heads, cap, positions):
+    rng = np.random.default_rng(cap + heads)
+    q = rng.standard_normal((bsz, heads, 1, 128)).astype(np.float16)
+    k = rng.standard_normal((bsz, heads, cap, 128)).astype(np.float16)
+    v = rng.standard_normal((bsz, heads, cap, 128)).astype(np.float16)
+    pos = np.asarray(positions, dtype=np.int32)
+    # rows beyond each position hold poison: they must not be read into the result
+    for b, p in enumerate(positions):
+        k[b, :, p + 1:] = 300.0
+        v[b, :, p + 1:] = -1000.0
+    out = gptq().decode_attention(torch.from_numpy(q).cuda(), torch.from_numpy(k).cuda(), torch.from_numpy(v).cuda(),
+                                  torch.from_numpy(pos).cuda())
+    assert out.shape == (bsz, 1, heads * 128) and out.dtype == torch.float16
+    ref = O.decode_attention_ref(q, k, v, positions)
+    err = np.abs(out.cpu().numpy().astype(np.float64) - ref)
+    assert (err <= 2e-3 + 1e-2 * np.abs(ref)).all(), err.max()
+    assert err.max() < 2e-3  # fp32 softmax of fp16 inputs, one fp16 rounding of the result
+
+
+def test_decode_attention_peaked_scores_do_not_overflow():
+    q = torch.zeros(1, 1, 1, 128).half(); q[..., :] = 30.0
+    k = torch.zeros(1, 1, 70, 128).half(); k[0, 0, 33] = 30.0; k[0, 0, 2] = -30.0
+    v = torch.randn(1, 1, 70, 128).half()
+    out = gptq().decode_attention(q.cuda(), k.cuda(), v.cuda(), torch.tensor([69], dtype=torch.int32).cuda())
+    assert torch.isfinite(out).all()
+    assert torch.equal(out.cpu().reshape(128), v[0, 0, 33])

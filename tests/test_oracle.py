@@ -256,3 +256,45 @@ def test_qkv_rotary_layout():
     # a rotated row equals the closed form on the projected row
     cos, sin = O.rotary_tables(8, Dh)
     assert np.allclose(k[0, 1, 2], O.apply_rotary(y[0, 2, hidden + Dh:hidden + 2 * Dh], cos[7], sin[7]), atol=1e-5)
+
+
+# ------------------------------------------------------------------ decoder-side operators
+def test_rmsnorm_oracle_special_cases():
+    rng = np.random.default_rng(0)
+    w = rng.standard_normal(64).astype(np.float16)
+    # a constant row normalises to +-1 exactly, so y = +-weight
+    for c in (3.0, -0.25):
+        y = O.rmsnorm_ref(np.full((2, 64), c, dtype=np.float16), w, 0.0)
+        assert (y == np.sign(c).astype(np.float16) * w).all()
+    # invariant under scaling of x when eps = 0 (powers of two keep fp16 inputs exact)
+    x = rng.standard_normal((3, 64)).astype(np.float16)
+    assert (O.rmsnorm_ref(x, w, 0.0) == O.rmsnorm_ref(x * np.float16(4.0), w, 0.0)).all()
+    # unit weight: the output row has mean square 1 up to fp16 rounding
+    y = O.rmsnorm_ref(x, np.ones(64, dtype=np.float16), 1e-6).astype(np.float64)
+    assert np.allclose((y * y).mean(-1), 1.0, atol=2e-3)
+    # eps matters for tiny rows: x = 0 gives 0, not NaN
+    assert (O.rmsnorm_ref(np.zeros((1, 64), dtype=np.float16), w, 1e-6) == 0).all()
+
+
+def test_decode_attention_oracle_special_cases():
+    rng = np.random.default_rng(1)
+    B, H, cap, D = 2, 3, 9, 128
+    q = rng.standard_normal((B, H, 1, D)).astype(np.float16)
+    k = rng.standard_normal((B, H, cap, D)).astype(np.float16)
+    v = rng.standard_normal((B, H, cap, D)).astype(np.float16)
+    # position 0: the only visible row
+    out = O.decode_attention_ref(q, k, v, [0, 0])
+    assert np.array_equal(out.reshape(B, H, D), v[:, :, 0].astype(np.float64))
+    # equal keys: uniform weights, the mean of the visible V rows
+    k_eq = np.broadcast_to(k[:, :, :1], k.shape)
+    out = O.decode_attention_ref(q, k_eq, v, [4, 8])
+    assert np.allclose(out[0].reshape(H, D), v[0, :, :5].astype(np.float64).mean(1))
+    assert np.allclose(out[1].reshape(H, D), v[1, :, :9].astype(np.float64).mean(1))
+    # one key aligned with a large query dominates: its V row comes out
+    qb = np.zeros((1, 1, 1, D), dtype=np.float16); qb[..., 0] = 200.0
+    kb = np.zeros((1, 1, cap, D), dtype=np.float16); kb[0, 0, 6, 0] = 10.0
+    out = O.decode_attention_ref(qb, kb, v[:1, :1], [8])
+    assert np.allclose(out.reshape(D), v[0, 0, 6].astype(np.float64), atol=1e-9)
+    # rows beyond the position are invisible
+    v2 = v.copy(); v2[:, :, 5:] = 1e4
+    assert np.array_equal(O.decode_attention_ref(q, k, v, [4, 4]), O.decode_attention_ref(q, k, v2, [4, 4]))
