@@ -9,7 +9,7 @@ from . import fused_mlp, quant_linear
 from .fused_attention import (LlamaConfigLite, QuantLlamaAttention, RotaryTable, make_quant_attn, qkv_rotary)
 from .fused_mlp import QuantLlamaMLP, llama_mlp_4, make_fused_mlp, triton_llama_mlp_4
 from .quant_linear import (QuantLinear, dequantize, make_quant, matmul4, prepare_act_order, triton_matmul4)
-from .decoder_ops import decode_attention, rms_norm
+from .decoder_ops import add_rms_norm, decode_attention, rms_norm
 from .llama import GreedyDecoder, LlamaForCausalLM, config_from_json
 from .loader import autotune_warmup, load_quant, save_quant
 from .pack import pack_linear, quantize_rtn
@@ -19,4 +19,5 @@ __all__ = [
     "QuantLlamaMLP", "make_fused_mlp", "llama_mlp_4", "triton_llama_mlp_4",
     "QuantLlamaAttention", "make_quant_attn", "qkv_rotary", "RotaryTable", "LlamaConfigLite",
     "load_quant", "save_quant", "autotune_warmup", "LlamaForCausalLM", "config_from_json", "pack_linear", "quantize_rtn",
+    "GreedyDecoder", "rms_norm", "add_rms_norm", "decode_attention",
 ]

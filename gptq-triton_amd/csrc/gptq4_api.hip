@@ -288,7 +288,18 @@ int gptq4_rmsnorm(const void *x, const void *weight, void *y, int M, int H, floa
     if (!x || !weight || !y) return -GPTQ4_E_NULL;
     if (M < 1 || H < 8 || (H % 8) != 0 || !(eps >= 0.f)) return -GPTQ4_E_SHAPE;
     if (misaligned16(x) || misaligned16(weight) || misaligned16(y)) return -GPTQ4_E_ALIGN;
-    return launch_rmsnorm(reinterpret_cast<const half_t *>(x), reinterpret_cast<const half_t *>(weight),
+    return launch_rmsnorm(reinterpret_cast<const half_t *>(x), nullptr, reinterpret_cast<const half_t *>(weight), nullptr,
+                          reinterpret_cast<half_t *>(y), M, H, eps, reinterpret_cast<hipStream_t>(stream));
+}
+
+int gptq4_add_rmsnorm(const void *x, const void *delta, const void *weight, void *sum_out, void *y, int M, int H, float eps,
+                      void *stream) {
+    if (!x || !delta || !weight || !sum_out || !y) return -GPTQ4_E_NULL;
+    if (M < 1 || H < 8 || (H % 8) != 0 || !(eps >= 0.f)) return -GPTQ4_E_SHAPE;
+    if (misaligned16(x) || misaligned16(delta) || misaligned16(weight) || misaligned16(sum_out) || misaligned16(y))
+        return -GPTQ4_E_ALIGN;
+    return launch_rmsnorm(reinterpret_cast<const half_t *>(x), reinterpret_cast<const half_t *>(delta),
+                          reinterpret_cast<const half_t *>(weight), reinterpret_cast<half_t *>(sum_out),
                           reinterpret_cast<half_t *>(y), M, H, eps, reinterpret_cast<hipStream_t>(stream));
 }
 
@@ -296,14 +307,15 @@ int gptq4_decode_attention(const void *q, const void *k_cache, const void *v_cac
                            int B, int H, int D, int kv_capacity, float scale, void *workspace, size_t workspace_bytes,
                            void *stream) {
     if (!q || !k_cache || !v_cache || !positions || !out) return -GPTQ4_E_NULL;
-    if (B < 1 || H < 1 || D != 128 || kv_capacity < 1 || (long)B * H > 65535) return -GPTQ4_E_SHAPE;
+    if (B < 1 || H < 1 || D != 128 || kv_capacity < 1 || (long)B * H > SKINNY_MAX_TILES) return -GPTQ4_E_SHAPE;
     if (misaligned16(q) || misaligned16(k_cache) || misaligned16(v_cache) || misaligned16(out)) return -GPTQ4_E_ALIGN;
     if (workspace == nullptr || workspace_bytes < GPTQ4_WS_COUNTER_BYTES + attn_decode_partial_bytes(B * H, kv_capacity))
         return -GPTQ4_E_WORKSPACE;
     float *partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_COUNTER_BYTES);
     return launch_attn_decode(reinterpret_cast<const half_t *>(q), reinterpret_cast<const half_t *>(k_cache),
                               reinterpret_cast<const half_t *>(v_cache), positions, reinterpret_cast<half_t *>(out), B, H,
-                              kv_capacity, scale, partials, reinterpret_cast<hipStream_t>(stream));
+                              kv_capacity, scale, reinterpret_cast<int *>(workspace), partials,
+                              reinterpret_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

@@ -11,55 +11,85 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
-// y[row] = weight * fp16( x[row] * rsqrt(mean(x[row]^2) + eps) ): statistics and the
-// normalisation in fp32, rounded to fp16, then an fp16 multiply by the weight - the
-// rounding order of the LLaMA RMSNorm module.  One workgroup per row, H % 8 == 0.
-__global__ __launch_bounds__(256) void gptq4_rmsnorm_kernel(const half_t *__restrict__ x, const half_t *__restrict__ w,
-                                                            half_t *__restrict__ y, int H, float eps) {
+// y[row] = weight * fp16( s[row] * rsqrt(mean(s[row]^2) + eps) ) with s = x (ADD false) or
+// s = fp16(x + delta), also written to sum_out (ADD true: the residual add that precedes
+// every RMSNorm of a decoder layer).  Statistics and the normalisation in fp32, rounded to
+// fp16, then an fp16 multiply by the weight - the rounding order of the LLaMA RMSNorm
+// module.  One workgroup per row, H % 8 == 0; sum_out may alias x.
+template <bool ADD>
+__global__ __launch_bounds__(256) void gptq4_rmsnorm_kernel(const half_t *x, const half_t *delta, const half_t *__restrict__ w,
+                                                            half_t *sum_out, half_t *__restrict__ y, int H, float eps) {
     __shared__ float part[4];
     const int tid = threadIdx.x;
-    const uint4 *xr = reinterpret_cast<const uint4 *>(x + (size_t)blockIdx.x * H);
+    const size_t row = (size_t)blockIdx.x * H;
+    const uint4 *xr = reinterpret_cast<const uint4 *>(x + row);
+    const uint4 *dr = reinterpret_cast<const uint4 *>(delta + (ADD ? row : 0));
     const uint4 *wr = reinterpret_cast<const uint4 *>(w);
-    uint4 *yr = reinterpret_cast<uint4 *>(y + (size_t)blockIdx.x * H);
+    uint4 *sr = reinterpret_cast<uint4 *>(sum_out + (ADD ? row : 0));
+    uint4 *yr = reinterpret_cast<uint4 *>(y + row);
     const int chunks = H >> 3;
+    constexpr int KEEP = 4;  // chunks per thread held in registers (covers H <= 8192); beyond that re-read
+    uint4 held[KEEP];
     float ss = 0.f;
-    for (int c = tid; c < chunks; c += 256) {
-        const uint4 v = xr[c];
+    auto take = [&](int c) {
+        uint4 v = xr[c];
+        if (ADD) {
+            const uint4 d = dr[c];
+            v.x = as_u32(as_h2(v.x) + as_h2(d.x));
+            v.y = as_u32(as_h2(v.y) + as_h2(d.y));
+            v.z = as_u32(as_h2(v.z) + as_h2(d.z));
+            v.w = as_u32(as_h2(v.w) + as_h2(d.w));
+            sr[c] = v;
+        }
         const h2_t p[4] = {as_h2(v.x), as_h2(v.y), as_h2(v.z), as_h2(v.w)};
 #pragma unroll
         for (int i = 0; i < 4; ++i) ss += (float)p[i].x * (float)p[i].x + (float)p[i].y * (float)p[i].y;
-    }
+        return v;
+    };
+#pragma unroll
+    for (int n = 0; n < KEEP; ++n)
+        if (tid + 256 * n < chunks) held[n] = take(tid + 256 * n);
+    for (int c = tid + 256 * KEEP; c < chunks; c += 256) take(c);
     ss = wave_sum(ss);
     if ((tid & 63) == 0) part[tid >> 6] = ss;
     __syncthreads();
     const float inv = rsqrtf((part[0] + part[1] + part[2] + part[3]) / (float)H + eps);
-    for (int c = tid; c < chunks; c += 256) {
-        const uint4 v = xr[c], g = wr[c];
+    auto put = [&](int c, uint4 v) {
+        const uint4 g = wr[c];
         const uint32_t vi[4] = {v.x, v.y, v.z, v.w}, gi[4] = {g.x, g.y, g.z, g.w};
         uint32_t o[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const h2_t p = as_h2(vi[i]);
-            const h2_t n = {(half_t)((float)p.x * inv), (half_t)((float)p.y * inv)};
-            o[i] = as_u32(as_h2(gi[i]) * n);
+            const h2_t nrm = {(half_t)((float)p.x * inv), (half_t)((float)p.y * inv)};
+            o[i] = as_u32(as_h2(gi[i]) * nrm);
         }
         yr[c] = make_uint4(o[0], o[1], o[2], o[3]);
-    }
+    };
+#pragma unroll
+    for (int n = 0; n < KEEP; ++n)
+        if (tid + 256 * n < chunks) put(tid + 256 * n, held[n]);
+    // chunks past the held ones: this thread wrote sr[c] itself (ADD), or x is unchanged
+    for (int c = tid + 256 * KEEP; c < chunks; c += 256) put(c, ADD ? sr[c] : xr[c]);
 }
 
 // Single-query attention, split over the cache length.  Workgroup (split, b*H + h) takes
 // rows [split*chunk, ...) of the valid prefix 0..positions[b]; 16 lanes share a row (8
 // head dimensions each, one 16-byte load of K and of V per lane), 16 rows per pass,
 // running (max, sum, weighted V) per thread in fp32; the 16 row slots are merged through
-// LDS and the partial [max, sum, acc[128]] goes to the workspace.
+// LDS and the partial [max, sum, acc[128]] goes to the workspace.  The splits of one (b, h)
+// meet through an arrival counter (agent-scope stores, completion wait, atomic count, as
+// in the matmul kernels); the last one merges the partials in split order and writes
+// out[b, h*128 + d].
 constexpr int ATT_PART = 130;  // floats per partial: max, sum, 128 accumulators
 
-__global__ __launch_bounds__(256) void gptq4_attn_partial_kernel(const half_t *__restrict__ q, const half_t *__restrict__ kc,
-                                                                 const half_t *__restrict__ vc, const int *__restrict__ positions,
-                                                                 float *__restrict__ part, int H, int capacity, int chunk,
-                                                                 float scale) {
+__global__ __launch_bounds__(256) void gptq4_attn_decode_kernel(const half_t *__restrict__ q, const half_t *__restrict__ kc,
+                                                                const half_t *__restrict__ vc, const int *__restrict__ positions,
+                                                                float *part, int *counters, half_t *__restrict__ out, int H,
+                                                                int capacity, int chunk, float scale) {
     __shared__ float s_m[16], s_l[16];
     __shared__ float s_acc[16][128];
+    __shared__ int s_is_last;
     const int tid = threadIdx.x;
     const int slot = tid >> 4, sub = tid & 15;
     const int bh = blockIdx.y, split = blockIdx.x, nsplit = gridDim.x;
@@ -123,46 +153,71 @@ __global__ __launch_bounds__(256) void gptq4_attn_partial_kernel(const half_t *_
 #pragma unroll
     for (int i = 0; i < 8; ++i) s_acc[slot][8 * sub + i] = acc[i];
     __syncthreads();
+    float mw = -INFINITY, lw = 0.f, a = 0.f;  // threads 0..127: this workgroup's partial for dimension tid
     if (tid < 128) {
-        float mw = -INFINITY;
 #pragma unroll
         for (int s = 0; s < 16; ++s) mw = fmaxf(mw, s_m[s]);
-        float lw = 0.f, a = 0.f;
 #pragma unroll
         for (int s = 0; s < 16; ++s) {
             const float f = (s_m[s] == -INFINITY) ? 0.f : __expf(s_m[s] - mw);
             lw += s_l[s] * f;
             a += s_acc[s][tid] * f;
         }
-        float *dst = part + ((size_t)bh * nsplit + split) * ATT_PART;
-        if (tid == 0) {
-            dst[0] = mw;
-            dst[1] = lw;
+    }
+    if (nsplit > 1) {
+        float *base = part + (size_t)bh * nsplit * ATT_PART;
+        if (tid < 128) {
+            float *dst = base + (size_t)split * ATT_PART;
+            if (tid == 0) {
+                __hip_atomic_store(dst, mw, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(dst + 1, lw, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            __hip_atomic_store(dst + 2 + tid, a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        dst[2 + tid] = a;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) {
+            const int old = __hip_atomic_fetch_add(&counters[bh * COUNTER_STRIDE], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s_is_last = (old == nsplit - 1);
+        }
+        __syncthreads();
+        if (!s_is_last) return;
+        if (tid == 0) __hip_atomic_store(&counters[bh * COUNTER_STRIDE], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (tid < 128) {
+            mw = -INFINITY, lw = 0.f, a = 0.f;
+            for (int s0 = 0; s0 < nsplit; s0 += 8) {
+                float ms[8], ls[8], as[8];
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {  // all loads issued together; slots past the end re-read the last
+                    const float *src = base + (size_t)min(s0 + k, nsplit - 1) * ATT_PART;
+                    ms[k] = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    ls[k] = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    as[k] = __hip_atomic_load(src + 2 + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    if (s0 + k < nsplit && ms[k] != -INFINITY) {
+                        const float mn = fmaxf(mw, ms[k]);
+                        const float f0 = __expf(mw - mn), f1 = __expf(ms[k] - mn);
+                        lw = lw * f0 + ls[k] * f1;
+                        a = a * f0 + as[k] * f1;
+                        mw = mn;
+                    }
+                }
+            }
+        }
     }
-}
-
-// out[b, h*128 + d] = sum over splits of acc * exp(max_s - max) / sum of sums likewise.
-__global__ __launch_bounds__(128) void gptq4_attn_combine_kernel(const float *__restrict__ part, half_t *__restrict__ out, int nsplit) {
-    const int bh = blockIdx.x, d = threadIdx.x;
-    const float *src = part + (size_t)bh * nsplit * ATT_PART;
-    float mw = -INFINITY;
-    for (int s = 0; s < nsplit; ++s) mw = fmaxf(mw, src[s * ATT_PART]);
-    float lw = 0.f, a = 0.f;
-    for (int s = 0; s < nsplit; ++s) {
-        const float ms = src[s * ATT_PART];
-        const float f = (ms == -INFINITY) ? 0.f : __expf(ms - mw);
-        lw += src[s * ATT_PART + 1] * f;
-        a += src[s * ATT_PART + 2 + d] * f;
-    }
-    out[(size_t)bh * 128 + d] = (half_t)(a / lw);
+    if (tid < 128) out[(size_t)bh * 128 + tid] = (half_t)(a / lw);
 }
 
 }  // namespace
 
-int launch_rmsnorm(const half_t *x, const half_t *w, half_t *y, int M, int H, float eps, hipStream_t stream) {
-    hipLaunchKernelGGL(gptq4_rmsnorm_kernel, dim3((unsigned)M), dim3(256), 0, stream, x, w, y, H, eps);
+int launch_rmsnorm(const half_t *x, const half_t *delta, const half_t *w, half_t *sum_out, half_t *y, int M, int H, float eps,
+                   hipStream_t stream) {
+    if (delta != nullptr)
+        hipLaunchKernelGGL(gptq4_rmsnorm_kernel<true>, dim3((unsigned)M), dim3(256), 0, stream, x, delta, w, sum_out, y, H, eps);
+    else
+        hipLaunchKernelGGL(gptq4_rmsnorm_kernel<false>, dim3((unsigned)M), dim3(256), 0, stream, x, x, w, y, y, H, eps);
     return (int)hipGetLastError();
 }
 
@@ -180,15 +235,12 @@ size_t attn_decode_partial_bytes(int BH, int capacity) {
 }
 
 int launch_attn_decode(const half_t *q, const half_t *kc, const half_t *vc, const int *positions, half_t *out, int B,
-                       int H, int capacity, float scale, float *partials, hipStream_t stream) {
+                       int H, int capacity, float scale, int *counters, float *partials, hipStream_t stream) {
     const int BH = B * H;
     const int nsplit = attn_decode_splits(BH, capacity);
     int chunk = (capacity + nsplit - 1) / nsplit;
     chunk = (chunk + 15) & ~15;
-    hipLaunchKernelGGL(gptq4_attn_partial_kernel, dim3((unsigned)nsplit, (unsigned)BH), dim3(256), 0, stream, q, kc, vc,
-                       positions, partials, H, capacity, chunk, scale);
-    int rc = (int)hipGetLastError();
-    if (rc) return rc;
-    hipLaunchKernelGGL(gptq4_attn_combine_kernel, dim3((unsigned)BH), dim3(128), 0, stream, partials, out, nsplit);
+    hipLaunchKernelGGL(gptq4_attn_decode_kernel, dim3((unsigned)nsplit, (unsigned)BH), dim3(256), 0, stream, q, kc, vc,
+                       positions, partials, counters, out, H, capacity, chunk, scale);
     return (int)hipGetLastError();
 }

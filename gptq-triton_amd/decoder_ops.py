@@ -32,6 +32,26 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     return y.reshape(x.shape)
 
 
+def add_rms_norm(x: torch.Tensor, delta: torch.Tensor, weight: torch.Tensor, eps: float):
+    """(x + delta, RMSNorm(x + delta)) in one launch; fp16 GPU tensors of equal shape [..., H]."""
+    for t, name in ((x, "x"), (delta, "delta"), (weight, "weight")):
+        _lib.require_cuda(t, name)
+        if t.dtype != torch.float16:
+            raise TypeError("add_rms_norm takes fp16 tensors")
+    h = x.shape[-1]
+    if delta.shape != x.shape or weight.shape != (h,) or h % 8 != 0:
+        raise ValueError("x and delta must have one shape [..., H], weight [H], H a multiple of 8")
+    x2 = x.reshape(-1, h).contiguous()
+    d2 = delta.reshape(-1, h).contiguous()
+    s = torch.empty_like(x2)
+    y = torch.empty_like(x2)
+    if x2.shape[0]:
+        rc = _lib.load().gptq4_add_rmsnorm(x2.data_ptr(), d2.data_ptr(), weight.data_ptr(), s.data_ptr(), y.data_ptr(),
+                                           x2.shape[0], h, float(eps), _lib.current_stream(x.device))
+        _lib.check(rc, "gptq4_add_rmsnorm")
+    return s.reshape(x.shape), y.reshape(x.shape)
+
+
 def decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
     """q fp16 [B, H, 1, 128]; caches fp16 [B, H, capacity, 128]; positions int32 [B] or [B, 1]:
     sequence b attends to cache rows 0..positions[b].  Returns fp16 [B, 1, H*128]."""

@@ -17,7 +17,7 @@ from typing import List, Optional, Tuple
 import torch
 import torch.nn as nn
 
-from .decoder_ops import decode_attention, rms_norm
+from .decoder_ops import add_rms_norm, decode_attention, rms_norm
 from .fused_attention import LlamaConfigLite
 
 
@@ -175,12 +175,18 @@ class GreedyDecoder:
         self.graph = None
 
     def _layers(self, h, position_ids, kv_offset, attend):
-        for layer, (kc, vc) in zip(self.model.model.layers, self.caches):
+        """The decoder stack on hidden states h [B, S, hidden]; every residual add is fused
+        with the RMSNorm that follows it.  Returns the greedy next token [B, 1]."""
+        layers = self.model.model.layers
+        x = layers[0].input_layernorm(h)
+        for i, (layer, (kc, vc)) in enumerate(zip(layers, self.caches)):
             attn = layer.self_attn
-            q, _, _ = attn.project_qkv(layer.input_layernorm(h), position_ids, kv_out=(kc, vc), kv_offset=kv_offset)
-            h = h + attn.o_proj(attend(q, kc, vc))  # attend -> [B, q_len, hidden]
-            h = h + layer.mlp(layer.post_attention_layernorm(h))
-        return self.model.lm_head(self.model.model.norm(h[:, -1:, :])).argmax(-1)
+            q, _, _ = attn.project_qkv(x, position_ids, kv_out=(kc, vc), kv_offset=kv_offset)
+            norm = layer.post_attention_layernorm
+            h, x = add_rms_norm(h, attn.o_proj(attend(q, kc, vc)), norm.weight, norm.variance_epsilon)  # attend -> [B, S, hidden]
+            norm = layers[i + 1].input_layernorm if i + 1 < len(layers) else self.model.model.norm
+            h, x = add_rms_norm(h, layer.mlp(x), norm.weight, norm.variance_epsilon)
+        return self.model.lm_head(x[:, -1:, :]).argmax(-1)
 
     @torch.no_grad()
     def prefill(self, input_ids: torch.Tensor) -> torch.Tensor:

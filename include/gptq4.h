@@ -131,11 +131,18 @@ int gptq4_qkv_rotary(const void *x, const int32_t *qweight, const int32_t *qzero
  * (src/gptq_triton/__init__.py:32-47; the quantised linears are the only modules it swaps). */
 int gptq4_rmsnorm(const void *x, const void *weight, void *y, int M, int H, float eps, void *stream);
 
+/* The residual add that precedes every RMSNorm of a decoder layer, fused with it:
+ * sum_out = fp16(x + delta) (may alias x), y = RMSNorm(sum_out).  Same shapes as above.  In
+ * the reference these are two torch ops of the HF decoder layer around its patched blocks. */
+int gptq4_add_rmsnorm(const void *x, const void *delta, const void *weight, void *sum_out, void *y,
+                      int M, int H, float eps, void *stream);
+
 /* Attention of ONE query token per sequence over a preallocated KV cache: for each (b, h)
  * softmax(q . K[0..positions[b]]^T * scale) . V[0..positions[b]], in fp32, written as fp16
  * out [B, H*D] (the layout o_proj consumes).  q fp16 [B, H, 1, D]; k_cache, v_cache fp16
  * [B, H, kv_capacity, D]; positions int32 [B] (clamped into [0, kv_capacity)); D must be
- * 128.  Replaces the attention core of QuantLlamaAttention.forward for q_len == 1
+ * 128; B * H <= 4096.  workspace as for the matmuls (zeroed head, gptq4_workspace_bytes with
+ * GPTQ4_OP_DECODE_ATTENTION).  Replaces the attention core of QuantLlamaAttention.forward for q_len == 1
  * (fused_attention.py:118-148: scores, mask, fp32 softmax, weighted sum, transpose). */
 int gptq4_decode_attention(const void *q, const void *k_cache, const void *v_cache,
                            const int32_t *positions, void *out, int B, int H, int D,

@@ -28,6 +28,23 @@ def test_rmsnorm(m, h):
     assert (bits(y) == bits(ref)).mean() > 0.98
 
 
+@pytest.mark.parametrize("m,h", [(1, 4096), (4, 5120), (300, 6656), (2, 8200)])
+def test_add_rmsnorm(m, h):
+    rng = np.random.default_rng(m * h)
+    x = (rng.standard_normal((m, h)) * 3).astype(np.float16)
+    d = rng.standard_normal((m, h)).astype(np.float16)
+    w = (1.0 + 0.1 * rng.standard_normal(h)).astype(np.float16)
+    s, y = gptq().add_rms_norm(torch.from_numpy(x).cuda(), torch.from_numpy(d).cuda(), torch.from_numpy(w).cuda(), 1e-6)
+    s_ref = (x + d).astype(np.float16)   # one fp16 add, as torch does
+    assert np.array_equal(bits(s.cpu().numpy()), bits(s_ref))
+    ref = O.rmsnorm_ref(s_ref, w, 1e-6)
+    diff = np.abs(y.cpu().numpy().astype(np.float64) - ref.astype(np.float64))
+    assert (diff <= 2 * np.spacing(np.abs(ref)).astype(np.float64)).all()
+    # and it is the unfused kernel applied to the sum, bit for bit
+    y2 = gptq().rms_norm(s, torch.from_numpy(w).cuda(), 1e-6)
+    assert torch.equal(y, y2)
+
+
 def test_rmsnorm_keeps_batch_dims_and_rejects_host_tensors():
     x = torch.randn(2, 3, 256).half()
     w = torch.ones(256).half()
