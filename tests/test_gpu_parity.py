@@ -304,3 +304,24 @@ def test_fused_qkv_equals_three_projections():
                 # the split-K factor depends on N, so the fp32 summation order may differ
                 d = (yf[:, i * hidden:(i + 1) * hidden].float() - yp.float()).abs().max().item()
                 assert d <= 2 ** -7
+
+
+def test_tiled_kernel_gathers_act_order_rows_itself_when_asked():
+    """The Python layer applies the permutation to tall inputs before the call; the C entry
+    point still accepts `perm` for any M (the tiled kernel then gathers in its A staging)."""
+    from gptq_triton_amd import _lib
+    k, n, g, m = 1024, 512, 128, 40
+    L = O.make_layer(k, n, g, seed=31, act_order=True)
+    x = O.make_x(m, k, seed=32)
+    G = gptq()
+    qs, perm = G.prepare_act_order(torch.from_numpy(L["qweight"]).cuda(), torch.from_numpy(L["g_idx"]).cuda(), g)
+    D = to_dev(L)
+    xd = torch.from_numpy(x).cuda()
+    y = torch.empty((m, n), dtype=torch.float16, device="cuda")
+    lib = _lib.load()
+    ws = _lib.workspace(xd.device, lib.gptq4_workspace_bytes(_lib.OP_MATMUL, m, k, n))
+    rc = lib.gptq4_matmul(xd.data_ptr(), qs.data_ptr(), D["qzeros"].data_ptr(), D["scales"].data_ptr(), perm.data_ptr(), None,
+                          y.data_ptr(), m, k, n, g, ws.data_ptr(), ws.numel(), _lib.current_stream(xd.device))
+    assert rc == 0
+    ref = O.quant_matmul_ref(x, L["qweight"], L["qzeros"], L["scales"], g, g_idx=L["g_idx"])
+    assert_close(y.cpu().numpy(), ref, "tiled kernel, in-kernel act-order gather")
