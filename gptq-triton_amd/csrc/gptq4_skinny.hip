@@ -404,12 +404,6 @@ int launch_epi(const MatmulArgs &a, const SkinnyPlan &pl, hipStream_t stream) {
         case 424: return launch_variant<EPI, 2, 4, 4>(a, stream);
         case 441: return launch_variant<EPI, 4, 1, 4>(a, stream);
         case 442: return launch_variant<EPI, 4, 2, 4>(a, stream);
-        case 821: return launch_variant<EPI, 2, 1, 8>(a, stream);
-        case 822: return launch_variant<EPI, 2, 2, 8>(a, stream);
-        case 841: return launch_variant<EPI, 4, 1, 8>(a, stream);
-        case 842: return launch_variant<EPI, 4, 2, 8>(a, stream);
-        case 1621: return launch_variant<EPI, 2, 1, 16>(a, stream);
-        case 1622: return launch_variant<EPI, 2, 2, 16>(a, stream);
         default: return launch_variant<EPI, 2, 2, 4>(a, stream);
     }
 }
