@@ -38,8 +38,19 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
     constexpr int BN = (EPI == EPI_SILU_MUL) ? 64 : 128;
     constexpr int A_UNITS = BM * (BK / 8) / 256;  // 16-byte units each thread stages per K tile
 
-    __shared__ __attribute__((aligned(16))) half_t As[2][BM][LDS_ROW];
-    static_assert(sizeof(As) >= 4 * 32 * 64 * sizeof(float), "epilogue exchange buffer does not fit");
+    // Activation tiles.  Plain path: two unpadded buffers of BM x 64 halves filled by
+    // LDS-direct loads (two separate objects, so that the compiler can tell a load into one
+    // from the reads of the other); act-order path: one padded double buffer filled through
+    // registers.  The epilogues reuse them as four 8 KiB exchange regions.
+    constexpr int A_HALVES = BM * BK;
+    __shared__ __attribute__((aligned(16))) half_t As0[PERM ? 2 * BM * LDS_ROW : A_HALVES];
+    __shared__ __attribute__((aligned(16))) half_t As1[PERM ? 8 : A_HALVES];
+    static_assert(PERM ? sizeof(As0) >= 4 * 32 * 64 * sizeof(float) : sizeof(As0) >= 2 * 32 * 64 * sizeof(float),
+                  "epilogue exchange regions do not fit");
+    auto region = [&](int w) -> float * {
+        if (PERM) return reinterpret_cast<float *>(As0) + w * (32 * 64);
+        return reinterpret_cast<float *>(w < 2 ? As0 : As1) + (w & 1) * (32 * 64);
+    };
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -91,7 +102,7 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
         const int row = min(a_row + 32 * u, M - 1 - m0);
         a_off[u] = (uint32_t)row * (uint32_t)K + 8u * a_ku;
     }
-    half_t *const a_lds = &As[0][a_row][8 * a_ku];
+    half_t *const a_lds = As0 + a_row * LDS_ROW + 8 * a_ku;  // act-order path
 
     uint4 a_stage[A_UNITS];
     uint2 bw[4];  // packed B words of the 4 K steps; refilled in place for the next K tile
@@ -145,56 +156,155 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
     const int nk = k_begin + p.slot_q + (split < p.slot_rem ? 1 : 0);
     int group = (p.splitk > 1) ? k_begin / tiles_per_group : 0;
     int left_in_group = tiles_per_group - (k_begin - group * tiles_per_group);  // K tiles left in the group
-    load_a(k_begin);
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) load_b_step(k_begin, ks);
-    load_group(group);
-    make_cd();
+    if constexpr (PERM) {
+        load_a(k_begin);
+    #pragma unroll
+        for (int ks = 0; ks < 4; ++ks) load_b_step(k_begin, ks);
+        load_group(group);
+        make_cd();
 
-    // B operands of the K step about to be multiplied.  They are decoded one step ahead,
-    // in place, right after the MFMAs that consumed the previous contents were issued, so
-    // the decode (VALU) of step s+1 runs under the MFMAs of step s.
-    h8_t bf[2];
-    bf[0] = decode_word_h8(bw[0].x, cd[0]);
-    bf[1] = decode_word_h8(bw[0].y, cd[1]);
-    load_b_step(min(k_begin + 1, nk - 1), 0);
+        // B operands of the K step about to be multiplied.  They are decoded one step ahead,
+        // in place, right after the MFMAs that consumed the previous contents were issued, so
+        // the decode (VALU) of step s+1 runs under the MFMAs of step s.
+        h8_t bf[2];
+        bf[0] = decode_word_h8(bw[0].x, cd[0]);
+        bf[1] = decode_word_h8(bw[0].y, cd[1]);
+        load_b_step(min(k_begin + 1, nk - 1), 0);
 
-    for (int kt = k_begin; kt < nk; ++kt) {
-        const int buf = kt & 1;
-        store_a(buf);
-        __syncthreads();
-        const int kn = min(kt + 1, nk - 1), kn2 = min(kt + 2, nk - 1);
-        const bool new_group = (left_in_group == 1);
-        load_a(kn);
-        load_group(min(group + (new_group ? 1 : 0), last_group));
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-            h8_t af[MT];
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                const int row = wm * (32 * MT) + mt * 32 + l32;
-                af[mt] = *reinterpret_cast<const h8_t *>(&As[buf][row][8 * (2 * ks + lhi)]);
+        for (int kt = k_begin; kt < nk; ++kt) {
+            const int buf = kt & 1;
+            store_a(buf);
+            __syncthreads();
+            const int kn = min(kt + 1, nk - 1), kn2 = min(kt + 2, nk - 1);
+            const bool new_group = (left_in_group == 1);
+            load_a(kn);
+            load_group(min(group + (new_group ? 1 : 0), last_group));
+    #pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                h8_t af[MT];
+    #pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    const int row = wm * (32 * MT) + mt * 32 + l32;
+                    af[mt] = *reinterpret_cast<const h8_t *>(As0 + (buf * BM + row) * LDS_ROW + 8 * (2 * ks + lhi));
+                }
+                if (ks == 3) make_cd();  // constants of the next K tile; this tile's decodes are all done
+                const uint2 nw = bw[(ks + 1) & 3];  // words of the next step (step 0 of the next tile when ks == 3)
+                // refill: step ks+1 of the next tile (step 0 of tile kt+2 when ks == 3)
+                if (ks < 3)
+                    load_b_step(kn, ks + 1);
+                else
+                    load_b_step(kn2, 0);
+    #pragma unroll
+                for (int mt = 0; mt < MT; ++mt) acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt], bf[0], acc[mt][0], 0, 0, 0);
+                bf[0] = decode_word_h8(nw.x, cd[0]);
+    #pragma unroll
+                for (int mt = 0; mt < MT; ++mt) acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt], bf[1], acc[mt][1], 0, 0, 0);
+                bf[1] = decode_word_h8(nw.y, cd[1]);
             }
-            if (ks == 3) make_cd();  // constants of the next K tile; this tile's decodes are all done
-            const uint2 nw = bw[(ks + 1) & 3];  // words of the next step (step 0 of the next tile when ks == 3)
-            // refill: step ks+1 of the next tile (step 0 of tile kt+2 when ks == 3)
-            if (ks < 3)
-                load_b_step(kn, ks + 1);
-            else
-                load_b_step(kn2, 0);
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt], bf[0], acc[mt][0], 0, 0, 0);
-            bf[0] = decode_word_h8(nw.x, cd[0]);
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt], bf[1], acc[mt][1], 0, 0, 0);
-            bf[1] = decode_word_h8(nw.y, cd[1]);
+            if (new_group) {
+                ++group;
+                left_in_group = tiles_per_group;
+            } else {
+                --left_in_group;
+            }
         }
-        if (new_group) {
-            ++group;
-            left_in_group = tiles_per_group;
-        } else {
-            --left_in_group;
+    } else {
+        // ---- plain path: activations go global -> LDS directly (no staging registers, so the
+        // loads of tile kt+1 are in flight under the MFMAs of tile kt).  A wave instruction
+        // fills 64 consecutive 16-byte chunks = 8 rows x 8 chunks; chunk c of row r sits at
+        // position c ^ ((r >> 1) & 7) of its row, which makes the 128-bit fragment reads
+        // (16 lanes = 16 rows, one position each) conflict-free without padding.  The lane
+        // picks the global chunk that belongs at its fixed LDS slot.
+        uint32_t a_goff[A_UNITS];
+#pragma unroll
+        for (int u = 0; u < A_UNITS; ++u) {
+            const int slot = (u * 4 + wave) * 64 + lane;
+            const int row = slot >> 3;
+            const int c = (slot & 7) ^ ((row >> 1) & 7);
+            a_goff[u] = (uint32_t)min(row, M - 1 - m0) * (uint32_t)K + 8u * c;
         }
+        // Buffer-addressed form of the LDS-direct load: unlike the flat/global form the compiler
+        // counts it in order with the other vector-memory loads, so its waits for the packed
+        // words stay exact while activation tiles are in flight.
+        const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)a_base, 0, (int)((uint32_t)min(BM, M - m0) * (uint32_t)K * 2u), 0x00020000);
+        auto dma_a = [&](half_t *dst, int kt) {
+#pragma unroll
+            for (int u = 0; u < A_UNITS; ++u)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (__attribute__((address_space(3))) void *)(dst + (u * 4 + wave) * 512),
+                                                         16, (int)(a_goff[u] * 2u), kt * (BK * 2), 0, 0);
+            asm volatile("" ::: "memory");  // the loads that follow stay behind these
+        };
+        const int sw = (l32 >> 1) & 7;  // (row >> 1) & 7 for every row this lane reads (rows = 32*j + l32)
+
+        dma_a(As0, k_begin);
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) load_b_step(k_begin, ks);
+        load_group(group);
+        make_cd();
+        h8_t bf[2];
+        bf[0] = decode_word_h8(bw[0].x, cd[0]);
+        bf[1] = decode_word_h8(bw[0].y, cd[1]);
+        load_b_step(min(k_begin + 1, nk - 1), 0);
+
+        // one K tile from buffer `cur`, while the next tile streams into `nxt`
+        auto k_tile = [&](const half_t *cur, half_t *nxt, int kt) {
+            // Every wave has issued at least 4 vector-memory loads after its LDS-direct loads
+            // of this tile (the scale/zero words and the packed words of 4 K steps), and
+            // loads complete in order: at most 4 outstanding means the tile has landed.
+            asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            const int kn = min(kt + 1, nk - 1), kn2 = min(kt + 2, nk - 1);
+            const bool new_group = (left_in_group == 1);
+            dma_a(nxt, kn);
+            load_group(min(group + (new_group ? 1 : 0), last_group));
+            // fragments of K step ks+1 are read from LDS before the MFMAs of step ks are issued
+            uint4 araw[MT];
+            auto read_a = [&](int ks) {
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    const int row = wm * (32 * MT) + mt * 32 + l32;
+                    araw[mt] = *reinterpret_cast<const uint4 *>(cur + row * BK + 8 * ((2 * ks + lhi) ^ sw));
+                }
+            };
+            read_a(0);
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                h8_t af[MT];
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) af[mt] = pair_order_a(araw[mt]);
+                if (ks < 3) read_a(ks + 1);
+                if (ks == 3) make_cd();
+                const uint2 nw = bw[(ks + 1) & 3];
+                if (ks < 3)
+                    load_b_step(kn, ks + 1);
+                else
+                    load_b_step(kn2, 0);
+                __builtin_amdgcn_sched_barrier(0);  // keep the loads above the MFMAs that hide them
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt], bf[0], acc[mt][0], 0, 0, 0);
+                bf[0] = decode_word_h8(nw.x, cd[0]);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt], bf[1], acc[mt][1], 0, 0, 0);
+                bf[1] = decode_word_h8(nw.y, cd[1]);
+            }
+            if (new_group) {
+                ++group;
+                left_in_group = tiles_per_group;
+            } else {
+                --left_in_group;
+            }
+        };
+        // pairs of tiles without a branch between them (a join there would make the compiler
+        // move packed words that are still in flight, and wait for them), then the odd one
+        int kt = k_begin;
+        for (; kt + 1 < nk; kt += 2) {
+            k_tile(As0, As1, kt);
+            k_tile(As1, As0, kt + 1);
+        }
+        if (kt < nk) k_tile(As0, As1, kt);
+        // all LDS-direct loads have landed and every wave is done reading before the
+        // epilogues reuse the buffers
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     }
 
     if (p.splitk > 1) {
@@ -232,11 +342,17 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-                for (int t = 0; t < 2; ++t)
+                for (int t = 0; t < 2; ++t) {
+                    // 16 loads in flight, then 16 adds (added as they are loaded, each would
+                    // wait for its own round trip)
+                    float got[16];
 #pragma unroll
                     for (int i = 0; i < 16; ++i)
-                        acc[mt][t][i] += __hip_atomic_load(all + ((size_t)sp * NREG + (mt * 2 + t) * 16 + i) * 256,
-                                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        got[i] = __hip_atomic_load(all + ((size_t)sp * NREG + (mt * 2 + t) * 16 + i) * 256,
+                                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) acc[mt][t][i] += got[i];
+                }
         }
         if (tid == 0) __hip_atomic_store(&p.counters[tile * COUNTER_STRIDE], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
@@ -245,7 +361,6 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
     //      column = 2*l32 + t of the wave.
     const int wrow0 = m0 + wm * (32 * MT);
     // exchange buffer: [wave][t*16 + i][lane], reusing the activation tiles
-    float *const ex = reinterpret_cast<float *>(&As[0][0][0]);
     if (EPI == EPI_PLAIN) {
         h2_t bias2 = {(half_t)0.f, (half_t)0.f};
         if (p.bias != nullptr) bias2 = as_h2(*reinterpret_cast<const uint32_t *>(p.bias + ncol));
@@ -262,7 +377,7 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
             }
     } else if (EPI == EPI_SILU_MUL) {
         // hand the up accumulators (wn == 1) to the gate wave (wn == 0) with the same wm
-        float *const mine = ex + wm * (32 * 64);
+        float *const mine = region(wm);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             __syncthreads();
@@ -294,8 +409,8 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
         const int head_col = n0 >> 7;
         const int which = head_col / r.H;
         const int head = head_col - which * r.H;
-        float *const mine = ex + wave * (32 * 64);
-        const float *const theirs = ex + (wave ^ 2) * (32 * 64);
+        float *const mine = region(wave);
+        const float *const theirs = region(wave ^ 2);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             if (which < 2) {
