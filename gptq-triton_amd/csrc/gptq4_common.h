@@ -74,6 +74,40 @@ __device__ __forceinline__ h8_t decode_word_h8(uint32_t w, const ColDecode &c) {
     return r;
 }
 
+// Natural-order variant for the tiled kernel, whose activation operand arrives in LDS
+// straight from memory and cannot be put in pair order on the way.  A byte permute puts
+// byte j of the word (nibbles 2j, 2j+1) into both halves; the mask 0x00F0000F then leaves
+// 1024 + q_{2j} in the low half and 1024 + 16 * q_{2j+1} in the high half, and one packed
+// fma with the per-half constants (1, 1/16) and (-(1025 + z), -(65 + z)) gives the exact
+// integers q - (z + 1) in both.  16 VALU ops per word instead of 13, but none per
+// activation fragment.
+struct ColDecodeNat {
+    h2_t neg;    // (-(1024 + z + 1), -(64 + z + 1))
+    h2_t scale;  // (s, s)
+};
+
+__device__ __forceinline__ ColDecodeNat make_col_decode_nat(uint32_t stored_zero, uint32_t scale_bits) {
+    ColDecodeNat c;
+    c.neg = as_h2((0xE401u + stored_zero) | ((0xD410u + (stored_zero << 4)) << 16));
+    c.scale = as_h2((scale_bits & 0xFFFFu) * 0x10001u);
+    return c;
+}
+
+// out = rows 0..7 of the word's 8-row block, in order.
+__device__ __forceinline__ h8_t decode_word_natural(uint32_t w, const ColDecodeNat &c) {
+    const h2_t unit = {(half_t)1.0f, (half_t)0.0625f};
+    const uint32_t magic = 0x64006400u;
+    h2_t p[4];
+    p[0] = as_h2(and_or_b32(__builtin_amdgcn_perm(w, w, 0x0c000c00u), 0x00F0000Fu, magic));
+    p[1] = as_h2(and_or_b32(__builtin_amdgcn_perm(w, w, 0x0c010c01u), 0x00F0000Fu, magic));
+    p[2] = as_h2(and_or_b32(__builtin_amdgcn_perm(w, w, 0x0c020c02u), 0x00F0000Fu, magic));
+    p[3] = as_h2(and_or_b32(__builtin_amdgcn_perm(w, w, 0x0c030c03u), 0x00F0000Fu, magic));
+#pragma unroll
+    for (int j = 0; j < 4; ++j) p[j] = __builtin_elementwise_fma(p[j], unit, c.neg) * c.scale;
+    h8_t r = {p[0].x, p[0].y, p[1].x, p[1].y, p[2].x, p[2].y, p[3].x, p[3].y};
+    return r;
+}
+
 // 8 consecutive activations a0..a7 (natural order, as a uint4) -> pair order
 // (a0,a4,a1,a5,a2,a6,a3,a7).
 __device__ __forceinline__ h8_t pair_order_a(uint4 v) {

@@ -7,22 +7,32 @@
 // step) straight from global memory, decodes them in registers and uses word t as the
 // B operand of column tile t, whose 32 columns are {2j + t}.
 //
-// The decode is VALU work (13 ops per word) that has to hide under the MFMAs, and each
-// decoded operand is reused only by the row tiles of its own wave.  The wave tile is
-// therefore tall and narrow: (32*MT) rows x 64 columns, MT = 4 by default - 8 MFMAs
-// per pair of decoded words, 128 accumulator registers, two waves per SIMD.  The
-// decode of K step s+1 is written between the MFMAs of step s; the packed words of a
-// step are refilled in place with the same step of the next K tile; every load in the
-// loop is unconditional (clamped indices) so the waits are exact vmcnt(N).
-// Only the activations go through LDS (stored in pair order, rows padded to 144 B,
-// double buffered, one barrier per K tile of 64).
+// The decode is VALU work that has to hide under the MFMAs, and each decoded operand is
+// reused only by the row tiles of its own wave.  The wave tile is therefore tall and
+// narrow: (32*MT) rows x 64 columns, MT = 4 by default - 8 MFMAs per pair of decoded
+// words, 128 accumulator registers, two waves per SIMD.  The decode of K step s+1 is
+// written between the MFMAs of step s.  Packed words and scale/zero words are loaded two
+// K tiles ahead into register slots that are refilled in place; every load in the loop is
+// unconditional (clamped indices), so the waits are exact vmcnt(N) and none of them
+// waits for a load younger than a whole K tile.
 //
-// Workgroup = 4 waves as 2 (M) x 2 (N): tile (64*MT) x 128.
-//   plain   : the two N waves take adjacent 64-column halves.
-//   rotary  : the 128 columns are one head; column d and its partner d + 64 sit in the
-//             two N waves at the same lane and register, and are swapped through LDS.
-//   SiLU*mul: the two N waves take the SAME 64 columns of the gate and of the up
-//             matrix (tile (64*MT) x 64 of the output); up is handed over through LDS.
+// Only the activations go through LDS, double buffered, one barrier per K tile of 64.
+// They are 4x the bytes of the 4-bit weights they meet, so the workgroup tile is wide:
+// one tile of 128 rows serves 4 waves side by side (256 columns).  They travel
+// global -> LDS directly (buffer_load ... lds: no staging registers, and - unlike the
+// flat form - counted in order by the compiler's wait insertion); rows are unpadded and
+// the 16-byte chunks of a row are XOR-swizzled for conflict-free fragment reads.  The
+// fragments come out in natural k order, so the weights are decoded in natural order too
+// (16 ops per word instead of 13, none per fragment).  With an act-order permutation the
+// activations are gathered through registers instead and stored in pair order.
+//
+// Workgroup = 4 waves.  MT = 4: 1 (M) x 4 (N), tile 128 x 256; MT = 2: 2 x 2, tile 128 x 128
+// (more tiles for mid-sized M).  N waves work in pairs:
+//   plain   : every N wave takes its own 64 columns.
+//   rotary  : a pair's 128 columns are one head; column d and its partner d + 64 sit in
+//             the two waves at the same lane and register, and are swapped through LDS.
+//   SiLU*mul: a pair takes the SAME 64 columns of the gate and of the up matrix (the
+//             output tile is half as wide); up is handed over through LDS.
 // blockIdx is remapped so each XCD (blockIdx % 8) owns a contiguous range of tiles:
 // the row tiles that share a weight panel then share one L2.
 #include "gptq4_internal.h"
@@ -34,29 +44,39 @@ constexpr int LDS_ROW = BK + 8;  // halves; 144-byte rows keep 128-bit reads con
 
 template <int EPI, int MT, bool PERM>
 __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
-    constexpr int BM = 64 * MT;
-    constexpr int BN = (EPI == EPI_SILU_MUL) ? 64 : 128;
-    constexpr int A_UNITS = BM * (BK / 8) / 256;  // 16-byte units each thread stages per K tile
+    constexpr int NW = 4;        // waves
+    constexpr int NT = 64 * NW;  // threads
+    constexpr int WM = (MT == 4) ? 1 : 2;  // waves along M
+    constexpr int WN = NW / WM;            // waves along N
+    constexpr int BM = 32 * MT * WM;
+    constexpr int BN = ((EPI == EPI_SILU_MUL) ? 32 : 64) * WN;
+    constexpr int A_UNITS = BM * (BK / 8) / NT;  // 16-byte units each thread stages per K tile
+    constexpr int A_ROWS = NT / 8;               // rows one pass of the workgroup stages (act-order path)
 
     // Activation tiles.  Plain path: two unpadded buffers of BM x 64 halves filled by
     // LDS-direct loads (two separate objects, so that the compiler can tell a load into one
     // from the reads of the other); act-order path: one padded double buffer filled through
     // registers.  The epilogues reuse them as four 8 KiB exchange regions.
+    constexpr int REGIONS = (EPI == EPI_ROPE) ? NW : NW / 2;  // 8 KiB each
+    constexpr int EX_HALVES = REGIONS * 32 * 64 * 2;          // all regions, in halves
     constexpr int A_HALVES = BM * BK;
-    __shared__ __attribute__((aligned(16))) half_t As0[PERM ? 2 * BM * LDS_ROW : A_HALVES];
-    __shared__ __attribute__((aligned(16))) half_t As1[PERM ? 8 : A_HALVES];
-    static_assert(PERM ? sizeof(As0) >= 4 * 32 * 64 * sizeof(float) : sizeof(As0) >= 2 * 32 * 64 * sizeof(float),
-                  "epilogue exchange regions do not fit");
+    constexpr int S0 = PERM ? (2 * BM * LDS_ROW > EX_HALVES ? 2 * BM * LDS_ROW : EX_HALVES)
+                            : (A_HALVES > EX_HALVES / 2 ? A_HALVES : EX_HALVES / 2);
+    constexpr int S1 = PERM ? 8 : S0;
+    __shared__ __attribute__((aligned(16))) half_t As0[S0];
+    __shared__ __attribute__((aligned(16))) half_t As1[S1];
     auto region = [&](int w) -> float * {
         if (PERM) return reinterpret_cast<float *>(As0) + w * (32 * 64);
-        return reinterpret_cast<float *>(w < 2 ? As0 : As1) + (w & 1) * (32 * 64);
+        constexpr int HALF = (REGIONS + 1) / 2;
+        return reinterpret_cast<float *>(w < HALF ? As0 : As1) + (w < HALF ? w : w - HALF) * (32 * 64);
     };
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave & 1;
-    const int wn = wave >> 1;
+    const int wm = (WM == 2) ? (wave & 1) : 0;
+    const int wn = (WM == 2) ? (wave >> 1) : wave;
+    const int wn_pair = wn >> 1, wn_odd = wn & 1;  // SiLU*mul and rotary work on pairs of N waves
     const int l32 = lane & 31;
     const int lhi = lane >> 5;
 
@@ -73,8 +93,8 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
     const int m0 = tile_m * BM;
     const int n0 = tile_n * BN;
 
-    const int mat = (EPI == EPI_SILU_MUL) ? wn : 0;
-    const int nw0 = n0 + ((EPI == EPI_SILU_MUL) ? 0 : wn * 64);  // first column of the wave
+    const int mat = (EPI == EPI_SILU_MUL) ? wn_odd : 0;
+    const int nw0 = n0 + ((EPI == EPI_SILU_MUL) ? wn_pair : wn) * 64;  // first column of the wave
     const int ncol = nw0 + 2 * l32;                               // lane's 2 columns
     const uint32_t *bptr = p.w[mat].qweight + (size_t)lhi * N + ncol;  // row lhi of K tile 0
     const uint32_t *qz = p.w[mat].qzeros + (ncol >> 3);
@@ -99,7 +119,7 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
     const int a_row = tid >> 3, a_ku = tid & 7;  // unit u of this thread: row a_row + 32*u, k-unit a_ku
 #pragma unroll
     for (int u = 0; u < A_UNITS; ++u) {
-        const int row = min(a_row + 32 * u, M - 1 - m0);
+        const int row = min(a_row + A_ROWS * u, M - 1 - m0);
         a_off[u] = (uint32_t)row * (uint32_t)K + 8u * a_ku;
     }
     half_t *const a_lds = As0 + a_row * LDS_ROW + 8 * a_ku;  // act-order path
@@ -131,7 +151,7 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
     auto store_a = [&](int buf) {
 #pragma unroll
         for (int u = 0; u < A_UNITS; ++u)
-            *reinterpret_cast<uint4 *>(a_lds + buf * (BM * LDS_ROW) + u * (32 * LDS_ROW)) = pair_order_u4(a_stage[u]);
+            *reinterpret_cast<uint4 *>(a_lds + buf * (BM * LDS_ROW) + u * (A_ROWS * LDS_ROW)) = pair_order_u4(a_stage[u]);
     };
     auto load_b_step = [&](int kt, int ks) {
         bw[ks] = *reinterpret_cast<const uint2 *>(bptr + ((size_t)kt * (BK / 8) + 2 * ks) * N);
@@ -218,7 +238,7 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
         uint32_t a_goff[A_UNITS];
 #pragma unroll
         for (int u = 0; u < A_UNITS; ++u) {
-            const int slot = (u * 4 + wave) * 64 + lane;
+            const int slot = (u * NW + wave) * 64 + lane;
             const int row = slot >> 3;
             const int c = (slot & 7) ^ ((row >> 1) & 7);
             a_goff[u] = (uint32_t)min(row, M - 1 - m0) * (uint32_t)K + 8u * c;
@@ -231,39 +251,72 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
         auto dma_a = [&](half_t *dst, int kt) {
 #pragma unroll
             for (int u = 0; u < A_UNITS; ++u)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (__attribute__((address_space(3))) void *)(dst + (u * 4 + wave) * 512),
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (__attribute__((address_space(3))) void *)(dst + (u * NW + wave) * 512),
                                                          16, (int)(a_goff[u] * 2u), kt * (BK * 2), 0, 0);
             asm volatile("" ::: "memory");  // the loads that follow stay behind these
         };
         const int sw = (l32 >> 1) & 7;  // (row >> 1) & 7 for every row this lane reads (rows = 32*j + l32)
 
+        // Packed words of two K tiles: slot [par][ks] holds step ks of a tile of parity par.  It
+        // is decoded during step ks - 1 and refilled during step ks - once its old contents
+        // are dead, so the load can land in place - with the same step two tiles on.
+        uint2 b2[2][4];
+        auto load_b2 = [&](int par, int kt, int ks) {
+            b2[par][ks] = *reinterpret_cast<const uint2 *>(bptr + ((size_t)min(kt, nk - 1) * (BK / 8) + 2 * ks) * N);
+        };
         dma_a(As0, k_begin);
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) load_b_step(k_begin, ks);
-        load_group(group);
-        make_cd();
+        for (int ks = 0; ks < 4; ++ks) load_b2(0, k_begin, ks);
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) load_b2(1, k_begin + 1, ks);
+        // Scale and zero words run two tiles ahead as well: slot [par] is loaded at the top of a
+        // tile of parity par with the group of the tile two on, and turned into the decode
+        // constants of that tile during the last step of the tile in between.  The group of
+        // the look-ahead tile is tracked by counting, like the current one.
+        uint32_t g_s[2], g_z[2];
+        int group2 = group, left2 = left_in_group;
+        auto load_group2 = [&](int par) {
+            const int g = min(group2, last_group);
+            g_s[par] = *reinterpret_cast<const uint32_t *>(sc + (size_t)g * N);
+            g_z[par] = qz[(size_t)g * (N >> 3)];
+            if (left2 == 1) {
+                ++group2;
+                left2 = tiles_per_group;
+            } else {
+                --left2;
+            }
+        };
+        // the activation fragments come out of LDS in natural k order, so the weights are
+        // decoded in natural order too
+        ColDecodeNat cn[2];
+        auto make_cn = [&](int par) {
+            const uint32_t z2 = g_z[par] >> (((2 * l32) & 7) * 4);
+            cn[0] = make_col_decode_nat(z2 & 0xFu, g_s[par]);
+            cn[1] = make_col_decode_nat((z2 >> 4) & 0xFu, g_s[par] >> 16);
+        };
+        load_group2(0);  // group of tile k_begin
+        make_cn(0);
+        load_group2(1);  // group of tile k_begin + 1, made into constants at the end of tile k_begin
         h8_t bf[2];
-        bf[0] = decode_word_h8(bw[0].x, cd[0]);
-        bf[1] = decode_word_h8(bw[0].y, cd[1]);
-        load_b_step(min(k_begin + 1, nk - 1), 0);
+        bf[0] = decode_word_natural(b2[0][0].x, cn[0]);
+        bf[1] = decode_word_natural(b2[0][0].y, cn[1]);
 
-        // one K tile from buffer `cur`, while the next tile streams into `nxt`
-        auto k_tile = [&](const half_t *cur, half_t *nxt, int kt) {
+        // one K tile (of parity `par` counted from k_begin) from buffer `cur`, while the next
+        // tile streams into `nxt`
+        auto k_tile = [&](const half_t *cur, half_t *nxt, int kt, int par) {
             // Every wave has issued at least 4 vector-memory loads after its LDS-direct loads
             // of this tile (the scale/zero words and the packed words of 4 K steps), and
             // loads complete in order: at most 4 outstanding means the tile has landed.
             asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-            const int kn = min(kt + 1, nk - 1), kn2 = min(kt + 2, nk - 1);
-            const bool new_group = (left_in_group == 1);
-            dma_a(nxt, kn);
-            load_group(min(group + (new_group ? 1 : 0), last_group));
+            dma_a(nxt, min(kt + 1, nk - 1));
+            load_group2(par);
             // fragments of K step ks+1 are read from LDS before the MFMAs of step ks are issued
-            uint4 araw[MT];
+            h8_t araw[MT];
             auto read_a = [&](int ks) {
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) {
                     const int row = wm * (32 * MT) + mt * 32 + l32;
-                    araw[mt] = *reinterpret_cast<const uint4 *>(cur + row * BK + 8 * ((2 * ks + lhi) ^ sw));
+                    araw[mt] = *reinterpret_cast<const h8_t *>(cur + row * BK + 8 * ((2 * ks + lhi) ^ sw));
                 }
             };
             read_a(0);
@@ -271,37 +324,31 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
             for (int ks = 0; ks < 4; ++ks) {
                 h8_t af[MT];
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) af[mt] = pair_order_a(araw[mt]);
+                for (int mt = 0; mt < MT; ++mt) {
+                    af[mt] = araw[mt];
+                }
                 if (ks < 3) read_a(ks + 1);
-                if (ks == 3) make_cd();
-                const uint2 nw = bw[(ks + 1) & 3];
-                if (ks < 3)
-                    load_b_step(kn, ks + 1);
-                else
-                    load_b_step(kn2, 0);
+                if (ks == 3) make_cn(par ^ 1);
+                load_b2(par, kt + 2, ks);  // this step's words were decoded during the previous step
                 __builtin_amdgcn_sched_barrier(0);  // keep the loads above the MFMAs that hide them
+                // words of the next step (step 0 of the next tile when ks == 3)
+                const uint2 nw = (ks < 3) ? b2[par][ks + 1] : b2[par ^ 1][0];
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt], bf[0], acc[mt][0], 0, 0, 0);
-                bf[0] = decode_word_h8(nw.x, cd[0]);
+                bf[0] = decode_word_natural(nw.x, cn[0]);
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt], bf[1], acc[mt][1], 0, 0, 0);
-                bf[1] = decode_word_h8(nw.y, cd[1]);
-            }
-            if (new_group) {
-                ++group;
-                left_in_group = tiles_per_group;
-            } else {
-                --left_in_group;
+                bf[1] = decode_word_natural(nw.y, cn[1]);
             }
         };
         // pairs of tiles without a branch between them (a join there would make the compiler
         // move packed words that are still in flight, and wait for them), then the odd one
         int kt = k_begin;
         for (; kt + 1 < nk; kt += 2) {
-            k_tile(As0, As1, kt);
-            k_tile(As1, As0, kt + 1);
+            k_tile(As0, As1, kt, 0);
+            k_tile(As1, As0, kt + 1, 1);
         }
-        if (kt < nk) k_tile(As0, As1, kt);
+        if (kt < nk) k_tile(As0, As1, kt, 0);
         // all LDS-direct loads have landed and every wave is done reading before the
         // epilogues reuse the buffers
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -314,14 +361,14 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
         __shared__ int s_is_last;
         constexpr int NREG = MT * 32;
         const int tile = logical;
-        float *const mine = p.partials + ((size_t)tile * p.splitk + split) * (NREG * 256) + tid;
+        float *const mine = p.partials + ((size_t)tile * p.splitk + split) * (NREG * NT) + tid;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int i = 0; i < 16; ++i)
-                    __hip_atomic_store(mine + ((mt * 2 + t) * 16 + i) * 256, acc[mt][t][i], __ATOMIC_RELAXED,
+                    __hip_atomic_store(mine + ((mt * 2 + t) * 16 + i) * NT, acc[mt][t][i], __ATOMIC_RELAXED,
                                        __HIP_MEMORY_SCOPE_AGENT);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
@@ -331,7 +378,7 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
         }
         __syncthreads();
         if (!s_is_last) return;
-        const float *const all = p.partials + (size_t)tile * p.splitk * (NREG * 256) + tid;
+        const float *const all = p.partials + (size_t)tile * p.splitk * (NREG * NT) + tid;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -348,7 +395,7 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
                     float got[16];
 #pragma unroll
                     for (int i = 0; i < 16; ++i)
-                        got[i] = __hip_atomic_load(all + ((size_t)sp * NREG + (mt * 2 + t) * 16 + i) * 256,
+                        got[i] = __hip_atomic_load(all + ((size_t)sp * NREG + (mt * 2 + t) * 16 + i) * NT,
                                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
                     for (int i = 0; i < 16; ++i) acc[mt][t][i] += got[i];
@@ -377,18 +424,18 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
             }
     } else if (EPI == EPI_SILU_MUL) {
         // hand the up accumulators (wn == 1) to the gate wave (wn == 0) with the same wm
-        float *const mine = region(wm);
+        float *const mine = region(WM == 2 ? wm : wn_pair);
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             __syncthreads();
-            if (wn == 1) {
+            if (wn_odd == 1) {
 #pragma unroll
                 for (int t = 0; t < 2; ++t)
 #pragma unroll
                     for (int i = 0; i < 16; ++i) mine[(t * 16 + i) * 64 + lane] = acc[mt][t][i];
             }
             __syncthreads();
-            if (wn == 0) {
+            if (wn_odd == 0) {
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const int row = wrow0 + mt * 32 + 8 * (i >> 2) + 4 * lhi + (i & 3);
@@ -406,11 +453,11 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
         // [64*wn, 64*wn + 64), the partner d +- 64 is the same lane and register of the
         // other N wave
         const RopeArgs &r = p.rope;
-        const int head_col = n0 >> 7;
+        const int head_col = (n0 >> 7) + wn_pair;
         const int which = head_col / r.H;
         const int head = head_col - which * r.H;
         float *const mine = region(wave);
-        const float *const theirs = region(wave ^ 2);
+        const float *const theirs = region(WM == 2 ? (wave ^ 2) : (wave ^ 1));
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             if (which < 2) {
@@ -444,7 +491,7 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
                 float o0 = acc[mt][0][i], o1 = acc[mt][1][i];
                 if (which < 2) {
                     const float p0 = theirs[(0 * 16 + i) * 64 + lane], p1 = theirs[(1 * 16 + i) * 64 + lane];
-                    if (wn == 0) {
+                    if (wn_odd == 0) {
                         o0 = o0 * cs[i].x - p0 * sn[i].x;
                         o1 = o1 * cs[i].y - p1 * sn[i].y;
                     } else {
@@ -467,7 +514,7 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
                         off = ((size_t)(bb * r.H + head) * r.kv_capacity + crow) * 128;
                     }
                     const h2_t o = {(half_t)o0, (half_t)o1};
-                    *reinterpret_cast<uint32_t *>(dst + off + 64 * wn + 2 * l32) = as_u32(o);
+                    *reinterpret_cast<uint32_t *>(dst + off + 64 * wn_odd + 2 * l32) = as_u32(o);
                 }
             }
         }
@@ -493,20 +540,31 @@ int launch_epi(const MatmulArgs &a, const GemmPlan &pl, hipStream_t stream) {
 
 GemmTuning g_gemm_tuning = {0, 0};
 
-// Tile height and split-K factor of the tiled kernel.  256-row tiles (MT = 4) once there
-// are enough of them to fill the chip twice over, otherwise 128-row tiles; K is split
-// only when even those leave most CUs idle (the M = 17..255 range on narrow layers).
+// Tile shape and split-K factor of the tiled kernel.  The wide tile (128 x 256, half as
+// wide for SiLU*mul) is the faster one as soon as there are enough of them to give three
+// CUs out of four a workgroup; from half the CUs on it still wins with K split in two.
+// Below that, 128 x 128 tiles, with K split when even those leave most CUs idle (the
+// M = 17..255 range on narrow layers).
 GemmPlan gemm_plan(int epi, int M, int N, int K) {
     GemmPlan pl;
-    const int bn = (epi == EPI_SILU_MUL) ? 64 : 128;
-    const long tiles4 = (long)((M + 255) / 256) * (N / bn);
-    pl.mt = g_gemm_tuning.mt ? g_gemm_tuning.mt : ((M > 128 && tiles4 >= 512) ? 4 : 2);
-    pl.tiles = ((M + 64 * pl.mt - 1) / (64 * pl.mt)) * (N / bn);
+    const int bn2 = (epi == EPI_SILU_MUL) ? 64 : 128;  // tile width at MT = 2; twice that at MT = 4
     const int nk = K / 64;
+    const long wide = (long)((M + 127) / 128) * (N / (2 * bn2));
     int s = 1;
+    if (g_gemm_tuning.mt) {
+        pl.mt = g_gemm_tuning.mt;
+    } else if (wide >= 192) {
+        pl.mt = 4;
+    } else if (wide >= 128 && nk >= 32) {
+        pl.mt = 4;
+        s = 2;
+    } else {
+        pl.mt = 2;
+    }
+    pl.tiles = ((M + 127) / 128) * (N / (pl.mt == 4 ? 2 * bn2 : bn2));
     if (g_gemm_tuning.splitk > 0) {
         s = g_gemm_tuning.splitk;
-    } else if (pl.tiles < 384) {
+    } else if (pl.mt == 2 && pl.tiles < 384) {
         s = (512 + pl.tiles / 2) / pl.tiles;  // aim for ~2 workgroups per CU
         if (s > nk / 8) s = nk / 8;            // keep at least 8 K tiles (512 k) per split
     }

@@ -77,7 +77,7 @@ size_t gemv_partial_bytes(const GemvPlan &plan, int M, int epi);
 int launch_gemv(int epi, MatmulArgs &a, const GemvPlan &plan, hipStream_t stream);
 // Launch shape of the tiled kernel.
 struct GemmPlan {
-    int mt;      // row tiles per wave: workgroup tile = (64 * mt) rows
+    int mt;      // 32-row tiles per wave: 2 = 128 x 128 workgroup tile (2 x 2 waves), 4 = 128 x 256 (1 x 4 waves)
     int splitk;  // workgroups sharing one tile along K
     int tiles;
 };

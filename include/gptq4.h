@@ -156,8 +156,8 @@ int gptq4_decode_attention(const void *q, const void *k_cache, const void *v_cac
  * tunes through Triton's autotuner, custom_autotune.py:12-172). */
 void gptq4_set_tuning(int words, int depth, int splitk);
 
-/* Same for the tiled (M > 16) kernel: rows per workgroup tile = 64 * mt (mt = 2 or 4) and
- * the split-K factor; 0 = automatic. */
+/* Same for the tiled (M > 16) kernel: workgroup tile (mt = 2: 128 x 128, mt = 4: 128 x 256
+ * outputs; half as wide for the fused gate/up) and the split-K factor; 0 = automatic. */
 void gptq4_set_gemm_tuning(int mt, int splitk);
 
 /* Same for the balanced decode GEMV (M <= 4): mode 0 = never use it, 1 = where it is the
