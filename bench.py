@@ -372,6 +372,29 @@ def main():
                    2 * m * HIDDEN * INTER, nsets=ns, reps=5)
             per_op(f"M={m} o_proj (4096x4096)", lambda L: o_op(xm, L), wo + 4 * m * HIDDEN, 2 * m * HIDDEN * HIDDEN,
                    nsets=ns, reps=5)
+        # Yardstick: the vendor library's DENSE fp16 GEMM (torch.matmul) on the same M = 2048
+        # shapes, weights already dequantised.  It does no 4-bit decode and reads 4x the
+        # weight bytes; it shows what fraction of the nominal MFMA peak a tuned kernel
+        # sustains on this chip at these shapes.
+        def dense(name, k, n, m=2048, reps=20):
+            a = torch.randn((m, k), device=dev, generator=gen).half()
+            ws = [(torch.randn((k, n), device=dev, generator=gen) * 0.02).half() for _ in range(2)]
+            for w in ws:
+                torch.matmul(a, w)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for i in range(reps):
+                torch.matmul(a, ws[i & 1])
+            e1.record()
+            torch.cuda.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / reps
+            extra[name] = {"us": round(us, 2), "TFLOPs": round(2.0 * m * k * n / us / 1e6, 2)}
+            log(f"  {name:34s} {us:9.2f} us  {'':8s}       {2.0 * m * k * n / us / 1e6:8.1f} TFLOP/s")
+        dense("dense fp16 library M=2048 qkv shape", HIDDEN, 3 * HIDDEN)
+        dense("dense fp16 library M=2048 gate+up shape", HIDDEN, 2 * INTER)
+        dense("dense fp16 library M=2048 down shape", INTER, HIDDEN)
+        dense("dense fp16 library M=2048 o_proj shape", HIDDEN, HIDDEN)
         best_prefill = max(v["TFLOPs"] for k, v in extra.items() if k.startswith("M=2048"))
         extra["prefill_best_TFLOPs"] = best_prefill
         extra["prefill_frac_of_fp16_mfma_peak"] = round(best_prefill / MFMA_FP16_PEAK_TFLOPS, 4)

@@ -131,7 +131,9 @@ __device__ __forceinline__ uint4 pair_order_u4(uint4 v) {
     return r;
 }
 
-__device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + __expf(-x)); }
+// x * sigmoid(x) with the hardware reciprocal (1 ulp) instead of an IEEE division: the result
+// is rounded to fp16 right after.
+__device__ __forceinline__ float silu_f32(float x) { return x * __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
 
 // Epilogue selectors shared by the small-M and the tiled kernels.
 enum { EPI_PLAIN = 0, EPI_SILU_MUL = 1, EPI_ROPE = 2 };

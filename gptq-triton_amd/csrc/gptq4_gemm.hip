@@ -57,7 +57,7 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
     // LDS-direct loads (two separate objects, so that the compiler can tell a load into one
     // from the reads of the other); act-order path: one padded double buffer filled through
     // registers.  The epilogues reuse them as four 8 KiB exchange regions.
-    constexpr int REGIONS = (EPI == EPI_ROPE) ? NW : NW / 2;  // 8 KiB each
+    constexpr int REGIONS = NW;                        // 8 KiB each
     constexpr int EX_HALVES = REGIONS * 32 * 64 * 2;          // all regions, in halves
     constexpr int A_HALVES = BM * BK;
     constexpr int S0 = PERM ? (2 * BM * LDS_ROW > EX_HALVES ? 2 * BM * LDS_ROW : EX_HALVES)
@@ -423,28 +423,39 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
                 }
             }
     } else if (EPI == EPI_SILU_MUL) {
-        // hand the up accumulators (wn == 1) to the gate wave (wn == 0) with the same wm
-        float *const mine = region(WM == 2 ? wm : wn_pair);
+        // The gate wave (even) and the up wave (odd) of a pair hold the same output tile.
+        // They split it by row blocks: in round r the up wave hands over block r and the
+        // gate wave block MT/2 + r, then each finishes the block it received a half of.
+        const int pair = (WM == 2) ? wm : wn_pair;
+        float *const to_gate = region(2 * pair), *const to_up = region(2 * pair + 1);
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
+        for (int r = 0; r < MT / 2; ++r) {
+            const int mt = wn_odd ? MT / 2 + r : r;  // the block this wave finishes
             __syncthreads();
-            if (wn_odd == 1) {
 #pragma unroll
-                for (int t = 0; t < 2; ++t)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) mine[(t * 16 + i) * 64 + lane] = acc[mt][t][i];
-            }
-            __syncthreads();
-            if (wn_odd == 0) {
+            for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
-                    const int row = wrow0 + mt * 32 + 8 * (i >> 2) + 4 * lhi + (i & 3);
-                    const float o0 = silu_f32(acc[mt][0][i]) * mine[(0 * 16 + i) * 64 + lane];
-                    const float o1 = silu_f32(acc[mt][1][i]) * mine[(1 * 16 + i) * 64 + lane];
-                    if (row < M) {
-                        const h2_t o = {(half_t)o0, (half_t)o1};
-                        *reinterpret_cast<uint32_t *>(p.y + (size_t)row * N + ncol) = as_u32(o);
-                    }
+                    if (wn_odd)
+                        to_gate[(t * 16 + i) * 64 + lane] = acc[r][t][i];
+                    else
+                        to_up[(t * 16 + i) * 64 + lane] = acc[MT / 2 + r][t][i];
+                }
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int row = wrow0 + mt * 32 + 8 * (i >> 2) + 4 * lhi + (i & 3);
+                float o0, o1;
+                if (wn_odd) {
+                    o0 = silu_f32(to_up[(0 * 16 + i) * 64 + lane]) * acc[MT / 2 + r][0][i];
+                    o1 = silu_f32(to_up[(1 * 16 + i) * 64 + lane]) * acc[MT / 2 + r][1][i];
+                } else {
+                    o0 = silu_f32(acc[r][0][i]) * to_gate[(0 * 16 + i) * 64 + lane];
+                    o1 = silu_f32(acc[r][1][i]) * to_gate[(1 * 16 + i) * 64 + lane];
+                }
+                if (row < M) {
+                    const h2_t o = {(half_t)o0, (half_t)o1};
+                    *reinterpret_cast<uint32_t *>(p.y + (size_t)row * N + ncol) = as_u32(o);
                 }
             }
         }
