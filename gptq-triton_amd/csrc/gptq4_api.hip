@@ -272,6 +272,13 @@ int gptq4_qkv_rotary(const void *x, const int32_t *qweight, const int32_t *qzero
     a.rope.kv_capacity = kv_capacity;
     a.rope.kv_offset = kv_offset;
     a.rope.max_pos = max_pos;
+    a.rope.s_magic = 0;
+    if (S > 1) {
+        // round-up reciprocal: exact for every row < M when (M - 1) * (magic * S - 2^32) < 2^32
+        const uint64_t magic = (1ull << 32) / (uint64_t)S + 1;
+        const uint64_t err = magic * (uint64_t)S - (1ull << 32);
+        if (magic < (1ull << 32) && (uint64_t)(a.M - 1) * err < (1ull << 32)) a.rope.s_magic = (uint32_t)magic;
+    }
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     if (a.M <= SKINNY_MAX_M) {
         return run_small(EPI_ROPE, a, 1, workspace, workspace_bytes, s);

@@ -150,4 +150,16 @@ struct RopeArgs {
     int kv_capacity;
     int kv_offset;
     int max_pos;  // rows of the tables; positions are clamped into [0, max_pos)
+    uint32_t s_magic;  // floor(2^32 / S) + 1 when umulhi(row, s_magic) == row / S for every row < M, else 0
 };
+
+// row -> (sequence, token within it)
+__device__ __forceinline__ void split_row(const RopeArgs &r, int row, int &b, int &s) {
+    if (r.S == 1) {
+        b = row;
+        s = 0;
+        return;
+    }
+    b = r.s_magic ? (int)__umulhi((unsigned)row, r.s_magic) : row / r.S;
+    s = row - b * r.S;
+}

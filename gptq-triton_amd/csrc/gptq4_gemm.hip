@@ -469,6 +469,12 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
         const int head = head_col - which * r.H;
         float *const mine = region(wave);
         const float *const theirs = region(WM == 2 ? (wave ^ 2) : (wave ^ 1));
+        // destination of this wave's head: q [B,H,S,128], k and v [B,H,kv_capacity,128]
+        const int cap = (which == 0) ? r.S : r.kv_capacity;
+        half_t *const dst = ((which == 0) ? r.q : (which == 1) ? r.k : r.v) + (size_t)head * cap * 128 + 64 * wn_odd + 2 * l32;
+        const size_t seq_stride = (size_t)r.H * cap * 128;
+        const bool at_position = (which != 0) && r.kv_offset < 0;  // cache row = the token's position
+        const int row_shift = (which == 0 || r.kv_offset < 0) ? 0 : r.kv_offset;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             if (which < 2) {
@@ -483,17 +489,20 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
             // unconditional (rows beyond M read row M-1) and issued together, so their
             // latencies overlap instead of forming 16 dependent chains
             float2 cs[16], sn[16];
-            if (which < 2) {
-                int pos[16];
+            int pos[16];
+            if (which < 2 || at_position) {
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const int row = min(wrow0 + mt * 32 + 8 * (i >> 2) + 4 * lhi + (i & 3), M - 1);
-                    pos[i] = min(max(r.position_ids[row], 0), r.max_pos - 1);
+                    pos[i] = max(r.position_ids[row], 0);
                 }
+            }
+            if (which < 2) {
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
-                    cs[i] = *reinterpret_cast<const float2 *>(r.cos_table + (size_t)pos[i] * 64 + 2 * l32);
-                    sn[i] = *reinterpret_cast<const float2 *>(r.sin_table + (size_t)pos[i] * 64 + 2 * l32);
+                    const int tp = min(pos[i], r.max_pos - 1);
+                    cs[i] = *reinterpret_cast<const float2 *>(r.cos_table + (size_t)tp * 64 + 2 * l32);
+                    sn[i] = *reinterpret_cast<const float2 *>(r.sin_table + (size_t)tp * 64 + 2 * l32);
                 }
             }
 #pragma unroll
@@ -511,21 +520,11 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
                     }
                 }
                 if (row < M) {
-                    const int bb = row / r.S;
-                    const int srow = row - bb * r.S;
-                    half_t *dst;
-                    size_t off;
-                    if (which == 0) {
-                        dst = r.q;
-                        off = ((size_t)(bb * r.H + head) * r.S + srow) * 128;
-                    } else {
-                        dst = (which == 1) ? r.k : r.v;
-                        // kv_offset < 0: the cache row is the token's position
-                        const int crow = r.kv_offset >= 0 ? r.kv_offset + srow : min(max(r.position_ids[row], 0), r.kv_capacity - 1);
-                        off = ((size_t)(bb * r.H + head) * r.kv_capacity + crow) * 128;
-                    }
+                    int bb, srow;
+                    split_row(r, row, bb, srow);
+                    const int crow = at_position ? min(pos[i], r.kv_capacity - 1) : srow + row_shift;
                     const h2_t o = {(half_t)o0, (half_t)o1};
-                    *reinterpret_cast<uint32_t *>(dst + off + 64 * wn_odd + 2 * l32) = as_u32(o);
+                    *reinterpret_cast<uint32_t *>(dst + (size_t)bb * seq_stride + (size_t)crow * 128) = as_u32(o);
                 }
             }
         }

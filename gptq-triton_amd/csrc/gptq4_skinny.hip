@@ -350,8 +350,8 @@ __global__ __launch_bounds__(64 * NW) void gptq4_skinny_kernel(MatmulArgs p) {
             const int d = (n0 & 127) + c;
             const int which = head_col / r.H;
             const int head = head_col - which * r.H;
-            const int bb = row / r.S;
-            const int ss = row - bb * r.S;
+            int bb, ss;
+            split_row(r, row, bb, ss);
             float o1 = val[q][0], o2 = val[q][NV - 1];
             if (which < 2) {
                 const int pos = min(max(r.position_ids[row], 0), r.max_pos - 1);
