@@ -241,7 +241,9 @@ def test_rope_table_matches_closed_form():
 
 
 @pytest.mark.parametrize("b,s,pos0,g", [(1, 1, 2047, -1), (2, 5, 10, 128), (1, 300, 0, -1), (3, 1, 77, 128),
-                                        (1, 16, 1000, -1), (1, 17, 0, 128)])
+                                        (1, 16, 1000, -1), (1, 17, 0, 128),
+                                        # tiled kernel: one token from each of 40 sequences; ragged S over several sequences
+                                        (40, 1, 500, 128), (3, 43, 7, 128), (5, 130, 0, -1)])
 def test_qkv_rotary(b, s, pos0, g):
     H, Dh, hidden = 8, 128, 1024
     L = O.make_layer(hidden, 3 * hidden, g, seed=200 + s)
@@ -281,6 +283,34 @@ def test_qkv_rotary_writes_into_kv_cache():
         untouched = torch.ones(cap, dtype=torch.bool)
         untouched[off:off + s] = False
         assert bool((kc[:, :, untouched] == 7.0).all()) and bool((vc[:, :, untouched] == 7.0).all())
+
+
+def test_qkv_rotary_places_rows_by_position_in_the_tiled_kernel():
+    """kv_offset = KV_AT_POSITION with more than 16 rows: every token lands in the cache row of
+    its own position id, whatever its place in the batch."""
+    from gptq_triton_amd.fused_attention import KV_AT_POSITION
+    H, Dh, hidden, g = 8, 128, 1024, 128
+    L = O.make_layer(hidden, 3 * hidden, g, seed=320)
+    D = to_dev(L)
+    G = gptq()
+    cos, sin = G.RotaryTable(Dh, 2048).get(torch.device("cuda"), 2048)
+    b, s, cap = 3, 11, 64
+    rng = np.random.default_rng(321)
+    pos = np.stack([rng.permutation(cap)[:s] for _ in range(b)]).astype(np.int64)   # distinct rows per sequence
+    x = O.make_x(b * s, hidden, seed=322).reshape(b, s, hidden)
+    kc = torch.full((b, H, cap, Dh), 7.0, dtype=torch.float16, device="cuda")
+    vc = torch.full((b, H, cap, Dh), 7.0, dtype=torch.float16, device="cuda")
+    xd, pd = torch.from_numpy(x).cuda(), torch.from_numpy(pos).cuda()
+    q, _, _ = G.qkv_rotary(g, xd, D["qweight"], D["scales"], D["qzeros"], pd, cos, sin, H, Dh,
+                           kv_out=(kc, vc), kv_offset=KV_AT_POSITION)
+    q0, k0, v0 = G.qkv_rotary(g, xd, D["qweight"], D["scales"], D["qzeros"], pd, cos, sin, H, Dh)
+    assert torch.equal(q, q0)
+    for bi in range(b):
+        rows = torch.from_numpy(pos[bi]).cuda()
+        assert torch.equal(kc[bi][:, rows], k0[bi]) and torch.equal(vc[bi][:, rows], v0[bi])
+        untouched = torch.ones(cap, dtype=torch.bool)
+        untouched[pos[bi]] = False
+        assert bool((kc[bi][:, untouched] == 7.0).all()) and bool((vc[bi][:, untouched] == 7.0).all())
 
 
 def test_fused_qkv_equals_three_projections():
