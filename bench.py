@@ -359,7 +359,7 @@ def main():
         per_op("decode M=1 o_proj", lambda L: o_op(x1, L), wo + 4 * HIDDEN, 2 * HIDDEN * HIDDEN)
         per_op("decode M=1 gate/up+silu*mul", lambda L: gateup_op(x1, L), gu_bytes, 4 * HIDDEN * INTER)
         per_op("decode M=1 down_proj", lambda L: down_op(h1, L), wd + 2 * INTER + 2 * HIDDEN, 2 * HIDDEN * INTER)
-        for m in (16, 128, 512, 2048):
+        for m in (16, 64, 128, 256, 512, 2048):
             xm = torch.randn((1, m, HIDDEN), device=dev, generator=gen).half()
             hm = torch.randn((m, INTER), device=dev, generator=gen).half()
             posm = torch.arange(m, device=dev, dtype=torch.int32).unsqueeze(0)

@@ -76,6 +76,37 @@ int setup_gemm(MatmulArgs &a, const GemmPlan &pl, void *workspace, size_t worksp
     return 0;
 }
 
+// M > 16: the mid-M kernel where it is the faster one, else the tiled kernel.
+bool prefer_kslice(const KslicePlan &kp, int epi, int M, int N) {
+    if (!kp.ok || g_kslice_tuning.mode == 0) return false;
+    if (g_kslice_tuning.mode == 2) return true;
+    // up to 768 rows, while the tiled kernel's wide tiles would leave a quarter of the CUs idle
+    const int wide_bn = (epi == EPI_SILU_MUL) ? 128 : 256;
+    return M <= 768 && (long)((M + 127) / 128) * (N / wide_bn) < 192;
+}
+
+int run_tiled(int epi, MatmulArgs &a, void *workspace, size_t workspace_bytes, hipStream_t s) {
+    const KslicePlan kp = kslice_plan(epi, a.M, a.N, a.K, a.perm != nullptr);
+    if (prefer_kslice(kp, epi, a.M, a.N)) {
+        a.tiles = kp.tiles;
+        a.splitk = kp.splitk;
+        const int nk = a.K / 64;
+        a.slot_q = nk / kp.splitk;
+        a.slot_rem = nk % kp.splitk;
+        if (kp.splitk > 1) {
+            if (workspace == nullptr || workspace_bytes < GPTQ4_WS_COUNTER_BYTES + kslice_partial_bytes(epi, kp))
+                return -GPTQ4_E_WORKSPACE;
+            a.counters = reinterpret_cast<int *>(workspace);
+            a.partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_COUNTER_BYTES);
+        }
+        return launch_kslice(epi, a, kp, s);
+    }
+    const GemmPlan pl = gemm_plan(epi, a.M, a.N, a.K);
+    const int rc = setup_gemm(a, pl, workspace, workspace_bytes);
+    if (rc) return rc;
+    return launch_gemm(epi, a, pl, s);
+}
+
 }  // namespace
 
 extern "C" {
@@ -104,6 +135,12 @@ const char *gptq4_strerror(int code) {
 void gptq4_set_gemm_tuning(int mt, int splitk) {
     g_gemm_tuning.mt = (mt == 2 || mt == 4) ? mt : 0;
     g_gemm_tuning.splitk = splitk > 0 ? splitk : 0;
+}
+
+void gptq4_set_midm_tuning(int mode, int mt, int splitk) {
+    g_kslice_tuning.mode = (mode >= 0 && mode <= 2) ? mode : 1;
+    g_kslice_tuning.mt = (mt == 1 || mt == 2 || mt == 4) ? mt : 0;
+    g_kslice_tuning.splitk = splitk > 0 ? splitk : 0;
 }
 
 void gptq4_set_gemv_tuning(int mode, int depth, int waves, int waves_per_cu) {
@@ -136,7 +173,11 @@ size_t gptq4_workspace_bytes(int op, int M, int K, int N) {
         bytes += need;
     } else if ((K % 64) == 0) {
         const int epi = (op == GPTQ4_OP_MLP_GATEUP) ? EPI_SILU_MUL : (op == GPTQ4_OP_QKV_ROTARY ? EPI_ROPE : EPI_PLAIN);
-        bytes += gemm_partial_bytes(gemm_plan(epi, M, N, K));  // for the current (automatic or forced) plan
+        // whichever kernel the current (automatic or forced) plans pick, with or without act-order
+        size_t need = gemm_partial_bytes(gemm_plan(epi, M, N, K));
+        const KslicePlan kp = kslice_plan(epi, M, N, K, false);
+        if (kp.ok && kslice_partial_bytes(epi, kp) > need) need = kslice_partial_bytes(epi, kp);
+        bytes += need;
     }
     return bytes;
 }
@@ -185,12 +226,7 @@ int gptq4_matmul(const void *x, const int32_t *qweight, const int32_t *qzeros, c
     if (M <= SKINNY_MAX_M) {
         return run_small(EPI_PLAIN, a, 1, workspace, workspace_bytes, s);
     }
-    {
-        const GemmPlan pl = gemm_plan(EPI_PLAIN, M, N, K);
-        rc = setup_gemm(a, pl, workspace, workspace_bytes);
-        if (rc) return rc;
-        return launch_gemm(EPI_PLAIN, a, pl, s);
-    }
+    return run_tiled(EPI_PLAIN, a, workspace, workspace_bytes, s);
 }
 
 int gptq4_mlp_gateup(const void *x, const int32_t *gate_qweight, const int32_t *gate_qzeros,
@@ -221,12 +257,7 @@ int gptq4_mlp_gateup(const void *x, const int32_t *gate_qweight, const int32_t *
     if (M <= SKINNY_MAX_M) {
         return run_small(EPI_SILU_MUL, a, 2, workspace, workspace_bytes, s);
     }
-    {
-        const GemmPlan pl = gemm_plan(EPI_SILU_MUL, M, I, K);
-        rc = setup_gemm(a, pl, workspace, workspace_bytes);
-        if (rc) return rc;
-        return launch_gemm(EPI_SILU_MUL, a, pl, s);
-    }
+    return run_tiled(EPI_SILU_MUL, a, workspace, workspace_bytes, s);
 }
 
 int gptq4_rope_table(float *cos_out, float *sin_out, int max_pos, int D, float base, void *stream) {
@@ -283,12 +314,7 @@ int gptq4_qkv_rotary(const void *x, const int32_t *qweight, const int32_t *qzero
     if (a.M <= SKINNY_MAX_M) {
         return run_small(EPI_ROPE, a, 1, workspace, workspace_bytes, s);
     }
-    {
-        const GemmPlan pl = gemm_plan(EPI_ROPE, a.M, N, K);
-        rc = setup_gemm(a, pl, workspace, workspace_bytes);
-        if (rc) return rc;
-        return launch_gemm(EPI_ROPE, a, pl, s);
-    }
+    return run_tiled(EPI_ROPE, a, workspace, workspace_bytes, s);
 }
 
 int gptq4_rmsnorm(const void *x, const void *weight, void *y, int M, int H, float eps, void *stream) {

@@ -90,6 +90,22 @@ size_t gemm_partial_bytes(const GemmPlan &plan);
 // Tiled matrix-core GEMM for any M.  Returns hipError_t.
 int launch_gemm(int epi, const MatmulArgs &a, const GemmPlan &plan, hipStream_t stream);
 
+// Launch shape of the mid-M kernel (K split across the waves of a workgroup).
+struct KslicePlan {
+    int mt;      // 32-row blocks per row tile (1, 2 or 4)
+    int splitk;  // workgroups sharing one tile along K, on top of the split inside the workgroup
+    int tiles;
+    bool ok;     // false: the shape needs another kernel
+};
+struct KsliceTuning {
+    int mode;        // 0 never, 1 where it is the faster kernel, 2 wherever it can run
+    int mt, splitk;  // 0 = automatic
+};
+extern KsliceTuning g_kslice_tuning;
+KslicePlan kslice_plan(int epi, int M, int N, int K, bool has_perm);
+size_t kslice_partial_bytes(int epi, const KslicePlan &plan);
+int launch_kslice(int epi, const MatmulArgs &a, const KslicePlan &plan, hipStream_t stream);
+
 int launch_dequant(const uint32_t *qweight, const uint32_t *qzeros, const half_t *scales,
                    const int32_t *g_idx, half_t *out, int K, int N, int groupsize,
                    hipStream_t stream);

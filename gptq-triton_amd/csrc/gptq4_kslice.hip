@@ -1,0 +1,435 @@
+// Dequant-fused matmul for mid-sized M (17 .. a few hundred rows) on gfx950.
+//
+// With so few rows there is one row tile (or a handful), so the tiled kernel's tile count
+// - N / 256 - leaves most CUs idle unless K is split across workgroups, and every split
+// costs a round trip of fp32 partial sums through memory.  Here the split along K happens
+// inside the workgroup: a workgroup owns a strip of only 64 output columns (128 for a
+// rotary head), and its four waves each run the tiled kernel's wave loop - the same
+// (32*MT) x 64 wave tile, 8 MFMAs per pair of decoded words at MT = 4 - over their own
+// contiguous quarter (half) of K.  The waves share nothing while they stream: each has
+// its own double-buffered activation tile in LDS, filled by its own LDS-direct loads, so
+// the loop has no barrier at all.  At the end the four accumulator sets meet in LDS:
+// row block mt is summed and finished by wave mt.
+//
+//   plain   : 4 K slices of one 64-column strip.
+//   SiLU*mul: waves 0,1 = the two K halves of the gate strip, waves 2,3 = of the up strip.
+//   rotary  : waves 0,1 = the two K halves of columns [0, 64) of a head, waves 2,3 = of
+//             [64, 128); the wave that finishes a row block holds d and d + 64 itself.
+//
+// Weights are decoded exactly once per row tile.  K can still be split across workgroups
+// on top (last-arriver protocol of the other kernels) when N / 64 strips do not fill the
+// chip; the partial sums exchanged are the workgroup's already reduced tile.
+#include "gptq4_internal.h"
+
+namespace {
+
+constexpr int BK = 64;
+
+template <int EPI, int MT>
+__global__ __launch_bounds__(256, (MT == 4) ? 1 : 2) void gptq4_kslice_kernel(MatmulArgs p) {
+    constexpr int BM = 32 * MT;
+    constexpr int KS = (EPI == EPI_PLAIN) ? 4 : 2;      // waves along K per strip
+    constexpr int BN = (EPI == EPI_ROPE) ? 128 : 64;    // output columns of the workgroup
+    constexpr int NSET = (EPI == EPI_PLAIN) ? 1 : 2;    // value sets the finishing wave combines
+    constexpr int A_HALVES = BM * BK;                   // one wave's K tile of activations
+    constexpr int A_UNITS = BM / 8;                     // LDS-direct loads per wave and K tile (8 rows each)
+
+    // Per-wave activation tiles (two objects, so that the compiler can tell the loads into one
+    // from the reads of the other).  Afterwards the same memory is MT * 4 exchange regions of
+    // 8 KiB: region (mt, w) = accumulators of row block mt from wave w.
+    __shared__ __attribute__((aligned(16))) half_t As0[4 * A_HALVES];
+    __shared__ __attribute__((aligned(16))) half_t As1[4 * A_HALVES];
+    static_assert(2 * 4 * A_HALVES * sizeof(half_t) >= (size_t)MT * 4 * 32 * 64 * sizeof(float), "exchange regions do not fit");
+    auto region = [&](int mt, int w) -> float * {
+        const int r = mt * 4 + w;
+        constexpr int HALF = MT * 2;
+        return reinterpret_cast<float *>(r < HALF ? As0 : As1) + (r < HALF ? r : r - HALF) * (32 * 64);
+    };
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int part = (KS == 4) ? 0 : (wave >> 1);  // gate / up, or the half of the head
+    const int ksl = (KS == 4) ? wave : (wave & 1);
+    const int l32 = lane & 31;
+    const int lhi = lane >> 5;
+
+    const int M = p.M, K = p.K, N = p.N;
+    const int tiles_m = (M + BM - 1) / BM;
+
+    // XCD-contiguous logical tile index, row tiles fastest
+    const int total = gridDim.x;
+    const int per = total >> 3, rem = total & 7;
+    const int xcd = blockIdx.x & 7;
+    const int logical = xcd * per + (xcd < rem ? xcd : rem) + (blockIdx.x >> 3);
+    const int tile_n = logical / tiles_m;
+    const int tile_m = logical - tile_n * tiles_m;
+    const int m0 = tile_m * BM;
+    const int n0 = tile_n * BN;
+
+    const int mat = (EPI == EPI_SILU_MUL) ? part : 0;
+    const int ncol = n0 + ((EPI == EPI_ROPE) ? part * 64 : 0) + 2 * l32;  // lane's 2 columns
+    const uint32_t *bptr = p.w[mat].qweight + (size_t)lhi * N + ncol;     // row lhi of K tile 0
+    const uint32_t *qz = p.w[mat].qzeros + (ncol >> 3);
+    const half_t *sc = p.w[mat].scales + ncol;
+    const int tiles_per_group = p.groupsize / BK;
+    const int last_group = K / p.groupsize - 1;
+
+    f16_t acc[MT][2];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[mt][t][i] = 0.f;
+
+    // K tiles of the workgroup (split across workgroups), then of this wave
+    const int split = blockIdx.y;
+    const int wg_begin = split * p.slot_q + min(split, p.slot_rem);
+    const int wg_len = p.slot_q + (split < p.slot_rem ? 1 : 0);
+    const int wq = wg_len / KS, wr = wg_len % KS;
+    const int k_begin = wg_begin + ksl * wq + min(ksl, wr);
+    const int nk = k_begin + wq + (ksl < wr ? 1 : 0);
+
+    if (nk > k_begin) {
+        half_t *const buf0 = As0 + wave * A_HALVES;
+        half_t *const buf1 = As1 + wave * A_HALVES;
+        // Activations global -> LDS directly.  One instruction fills 8 rows x 8 chunks of 16
+        // bytes; the chunk that lands at position c of row r is global chunk c ^ ((r >> 1) & 7),
+        // which makes the 128-bit fragment reads conflict-free without padding.  Rows of a
+        // unit are 8u + lane / 8, so the swizzle term is (lane >> 4) for even u and that ^ 4
+        // for odd u: two per-lane offsets, everything else is a scalar offset.
+        const int valid = min(BM, M - m0);
+        const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)(p.x + (size_t)m0 * K), 0, (int)((uint32_t)valid * (uint32_t)K * 2u), 0x00020000);
+        const int r8 = lane >> 3, c8 = lane & 7;
+        const int voff_even = (r8 * K + 8 * (c8 ^ (r8 >> 1))) * 2;
+        const int voff_odd = (r8 * K + 8 * (c8 ^ (r8 >> 1) ^ 4)) * 2;
+        const bool full = (valid == BM);
+        auto dma_a = [&](half_t *dst, int kt) {
+            if (full) {
+#pragma unroll
+                for (int u = 0; u < A_UNITS; ++u)
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (__attribute__((address_space(3))) void *)(dst + u * 512), 16,
+                                                             (u & 1) ? voff_odd : voff_even, (8 * u * K + kt * BK) * 2, 0, 0);
+            } else {
+                // last row tile: rows beyond M load row M-1 instead (the scalar offset is not
+                // covered by the buffer's range check, so the row has to be clamped per lane)
+#pragma unroll
+                for (int u = 0; u < A_UNITS; ++u) {
+                    const int row = min(8 * u + r8, valid - 1);
+                    const int chunk = c8 ^ (r8 >> 1) ^ ((u & 1) ? 4 : 0);
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (__attribute__((address_space(3))) void *)(dst + u * 512), 16,
+                                                             (row * K + 8 * chunk) * 2, kt * (BK * 2), 0, 0);
+                }
+            }
+            asm volatile("" ::: "memory");  // the loads that follow stay behind these
+        };
+        const int sw = (l32 >> 1) & 7;  // (row >> 1) & 7 for every row this lane reads (rows = 32*j + l32)
+
+        // Packed words of two K tiles: slot [par][ks] holds step ks of a tile of parity par.  It
+        // is decoded during step ks - 1 and refilled during step ks - once its old contents
+        // are dead, so the load can land in place - with the same step two tiles on.
+        uint2 b2[2][4];
+        auto load_b2 = [&](int par, int kt, int ks) {
+            b2[par][ks] = *reinterpret_cast<const uint2 *>(bptr + ((size_t)min(kt, nk - 1) * (BK / 8) + 2 * ks) * N);
+        };
+        // Scale and zero words two tiles ahead as well; the group of the look-ahead tile is
+        // tracked by counting.
+        int group2 = k_begin / tiles_per_group;
+        int left2 = tiles_per_group - (k_begin - group2 * tiles_per_group);
+        uint32_t g_s[2], g_z[2];
+        auto load_group2 = [&](int par) {
+            const int g = min(group2, last_group);
+            g_s[par] = *reinterpret_cast<const uint32_t *>(sc + (size_t)g * N);
+            g_z[par] = qz[(size_t)g * (N >> 3)];
+            if (left2 == 1) {
+                ++group2;
+                left2 = tiles_per_group;
+            } else {
+                --left2;
+            }
+        };
+        ColDecodeNat cn[2];
+        auto make_cn = [&](int par) {
+            const uint32_t z2 = g_z[par] >> (((2 * l32) & 7) * 4);
+            cn[0] = make_col_decode_nat(z2 & 0xFu, g_s[par]);
+            cn[1] = make_col_decode_nat((z2 >> 4) & 0xFu, g_s[par] >> 16);
+        };
+
+        dma_a(buf0, k_begin);
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) load_b2(0, k_begin, ks);
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) load_b2(1, k_begin + 1, ks);
+        load_group2(0);  // group of tile k_begin
+        make_cn(0);
+        load_group2(1);  // group of tile k_begin + 1, made into constants at the end of tile k_begin
+        h8_t bf[2];
+        bf[0] = decode_word_natural(b2[0][0].x, cn[0]);
+        bf[1] = decode_word_natural(b2[0][0].y, cn[1]);
+
+        // one K tile (of parity `par` counted from k_begin) from buffer `cur`, while the next
+        // tile streams into `nxt`
+        auto k_tile = [&](const half_t *cur, half_t *nxt, int kt, int par) {
+            // Loads complete in order and this wave issued 4 packed-word loads after the
+            // scale/zero words that followed its LDS-direct loads of this tile: at most 4
+            // outstanding means the tile has landed.  It is this wave's own tile: no barrier.
+            asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+            dma_a(nxt, min(kt + 1, nk - 1));
+            load_group2(par);
+            h8_t araw[MT];
+            auto read_a = [&](int ks) {
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                    araw[mt] = *reinterpret_cast<const h8_t *>(cur + (mt * 32 + l32) * BK + 8 * ((2 * ks + lhi) ^ sw));
+            };
+            read_a(0);
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                h8_t af[MT];
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) af[mt] = araw[mt];
+                if (ks < 3) read_a(ks + 1);
+                if (ks == 3) make_cn(par ^ 1);
+                load_b2(par, kt + 2, ks);           // this step's words were decoded during the previous step
+                __builtin_amdgcn_sched_barrier(0);  // keep the loads above the MFMAs that hide them
+                const uint2 nw = (ks < 3) ? b2[par][ks + 1] : b2[par ^ 1][0];
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt], bf[0], acc[mt][0], 0, 0, 0);
+                bf[0] = decode_word_natural(nw.x, cn[0]);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt], bf[1], acc[mt][1], 0, 0, 0);
+                bf[1] = decode_word_natural(nw.y, cn[1]);
+            }
+        };
+        int kt = k_begin;
+        for (; kt + 1 < nk; kt += 2) {
+            k_tile(buf0, buf1, kt, 0);
+            k_tile(buf1, buf0, kt + 1, 1);
+        }
+        if (kt < nk) k_tile(buf0, buf1, kt, 0);
+    }
+    // every LDS-direct load has landed and every wave is done reading before the tiles are
+    // reused for the exchange
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __syncthreads();
+
+    // ---- the four accumulator sets meet: row block mt goes to wave mt.
+    // acc[mt][t][i]: row = 32*mt + 8*(i/4) + 4*lhi + i%4 of the tile, column = 2*l32 + t of the strip.
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        float *const dst = region(mt, wave);
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) dst[(t * 16 + i) * 64 + lane] = acc[mt][t][i];
+    }
+    __syncthreads();
+
+    // vals[0] (and vals[1]): the sums the epilogue combines - plain: the strip; SiLU*mul: gate
+    // and up; rotary: columns d < 64 and d >= 64 of the head.  Only waves < MT hold any.
+    float vals[NSET][2][16];
+    const bool owner = wave < MT;
+    if (owner) {
+        const float *src[4];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) src[w] = region(wave, w) + lane;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                float v[4];
+#pragma unroll
+                for (int w = 0; w < 4; ++w) v[w] = src[w][(t * 16 + i) * 64];
+                if (NSET == 1) {
+                    vals[0][t][i] = ((v[0] + v[1]) + v[2]) + v[3];
+                } else {
+                    vals[0][t][i] = v[0] + v[1];
+                    vals[NSET - 1][t][i] = v[2] + v[3];
+                }
+            }
+    }
+
+    if (p.splitk > 1) {
+        // K split across workgroups as well: each publishes its reduced tile (agent-scope
+        // atomics, no cache maintenance), the last one to arrive sums them in split order.
+        __shared__ int s_is_last;
+        constexpr int NREG = NSET * 32;
+        const int tile = logical;
+        const size_t per_split = (size_t)MT * NREG * 64;
+        float *const mine = p.partials + ((size_t)tile * p.splitk + split) * per_split + (size_t)wave * NREG * 64 + lane;
+        if (owner) {
+#pragma unroll
+            for (int s = 0; s < NSET; ++s)
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i)
+                        __hip_atomic_store(mine + ((s * 2 + t) * 16 + i) * 64, vals[s][t][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) {
+            const int old = __hip_atomic_fetch_add(&p.counters[tile * COUNTER_STRIDE], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s_is_last = (old == p.splitk - 1);
+        }
+        __syncthreads();
+        if (!s_is_last) return;
+        if (owner) {
+            const float *const all = p.partials + (size_t)tile * p.splitk * per_split + (size_t)wave * NREG * 64 + lane;
+#pragma unroll
+            for (int s = 0; s < NSET; ++s)
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) vals[s][t][i] = 0.f;
+            for (int sp = 0; sp < p.splitk; ++sp) {
+#pragma unroll
+                for (int s = 0; s < NSET; ++s)
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) {
+                        float got[16];
+#pragma unroll
+                        for (int i = 0; i < 16; ++i)
+                            got[i] = __hip_atomic_load(all + (size_t)sp * per_split + ((s * 2 + t) * 16 + i) * 64, __ATOMIC_RELAXED,
+                                                       __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) vals[s][t][i] += got[i];
+                    }
+            }
+        }
+        if (tid == 0) __hip_atomic_store(&p.counters[tile * COUNTER_STRIDE], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (!owner) return;
+
+    // ---- epilogue of row block `wave`
+    const int row0 = m0 + wave * 32 + 4 * lhi;
+    if (EPI == EPI_PLAIN) {
+        h2_t bias2 = {(half_t)0.f, (half_t)0.f};
+        if (p.bias != nullptr) bias2 = as_h2(*reinterpret_cast<const uint32_t *>(p.bias + ncol));
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int row = row0 + 8 * (i >> 2) + (i & 3);
+            if (row < M) {
+                h2_t o = {(half_t)vals[0][0][i], (half_t)vals[0][1][i]};
+                if (p.bias != nullptr) o = o + bias2;
+                *reinterpret_cast<uint32_t *>(p.y + (size_t)row * N + ncol) = as_u32(o);
+            }
+        }
+    } else if (EPI == EPI_SILU_MUL) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int row = row0 + 8 * (i >> 2) + (i & 3);
+            if (row < M) {
+                const h2_t o = {(half_t)(silu_f32(vals[0][0][i]) * vals[NSET - 1][0][i]),
+                                (half_t)(silu_f32(vals[0][1][i]) * vals[NSET - 1][1][i])};
+                *reinterpret_cast<uint32_t *>(p.y + (size_t)row * N + n0 + 2 * l32) = as_u32(o);
+            }
+        }
+    } else {
+        // the workgroup's 128 columns are one head of q, k or v
+        const RopeArgs &r = p.rope;
+        const int head_col = n0 >> 7;
+        const int which = head_col / r.H;
+        const int head = head_col - which * r.H;
+        const int cap = (which == 0) ? r.S : r.kv_capacity;
+        half_t *const dst = ((which == 0) ? r.q : (which == 1) ? r.k : r.v) + (size_t)head * cap * 128 + 2 * l32;
+        const size_t seq_stride = (size_t)r.H * cap * 128;
+        const bool at_position = (which != 0) && r.kv_offset < 0;  // cache row = the token's position
+        const int row_shift = (which == 0 || r.kv_offset < 0) ? 0 : r.kv_offset;
+        float2 cs[16], sn[16];
+        int pos[16];
+        if (which < 2 || at_position) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) pos[i] = max(r.position_ids[min(row0 + 8 * (i >> 2) + (i & 3), M - 1)], 0);
+        }
+        if (which < 2) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int tp = min(pos[i], r.max_pos - 1);
+                cs[i] = *reinterpret_cast<const float2 *>(r.cos_table + (size_t)tp * 64 + 2 * l32);
+                sn[i] = *reinterpret_cast<const float2 *>(r.sin_table + (size_t)tp * 64 + 2 * l32);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int row = row0 + 8 * (i >> 2) + (i & 3);
+            float lo0 = vals[0][0][i], lo1 = vals[0][1][i], hi0 = vals[NSET - 1][0][i], hi1 = vals[NSET - 1][1][i];
+            if (which < 2) {
+                const float a0 = lo0 * cs[i].x - hi0 * sn[i].x, a1 = lo1 * cs[i].y - hi1 * sn[i].y;
+                const float b0 = hi0 * cs[i].x + lo0 * sn[i].x, b1 = hi1 * cs[i].y + lo1 * sn[i].y;
+                lo0 = a0, lo1 = a1, hi0 = b0, hi1 = b1;
+            }
+            if (row < M) {
+                int bb, srow;
+                split_row(r, row, bb, srow);
+                const int crow = at_position ? min(pos[i], r.kv_capacity - 1) : srow + row_shift;
+                half_t *const at = dst + (size_t)bb * seq_stride + (size_t)crow * 128;
+                const h2_t olo = {(half_t)lo0, (half_t)lo1}, ohi = {(half_t)hi0, (half_t)hi1};
+                *reinterpret_cast<uint32_t *>(at) = as_u32(olo);
+                *reinterpret_cast<uint32_t *>(at + 64) = as_u32(ohi);
+            }
+        }
+    }
+}
+
+template <int EPI, int MT>
+int launch_one(const MatmulArgs &a, int tiles, hipStream_t stream) {
+    dim3 grid((unsigned)tiles, (unsigned)a.splitk), block(256);
+    hipLaunchKernelGGL((gptq4_kslice_kernel<EPI, MT>), grid, block, 0, stream, a);
+    return (int)hipGetLastError();
+}
+
+template <int EPI>
+int launch_epi(const MatmulArgs &a, const KslicePlan &pl, hipStream_t stream) {
+    switch (pl.mt) {
+        case 1: return launch_one<EPI, 1>(a, pl.tiles, stream);
+        case 2: return launch_one<EPI, 2>(a, pl.tiles, stream);
+        default: return launch_one<EPI, 4>(a, pl.tiles, stream);
+    }
+}
+
+}  // namespace
+
+KsliceTuning g_kslice_tuning = {1, 0, 0};
+
+// Row tile: 32 rows up to M = 32, else 64 (128-row tiles decode each weight once instead of
+// twice at M = 128, but their 128 KiB of LDS leaves one wave per SIMD and they come out no
+// faster).  K is split across workgroups only while all of them still fit on the chip at
+// once (two workgroups per CU), and never below 4 K tiles per wave.
+KslicePlan kslice_plan(int epi, int M, int N, int K, bool has_perm) {
+    KslicePlan pl = {};
+    const int ks = (epi == EPI_PLAIN) ? 4 : 2;
+    const int bn = (epi == EPI_ROPE) ? 128 : 64;
+    const int nk = K / 64;
+    pl.mt = g_kslice_tuning.mt ? g_kslice_tuning.mt : (M <= 32 ? 1 : 2);
+    const int bm = 32 * pl.mt;
+    pl.tiles = ((M + bm - 1) / bm) * (N / bn);
+    int s = 1;
+    if (g_kslice_tuning.splitk > 0) {
+        s = g_kslice_tuning.splitk;
+    } else {
+        s = (pl.mt == 4 ? 256 : 512) / pl.tiles;
+        if (s > nk / (4 * ks)) s = nk / (4 * ks);
+    }
+    if (s > GEMM_MAX_SPLITK) s = GEMM_MAX_SPLITK;
+    if (s < 1 || pl.tiles > SKINNY_MAX_TILES) s = 1;
+    pl.splitk = s;
+    // the wave loop needs the activations unpermuted and at least one K tile per wave
+    pl.ok = !has_perm && (N % bn) == 0 && nk / s >= ks;
+    return pl;
+}
+
+size_t kslice_partial_bytes(int epi, const KslicePlan &pl) {
+    const int nset = (epi == EPI_PLAIN) ? 1 : 2;
+    return pl.splitk > 1 ? (size_t)pl.tiles * pl.splitk * pl.mt * nset * 32 * 64 * sizeof(float) : 0;
+}
+
+int launch_kslice(int epi, const MatmulArgs &a, const KslicePlan &pl, hipStream_t stream) {
+    switch (epi) {
+        case EPI_PLAIN: return launch_epi<EPI_PLAIN>(a, pl, stream);
+        case EPI_SILU_MUL: return launch_epi<EPI_SILU_MUL>(a, pl, stream);
+        default: return launch_epi<EPI_ROPE>(a, pl, stream);
+    }
+}

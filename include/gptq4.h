@@ -160,6 +160,12 @@ void gptq4_set_tuning(int words, int depth, int splitk);
  * outputs; half as wide for the fused gate/up) and the split-K factor; 0 = automatic. */
 void gptq4_set_gemm_tuning(int mt, int splitk);
 
+/* Same for the mid-M kernel (M > 16 with too few wide tiles for the tiled kernel; K is split
+ * across the four waves of a workgroup): mode 0 = never use it, 1 = where it is the faster
+ * kernel, 2 = wherever it can run; 32-row blocks per row tile (1, 2, 4) and the split-K
+ * factor across workgroups; 0 = automatic. */
+void gptq4_set_midm_tuning(int mode, int mt, int splitk);
+
 /* Same for the balanced decode GEMV (M <= 4): mode 0 = never use it, 1 = where it is the
  * faster kernel (one row, SiLU*mul epilogue), 2 = wherever it can run; units in
  * flight per wave (2, 3), waves per workgroup (4, 8, 16), waves per CU (4..32), 0 =
