@@ -139,7 +139,7 @@ void gptq4_set_gemm_tuning(int mt, int splitk) {
 
 void gptq4_set_midm_tuning(int mode, int mt, int splitk) {
     g_kslice_tuning.mode = (mode >= 0 && mode <= 2) ? mode : 1;
-    g_kslice_tuning.mt = (mt == 1 || mt == 2 || mt == 4) ? mt : 0;
+    g_kslice_tuning.mt = (mt == 1 || mt == 2) ? mt : 0;
     g_kslice_tuning.splitk = splitk > 0 ? splitk : 0;
 }
 

@@ -92,7 +92,7 @@ int launch_gemm(int epi, const MatmulArgs &a, const GemmPlan &plan, hipStream_t 
 
 // Launch shape of the mid-M kernel (K split across the waves of a workgroup).
 struct KslicePlan {
-    int mt;      // 32-row blocks per row tile (1, 2 or 4)
+    int mt;      // 32-row blocks per row tile (1 or 2)
     int splitk;  // workgroups sharing one tile along K, on top of the split inside the workgroup
     int tiles;
     bool ok;     // false: the shape needs another kernel

@@ -5,8 +5,8 @@
 // costs a round trip of fp32 partial sums through memory.  Here the split along K happens
 // inside the workgroup: a workgroup owns a strip of only 64 output columns (128 for a
 // rotary head), and its four waves each run the tiled kernel's wave loop - the same
-// (32*MT) x 64 wave tile, 8 MFMAs per pair of decoded words at MT = 4 - over their own
-// contiguous quarter (half) of K.  The waves share nothing while they stream: each has
+// (32*MT) x 64 wave tile, here with MT = 1 or 2 - over their own contiguous quarter
+// (half) of K.  The waves share nothing while they stream: each has
 // its own double-buffered activation tile in LDS, filled by its own LDS-direct loads, so
 // the loop has no barrier at all.  At the end the four accumulator sets meet in LDS:
 // row block mt is summed and finished by wave mt.
@@ -26,7 +26,7 @@ namespace {
 constexpr int BK = 64;
 
 template <int EPI, int MT>
-__global__ __launch_bounds__(256, (MT == 4) ? 1 : 2) void gptq4_kslice_kernel(MatmulArgs p) {
+__global__ __launch_bounds__(256, 2) void gptq4_kslice_kernel(MatmulArgs p) {
     constexpr int BM = 32 * MT;
     constexpr int KS = (EPI == EPI_PLAIN) ? 4 : 2;      // waves along K per strip
     constexpr int BN = (EPI == EPI_ROPE) ? 128 : 64;    // output columns of the workgroup
@@ -383,11 +383,7 @@ int launch_one(const MatmulArgs &a, int tiles, hipStream_t stream) {
 
 template <int EPI>
 int launch_epi(const MatmulArgs &a, const KslicePlan &pl, hipStream_t stream) {
-    switch (pl.mt) {
-        case 1: return launch_one<EPI, 1>(a, pl.tiles, stream);
-        case 2: return launch_one<EPI, 2>(a, pl.tiles, stream);
-        default: return launch_one<EPI, 4>(a, pl.tiles, stream);
-    }
+    return pl.mt == 1 ? launch_one<EPI, 1>(a, pl.tiles, stream) : launch_one<EPI, 2>(a, pl.tiles, stream);
 }
 
 }  // namespace
@@ -410,7 +406,7 @@ KslicePlan kslice_plan(int epi, int M, int N, int K, bool has_perm) {
     if (g_kslice_tuning.splitk > 0) {
         s = g_kslice_tuning.splitk;
     } else {
-        s = (pl.mt == 4 ? 256 : 512) / pl.tiles;
+        s = 512 / pl.tiles;
         if (s > nk / (4 * ks)) s = nk / (4 * ks);
     }
     if (s > GEMM_MAX_SPLITK) s = GEMM_MAX_SPLITK;
