@@ -4,20 +4,21 @@
 // - N / 256 - leaves most CUs idle unless K is split across workgroups, and every split
 // costs a round trip of fp32 partial sums through memory.  Here the split along K happens
 // inside the workgroup: a workgroup owns a strip of only 64 output columns (128 for a
-// rotary head), and its four waves each run the tiled kernel's wave loop - the same
-// (32*MT) x 64 wave tile, here with MT = 1 or 2 - over their own contiguous quarter
-// (half) of K.  The waves share nothing while they stream: each has
-// its own double-buffered activation tile in LDS, filled by its own LDS-direct loads, so
-// the loop has no barrier at all.  At the end the four accumulator sets meet in LDS:
-// row block mt is summed and finished by wave mt.
+// rotary head), and its four waves each run the tiled kernel's wave loop over their own
+// contiguous quarter of K.  The waves share nothing while they stream: each has its own
+// double-buffered activation tile in LDS, filled by its own LDS-direct loads, so the loop
+// has no barrier at all.  At the end the four accumulator sets meet in LDS: row block mt
+// is summed and finished by wave mt.
 //
-//   plain   : 4 K slices of one 64-column strip.
-//   SiLU*mul: waves 0,1 = the two K halves of the gate strip, waves 2,3 = of the up strip.
-//   rotary  : waves 0,1 = the two K halves of columns [0, 64) of a head, waves 2,3 = of
-//             [64, 128); the wave that finishes a row block holds d and d + 64 itself.
+// Wave tile: (32*MT) rows x NB blocks of 64 columns.
+//   plain   : NB = 1, one 64-column strip.
+//   SiLU*mul: NB = 2, the same 64 columns of the gate and of the up matrix.
+//   rotary  : NB = 2, columns [0, 64) and [64, 128) of one head, so the wave that finishes
+//             a row block holds d and d + 64 itself.
+// With NB = 2 every activation fragment read from LDS feeds twice as many MFMAs.
 //
 // Weights are decoded exactly once per row tile.  K can still be split across workgroups
-// on top (last-arriver protocol of the other kernels) when N / 64 strips do not fill the
+// on top (last-arriver protocol of the other kernels) when the strips do not fill the
 // chip; the partial sums exchanged are the workgroup's already reduced tile.
 #include "gptq4_internal.h"
 
@@ -28,9 +29,10 @@ constexpr int BK = 64;
 template <int EPI, int MT>
 __global__ __launch_bounds__(256, 2) void gptq4_kslice_kernel(MatmulArgs p) {
     constexpr int BM = 32 * MT;
-    constexpr int KS = (EPI == EPI_PLAIN) ? 4 : 2;      // waves along K per strip
+    constexpr int KS = 4;                               // all four waves along K
+    constexpr int NB = (EPI == EPI_PLAIN) ? 1 : 2;      // 64-column blocks of the wave tile
     constexpr int BN = (EPI == EPI_ROPE) ? 128 : 64;    // output columns of the workgroup
-    constexpr int NSET = (EPI == EPI_PLAIN) ? 1 : 2;    // value sets the finishing wave combines
+    constexpr int NSET = NB;                            // value sets the finishing wave combines
     constexpr int A_HALVES = BM * BK;                   // one wave's K tile of activations
     constexpr int A_UNITS = BM / 8;                     // LDS-direct loads per wave and K tile (8 rows each)
 
@@ -49,8 +51,7 @@ __global__ __launch_bounds__(256, 2) void gptq4_kslice_kernel(MatmulArgs p) {
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int part = (KS == 4) ? 0 : (wave >> 1);  // gate / up, or the half of the head
-    const int ksl = (KS == 4) ? wave : (wave & 1);
+    const int ksl = wave;
     const int l32 = lane & 31;
     const int lhi = lane >> 5;
 
@@ -67,21 +68,35 @@ __global__ __launch_bounds__(256, 2) void gptq4_kslice_kernel(MatmulArgs p) {
     const int m0 = tile_m * BM;
     const int n0 = tile_n * BN;
 
-    const int mat = (EPI == EPI_SILU_MUL) ? part : 0;
-    const int ncol = n0 + ((EPI == EPI_ROPE) ? part * 64 : 0) + 2 * l32;  // lane's 2 columns
-    const uint32_t *bptr = p.w[mat].qweight + (size_t)lhi * N + ncol;     // row lhi of K tile 0
-    const uint32_t *qz = p.w[mat].qzeros + (ncol >> 3);
-    const half_t *sc = p.w[mat].scales + ncol;
+    // block j of the wave tile: matrix j at the strip's columns (SiLU*mul), or columns
+    // 64*j .. 64*j + 63 of the head (rotary); the lane's 2 columns of it
+    const int ncol = n0 + 2 * l32;
+    // (for rotary the second block is a constant offset from the first: no second set of pointers)
+    constexpr int NPTR = (EPI == EPI_SILU_MUL) ? 2 : 1;
+    const uint32_t *bptr_[NPTR];
+    const uint32_t *qz_[NPTR];
+    const half_t *sc_[NPTR];
+#pragma unroll
+    for (int j = 0; j < NPTR; ++j) {
+        bptr_[j] = p.w[j].qweight + (size_t)lhi * N + ncol;  // row lhi of K tile 0
+        qz_[j] = p.w[j].qzeros + (ncol >> 3);
+        sc_[j] = p.w[j].scales + ncol;
+    }
+    auto bptr = [&](int j) { return (EPI == EPI_ROPE) ? bptr_[0] + 64 * j : bptr_[j < NPTR ? j : 0]; };
+    auto qz = [&](int j) { return (EPI == EPI_ROPE) ? qz_[0] + 8 * j : qz_[j < NPTR ? j : 0]; };
+    auto sc = [&](int j) { return (EPI == EPI_ROPE) ? sc_[0] + 64 * j : sc_[j < NPTR ? j : 0]; };
     const int tiles_per_group = p.groupsize / BK;
     const int last_group = K / p.groupsize - 1;
 
-    f16_t acc[MT][2];
+    f16_t acc[NB][MT][2];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+    for (int j = 0; j < NB; ++j)
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+        for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) acc[mt][t][i] = 0.f;
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) acc[j][mt][t][i] = 0.f;
 
     // K tiles of the workgroup (split across workgroups), then of this wave
     const int split = blockIdx.y;
@@ -130,19 +145,24 @@ __global__ __launch_bounds__(256, 2) void gptq4_kslice_kernel(MatmulArgs p) {
         // Packed words of two K tiles: slot [par][ks] holds step ks of a tile of parity par.  It
         // is decoded during step ks - 1 and refilled during step ks - once its old contents
         // are dead, so the load can land in place - with the same step two tiles on.
-        uint2 b2[2][4];
+        uint2 b2[NB][2][4];
         auto load_b2 = [&](int par, int kt, int ks) {
-            b2[par][ks] = *reinterpret_cast<const uint2 *>(bptr + ((size_t)min(kt, nk - 1) * (BK / 8) + 2 * ks) * N);
+            const size_t off = ((size_t)min(kt, nk - 1) * (BK / 8) + 2 * ks) * N;
+#pragma unroll
+            for (int j = 0; j < NB; ++j) b2[j][par][ks] = *reinterpret_cast<const uint2 *>(bptr(j) + off);
         };
         // Scale and zero words two tiles ahead as well; the group of the look-ahead tile is
         // tracked by counting.
         int group2 = k_begin / tiles_per_group;
         int left2 = tiles_per_group - (k_begin - group2 * tiles_per_group);
-        uint32_t g_s[2], g_z[2];
+        uint32_t g_s[NB][2], g_z[NB][2];
         auto load_group2 = [&](int par) {
             const int g = min(group2, last_group);
-            g_s[par] = *reinterpret_cast<const uint32_t *>(sc + (size_t)g * N);
-            g_z[par] = qz[(size_t)g * (N >> 3)];
+#pragma unroll
+            for (int j = 0; j < NB; ++j) {
+                g_s[j][par] = *reinterpret_cast<const uint32_t *>(sc(j) + (size_t)g * N);
+                g_z[j][par] = qz(j)[(size_t)g * (N >> 3)];
+            }
             if (left2 == 1) {
                 ++group2;
                 left2 = tiles_per_group;
@@ -150,11 +170,14 @@ __global__ __launch_bounds__(256, 2) void gptq4_kslice_kernel(MatmulArgs p) {
                 --left2;
             }
         };
-        ColDecodeNat cn[2];
+        ColDecodeNat cn[NB][2];
         auto make_cn = [&](int par) {
-            const uint32_t z2 = g_z[par] >> (((2 * l32) & 7) * 4);
-            cn[0] = make_col_decode_nat(z2 & 0xFu, g_s[par]);
-            cn[1] = make_col_decode_nat((z2 >> 4) & 0xFu, g_s[par] >> 16);
+#pragma unroll
+            for (int j = 0; j < NB; ++j) {
+                const uint32_t z2 = g_z[j][par] >> (((2 * l32) & 7) * 4);
+                cn[j][0] = make_col_decode_nat(z2 & 0xFu, g_s[j][par]);
+                cn[j][1] = make_col_decode_nat((z2 >> 4) & 0xFu, g_s[j][par] >> 16);
+            }
         };
 
         dma_a(buf0, k_begin);
@@ -165,17 +188,23 @@ __global__ __launch_bounds__(256, 2) void gptq4_kslice_kernel(MatmulArgs p) {
         load_group2(0);  // group of tile k_begin
         make_cn(0);
         load_group2(1);  // group of tile k_begin + 1, made into constants at the end of tile k_begin
-        h8_t bf[2];
-        bf[0] = decode_word_natural(b2[0][0].x, cn[0]);
-        bf[1] = decode_word_natural(b2[0][0].y, cn[1]);
+        h8_t bf[NB][2];
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+            bf[j][0] = decode_word_natural(b2[j][0][0].x, cn[j][0]);
+            bf[j][1] = decode_word_natural(b2[j][0][0].y, cn[j][1]);
+        }
 
         // one K tile (of parity `par` counted from k_begin) from buffer `cur`, while the next
         // tile streams into `nxt`
         auto k_tile = [&](const half_t *cur, half_t *nxt, int kt, int par) {
-            // Loads complete in order and this wave issued 4 packed-word loads after the
-            // scale/zero words that followed its LDS-direct loads of this tile: at most 4
-            // outstanding means the tile has landed.  It is this wave's own tile: no barrier.
-            asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+            // Loads complete in order and this wave issued 4 * NB packed-word loads after the
+            // scale/zero words that followed its LDS-direct loads of this tile: at most that
+            // many outstanding means the tile has landed.  It is this wave's own tile: no barrier.
+            if (NB == 1)
+                asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+            else
+                asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
             dma_a(nxt, min(kt + 1, nk - 1));
             load_group2(par);
             h8_t araw[MT];
@@ -194,13 +223,18 @@ __global__ __launch_bounds__(256, 2) void gptq4_kslice_kernel(MatmulArgs p) {
                 if (ks == 3) make_cn(par ^ 1);
                 load_b2(par, kt + 2, ks);           // this step's words were decoded during the previous step
                 __builtin_amdgcn_sched_barrier(0);  // keep the loads above the MFMAs that hide them
-                const uint2 nw = (ks < 3) ? b2[par][ks + 1] : b2[par ^ 1][0];
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt], bf[0], acc[mt][0], 0, 0, 0);
-                bf[0] = decode_word_natural(nw.x, cn[0]);
+                for (int j = 0; j < NB; ++j) {
+                    const uint2 nw = (ks < 3) ? b2[j][par][ks + 1] : b2[j][par ^ 1][0];
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt], bf[1], acc[mt][1], 0, 0, 0);
-                bf[1] = decode_word_natural(nw.y, cn[1]);
+                    for (int mt = 0; mt < MT; ++mt)
+                        acc[j][mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt], bf[j][0], acc[j][mt][0], 0, 0, 0);
+                    bf[j][0] = decode_word_natural(nw.x, cn[j][0]);
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
+                        acc[j][mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt], bf[j][1], acc[j][mt][1], 0, 0, 0);
+                    bf[j][1] = decode_word_natural(nw.y, cn[j][1]);
+                }
             }
         };
         int kt = k_begin;
@@ -215,40 +249,38 @@ __global__ __launch_bounds__(256, 2) void gptq4_kslice_kernel(MatmulArgs p) {
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
 
-    // ---- the four accumulator sets meet: row block mt goes to wave mt.
-    // acc[mt][t][i]: row = 32*mt + 8*(i/4) + 4*lhi + i%4 of the tile, column = 2*l32 + t of the strip.
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        float *const dst = region(mt, wave);
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) dst[(t * 16 + i) * 64 + lane] = acc[mt][t][i];
-    }
-    __syncthreads();
-
-    // vals[0] (and vals[1]): the sums the epilogue combines - plain: the strip; SiLU*mul: gate
-    // and up; rotary: columns d < 64 and d >= 64 of the head.  Only waves < MT hold any.
+    // ---- the four accumulator sets meet: row block mt goes to wave mt, one column block at a time.
+    // acc[j][mt][t][i]: row = 32*mt + 8*(i/4) + 4*lhi + i%4 of the tile, column = 2*l32 + t of block j.
+    // vals[j]: the sums the epilogue combines - plain: the strip; SiLU*mul: gate and up; rotary:
+    // columns d < 64 and d >= 64 of the head.  Only waves < MT hold any.
     float vals[NSET][2][16];
     const bool owner = wave < MT;
-    if (owner) {
-        const float *src[4];
 #pragma unroll
-        for (int w = 0; w < 4; ++w) src[w] = region(wave, w) + lane;
+    for (int j = 0; j < NB; ++j) {
+        if (j > 0) __syncthreads();  // the owners are done reading the previous block
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+        for (int mt = 0; mt < MT; ++mt) {
+            float *const dst = region(mt, wave);
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                float v[4];
+            for (int t = 0; t < 2; ++t)
 #pragma unroll
-                for (int w = 0; w < 4; ++w) v[w] = src[w][(t * 16 + i) * 64];
-                if (NSET == 1) {
-                    vals[0][t][i] = ((v[0] + v[1]) + v[2]) + v[3];
-                } else {
-                    vals[0][t][i] = v[0] + v[1];
-                    vals[NSET - 1][t][i] = v[2] + v[3];
+                for (int i = 0; i < 16; ++i) dst[(t * 16 + i) * 64 + lane] = acc[j][mt][t][i];
+        }
+        __syncthreads();
+        if (owner) {
+            const float *src[4];
+#pragma unroll
+            for (int w = 0; w < 4; ++w) src[w] = region(wave, w) + lane;
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    float v[4];
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) v[w] = src[w][(t * 16 + i) * 64];
+                    vals[j][t][i] = ((v[0] + v[1]) + v[2]) + v[3];
                 }
-            }
+        }
     }
 
     if (p.splitk > 1) {
@@ -393,10 +425,11 @@ KsliceTuning g_kslice_tuning = {1, 0, 0};
 // Row tile: 32 rows up to M = 32, else 64 (128-row tiles decode each weight once instead of
 // twice at M = 128, but their 128 KiB of LDS leaves one wave per SIMD and they come out no
 // faster).  K is split across workgroups only while all of them still fit on the chip at
-// once (two workgroups per CU), and never below 4 K tiles per wave.
+// once (two workgroups per CU; measured best at one per CU for the two-block wave tiles),
+// and never below 4 K tiles per wave.
 KslicePlan kslice_plan(int epi, int M, int N, int K, bool has_perm) {
     KslicePlan pl = {};
-    const int ks = (epi == EPI_PLAIN) ? 4 : 2;
+    const int ks = 4;
     const int bn = (epi == EPI_ROPE) ? 128 : 64;
     const int nk = K / 64;
     pl.mt = g_kslice_tuning.mt ? g_kslice_tuning.mt : (M <= 32 ? 1 : 2);
@@ -406,7 +439,7 @@ KslicePlan kslice_plan(int epi, int M, int N, int K, bool has_perm) {
     if (g_kslice_tuning.splitk > 0) {
         s = g_kslice_tuning.splitk;
     } else {
-        s = 512 / pl.tiles;
+        s = ((epi == EPI_PLAIN) ? 512 : 256) / pl.tiles;  // the two-block wave tiles: one workgroup per CU
         if (s > nk / (4 * ks)) s = nk / (4 * ks);
     }
     if (s > GEMM_MAX_SPLITK) s = GEMM_MAX_SPLITK;
