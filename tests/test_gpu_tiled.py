@@ -1,0 +1,105 @@
+"""GPU parity of the tiled kernel with the mid-M kernel switched off, so that every row count
+above 16 reaches it: both workgroup tiles (128 x 128 and 128 x 256), with and without K split
+across workgroups, all three epilogues, ragged last row tiles, and the automatic plan on a
+shape with enough wide tiles.  Same bars as test_gpu_parity.py."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import to_dev
+from oracle import gptq_oracle as O
+from test_gpu_parity import assert_close, gptq
+
+pytestmark = pytest.mark.gpu
+
+# (32-row blocks per wave: 2 = 128 x 128 tile, 4 = 128 x 256 tile; split-K); 0 = automatic
+CONFIGS = [(2, 1), (4, 1), (2, 3), (4, 2), (0, 0)]
+
+
+@pytest.fixture(params=CONFIGS, ids=lambda c: "mt%d_s%d" % c)
+def forced_tiled(request):
+    from gptq_triton_amd import _lib
+    lib = _lib.load()
+    lib.gptq4_set_midm_tuning(0, 0, 0)
+    lib.gptq4_set_gemm_tuning(*request.param)
+    yield lib
+    lib.gptq4_set_gemm_tuning(0, 0)
+    lib.gptq4_set_midm_tuning(1, 0, 0)
+
+
+@pytest.mark.parametrize("k,n,g", [(1024, 512, 128), (1536, 256, -1), (2048, 768, 512)])
+@pytest.mark.parametrize("m", [17, 128, 130, 300])
+def test_tiled_matmul(forced_tiled, k, n, g, m):
+    L = O.make_layer(k, n, g, seed=k + n + m, bias=(m % 2 == 0))
+    x = O.make_x(m, k, seed=m + 5)
+    D = to_dev(L)
+    xd = torch.from_numpy(x).cuda()
+    y = gptq().matmul4(k if g == -1 else g, xd, D["qweight"], D["scales"], D["qzeros"], D.get("bias"))
+    y2 = gptq().matmul4(k if g == -1 else g, xd, D["qweight"], D["scales"], D["qzeros"], D.get("bias"))
+    assert torch.equal(y, y2)
+    ref = O.quant_matmul_ref(x, L["qweight"], L["qzeros"], L["scales"], g, bias=L["bias"])
+    if L["bias"] is None:
+        assert_close(y.cpu().numpy(), ref, f"tiled matmul K={k} N={n} g={g} M={m}")
+    else:
+        ok, max_abs, _ = O.within_tolerance(y.cpu().numpy(), ref)
+        assert ok, max_abs
+
+
+@pytest.mark.parametrize("m", [40, 200])
+def test_tiled_gateup(forced_tiled, m):
+    k, n, g = 1024, 1280, 128
+    gate = O.make_layer(k, n, g, seed=100)
+    up = O.make_layer(k, n, g, seed=101)
+    x = O.make_x(m, k, seed=102 + m)
+    Dg, Du = to_dev(gate), to_dev(up)
+    h = gptq().llama_mlp_4(g, torch.from_numpy(x).cuda(), Dg["qweight"], Dg["scales"], Dg["qzeros"],
+                           Du["qweight"], Du["scales"], Du["qzeros"])
+    ref = O.mlp_gateup_ref(x, (gate["qweight"], gate["qzeros"], gate["scales"]),
+                           (up["qweight"], up["qzeros"], up["scales"]), g)
+    assert_close(h.cpu().numpy(), ref, f"tiled gate/up M={m}")
+
+
+@pytest.mark.parametrize("b,s,pos0,g", [(2, 33, 10, 128), (40, 1, 500, -1), (1, 150, 1800, 128)])
+def test_tiled_qkv_rotary(forced_tiled, b, s, pos0, g):
+    H, Dh, hidden = 8, 128, 1024
+    L = O.make_layer(hidden, 3 * hidden, g, seed=200 + s)
+    x = O.make_x(b * s, hidden, seed=201 + s).reshape(b, s, hidden)
+    pos = (pos0 + np.arange(s))[None, :].repeat(b, 0) + np.arange(b)[:, None] * 3
+    D = to_dev(L)
+    G = gptq()
+    cos, sin = G.RotaryTable(Dh, 2048).get(torch.device("cuda"), 2048)
+    q, k, v = G.qkv_rotary(hidden if g == -1 else g, torch.from_numpy(x).cuda(), D["qweight"], D["scales"],
+                           D["qzeros"], torch.from_numpy(pos).cuda(), cos, sin, H, Dh)
+    qr, kr, vr = O.qkv_rotary_ref(x, L["qweight"], L["qzeros"], L["scales"], g, pos, H, Dh, max_pos=2048)
+    for got, ref, name in ((q, qr, "q"), (k, kr, "k"), (v, vr, "v")):
+        assert_close(got.cpu().numpy(), ref, f"tiled {name} b={b} s={s} g={g}")
+
+
+def test_prefill_sized_call_takes_the_wide_tiles_by_itself():
+    """2048 rows x 3072 columns = 192 wide tiles: the automatic plan picks the 128 x 256 tile
+    without any forcing; K is small so that the oracle finishes in seconds."""
+    k, n, g, m = 256, 3072, 128, 2048
+    L = O.make_layer(k, n, g, seed=77)
+    x = O.make_x(m, k, seed=78)
+    D = to_dev(L)
+    y = gptq().matmul4(g, torch.from_numpy(x).cuda(), D["qweight"], D["scales"], D["qzeros"])
+    ref = O.quant_matmul_ref(x, L["qweight"], L["qzeros"], L["scales"], g)
+    assert_close(y.cpu().numpy(), ref, "prefill-sized matmul")
+
+
+def test_hand_over_between_the_mid_m_and_the_tiled_kernel():
+    """768 rows is the last row count the mid-M kernel takes on a narrow layer, 769 the first
+    for the tiled kernel: both sides of the boundary against the oracle, and the rows they
+    share against each other within fp32 summation-order noise."""
+    k, n, g = 512, 512, 128
+    L = O.make_layer(k, n, g, seed=91)
+    x = O.make_x(769, k, seed=92)
+    D = to_dev(L)
+    ref = O.quant_matmul_ref(x, L["qweight"], L["qzeros"], L["scales"], g)
+    ya = gptq().matmul4(g, torch.from_numpy(x[:768].copy()).cuda(), D["qweight"], D["scales"], D["qzeros"])
+    yb = gptq().matmul4(g, torch.from_numpy(x).cuda(), D["qweight"], D["scales"], D["qzeros"])
+    assert_close(ya.cpu().numpy(), ref[:768], "768 rows")
+    assert_close(yb.cpu().numpy(), ref, "769 rows")
+    big = torch.maximum(ya.abs(), yb[:768].abs()).float().cpu().numpy().astype(np.float16)
+    ulp = torch.from_numpy(np.spacing(big).astype(np.float32)).cuda()
+    assert bool(((ya.float() - yb[:768].float()).abs() <= ulp + 1e-4).all())
