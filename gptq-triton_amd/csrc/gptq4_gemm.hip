@@ -110,64 +110,7 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[mt][t][i] = 0.f;
 
-    // Activation staging: each thread owns A_UNITS 16-byte units (row, 8 k) of the tile.
-    // Rows beyond M read row M-1 instead of branching: A row m only feeds output row m and
-    // rows >= M are never stored.  Addresses: one uniform base (scalar registers) plus a
-    // small per-lane element offset.
     const half_t *a_base = p.x + (size_t)m0 * K;
-    uint32_t a_off[A_UNITS];
-    const int a_row = tid >> 3, a_ku = tid & 7;  // unit u of this thread: row a_row + 32*u, k-unit a_ku
-#pragma unroll
-    for (int u = 0; u < A_UNITS; ++u) {
-        const int row = min(a_row + A_ROWS * u, M - 1 - m0);
-        a_off[u] = (uint32_t)row * (uint32_t)K + 8u * a_ku;
-    }
-    half_t *const a_lds = As0 + a_row * LDS_ROW + 8 * a_ku;  // act-order path
-
-    uint4 a_stage[A_UNITS];
-    uint2 bw[4];  // packed B words of the 4 K steps; refilled in place for the next K tile
-    uint32_t raw_s, raw_z;
-    ColDecode cd[2];
-
-    auto load_a = [&](int kt) {
-#pragma unroll
-        for (int u = 0; u < A_UNITS; ++u) {
-            if (!PERM) {
-                a_stage[u] = *reinterpret_cast<const uint4 *>(a_base + a_off[u] + kt * BK);
-            } else {
-                const int k = kt * BK + 8 * a_ku;
-                const int4 i0 = *reinterpret_cast<const int4 *>(p.perm + k);
-                const int4 i1 = *reinterpret_cast<const int4 *>(p.perm + k + 4);
-                const uint16_t *xs = reinterpret_cast<const uint16_t *>(a_base + (a_off[u] - 8u * a_ku));
-                uint4 a;
-                a.x = (uint32_t)xs[i0.x] | ((uint32_t)xs[i0.y] << 16);
-                a.y = (uint32_t)xs[i0.z] | ((uint32_t)xs[i0.w] << 16);
-                a.z = (uint32_t)xs[i1.x] | ((uint32_t)xs[i1.y] << 16);
-                a.w = (uint32_t)xs[i1.z] | ((uint32_t)xs[i1.w] << 16);
-                a_stage[u] = a;
-            }
-        }
-    };
-    auto store_a = [&](int buf) {
-#pragma unroll
-        for (int u = 0; u < A_UNITS; ++u)
-            *reinterpret_cast<uint4 *>(a_lds + buf * (BM * LDS_ROW) + u * (A_ROWS * LDS_ROW)) = pair_order_u4(a_stage[u]);
-    };
-    auto load_b_step = [&](int kt, int ks) {
-        bw[ks] = *reinterpret_cast<const uint2 *>(bptr + ((size_t)kt * (BK / 8) + 2 * ks) * N);
-    };
-    auto load_group = [&](int g) {
-        raw_s = *reinterpret_cast<const uint32_t *>(sc + (size_t)g * N);
-        raw_z = qz[(size_t)g * (N >> 3)];
-    };
-    // Decode constants from the raw scale / zero words.  Recomputed for every K tile from
-    // that tile's own group (a few integer ops) rather than only at group boundaries:
-    // with no branch around the loads that feed them, every wait in the loop is exact.
-    auto make_cd = [&]() {
-        const uint32_t z2 = raw_z >> (((2 * l32) & 7) * 4);
-        cd[0] = make_col_decode(z2 & 0xFu, raw_s);
-        cd[1] = make_col_decode((z2 >> 4) & 0xFu, raw_s >> 16);
-    };
 
     // K tiles [k_begin, nk) of this split (host-side quotient / remainder, no division here
     // except the one that finds the first group)
@@ -177,8 +120,60 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
     int group = (p.splitk > 1) ? k_begin / tiles_per_group : 0;
     int left_in_group = tiles_per_group - (k_begin - group * tiles_per_group);  // K tiles left in the group
     if constexpr (PERM) {
+        // ---- act-order path: the activations are gathered through registers (x_sorted[k] =
+        // x[perm[k]]) and stored to LDS in pair order, rows padded to 144 bytes; the weights are
+        // decoded in pair order.  Each thread owns A_UNITS 16-byte units (row, 8 k) of the tile;
+        // rows beyond M read row M-1 instead of branching (A row m only feeds output row m and
+        // rows >= M are never stored).
+        uint32_t a_rowoff[A_UNITS];
+        const int a_row = tid >> 3, a_ku = tid & 7;  // unit u of this thread: row a_row + A_ROWS*u, k-unit a_ku
+#pragma unroll
+        for (int u = 0; u < A_UNITS; ++u) a_rowoff[u] = (uint32_t)min(a_row + A_ROWS * u, M - 1 - m0) * (uint32_t)K;
+        half_t *const a_lds = As0 + a_row * LDS_ROW + 8 * a_ku;
+
+        uint4 a_stage[A_UNITS];
+        uint2 bw[4];  // packed B words of the 4 K steps; refilled in place for the next K tile
+        uint32_t raw_s, raw_z;
+        ColDecode cd[2];
+
+        auto load_a = [&](int kt) {
+#pragma unroll
+            for (int u = 0; u < A_UNITS; ++u) {
+                const int k = kt * BK + 8 * a_ku;
+                const int4 i0 = *reinterpret_cast<const int4 *>(p.perm + k);
+                const int4 i1 = *reinterpret_cast<const int4 *>(p.perm + k + 4);
+                const uint16_t *xs = reinterpret_cast<const uint16_t *>(a_base + a_rowoff[u]);
+                uint4 a;
+                a.x = (uint32_t)xs[i0.x] | ((uint32_t)xs[i0.y] << 16);
+                a.y = (uint32_t)xs[i0.z] | ((uint32_t)xs[i0.w] << 16);
+                a.z = (uint32_t)xs[i1.x] | ((uint32_t)xs[i1.y] << 16);
+                a.w = (uint32_t)xs[i1.z] | ((uint32_t)xs[i1.w] << 16);
+                a_stage[u] = a;
+            }
+        };
+        auto store_a = [&](int buf) {
+#pragma unroll
+            for (int u = 0; u < A_UNITS; ++u)
+                *reinterpret_cast<uint4 *>(a_lds + buf * (BM * LDS_ROW) + u * (A_ROWS * LDS_ROW)) = pair_order_u4(a_stage[u]);
+        };
+        auto load_b_step = [&](int kt, int ks) {
+            bw[ks] = *reinterpret_cast<const uint2 *>(bptr + ((size_t)kt * (BK / 8) + 2 * ks) * N);
+        };
+        auto load_group = [&](int g) {
+            raw_s = *reinterpret_cast<const uint32_t *>(sc + (size_t)g * N);
+            raw_z = qz[(size_t)g * (N >> 3)];
+        };
+        // Decode constants from the raw scale / zero words.  Recomputed for every K tile from
+        // that tile's own group (a few integer ops) rather than only at group boundaries:
+        // with no branch around the loads that feed them, every wait in the loop is exact.
+        auto make_cd = [&]() {
+            const uint32_t z2 = raw_z >> (((2 * l32) & 7) * 4);
+            cd[0] = make_col_decode(z2 & 0xFu, raw_s);
+            cd[1] = make_col_decode((z2 >> 4) & 0xFu, raw_s >> 16);
+        };
+
         load_a(k_begin);
-    #pragma unroll
+#pragma unroll
         for (int ks = 0; ks < 4; ++ks) load_b_step(k_begin, ks);
         load_group(group);
         make_cd();
@@ -199,10 +194,10 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
             const bool new_group = (left_in_group == 1);
             load_a(kn);
             load_group(min(group + (new_group ? 1 : 0), last_group));
-    #pragma unroll
+#pragma unroll
             for (int ks = 0; ks < 4; ++ks) {
                 h8_t af[MT];
-    #pragma unroll
+#pragma unroll
                 for (int mt = 0; mt < MT; ++mt) {
                     const int row = wm * (32 * MT) + mt * 32 + l32;
                     af[mt] = *reinterpret_cast<const h8_t *>(As0 + (buf * BM + row) * LDS_ROW + 8 * (2 * ks + lhi));
@@ -214,10 +209,10 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
                     load_b_step(kn, ks + 1);
                 else
                     load_b_step(kn2, 0);
-    #pragma unroll
+#pragma unroll
                 for (int mt = 0; mt < MT; ++mt) acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt], bf[0], acc[mt][0], 0, 0, 0);
                 bf[0] = decode_word_h8(nw.x, cd[0]);
-    #pragma unroll
+#pragma unroll
                 for (int mt = 0; mt < MT; ++mt) acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt], bf[1], acc[mt][1], 0, 0, 0);
                 bf[1] = decode_word_h8(nw.y, cd[1]);
             }
