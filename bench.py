@@ -17,7 +17,8 @@ Also reported on the same line:
                 the 8 TB/s HBM peak
   cpu_baseline  the PyTorch CPU dequantise-then-fp32-matmul path (oracle/torch_cpu.py)
                 on the host cores for 1 of the 32 layers, extrapolated to a token
-  extra         per-operator decode timings and prefill TFLOP/s (M = 128 / 512 / 2048)
+  extra         per-operator decode timings, batched and prefill TFLOP/s (M = 16 ... 8192) and
+                the vendor library's dense fp16 GEMM on the M = 2048 shapes
 
 Other workloads (--workload llama7b | llama13b | llama30b): a full random-init decoder of
 that shape (embedding, RMSNorm, fused QKV + rotary into a preallocated KV cache, torch
@@ -359,11 +360,11 @@ def main():
         per_op("decode M=1 o_proj", lambda L: o_op(x1, L), wo + 4 * HIDDEN, 2 * HIDDEN * HIDDEN)
         per_op("decode M=1 gate/up+silu*mul", lambda L: gateup_op(x1, L), gu_bytes, 4 * HIDDEN * INTER)
         per_op("decode M=1 down_proj", lambda L: down_op(h1, L), wd + 2 * INTER + 2 * HIDDEN, 2 * HIDDEN * INTER)
-        for m in (16, 64, 128, 256, 512, 2048):
+        for m in (16, 64, 128, 256, 512, 2048, 8192):
             xm = torch.randn((1, m, HIDDEN), device=dev, generator=gen).half()
             hm = torch.randn((m, INTER), device=dev, generator=gen).half()
             posm = torch.arange(m, device=dev, dtype=torch.int32).unsqueeze(0)
-            ns = 8 if m <= 128 else 4
+            ns = 8 if m <= 128 else (4 if m <= 2048 else 2)
             per_op(f"M={m} qkv+rotary", lambda L: qkv_op(xm, L, posm), wq + 2 * m * HIDDEN + 6 * m * HIDDEN,
                    2 * m * HIDDEN * 3 * HIDDEN, nsets=ns, reps=5)
             per_op(f"M={m} gate/up+silu*mul", lambda L: gateup_op(xm, L), 2 * wg + 2 * m * HIDDEN + 2 * m * INTER,
