@@ -33,8 +33,9 @@
 //             the two waves at the same lane and register, and are swapped through LDS.
 //   SiLU*mul: a pair takes the SAME 64 columns of the gate and of the up matrix (the
 //             output tile is half as wide); up is handed over through LDS.
-// blockIdx is remapped so each XCD (blockIdx % 8) owns a contiguous range of tiles:
-// the row tiles that share a weight panel then share one L2.
+// blockIdx is remapped so each XCD (blockIdx % 8) owns a contiguous range of tiles, ordered
+// so that the workgroups resident on it at one time share both activation tiles and weight
+// panels in its L2.
 #include "gptq4_internal.h"
 
 namespace {
@@ -83,13 +84,24 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
     const int M = p.M, K = p.K, N = p.N;
     const int tiles_m = (M + BM - 1) / BM;
 
-    // XCD-contiguous logical tile index, row tiles fastest
+    // XCD-contiguous logical tile index: workgroups that run at the same time on one XCD (one
+    // L2) have consecutive logical indices.  These walk GROUP_M row tiles, then move to the
+    // next column panel, and only after the last panel to the next GROUP_M row tiles: the
+    // ~64 workgroups resident on an XCD then cover about 8 row tiles x 8 column panels, so
+    // every activation tile and every weight panel they stream is shared by 8 of them in
+    // the L2 (row tiles fastest over all of M left a weight panel shared by many but an
+    // activation tile by two, and the activation tiles are the larger stream).
+    constexpr int GROUP_M = 8;
+    const int tiles_n = N / BN;
     const int total = gridDim.x;
     const int per = total >> 3, rem = total & 7;
     const int xcd = blockIdx.x & 7;
     const int logical = xcd * per + (xcd < rem ? xcd : rem) + (blockIdx.x >> 3);
-    const int tile_n = logical / tiles_m;
-    const int tile_m = logical - tile_n * tiles_m;
+    const int band = logical / (GROUP_M * tiles_n);  // band of GROUP_M row tiles
+    const int in_band = logical - band * (GROUP_M * tiles_n);
+    const int band_rows = min(GROUP_M, tiles_m - band * GROUP_M);
+    const int tile_n = in_band / band_rows;
+    const int tile_m = band * GROUP_M + (in_band - tile_n * band_rows);
     const int m0 = tile_m * BM;
     const int n0 = tile_n * BN;
 
