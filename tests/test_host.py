@@ -185,3 +185,25 @@ def test_product_code_never_touches_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".cpp")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in text.lower() or f == "never", f"{f} mentions the oracle"
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """Every box has one GPU: `bench.py --gpus N` with N > 1 must say so and exit non-zero
+    without touching a device."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "one GPU" in (r.stderr + r.stdout) or "single GPU" in (r.stderr + r.stdout) or "--gpus 1" in (r.stderr + r.stdout)
+
+
+def test_mid_m_plan_is_declared_and_tunable():
+    """The launch-plan hooks exist with the documented arity (no compute is launched)."""
+    from gptq_triton_amd import _lib
+    lib = _lib.load()
+    for args in ((0, 0, 0), (2, 1, 3), (1, 0, 0)):
+        lib.gptq4_set_midm_tuning(*args)
+    # the workspace query covers whichever kernel the plans pick for a mid-sized call
+    assert lib.gptq4_workspace_bytes(_lib.OP_MATMUL, 64, 4096, 4096) >= _lib.WS_COUNTER_BYTES
+    assert lib.gptq4_workspace_bytes(_lib.OP_QKV_ROTARY, 128, 4096, 12288) >= _lib.WS_COUNTER_BYTES
