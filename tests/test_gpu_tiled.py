@@ -103,3 +103,19 @@ def test_hand_over_between_the_mid_m_and_the_tiled_kernel():
     big = torch.maximum(ya.abs(), yb[:768].abs()).float().cpu().numpy().astype(np.float16)
     ulp = torch.from_numpy(np.spacing(big).astype(np.float32)).cuda()
     assert bool(((ya.float() - yb[:768].float()).abs() <= ulp + 1e-4).all())
+
+
+def test_tiled_one_hot_rows_reproduce_weight_rows(forced_tiled):
+    """x = e_k picks row k of the dequantised weight: a single product, so the tiled kernel's own
+    in-register decode (natural k order) must give the canonical fp16 weight bit for bit, for
+    every nibble position and both column halves of a word pair."""
+    k, n, g = 1024, 512, 128
+    L = O.make_layer(k, n, g, seed=19)
+    D = to_dev(L)
+    rows = np.array(list(range(0, 16)) + [63, 64, 127, 128, 255, 256, 511, 512, 700, 767, 768, 1000, 1016, 1017, 1022, 1023]
+                    + list(range(320, 328)))
+    x = np.zeros((len(rows), k), dtype=np.float16)
+    x[np.arange(len(rows)), rows] = 1.0
+    y = gptq().matmul4(g, torch.from_numpy(x).cuda(), D["qweight"], D["scales"], D["qzeros"])
+    W = O.dequant_fp16(L["qweight"], L["qzeros"], L["scales"], g)
+    assert (y.cpu().numpy().view(np.uint16) == W[rows].view(np.uint16)).all()
