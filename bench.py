@@ -17,8 +17,10 @@ Also reported on the same line:
                 the 8 TB/s HBM peak
   cpu_baseline  the PyTorch CPU dequantise-then-fp32-matmul path (oracle/torch_cpu.py)
                 on the host cores for 1 of the 32 layers, extrapolated to a token
-  extra         per-operator decode timings, batched and prefill TFLOP/s (M = 16 ... 8192) and
-                the vendor library's dense fp16 GEMM on the M = 2048 shapes
+  extra         per-operator decode timings ("hot" = one layer's weights over and over, served by
+                the Infinity Cache; everything else streams from HBM), batched and prefill
+                TFLOP/s (M = 16 ... 8192) and the vendor library's dense fp16 GEMM on the
+                M = 2048 shapes
 
 Other workloads (--workload llama7b | llama13b | llama30b): a full random-init decoder of
 that shape (embedding, RMSNorm, fused QKV + rotary into a preallocated KV cache, torch
@@ -360,6 +362,18 @@ def main():
         per_op("decode M=1 o_proj", lambda L: o_op(x1, L), wo + 4 * HIDDEN, 2 * HIDDEN * HIDDEN)
         per_op("decode M=1 gate/up+silu*mul", lambda L: gateup_op(x1, L), gu_bytes, 4 * HIDDEN * INTER)
         per_op("decode M=1 down_proj", lambda L: down_op(h1, L), wd + 2 * INTER + 2 * HIDDEN, 2 * HIDDEN * INTER)
+        # "hot": the same launches on ONE layer's weights over and over, so that they come out of the
+        # 256 MB Infinity Cache instead of HBM.  Not an HBM figure; it shows what the memory side costs.
+        def per_op_hot(name, fn, nbytes, flops, reps=10):
+            g, _ = capture(lambda: [fn(layers[0]) for _ in range(LAYERS)])
+            us = statistics.median(time_graph(g, reps)) * 1e3 / LAYERS
+            extra[name] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1), "TFLOPs": round(flops / us / 1e6, 2)}
+            log(f"  {name:34s} {us:9.2f} us  {nbytes / us / 1e3:8.0f} GB/s  {flops / us / 1e6:8.1f} TFLOP/s")
+            del g
+        per_op_hot("hot M=1 qkv+rotary", lambda L: qkv_op(x1, L, pos1), wq + 2 * HIDDEN + 6 * HIDDEN, 2 * HIDDEN * 3 * HIDDEN)
+        per_op_hot("hot M=1 o_proj", lambda L: o_op(x1, L), wo + 4 * HIDDEN, 2 * HIDDEN * HIDDEN)
+        per_op_hot("hot M=1 gate/up+silu*mul", lambda L: gateup_op(x1, L), gu_bytes, 4 * HIDDEN * INTER)
+        per_op_hot("hot M=1 down_proj", lambda L: down_op(h1, L), wd + 2 * INTER + 2 * HIDDEN, 2 * HIDDEN * INTER)
         for m in (16, 64, 128, 256, 512, 2048, 8192):
             xm = torch.randn((1, m, HIDDEN), device=dev, generator=gen).half()
             hm = torch.randn((m, INTER), device=dev, generator=gen).half()
