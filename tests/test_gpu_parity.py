@@ -355,3 +355,30 @@ def test_tiled_kernel_gathers_act_order_rows_itself_when_asked():
     assert rc == 0
     ref = O.quant_matmul_ref(x, L["qweight"], L["qzeros"], L["scales"], g, g_idx=L["g_idx"])
     assert_close(y.cpu().numpy(), ref, "tiled kernel, in-kernel act-order gather")
+
+
+def test_empty_inputs_give_empty_outputs():
+    """Zero rows: every functional returns a tensor of the right shape and launches nothing;
+    the C entry points themselves reject M < 1."""
+    from gptq_triton_amd import _lib
+    k, n, g = 256, 512, 128
+    L = O.make_layer(k, n, g, seed=900)
+    D = to_dev(L)
+    G = gptq()
+    x0 = torch.empty((0, k), dtype=torch.float16, device="cuda")
+    assert G.matmul4(g, x0, D["qweight"], D["scales"], D["qzeros"]).shape == (0, n)
+    assert G.matmul4(g, x0.view(2, 0, k), D["qweight"], D["scales"], D["qzeros"]).shape == (2, 0, n)
+    assert G.llama_mlp_4(g, x0, D["qweight"], D["scales"], D["qzeros"], D["qweight"], D["scales"], D["qzeros"]).shape == (0, n)
+    Lq = O.make_layer(256, 768, g, seed=901)
+    Dq = to_dev(Lq)
+    cos, sin = G.RotaryTable(128, 64).get(torch.device("cuda"), 64)
+    pos0 = torch.empty((1, 0), dtype=torch.int64, device="cuda")
+    q, kk, vv = G.qkv_rotary(g, x0.view(1, 0, k), Dq["qweight"], Dq["scales"], Dq["qzeros"], pos0, cos, sin, 2, 128)
+    assert q.shape == kk.shape == vv.shape == (1, 2, 0, 128)
+    lib = _lib.load()
+    ws = _lib.workspace(x0.device, lib.gptq4_workspace_bytes(_lib.OP_MATMUL, 1, k, n))
+    y = torch.empty((1, n), dtype=torch.float16, device="cuda")
+    x1 = torch.zeros((1, k), dtype=torch.float16, device="cuda")
+    rc = lib.gptq4_matmul(x1.data_ptr(), D["qweight"].data_ptr(), D["qzeros"].data_ptr(), D["scales"].data_ptr(), None, None,
+                          y.data_ptr(), 0, k, n, g, ws.data_ptr(), ws.numel(), _lib.current_stream(x0.device))
+    assert rc < 0 and b"shape" in lib.gptq4_strerror(rc).lower()

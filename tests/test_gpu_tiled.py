@@ -119,3 +119,37 @@ def test_tiled_one_hot_rows_reproduce_weight_rows(forced_tiled):
     y = gptq().matmul4(g, torch.from_numpy(x).cuda(), D["qweight"], D["scales"], D["qzeros"])
     W = O.dequant_fp16(L["qweight"], L["qzeros"], L["scales"], g)
     assert (y.cpu().numpy().view(np.uint16) == W[rows].view(np.uint16)).all()
+
+
+@pytest.mark.parametrize("m", [64, 300, 1100])
+def test_graph_replays_equal_eager_launches(m):
+    """The K-sliced and tiled kernels under HIP-graph capture (split-K counters included): every replay,
+    with new input values and eager launches in between, gives the bits of an eager call."""
+    k, n, g = 2048, 1024, 128
+    L, L2 = O.make_layer(k, n, g, seed=70), O.make_layer(k, n, g, seed=71)
+    D, D2 = to_dev(L), to_dev(L2)
+    G = gptq()
+    x = torch.from_numpy(O.make_x(m, k, seed=72)).cuda()
+
+    def ops():
+        return (G.matmul4(g, x, D["qweight"], D["scales"], D["qzeros"]),
+                G.llama_mlp_4(g, x, D["qweight"], D["scales"], D["qzeros"], D2["qweight"], D2["scales"], D2["qzeros"]))
+
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        ops()                                   # sizes this stream's workspace outside the capture
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=s):
+        y, h = ops()
+    for i in range(4):
+        x.copy_(torch.from_numpy(O.make_x(m, k, seed=80 + i)).cuda())
+        graph.replay()
+        torch.cuda.synchronize()
+        y_e, h_e = ops()
+        assert torch.equal(y, y_e) and torch.equal(h, h_e), f"replay {i}"
+    ref = O.quant_matmul_ref(x.cpu().numpy(), L["qweight"], L["qzeros"], L["scales"], g)
+    ok, max_abs, _ = O.within_tolerance(y.cpu().numpy(), ref)
+    assert ok, max_abs
