@@ -339,7 +339,7 @@ def main():
                 "frac": round(gu_gbs / HBM_PEAK_GBS, 4),
                 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
                 # `bench.py --traffic-probe`, scaled by a 256 MiB copy (x2.000 / x1.000)
-                "traffic": 50_651_000 + 1_286_000,
+                "traffic": 50_601_000 + 1_286_000,
                 "kernel": "gptq4_gemv_kernel<SILU_MUL> (gate/up GEMV, M=1, K=4096, I=11008, g=128)",
                 "bytes_per_launch": gu_bytes, "avg_launch_us": round(gu_us, 2)}
     log(f"gate/up GEMV: {gu_us:.2f} us/launch, {gu_gbs:.0f} GB/s = {100 * gu_gbs / HBM_PEAK_GBS:.1f}% of HBM peak")

@@ -145,7 +145,7 @@ void gptq4_set_midm_tuning(int mode, int mt, int splitk) {
 
 void gptq4_set_gemv_tuning(int mode, int depth, int waves, int waves_per_cu) {
     g_gemv_tuning.mode = (mode >= 0 && mode <= 2) ? mode : 1;
-    g_gemv_tuning.depth = (depth == 2 || depth == 3) ? depth : 0;
+    g_gemv_tuning.depth = (depth >= 1 && depth <= 3) ? depth : 0;
     g_gemv_tuning.waves = (waves == 4 || waves == 8 || waves == 16) ? waves : 0;
     g_gemv_tuning.waves_per_cu = (waves_per_cu >= 4 && waves_per_cu <= 32) ? waves_per_cu : 0;
 }

@@ -168,7 +168,7 @@ void gptq4_set_midm_tuning(int mode, int mt, int splitk);
 
 /* Same for the balanced decode GEMV (M <= 4): mode 0 = never use it, 1 = where it is the
  * faster kernel (one row, SiLU*mul epilogue), 2 = wherever it can run; units in
- * flight per wave (2, 3), waves per workgroup (4, 8, 16), waves per CU (4..32), 0 =
+ * flight per wave (1..3), waves per workgroup (4, 8, 16), waves per CU (4..32), 0 =
  * automatic. */
 void gptq4_set_gemv_tuning(int mode, int depth, int waves, int waves_per_cu);
 

@@ -13,7 +13,7 @@ from test_gpu_parity import assert_close, gptq
 pytestmark = pytest.mark.gpu
 
 # (units in flight, waves per workgroup, waves per CU); 0 = automatic
-CONFIGS = [(0, 0, 0), (3, 8, 16), (2, 16, 16), (2, 8, 4)]
+CONFIGS = [(0, 0, 0), (3, 8, 16), (2, 16, 16), (2, 8, 4), (1, 8, 8), (2, 4, 8)]
 
 
 @pytest.fixture(params=CONFIGS, ids=lambda c: "d%d_w%d_cu%d" % c)
