@@ -207,3 +207,14 @@ def test_mid_m_plan_is_declared_and_tunable():
     # the workspace query covers whichever kernel the plans pick for a mid-sized call
     assert lib.gptq4_workspace_bytes(_lib.OP_MATMUL, 64, 4096, 4096) >= _lib.WS_COUNTER_BYTES
     assert lib.gptq4_workspace_bytes(_lib.OP_QKV_ROTARY, 128, 4096, 12288) >= _lib.WS_COUNTER_BYTES
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    """No CPU fallback: with the shared object absent, loading raises and names the build command."""
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", tmp_path / "libgptq4.so")
+    with pytest.raises(_lib.LibraryMissing, match="build"):
+        _lib.load()
+    layer = G.QuantLinear(4, 128, 256, 256, bias=False)
+    with pytest.raises((_lib.LibraryMissing, RuntimeError, AssertionError)):
+        layer(torch.zeros((1, 256), dtype=torch.float16))
