@@ -4,6 +4,7 @@
 #include "../../include/gptq4.h"
 
 #include "gptq4_internal.h"
+#include "gptq4_norm.h"
 
 namespace {
 
@@ -44,6 +45,23 @@ int setup_skinny(MatmulArgs &a, const SkinnyPlan &pl, int nmat, void *workspace,
 // M <= 16: the balanced GEMV where its plan says so (by default the one-row gate/up pair),
 // the split-K kernel otherwise.
 int run_small(int epi, MatmulArgs &a, int nmat, void *workspace, size_t workspace_bytes, hipStream_t s) {
+    if (a.nrm_weight != nullptr) {
+        // the variants that normalise their own input exist for the automatic launch shapes only
+        if (a.M <= GEMV_MAX_M) {
+            const GemvPlan gp = gemv_plan(epi, a.M, a.N, a.K, true);
+            if (gp.ok) {
+                if (workspace == nullptr || workspace_bytes < GPTQ4_WS_COUNTER_BYTES + gemv_partial_bytes(gp, a.M, epi))
+                    return -GPTQ4_E_WORKSPACE;
+                a.counters = reinterpret_cast<int *>(workspace);
+                a.partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_COUNTER_BYTES);
+                return launch_gemv(epi, a, gp, s);
+            }
+        }
+        const SkinnyPlan pl = skinny_plan(epi, a.N, a.K, true);
+        int rc = setup_skinny(a, pl, nmat, workspace, workspace_bytes);
+        if (rc) return rc;
+        return launch_skinny(epi, a, pl, s);
+    }
     if (a.M <= GEMV_MAX_M) {
         const GemvPlan pl = gemv_plan(epi, a.M, a.N, a.K);
         if (pl.ok) {
@@ -73,6 +91,21 @@ int setup_gemm(MatmulArgs &a, const GemmPlan &pl, void *workspace, size_t worksp
         a.counters = reinterpret_cast<int *>(workspace);
         a.partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_COUNTER_BYTES);
     }
+    return 0;
+}
+
+// Fused residual add + RMSNorm of the input: decode-sized calls only (the workgroups of the small-M
+// kernel each normalise all M rows into their LDS), unpermuted rows, and a sum_out that no
+// workgroup still reads from.
+int setup_norm(MatmulArgs &a, const void *delta, const void *norm_weight, void *sum_out, float eps) {
+    if (!norm_weight || (delta && !sum_out)) return -GPTQ4_E_NULL;
+    if (a.M > NORM_MAX_M || a.K > NORM_MAX_H || a.perm != nullptr || !(eps >= 0.f)) return -GPTQ4_E_SHAPE;
+    if (delta && (sum_out == static_cast<const void *>(a.x) || sum_out == delta)) return -GPTQ4_E_SHAPE;
+    if (misaligned16(norm_weight) || (delta && (misaligned16(delta) || misaligned16(sum_out)))) return -GPTQ4_E_ALIGN;
+    a.nrm_delta = reinterpret_cast<const half_t *>(delta);
+    a.nrm_weight = reinterpret_cast<const half_t *>(norm_weight);
+    a.nrm_sum_out = delta ? reinterpret_cast<half_t *>(sum_out) : nullptr;
+    a.nrm_eps = eps;
     return 0;
 }
 
@@ -167,8 +200,11 @@ size_t gptq4_workspace_bytes(int op, int M, int K, int N) {
         size_t need = partial_bytes(SKINNY_MAX_SPLITK, M, cols);
         if (M <= GEMV_MAX_M && (K % 128) == 0 && (N % 256) == 0) {
             const int epi = (op == GPTQ4_OP_MLP_GATEUP) ? EPI_SILU_MUL : (op == GPTQ4_OP_QKV_ROTARY ? EPI_ROPE : EPI_PLAIN);
-            const GemvPlan pl = gemv_plan(epi, M, N, K);
-            if (pl.ok && gemv_partial_bytes(pl, M, epi) > need) need = gemv_partial_bytes(pl, M, epi);
+            // whichever launch shape runs: the tuned one, or the automatic one of the self-normalising variant
+            for (int norm = 0; norm < 2; ++norm) {
+                const GemvPlan pl = gemv_plan(epi, M, N, K, norm != 0);
+                if (pl.ok && gemv_partial_bytes(pl, M, epi) > need) need = gemv_partial_bytes(pl, M, epi);
+            }
         }
         bytes += need;
     } else if ((K % 64) == 0) {
@@ -229,10 +265,11 @@ int gptq4_matmul(const void *x, const int32_t *qweight, const int32_t *qzeros, c
     return run_tiled(EPI_PLAIN, a, workspace, workspace_bytes, s);
 }
 
-int gptq4_mlp_gateup(const void *x, const int32_t *gate_qweight, const int32_t *gate_qzeros,
-                     const void *gate_scales, const int32_t *up_qweight, const int32_t *up_qzeros,
-                     const void *up_scales, const int32_t *perm, void *h, int M, int K, int I, int groupsize,
-                     void *workspace, size_t workspace_bytes, void *stream) {
+static int mlp_gateup_impl(const void *x, const void *delta, const void *norm_weight, void *sum_out, float eps,
+                           const int32_t *gate_qweight, const int32_t *gate_qzeros, const void *gate_scales,
+                           const int32_t *up_qweight, const int32_t *up_qzeros, const void *up_scales,
+                           const int32_t *perm, void *h, int M, int K, int I, int groupsize, void *workspace,
+                           size_t workspace_bytes, void *stream, bool norm) {
     if (!x || !gate_qweight || !gate_qzeros || !gate_scales || !up_qweight || !up_qzeros || !up_scales || !h)
         return -GPTQ4_E_NULL;
     if (M < 1) return -GPTQ4_E_SHAPE;
@@ -253,11 +290,31 @@ int gptq4_mlp_gateup(const void *x, const int32_t *gate_qweight, const int32_t *
     a.K = K;
     a.N = I;
     a.groupsize = groupsize;
+    if (norm) {
+        rc = setup_norm(a, delta, norm_weight, sum_out, eps);
+        if (rc) return rc;
+    }
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     if (M <= SKINNY_MAX_M) {
         return run_small(EPI_SILU_MUL, a, 2, workspace, workspace_bytes, s);
     }
     return run_tiled(EPI_SILU_MUL, a, workspace, workspace_bytes, s);
+}
+
+int gptq4_mlp_gateup(const void *x, const int32_t *gate_qweight, const int32_t *gate_qzeros,
+                     const void *gate_scales, const int32_t *up_qweight, const int32_t *up_qzeros,
+                     const void *up_scales, const int32_t *perm, void *h, int M, int K, int I, int groupsize,
+                     void *workspace, size_t workspace_bytes, void *stream) {
+    return mlp_gateup_impl(x, nullptr, nullptr, nullptr, 0.f, gate_qweight, gate_qzeros, gate_scales, up_qweight, up_qzeros,
+                           up_scales, perm, h, M, K, I, groupsize, workspace, workspace_bytes, stream, false);
+}
+
+int gptq4_norm_mlp_gateup(const void *x, const void *delta, const void *norm_weight, float eps, void *sum_out,
+                          const int32_t *gate_qweight, const int32_t *gate_qzeros, const void *gate_scales,
+                          const int32_t *up_qweight, const int32_t *up_qzeros, const void *up_scales, void *h, int M,
+                          int K, int I, int groupsize, void *workspace, size_t workspace_bytes, void *stream) {
+    return mlp_gateup_impl(x, delta, norm_weight, sum_out, eps, gate_qweight, gate_qzeros, gate_scales, up_qweight,
+                           up_qzeros, up_scales, nullptr, h, M, K, I, groupsize, workspace, workspace_bytes, stream, true);
 }
 
 int gptq4_rope_table(float *cos_out, float *sin_out, int max_pos, int D, float base, void *stream) {
@@ -266,11 +323,11 @@ int gptq4_rope_table(float *cos_out, float *sin_out, int max_pos, int D, float b
     return launch_rope_table(cos_out, sin_out, max_pos, D, base, reinterpret_cast<hipStream_t>(stream));
 }
 
-int gptq4_qkv_rotary(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
-                     const int32_t *perm, const int32_t *position_ids, const float *cos_table,
-                     const float *sin_table, int max_pos, void *q, void *k, void *v, int B, int S, int H, int D,
-                     int K, int groupsize, int kv_capacity, int kv_offset, void *workspace,
-                     size_t workspace_bytes, void *stream) {
+static int qkv_rotary_impl(const void *x, const void *delta, const void *norm_weight, void *sum_out, float eps,
+                           const int32_t *qweight, const int32_t *qzeros, const void *scales, const int32_t *perm,
+                           const int32_t *position_ids, const float *cos_table, const float *sin_table, int max_pos,
+                           void *q, void *k, void *v, int B, int S, int H, int D, int K, int groupsize, int kv_capacity,
+                           int kv_offset, void *workspace, size_t workspace_bytes, void *stream, bool norm) {
     if (!x || !qweight || !qzeros || !scales || !position_ids || !cos_table || !sin_table || !q || !k || !v)
         return -GPTQ4_E_NULL;
     if (B < 1 || S < 1 || H < 1 || D != 128 || max_pos < 1) return -GPTQ4_E_SHAPE;
@@ -310,11 +367,35 @@ int gptq4_qkv_rotary(const void *x, const int32_t *qweight, const int32_t *qzero
         const uint64_t err = magic * (uint64_t)S - (1ull << 32);
         if (magic < (1ull << 32) && (uint64_t)(a.M - 1) * err < (1ull << 32)) a.rope.s_magic = (uint32_t)magic;
     }
+    if (norm) {
+        rc = setup_norm(a, delta, norm_weight, sum_out, eps);
+        if (rc) return rc;
+    }
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     if (a.M <= SKINNY_MAX_M) {
         return run_small(EPI_ROPE, a, 1, workspace, workspace_bytes, s);
     }
     return run_tiled(EPI_ROPE, a, workspace, workspace_bytes, s);
+}
+
+int gptq4_qkv_rotary(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
+                     const int32_t *perm, const int32_t *position_ids, const float *cos_table,
+                     const float *sin_table, int max_pos, void *q, void *k, void *v, int B, int S, int H, int D,
+                     int K, int groupsize, int kv_capacity, int kv_offset, void *workspace,
+                     size_t workspace_bytes, void *stream) {
+    return qkv_rotary_impl(x, nullptr, nullptr, nullptr, 0.f, qweight, qzeros, scales, perm, position_ids, cos_table,
+                           sin_table, max_pos, q, k, v, B, S, H, D, K, groupsize, kv_capacity, kv_offset, workspace,
+                           workspace_bytes, stream, false);
+}
+
+int gptq4_norm_qkv_rotary(const void *x, const void *delta, const void *norm_weight, float eps, void *sum_out,
+                          const int32_t *qweight, const int32_t *qzeros, const void *scales,
+                          const int32_t *position_ids, const float *cos_table, const float *sin_table, int max_pos,
+                          void *q, void *k, void *v, int B, int S, int H, int D, int K, int groupsize, int kv_capacity,
+                          int kv_offset, void *workspace, size_t workspace_bytes, void *stream) {
+    return qkv_rotary_impl(x, delta, norm_weight, sum_out, eps, qweight, qzeros, scales, nullptr, position_ids, cos_table,
+                           sin_table, max_pos, q, k, v, B, S, H, D, K, groupsize, kv_capacity, kv_offset, workspace,
+                           workspace_bytes, stream, true);
 }
 
 int gptq4_rmsnorm(const void *x, const void *weight, void *y, int M, int H, float eps, void *stream) {

@@ -2,20 +2,16 @@
 // whole step is a short chain of HIP launches: RMSNorm and single-query attention over a
 // preallocated KV cache.  Both are HBM/L2-bound elementwise-and-reduce kernels.
 #include "gptq4_internal.h"
+#include "gptq4_norm.h"
 
 namespace {
-
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o);
-    return v;
-}
 
 // y[row] = weight * fp16( s[row] * rsqrt(mean(s[row]^2) + eps) ) with s = x (ADD false) or
 // s = fp16(x + delta), also written to sum_out (ADD true: the residual add that precedes
 // every RMSNorm of a decoder layer).  Statistics and the normalisation in fp32, rounded to
 // fp16, then an fp16 multiply by the weight - the rounding order of the LLaMA RMSNorm
-// module.  One workgroup per row, H % 8 == 0; sum_out may alias x.
+// module.  One workgroup per row, H % 8 == 0; sum_out may alias x.  The arithmetic lives in
+// gptq4_norm.h, shared with the matmul kernels that normalise their own input.
 template <bool ADD>
 __global__ __launch_bounds__(256) void gptq4_rmsnorm_kernel(const half_t *x, const half_t *delta, const half_t *__restrict__ w,
                                                             half_t *sum_out, half_t *__restrict__ y, int H, float eps) {
@@ -28,44 +24,21 @@ __global__ __launch_bounds__(256) void gptq4_rmsnorm_kernel(const half_t *x, con
     uint4 *sr = reinterpret_cast<uint4 *>(sum_out + (ADD ? row : 0));
     uint4 *yr = reinterpret_cast<uint4 *>(y + row);
     const int chunks = H >> 3;
-    constexpr int KEEP = 4;  // chunks per thread held in registers (covers H <= 8192); beyond that re-read
+    constexpr int KEEP = NORM_KEEP;  // chunks per thread held in registers (covers H <= 8192); beyond that re-read
     uint4 held[KEEP];
     float ss = 0.f;
     auto take = [&](int c) {
-        uint4 v = xr[c];
-        if (ADD) {
-            const uint4 d = dr[c];
-            v.x = as_u32(as_h2(v.x) + as_h2(d.x));
-            v.y = as_u32(as_h2(v.y) + as_h2(d.y));
-            v.z = as_u32(as_h2(v.z) + as_h2(d.z));
-            v.w = as_u32(as_h2(v.w) + as_h2(d.w));
-            sr[c] = v;
-        }
-        const h2_t p[4] = {as_h2(v.x), as_h2(v.y), as_h2(v.z), as_h2(v.w)};
-#pragma unroll
-        for (int i = 0; i < 4; ++i) ss += (float)p[i].x * (float)p[i].x + (float)p[i].y * (float)p[i].y;
+        const uint4 v0 = xr[c];
+        const uint4 v = norm_take<ADD>(v0, ADD ? dr[c] : v0, ss);
+        if (ADD) sr[c] = v;
         return v;
     };
 #pragma unroll
     for (int n = 0; n < KEEP; ++n)
         if (tid + 256 * n < chunks) held[n] = take(tid + 256 * n);
     for (int c = tid + 256 * KEEP; c < chunks; c += 256) take(c);
-    ss = wave_sum(ss);
-    if ((tid & 63) == 0) part[tid >> 6] = ss;
-    __syncthreads();
-    const float inv = rsqrtf((part[0] + part[1] + part[2] + part[3]) / (float)H + eps);
-    auto put = [&](int c, uint4 v) {
-        const uint4 g = wr[c];
-        const uint32_t vi[4] = {v.x, v.y, v.z, v.w}, gi[4] = {g.x, g.y, g.z, g.w};
-        uint32_t o[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const h2_t p = as_h2(vi[i]);
-            const h2_t nrm = {(half_t)((float)p.x * inv), (half_t)((float)p.y * inv)};
-            o[i] = as_u32(as_h2(gi[i]) * nrm);
-        }
-        yr[c] = make_uint4(o[0], o[1], o[2], o[3]);
-    };
+    const float inv = norm_inv_rms(ss, part, tid, H, eps);
+    auto put = [&](int c, uint4 v) { yr[c] = norm_put(v, wr[c], inv); };
 #pragma unroll
     for (int n = 0; n < KEEP; ++n)
         if (tid + 256 * n < chunks) put(tid + 256 * n, held[n]);

@@ -26,6 +26,7 @@
 // redirected to the first bytes of the matrix (one cache line) and never used, so the
 // compiler's wait counters stay exact and DEPTH units are really in flight.
 #include "gptq4_internal.h"
+#include "gptq4_norm.h"
 
 #ifdef GPTQ4_PHASE_TIMERS
 #define WSTAMP(i)                                                                                          \
@@ -64,8 +65,13 @@ struct UnitRegs {
 
 constexpr int XROW = 17;  // 16-byte chunks per (unit, row) of the x slice: 16 + 1 pad
 
-template <int EPI, int DEPTH, bool PERM, int NW>
+// NORM (2 or 4 chunks of 8 values per thread cover a row; 0 = off): p.x is the residual stream; the
+// workgroup first writes weight * rmsnorm(x (+ delta)) of all rows to LDS (gptq4_norm.h; workgroup 0
+// also writes the sums out) and its waves stage their x slices from there instead of from memory.
+template <int EPI, int DEPTH, bool PERM, int NW, int NORM>
 __global__ __launch_bounds__(64 * NW) void gptq4_gemv_kernel(MatmulArgs p) {
+    static_assert(!NORM || (NW == 4 && !PERM), "the fused norm is written for 256 threads and unpermuted rows");
+    __shared__ float norm_part[NORM ? NORM_MAX_M * 4 : 1];
     constexpr int NV = (EPI == EPI_PLAIN) ? 1 : 2;
     constexpr int W = 2;
     constexpr int SW = 32;
@@ -85,7 +91,7 @@ __global__ __launch_bounds__(64 * NW) void gptq4_gemv_kernel(MatmulArgs p) {
     const int v = blockIdx.x * NW + wave;  // this wave's rank in the grid
     const int u0 = v * q + min(v, r);      // first unit
     const int n = q + (v < r ? 1 : 0);     // units of this wave
-    if (n == 0) return;                    // (waves never wait for each other)
+    if (n == 0 && !NORM) return;           // (waves never wait for each other; with NORM they share the row first)
     WSTAMP(0);
     const int t0 = div_magic(u0, NB, p.nb_magic);
     const int bs = u0 - t0 * NB;  // first batch inside tile t0
@@ -109,8 +115,16 @@ __global__ __launch_bounds__(64 * NW) void gptq4_gemv_kernel(MatmulArgs p) {
         off = ok ? (uint32_t)(rr * K + batch_of(i) * 128 + 8 * j) * 2u : OFF_RANGE;
         return ok;
     };
+    uint4 *const xs = smem + NW * p.lds_wave_chunks;  // NORM: [M][K / 8] normalised activations, behind the slices
+    NormLoads<NORM ? NORM : 1> nl;
+    if (NORM) {
+        if (p.nrm_delta != nullptr)
+            norm_issue_row0<true>(p.x, p.nrm_delta, p.nrm_weight, K, (int)threadIdx.x, nl);
+        else
+            norm_issue_row0<false>(p.x, p.x, p.nrm_weight, K, (int)threadIdx.x, nl);
+    }
     u32x4_t xv0, xv1;
-    if (!PERM) {
+    if (!PERM && !NORM) {
         int dst;
         uint32_t off;
         x_chunk(lane, dst, off);
@@ -165,6 +179,19 @@ __global__ __launch_bounds__(64 * NW) void gptq4_gemv_kernel(MatmulArgs p) {
     for (int d = 0; d < DEPTH; ++d) load_unit(ring[d], d);
     WSTAMP(1);
 
+    if (NORM) {
+        half_t *const sums = (blockIdx.x == 0) ? p.nrm_sum_out : nullptr;
+        if (p.nrm_delta != nullptr)
+            norm_rows_to_lds<true>(p.x, p.nrm_delta, p.nrm_weight, sums, xs, norm_part, M, K, p.nrm_eps, (int)threadIdx.x, nl);
+        else
+            norm_rows_to_lds<false>(p.x, p.x, p.nrm_weight, nullptr, xs, norm_part, M, K, p.nrm_eps, (int)threadIdx.x, nl);
+        if (n == 0) return;
+        for (int c = lane; c < p.x_chunks_max; c += 64) {
+            int dst;
+            uint32_t off;
+            if (x_chunk(c, dst, off)) xw[dst] = pair_order_u4(xs[off >> 4]);
+        }
+    } else
     // ---- finish the x slice (its first loads were issued before the weights, so they
     //      arrive first)
     if (!PERM) {
@@ -381,14 +408,26 @@ template <int EPI, int DEPTH, int NW>
 int launch_variant(const MatmulArgs &a, const GemvPlan &pl, hipStream_t stream) {
     dim3 grid((unsigned)pl.workgroups), block(64 * NW);
     if (a.perm == nullptr)
-        hipLaunchKernelGGL((gptq4_gemv_kernel<EPI, DEPTH, false, NW>), grid, block, pl.lds_bytes, stream, a);
+        hipLaunchKernelGGL((gptq4_gemv_kernel<EPI, DEPTH, false, NW, 0>), grid, block, pl.lds_bytes, stream, a);
     else
-        hipLaunchKernelGGL((gptq4_gemv_kernel<EPI, DEPTH, true, NW>), grid, block, pl.lds_bytes, stream, a);
+        hipLaunchKernelGGL((gptq4_gemv_kernel<EPI, DEPTH, true, NW, 0>), grid, block, pl.lds_bytes, stream, a);
+    return (int)hipGetLastError();
+}
+
+// The variant that normalises its own input: 4 waves, one unit in flight.
+template <int EPI>
+int launch_norm_variant(const MatmulArgs &a, const GemvPlan &pl, hipStream_t stream) {
+    dim3 grid((unsigned)pl.workgroups), block(256);
+    if (a.K <= 4096)
+        hipLaunchKernelGGL((gptq4_gemv_kernel<EPI, 1, false, 4, 2>), grid, block, pl.lds_bytes, stream, a);
+    else
+        hipLaunchKernelGGL((gptq4_gemv_kernel<EPI, 1, false, 4, 4>), grid, block, pl.lds_bytes, stream, a);
     return (int)hipGetLastError();
 }
 
 template <int EPI>
 int launch_epi(const MatmulArgs &a, const GemvPlan &pl, hipStream_t stream) {
+    if (a.nrm_weight != nullptr) return launch_norm_variant<EPI>(a, pl, stream);
     const int key = pl.waves * 10 + pl.depth;
     switch (key) {
         case 41: return launch_variant<EPI, 1, 4>(a, pl, stream);
@@ -410,13 +449,14 @@ GemvTuning g_gemv_tuning = {1, 0, 0, 0};
 
 // Launch shape: the grid holds `waves_per_cu` waves per CU on all 256 CUs (or fewer
 // waves when there are fewer units than that), each wave owning q or q+1 units.
-GemvPlan gemv_plan(int epi, int M, int N, int K) {
+GemvPlan gemv_plan(int epi, int M, int N, int K, bool norm) {
     GemvPlan pl = {};
     // one unit in flight per wave: with 8 waves per CU a deeper ring only queues requests the CU cannot
-    // have outstanding anyway (measured 15.2 us against 15.9 at two units for the LLaMA-7B gate/up pair)
-    pl.depth = g_gemv_tuning.depth > 0 ? g_gemv_tuning.depth : 1;
-    pl.waves = g_gemv_tuning.waves > 0 ? g_gemv_tuning.waves : 4;
-    const int waves_per_cu = g_gemv_tuning.waves_per_cu > 0 ? g_gemv_tuning.waves_per_cu : 8;
+    // have outstanding anyway (measured 15.2 us against 15.9 at two units for the LLaMA-7B gate/up pair).
+    // The variant that normalises its own input exists for the automatic shape only.
+    pl.depth = (!norm && g_gemv_tuning.depth > 0) ? g_gemv_tuning.depth : 1;
+    pl.waves = (!norm && g_gemv_tuning.waves > 0) ? g_gemv_tuning.waves : 4;
+    const int waves_per_cu = (!norm && g_gemv_tuning.waves_per_cu > 0) ? g_gemv_tuning.waves_per_cu : 8;
     const int sw = 32;
     pl.tiles = (epi == EPI_ROPE) ? (N / 128) * (64 / sw) : N / sw;
     pl.nb = K / 128;
@@ -440,6 +480,7 @@ GemvPlan gemv_plan(int epi, int M, int N, int K) {
     const int max_units = pl.q + (pl.r ? 1 : 0);
     pl.lds_wave_chunks = (max_units << mshift) * XROW;
     size_t lds = (size_t)pl.waves * pl.lds_wave_chunks * 16;
+    if (norm) lds += (size_t)M * K * sizeof(half_t);  // the normalised rows, shared by the workgroup
     // no CU may take more than its share of workgroups: ask for so much LDS (160 KiB per
     // CU) that one more workgroup would not fit
     const int wgs_per_cu = (waves_per_cu + pl.waves - 1) / pl.waves;

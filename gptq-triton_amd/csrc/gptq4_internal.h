@@ -40,6 +40,13 @@ struct MatmulArgs {
     int x_chunks_max;     // chunks of the largest x slice: (slot_q + 1) << (4 + m_shift)
     int max_contrib;      // partial-sum slots per tile
     RopeArgs rope;          // EPI_ROPE only
+    // fused residual add + RMSNorm of the input (small-M kernels): when nrm_weight is set, x is the
+    // residual stream and the kernel multiplies with nrm_weight * rmsnorm(x (+ nrm_delta)); the sums
+    // x + nrm_delta go to nrm_sum_out (not aliasing x or nrm_delta: other workgroups still read them)
+    const half_t *nrm_delta;
+    const half_t *nrm_weight;
+    half_t *nrm_sum_out;
+    float nrm_eps;
 };
 
 // Launch shape of the small-M kernel.
@@ -54,7 +61,8 @@ struct SkinnyTuning {
     int words, depth, splitk, waves;  // 0 = automatic
 };
 extern SkinnyTuning g_skinny_tuning;
-SkinnyPlan skinny_plan(int epi, int N, int K);
+// standard_shape: ignore the tuning overrides of words, depth and waves (the split is still tunable)
+SkinnyPlan skinny_plan(int epi, int N, int K, bool standard_shape = false);
 // Small-M (M <= 16) split-K matrix-core GEMV.  Returns hipError_t.
 int launch_skinny(int epi, const MatmulArgs &a, const SkinnyPlan &plan, hipStream_t stream);
 // Balanced decode GEMV (M <= GEMV_MAX_M): (tile, batch) units dealt evenly to waves.
@@ -72,7 +80,8 @@ struct GemvTuning {
     int depth, waves, waves_per_cu;  // 0 = automatic
 };
 extern GemvTuning g_gemv_tuning;
-GemvPlan gemv_plan(int epi, int M, int N, int K);
+// norm: plan for the variant that normalises its own input (automatic launch shape, room for the rows in LDS)
+GemvPlan gemv_plan(int epi, int M, int N, int K, bool norm = false);
 size_t gemv_partial_bytes(const GemvPlan &plan, int M, int epi);
 int launch_gemv(int epi, MatmulArgs &a, const GemvPlan &plan, hipStream_t stream);
 // Launch shape of the tiled kernel.

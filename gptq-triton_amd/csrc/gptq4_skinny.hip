@@ -25,6 +25,7 @@
 //   blockIdx -> (tile, split): all splits of a tile, and tiles that share a 128-byte
 //   line of a qweight row, land on one XCD (blockIdx % 8) and hence one L2.
 #include "gptq4_internal.h"
+#include "gptq4_norm.h"
 
 // Development aid, compiled out of the product build: per-workgroup cycle stamps at
 // the phase boundaries of the kernel, written 32 MiB into the workspace (size it so).
@@ -67,10 +68,16 @@ struct Batch {
     uint2 raw_s[NV];                     // W fp16 scales of the lane's columns (low halves first)
     uint32_t raw_z[NV];
     int group;
+    int b;                               // the batch (uniform over the wave)
 };
 
-template <int EPI, int W, int DEPTH, bool PERM, int NW>
+// NORM: p.x is the residual stream; the workgroup first computes weight * rmsnorm(x (+ delta)) of
+// all M rows into LDS (gptq4_norm.h; the workgroup of tile 0, split 0 also writes the sums out)
+// and takes its A operand from there instead of from memory.
+// NORM = chunks of 8 values per thread that cover a row (2: K <= 4096, 4: K <= 8192), 0 = off.
+template <int EPI, int W, int DEPTH, bool PERM, int NW, int NORM>
 __global__ __launch_bounds__(64 * NW) void gptq4_skinny_kernel(MatmulArgs p) {
+    static_assert(!NORM || (NW == 4 && !PERM), "the fused norm is written for 256 threads and unpermuted rows");
     constexpr int NV = (EPI == EPI_PLAIN) ? 1 : 2;  // strips loaded per K step
     constexpr int SW = 16 * W;                      // strip width in columns
     constexpr int TILE_COLS = SW * NV;              // columns of the LDS tile
@@ -79,6 +86,8 @@ __global__ __launch_bounds__(64 * NW) void gptq4_skinny_kernel(MatmulArgs p) {
 
     __shared__ float red[NW][SKINNY_MAX_M][TILE_COLS];
     __shared__ int s_is_last;
+    __shared__ float norm_part[NORM ? NORM_MAX_M * 4 : 1];
+    extern __shared__ uint4 xs[];  // NORM: [M][K / 8] normalised activations
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -153,8 +162,10 @@ __global__ __launch_bounds__(64 * NW) void gptq4_skinny_kernel(MatmulArgs p) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) B.w[v][i] = *reinterpret_cast<const wvec_t *>(base + (size_t)(4 * i) * N);
         }
+        B.b = b;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
+            if (NORM) break;  // the A operand comes from LDS at compute time
             const int k = b * 128 + 32 * i + 8 * lrow;
             uint4 a;
             if (!PERM) {
@@ -188,6 +199,7 @@ __global__ __launch_bounds__(64 * NW) void gptq4_skinny_kernel(MatmulArgs p) {
         }
     };
 
+    const int xs_row = (lcol < M ? lcol : M - 1) * (K >> 3);  // NORM: the lane's row of xs
     auto compute_batch = [&](const batch_t &B) {
         if (B.group != cur_group) {
             cur_group = B.group;
@@ -204,7 +216,7 @@ __global__ __launch_bounds__(64 * NW) void gptq4_skinny_kernel(MatmulArgs p) {
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const h8_t a = pair_order_a(B.a[i]);
+            const h8_t a = pair_order_a(NORM ? xs[xs_row + B.b * 16 + 4 * i + lrow] : B.a[i]);
 #pragma unroll
             for (int v = 0; v < NV; ++v) {
 #pragma unroll
@@ -218,6 +230,15 @@ __global__ __launch_bounds__(64 * NW) void gptq4_skinny_kernel(MatmulArgs p) {
 
     // software pipeline: DEPTH batches of loads in flight per wave
     {
+        // NORM: the loads of the first row go out ahead of the weights, so that the row is
+        // normalised while the weights are still on their way
+        NormLoads<NORM ? NORM : 1> nl;
+        if (NORM) {
+            if (p.nrm_delta != nullptr)
+                norm_issue_row0<true>(p.x, p.nrm_delta, p.nrm_weight, K, tid, nl);
+            else
+                norm_issue_row0<false>(p.x, p.x, p.nrm_weight, K, tid, nl);
+        }
         batch_t ring[DEPTH];
 #pragma unroll
         for (int d = 0; d < DEPTH; ++d)
@@ -227,6 +248,13 @@ __global__ __launch_bounds__(64 * NW) void gptq4_skinny_kernel(MatmulArgs p) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         PHASE_STAMP(5);
 #endif
+        if (NORM) {
+            half_t *const sums = (tile == 0 && split == 0) ? p.nrm_sum_out : nullptr;
+            if (p.nrm_delta != nullptr)
+                norm_rows_to_lds<true>(p.x, p.nrm_delta, p.nrm_weight, sums, xs, norm_part, M, K, p.nrm_eps, tid, nl);
+            else
+                norm_rows_to_lds<false>(p.x, p.x, p.nrm_weight, nullptr, xs, norm_part, M, K, p.nrm_eps, tid, nl);
+        }
         for (int b = b0; b < b1; b += DEPTH) {
 #pragma unroll
             for (int d = 0; d < DEPTH; ++d) {
@@ -387,9 +415,22 @@ int launch_variant(const MatmulArgs &a, hipStream_t stream) {
     const int groups = (a.tiles + per_xcd - 1) / per_xcd;
     dim3 grid((unsigned)(groups * per_xcd), (unsigned)a.splitk), block(64 * NW);
     if (a.perm == nullptr)
-        hipLaunchKernelGGL((gptq4_skinny_kernel<EPI, W, DEPTH, false, NW>), grid, block, 0, stream, a);
+        hipLaunchKernelGGL((gptq4_skinny_kernel<EPI, W, DEPTH, false, NW, 0>), grid, block, 0, stream, a);
     else
-        hipLaunchKernelGGL((gptq4_skinny_kernel<EPI, W, DEPTH, true, NW>), grid, block, 0, stream, a);
+        hipLaunchKernelGGL((gptq4_skinny_kernel<EPI, W, DEPTH, true, NW, 0>), grid, block, 0, stream, a);
+    return (int)hipGetLastError();
+}
+
+// The variant that normalises its own input: the automatic launch shape only.
+template <int EPI, int DEPTH>
+int launch_norm_variant(const MatmulArgs &a, hipStream_t stream) {
+    const int groups = (a.tiles + 7) / 8;
+    dim3 grid((unsigned)(groups * 8), (unsigned)a.splitk), block(256);
+    const size_t lds = (size_t)a.M * a.K * sizeof(half_t);
+    if (a.K <= 4096)
+        hipLaunchKernelGGL((gptq4_skinny_kernel<EPI, 2, DEPTH, false, 4, 2>), grid, block, lds, stream, a);
+    else
+        hipLaunchKernelGGL((gptq4_skinny_kernel<EPI, 2, DEPTH, false, 4, 4>), grid, block, lds, stream, a);
     return (int)hipGetLastError();
 }
 
@@ -416,11 +457,12 @@ SkinnyTuning g_skinny_tuning = {0, 0, 0, 0};
 // strips, full 128-byte lines per row) beat 16-byte loads because they give twice the
 // tiles; two batches in flight per wave, one for the gate/up pair (register budget);
 // split K until there are ~1024 workgroups (4 per CU) but keep >= 2 batches per wave.
-SkinnyPlan skinny_plan(int epi, int N, int K) {
+SkinnyPlan skinny_plan(int epi, int N, int K, bool standard_shape) {
     SkinnyPlan pl;
-    pl.words = g_skinny_tuning.words > 0 ? g_skinny_tuning.words : 2;
-    pl.depth = g_skinny_tuning.depth > 0 ? g_skinny_tuning.depth : (epi == EPI_SILU_MUL ? 1 : 2);
-    pl.waves = g_skinny_tuning.waves > 0 ? g_skinny_tuning.waves : 4;
+    const bool tuned = !standard_shape;
+    pl.words = (tuned && g_skinny_tuning.words > 0) ? g_skinny_tuning.words : 2;
+    pl.depth = (tuned && g_skinny_tuning.depth > 0) ? g_skinny_tuning.depth : (epi == EPI_SILU_MUL ? 1 : 2);
+    pl.waves = (tuned && g_skinny_tuning.waves > 0) ? g_skinny_tuning.waves : 4;
     const int sw = 16 * pl.words;
     pl.tiles = (epi == EPI_ROPE) ? (N / 128) * (64 / sw) : N / sw;
     const int k_batches = K / 128;
@@ -439,6 +481,12 @@ SkinnyPlan skinny_plan(int epi, int N, int K) {
 }
 
 int launch_skinny(int epi, const MatmulArgs &a, const SkinnyPlan &pl, hipStream_t stream) {
+    if (a.nrm_weight != nullptr) {
+        // checked by the caller: automatic plan (8-byte loads, 4 waves), M <= NORM_MAX_M, K <= NORM_MAX_H, no perm
+        if (epi == EPI_SILU_MUL) return launch_norm_variant<EPI_SILU_MUL, 1>(a, stream);
+        if (epi == EPI_ROPE) return launch_norm_variant<EPI_ROPE, 2>(a, stream);
+        return launch_norm_variant<EPI_PLAIN, 2>(a, stream);
+    }
     switch (epi) {
         case EPI_PLAIN: return launch_epi<EPI_PLAIN>(a, pl, stream);
         case EPI_SILU_MUL: return launch_epi<EPI_SILU_MUL>(a, pl, stream);

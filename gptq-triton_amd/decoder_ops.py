@@ -5,10 +5,39 @@ so that a whole decode step is a short chain of HIP launches that a graph can re
 from __future__ import annotations
 
 import math
+import os
 
 import torch
 
 from . import _lib
+
+
+# limits of the matmul kernels that normalise their own input (gptq4_norm_qkv_rotary, gptq4_norm_mlp_gateup)
+NORM_MAX_ROWS, NORM_MAX_HIDDEN = 4, 8192
+# GPTQ4_NORM_FUSION=0 in the environment keeps the norms as launches of their own (for A/B timing)
+NORM_FUSION = os.environ.get("GPTQ4_NORM_FUSION", "1") != "0"
+
+
+def norm_fusable(rows: int, hidden: int, perm=None) -> bool:
+    """Whether a projection of `rows` rows can take the residual add + RMSNorm of its input along."""
+    return NORM_FUSION and 0 < rows <= NORM_MAX_ROWS and hidden <= NORM_MAX_HIDDEN and hidden % 8 == 0 and perm is None
+
+
+def check_norm_args(h: torch.Tensor, delta, weight: torch.Tensor):
+    """Validate (h, delta, norm weight) of a fused call; returns the [rows, hidden] views and the sum buffer."""
+    for t, name in ((h, "h"), (delta, "delta"), (weight, "norm weight")):
+        if t is None:
+            continue
+        _lib.require_cuda(t, name)
+        if t.dtype != torch.float16:
+            raise TypeError("the fused residual add + RMSNorm takes fp16 tensors")
+    hidden = h.shape[-1]
+    if weight.shape != (hidden,) or (delta is not None and delta.shape != h.shape):
+        raise ValueError("h and delta must have one shape [..., H] and the norm weight [H]")
+    h2 = h.reshape(-1, hidden).contiguous()
+    d2 = None if delta is None else delta.reshape(-1, hidden).contiguous()
+    s = None if delta is None else torch.empty_like(h2)  # never aliases h or delta: other workgroups still read them
+    return h2, d2, s
 
 
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:

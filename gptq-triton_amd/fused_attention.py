@@ -64,8 +64,11 @@ KV_AT_POSITION = -1  # GPTQ4_KV_AT_POSITION of the C ABI
 def qkv_rotary(groupsize: int, hidden_states: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor,
                qzeros: torch.Tensor, position_ids: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
                num_heads: int, head_dim: int = 128, perm: Optional[torch.Tensor] = None,
-               kv_out: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, kv_offset: int = 0):
+               kv_out: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, kv_offset: int = 0, norm=None):
     """hidden_states fp16 [B, S, K]; packed weights with N = 3*H*D in q, k, v order.
+    norm = (delta or None, norm_weight, eps): hidden_states is the residual stream h and the
+    kernel projects RMSNorm(h + delta) * norm_weight, normalising its own input (decode-sized
+    calls only, decoder_ops.norm_fusable); a fourth value is returned then, h + delta.
     Returns (q, k, v): q [B,H,S,D] rotated; k, v [B,H,S,D], or - when `kv_out` gives
     preallocated [B,H,cap,D] buffers - those buffers with rows kv_offset..kv_offset+S
     filled (kv_offset = KV_AT_POSITION: row position_ids[b, s] for token (b, s), so that a
@@ -93,6 +96,21 @@ def qkv_rotary(groupsize: int, hidden_states: torch.Tensor, qweight: torch.Tenso
         if kk.shape != vv.shape or kk.shape[0] != bsz or kk.shape[1] != num_heads or kk.shape[3] != head_dim \
                 or not kk.is_contiguous() or not vv.is_contiguous() or off < KV_AT_POSITION or off + q_len > cap:
             raise ValueError("kv_out buffers must be contiguous [B, H, capacity, D] with room for the new rows")
+    if norm is not None:
+        from .decoder_ops import check_norm_args, norm_fusable
+        delta, norm_weight, eps = norm
+        if not norm_fusable(bsz * q_len, k_in, perm):
+            raise ValueError("outside what the fused norm takes; run add_rms_norm and the plain call")
+        h2, d2, s = check_norm_args(hidden_states, delta, norm_weight)
+        lib = _lib.load()
+        ws = _lib.workspace(dev, lib.gptq4_workspace_bytes(_lib.OP_QKV_ROTARY, bsz * q_len, k_in, n))
+        rc = lib.gptq4_norm_qkv_rotary(h2.data_ptr(), _lib.ptr(d2), norm_weight.data_ptr(), float(eps), _lib.ptr(s),
+                                       qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(), pos.data_ptr(),
+                                       cos.data_ptr(), sin.data_ptr(), cos.shape[0], q.data_ptr(), kk.data_ptr(),
+                                       vv.data_ptr(), bsz, q_len, num_heads, head_dim, k_in, groupsize, cap, off,
+                                       ws.data_ptr(), ws.numel(), _lib.current_stream(dev))
+        _lib.check(rc, "gptq4_norm_qkv_rotary")
+        return q, kk, vv, (hidden_states if s is None else s.view(hidden_states.shape))
     if bsz * q_len == 0:
         return q, kk, vv
     lib = _lib.load()
@@ -169,13 +187,18 @@ class QuantLlamaAttention(nn.Module):
                                 float(getattr(config, 'rope_theta', 10000.0)))
 
     def project_qkv(self, hidden_states: torch.Tensor, position_ids: torch.Tensor,
-                    kv_out=None, kv_offset: int = 0):
+                    kv_out=None, kv_offset: int = 0, norm=None):
+        """norm = (delta or None, norm_weight, eps): see qkv_rotary."""
         need = max(kv_offset, 0) + hidden_states.shape[1]
         cos, sin = self.rope.get(hidden_states.device, max(need, self.max_position_embeddings))
         qweight, perm = self.qkv_proj.kernel_weights()
         return qkv_rotary(self.qkv_proj.groupsize, hidden_states, qweight, self.qkv_proj.scales,
                           self.qkv_proj.qzeros, position_ids, cos, sin, self.num_heads, self.head_dim,
-                          perm=perm, kv_out=kv_out, kv_offset=kv_offset)
+                          perm=perm, kv_out=kv_out, kv_offset=kv_offset, norm=norm)
+
+    def norm_fusable(self, rows: int) -> bool:
+        from .decoder_ops import norm_fusable
+        return norm_fusable(rows, self.hidden_size, self.qkv_proj.kernel_weights()[1])
 
     def forward(
         self,

@@ -178,6 +178,10 @@ class GreedyDecoder:
         """The decoder stack on hidden states h [B, S, hidden]; every residual add is fused
         with the RMSNorm that follows it.  Returns the greedy next token [B, 1]."""
         layers = self.model.model.layers
+        rows = h.shape[0] * h.shape[1]
+        if all(getattr(l.self_attn, "norm_fusable", lambda r: False)(rows) and getattr(l.mlp, "norm_fusable", lambda r: False)(rows)
+               for l in layers):
+            return self._layers_norm_in_matmul(h, position_ids, kv_offset, attend)
         x = layers[0].input_layernorm(h)
         for i, (layer, (kc, vc)) in enumerate(zip(layers, self.caches)):
             attn = layer.self_attn
@@ -186,6 +190,21 @@ class GreedyDecoder:
             h, x = add_rms_norm(h, attn.o_proj(attend(q, kc, vc)), norm.weight, norm.variance_epsilon)  # attend -> [B, S, hidden]
             norm = layers[i + 1].input_layernorm if i + 1 < len(layers) else self.model.model.norm
             h, x = add_rms_norm(h, layer.mlp(x), norm.weight, norm.variance_epsilon)
+        return self.model.lm_head(x[:, -1:, :]).argmax(-1)
+
+    def _layers_norm_in_matmul(self, h, position_ids, kv_offset, attend):
+        """The same stack for a handful of rows: the QKV and the gate/up launch each do the residual
+        add and the RMSNorm of their own input (same bits as _layers' separate launches), so a
+        layer is 5 launches instead of 7."""
+        layers = self.model.model.layers
+        delta = None
+        for layer, (kc, vc) in zip(layers, self.caches):
+            attn, n1, n2 = layer.self_attn, layer.input_layernorm, layer.post_attention_layernorm
+            q, _, _, h = attn.project_qkv(h, position_ids, kv_out=(kc, vc), kv_offset=kv_offset,
+                                          norm=(delta, n1.weight, n1.variance_epsilon))
+            h, delta = layer.mlp.forward_normed(h, attn.o_proj(attend(q, kc, vc)), n2.weight, n2.variance_epsilon)
+        norm = self.model.model.norm
+        h, x = add_rms_norm(h, delta, norm.weight, norm.variance_epsilon)
         return self.model.lm_head(x[:, -1:, :]).argmax(-1)
 
     @torch.no_grad()
