@@ -27,9 +27,9 @@ SIGNATURES = {
     "gptq4_mlp_gateup": (c_int, [c_void_p] * 9 + [c_int] * 4 + [c_void_p, c_size_t, c_void_p]),
     "gptq4_rope_table": (c_int, [c_void_p, c_void_p, c_int, c_int, c_float, c_void_p]),
     "gptq4_qkv_rotary": (c_int, [c_void_p] * 8 + [c_int] + [c_void_p] * 3 + [c_int] * 8 + [c_void_p, c_size_t, c_void_p]),
-    "gptq4_norm_qkv_rotary": (c_int, [c_void_p] * 3 + [c_float] + [c_void_p] * 7 + [c_int] + [c_void_p] * 3 + [c_int] * 8
+    "gptq4_norm_qkv_rotary": (c_int, [c_void_p] * 3 + [c_float] + [c_void_p] * 8 + [c_int] + [c_void_p] * 3 + [c_int] * 8
                               + [c_void_p, c_size_t, c_void_p]),
-    "gptq4_norm_mlp_gateup": (c_int, [c_void_p] * 3 + [c_float] + [c_void_p] * 8 + [c_int] * 4 + [c_void_p, c_size_t, c_void_p]),
+    "gptq4_norm_mlp_gateup": (c_int, [c_void_p] * 3 + [c_float] + [c_void_p] * 9 + [c_int] * 4 + [c_void_p, c_size_t, c_void_p]),
     "gptq4_rmsnorm": (c_int, [c_void_p] * 3 + [c_int, c_int, c_float, c_void_p]),
     "gptq4_add_rmsnorm": (c_int, [c_void_p] * 5 + [c_int, c_int, c_float, c_void_p]),
     "gptq4_decode_attention": (c_int, [c_void_p] * 5 + [c_int] * 4 + [c_float, c_void_p, c_size_t, c_void_p]),

@@ -95,11 +95,10 @@ int setup_gemm(MatmulArgs &a, const GemmPlan &pl, void *workspace, size_t worksp
 }
 
 // Fused residual add + RMSNorm of the input: decode-sized calls only (the workgroups of the small-M
-// kernel each normalise all M rows into their LDS), unpermuted rows, and a sum_out that no
-// workgroup still reads from.
+// kernel each normalise all M rows into their LDS), and a sum_out that no workgroup still reads from.
 int setup_norm(MatmulArgs &a, const void *delta, const void *norm_weight, void *sum_out, float eps) {
     if (!norm_weight || (delta && !sum_out)) return -GPTQ4_E_NULL;
-    if (a.M > NORM_MAX_M || a.K > NORM_MAX_H || a.perm != nullptr || !(eps >= 0.f)) return -GPTQ4_E_SHAPE;
+    if (a.M > NORM_MAX_M || a.K > NORM_MAX_H || !(eps >= 0.f)) return -GPTQ4_E_SHAPE;
     if (delta && (sum_out == static_cast<const void *>(a.x) || sum_out == delta)) return -GPTQ4_E_SHAPE;
     if (misaligned16(norm_weight) || (delta && (misaligned16(delta) || misaligned16(sum_out)))) return -GPTQ4_E_ALIGN;
     a.nrm_delta = reinterpret_cast<const half_t *>(delta);
@@ -311,10 +310,11 @@ int gptq4_mlp_gateup(const void *x, const int32_t *gate_qweight, const int32_t *
 
 int gptq4_norm_mlp_gateup(const void *x, const void *delta, const void *norm_weight, float eps, void *sum_out,
                           const int32_t *gate_qweight, const int32_t *gate_qzeros, const void *gate_scales,
-                          const int32_t *up_qweight, const int32_t *up_qzeros, const void *up_scales, void *h, int M,
-                          int K, int I, int groupsize, void *workspace, size_t workspace_bytes, void *stream) {
+                          const int32_t *up_qweight, const int32_t *up_qzeros, const void *up_scales,
+                          const int32_t *perm, void *h, int M, int K, int I, int groupsize, void *workspace,
+                          size_t workspace_bytes, void *stream) {
     return mlp_gateup_impl(x, delta, norm_weight, sum_out, eps, gate_qweight, gate_qzeros, gate_scales, up_qweight,
-                           up_qzeros, up_scales, nullptr, h, M, K, I, groupsize, workspace, workspace_bytes, stream, true);
+                           up_qzeros, up_scales, perm, h, M, K, I, groupsize, workspace, workspace_bytes, stream, true);
 }
 
 int gptq4_rope_table(float *cos_out, float *sin_out, int max_pos, int D, float base, void *stream) {
@@ -389,11 +389,11 @@ int gptq4_qkv_rotary(const void *x, const int32_t *qweight, const int32_t *qzero
 }
 
 int gptq4_norm_qkv_rotary(const void *x, const void *delta, const void *norm_weight, float eps, void *sum_out,
-                          const int32_t *qweight, const int32_t *qzeros, const void *scales,
+                          const int32_t *qweight, const int32_t *qzeros, const void *scales, const int32_t *perm,
                           const int32_t *position_ids, const float *cos_table, const float *sin_table, int max_pos,
                           void *q, void *k, void *v, int B, int S, int H, int D, int K, int groupsize, int kv_capacity,
                           int kv_offset, void *workspace, size_t workspace_bytes, void *stream) {
-    return qkv_rotary_impl(x, delta, norm_weight, sum_out, eps, qweight, qzeros, scales, nullptr, position_ids, cos_table,
+    return qkv_rotary_impl(x, delta, norm_weight, sum_out, eps, qweight, qzeros, scales, perm, position_ids, cos_table,
                            sin_table, max_pos, q, k, v, B, S, H, D, K, groupsize, kv_capacity, kv_offset, workspace,
                            workspace_bytes, stream, true);
 }

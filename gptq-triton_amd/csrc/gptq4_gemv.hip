@@ -70,7 +70,7 @@ constexpr int XROW = 17;  // 16-byte chunks per (unit, row) of the x slice: 16 +
 // also writes the sums out) and its waves stage their x slices from there instead of from memory.
 template <int EPI, int DEPTH, bool PERM, int NW, int NORM>
 __global__ __launch_bounds__(64 * NW) void gptq4_gemv_kernel(MatmulArgs p) {
-    static_assert(!NORM || (NW == 4 && !PERM), "the fused norm is written for 256 threads and unpermuted rows");
+    static_assert(!NORM || NW == 4, "the fused norm is written for 256 threads");
     __shared__ float norm_part[NORM ? NORM_MAX_M * 4 : 1];
     constexpr int NV = (EPI == EPI_PLAIN) ? 1 : 2;
     constexpr int W = 2;
@@ -189,7 +189,25 @@ __global__ __launch_bounds__(64 * NW) void gptq4_gemv_kernel(MatmulArgs p) {
         for (int c = lane; c < p.x_chunks_max; c += 64) {
             int dst;
             uint32_t off;
-            if (x_chunk(c, dst, off)) xw[dst] = pair_order_u4(xs[off >> 4]);
+            if (x_chunk(c, dst, off)) {
+                if (!PERM) {
+                    xw[dst] = pair_order_u4(xs[off >> 4]);
+                } else {
+                    // act-order: x_sorted[k] = x[perm[k]], gathered from the row in LDS, directly in pair order
+                    const int rowk = (int)(off >> 1);
+                    const int row = (c >> 4) & ((1 << mshift) - 1);
+                    const int k = rowk - row * K;
+                    const uint16_t *xh = reinterpret_cast<const uint16_t *>(xs) + (size_t)row * K;
+                    const int4 i0 = *reinterpret_cast<const int4 *>(p.perm + k);
+                    const int4 i1 = *reinterpret_cast<const int4 *>(p.perm + k + 4);
+                    uint4 val;
+                    val.x = (uint32_t)xh[i0.x] | ((uint32_t)xh[i1.x] << 16);
+                    val.y = (uint32_t)xh[i0.y] | ((uint32_t)xh[i1.y] << 16);
+                    val.z = (uint32_t)xh[i0.z] | ((uint32_t)xh[i1.z] << 16);
+                    val.w = (uint32_t)xh[i0.w] | ((uint32_t)xh[i1.w] << 16);
+                    xw[dst] = val;
+                }
+            }
         }
     } else
     // ---- finish the x slice (its first loads were issued before the weights, so they
@@ -418,10 +436,15 @@ int launch_variant(const MatmulArgs &a, const GemvPlan &pl, hipStream_t stream) 
 template <int EPI>
 int launch_norm_variant(const MatmulArgs &a, const GemvPlan &pl, hipStream_t stream) {
     dim3 grid((unsigned)pl.workgroups), block(256);
-    if (a.K <= 4096)
+    const bool perm = a.perm != nullptr;
+    if (a.K <= 4096 && !perm)
         hipLaunchKernelGGL((gptq4_gemv_kernel<EPI, 1, false, 4, 2>), grid, block, pl.lds_bytes, stream, a);
-    else
+    else if (a.K <= 4096)
+        hipLaunchKernelGGL((gptq4_gemv_kernel<EPI, 1, true, 4, 2>), grid, block, pl.lds_bytes, stream, a);
+    else if (!perm)
         hipLaunchKernelGGL((gptq4_gemv_kernel<EPI, 1, false, 4, 4>), grid, block, pl.lds_bytes, stream, a);
+    else
+        hipLaunchKernelGGL((gptq4_gemv_kernel<EPI, 1, true, 4, 4>), grid, block, pl.lds_bytes, stream, a);
     return (int)hipGetLastError();
 }
 

@@ -77,7 +77,7 @@ struct Batch {
 // NORM = chunks of 8 values per thread that cover a row (2: K <= 4096, 4: K <= 8192), 0 = off.
 template <int EPI, int W, int DEPTH, bool PERM, int NW, int NORM>
 __global__ __launch_bounds__(64 * NW) void gptq4_skinny_kernel(MatmulArgs p) {
-    static_assert(!NORM || (NW == 4 && !PERM), "the fused norm is written for 256 threads and unpermuted rows");
+    static_assert(!NORM || NW == 4, "the fused norm is written for 256 threads");
     constexpr int NV = (EPI == EPI_PLAIN) ? 1 : 2;  // strips loaded per K step
     constexpr int SW = 16 * W;                      // strip width in columns
     constexpr int TILE_COLS = SW * NV;              // columns of the LDS tile
@@ -165,10 +165,19 @@ __global__ __launch_bounds__(64 * NW) void gptq4_skinny_kernel(MatmulArgs p) {
         B.b = b;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            if (NORM) break;  // the A operand comes from LDS at compute time
             const int k = b * 128 + 32 * i + 8 * lrow;
             uint4 a;
-            if (!PERM) {
+            if (NORM) {
+                // the A operand comes from LDS at compute time; act-order: keep the 8 source
+                // positions (below 8192, two per word)
+                if (!PERM) break;
+                const int4 i0 = *reinterpret_cast<const int4 *>(p.perm + k);
+                const int4 i1 = *reinterpret_cast<const int4 *>(p.perm + k + 4);
+                a.x = (uint32_t)i0.x | ((uint32_t)i0.y << 16);
+                a.y = (uint32_t)i0.z | ((uint32_t)i0.w << 16);
+                a.z = (uint32_t)i1.x | ((uint32_t)i1.y << 16);
+                a.w = (uint32_t)i1.z | ((uint32_t)i1.w << 16);
+            } else if (!PERM) {
                 a = *reinterpret_cast<const uint4 *>(xrow + k);
             } else {
                 const int4 i0 = *reinterpret_cast<const int4 *>(p.perm + k);
@@ -216,7 +225,17 @@ __global__ __launch_bounds__(64 * NW) void gptq4_skinny_kernel(MatmulArgs p) {
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const h8_t a = pair_order_a(NORM ? xs[xs_row + B.b * 16 + 4 * i + lrow] : B.a[i]);
+            uint4 av = B.a[i];
+            if (NORM && !PERM) av = xs[xs_row + B.b * 16 + 4 * i + lrow];
+            if (NORM && PERM) {
+                const uint16_t *xh = reinterpret_cast<const uint16_t *>(xs + xs_row);
+                const uint32_t ix[4] = {av.x, av.y, av.z, av.w};
+                uint32_t o[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = (uint32_t)xh[ix[e] & 0xFFFFu] | ((uint32_t)xh[ix[e] >> 16] << 16);
+                av = make_uint4(o[0], o[1], o[2], o[3]);
+            }
+            const h8_t a = pair_order_a(av);
 #pragma unroll
             for (int v = 0; v < NV; ++v) {
 #pragma unroll
@@ -427,10 +446,15 @@ int launch_norm_variant(const MatmulArgs &a, hipStream_t stream) {
     const int groups = (a.tiles + 7) / 8;
     dim3 grid((unsigned)(groups * 8), (unsigned)a.splitk), block(256);
     const size_t lds = (size_t)a.M * a.K * sizeof(half_t);
-    if (a.K <= 4096)
+    const bool perm = a.perm != nullptr;
+    if (a.K <= 4096 && !perm)
         hipLaunchKernelGGL((gptq4_skinny_kernel<EPI, 2, DEPTH, false, 4, 2>), grid, block, lds, stream, a);
-    else
+    else if (a.K <= 4096)
+        hipLaunchKernelGGL((gptq4_skinny_kernel<EPI, 2, DEPTH, true, 4, 2>), grid, block, lds, stream, a);
+    else if (!perm)
         hipLaunchKernelGGL((gptq4_skinny_kernel<EPI, 2, DEPTH, false, 4, 4>), grid, block, lds, stream, a);
+    else
+        hipLaunchKernelGGL((gptq4_skinny_kernel<EPI, 2, DEPTH, true, 4, 4>), grid, block, lds, stream, a);
     return (int)hipGetLastError();
 }
 
@@ -482,7 +506,7 @@ SkinnyPlan skinny_plan(int epi, int N, int K, bool standard_shape) {
 
 int launch_skinny(int epi, const MatmulArgs &a, const SkinnyPlan &pl, hipStream_t stream) {
     if (a.nrm_weight != nullptr) {
-        // checked by the caller: automatic plan (8-byte loads, 4 waves), M <= NORM_MAX_M, K <= NORM_MAX_H, no perm
+        // checked by the caller: automatic plan (8-byte loads, 4 waves), M <= NORM_MAX_M, K <= NORM_MAX_H
         if (epi == EPI_SILU_MUL) return launch_norm_variant<EPI_SILU_MUL, 1>(a, stream);
         if (epi == EPI_ROPE) return launch_norm_variant<EPI_ROPE, 2>(a, stream);
         return launch_norm_variant<EPI_PLAIN, 2>(a, stream);

@@ -18,9 +18,9 @@ NORM_MAX_ROWS, NORM_MAX_HIDDEN = 4, 8192
 NORM_FUSION = os.environ.get("GPTQ4_NORM_FUSION", "1") != "0"
 
 
-def norm_fusable(rows: int, hidden: int, perm=None) -> bool:
+def norm_fusable(rows: int, hidden: int) -> bool:
     """Whether a projection of `rows` rows can take the residual add + RMSNorm of its input along."""
-    return NORM_FUSION and 0 < rows <= NORM_MAX_ROWS and hidden <= NORM_MAX_HIDDEN and hidden % 8 == 0 and perm is None
+    return NORM_FUSION and 0 < rows <= NORM_MAX_ROWS and hidden <= NORM_MAX_HIDDEN and hidden % 8 == 0
 
 
 def check_norm_args(h: torch.Tensor, delta, weight: torch.Tensor):

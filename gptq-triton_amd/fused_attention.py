@@ -99,13 +99,13 @@ def qkv_rotary(groupsize: int, hidden_states: torch.Tensor, qweight: torch.Tenso
     if norm is not None:
         from .decoder_ops import check_norm_args, norm_fusable
         delta, norm_weight, eps = norm
-        if not norm_fusable(bsz * q_len, k_in, perm):
+        if not norm_fusable(bsz * q_len, k_in):
             raise ValueError("outside what the fused norm takes; run add_rms_norm and the plain call")
         h2, d2, s = check_norm_args(hidden_states, delta, norm_weight)
         lib = _lib.load()
         ws = _lib.workspace(dev, lib.gptq4_workspace_bytes(_lib.OP_QKV_ROTARY, bsz * q_len, k_in, n))
         rc = lib.gptq4_norm_qkv_rotary(h2.data_ptr(), _lib.ptr(d2), norm_weight.data_ptr(), float(eps), _lib.ptr(s),
-                                       qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(), pos.data_ptr(),
+                                       qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(), _lib.ptr(perm), pos.data_ptr(),
                                        cos.data_ptr(), sin.data_ptr(), cos.shape[0], q.data_ptr(), kk.data_ptr(),
                                        vv.data_ptr(), bsz, q_len, num_heads, head_dim, k_in, groupsize, cap, off,
                                        ws.data_ptr(), ws.numel(), _lib.current_stream(dev))
@@ -198,7 +198,7 @@ class QuantLlamaAttention(nn.Module):
 
     def norm_fusable(self, rows: int) -> bool:
         from .decoder_ops import norm_fusable
-        return norm_fusable(rows, self.hidden_size, self.qkv_proj.kernel_weights()[1])
+        return norm_fusable(rows, self.hidden_size)
 
     def forward(
         self,

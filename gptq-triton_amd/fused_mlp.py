@@ -49,7 +49,8 @@ triton_llama_mlp_4 = llama_mlp_4
 
 def norm_llama_mlp_4(groupsize: int, h: torch.Tensor, delta: Optional[torch.Tensor], norm_weight: torch.Tensor, eps: float,
                      gate_qweight: torch.Tensor, gate_scales: torch.Tensor, gate_qzeros: torch.Tensor,
-                     up_qweight: torch.Tensor, up_scales: torch.Tensor, up_qzeros: torch.Tensor):
+                     up_qweight: torch.Tensor, up_scales: torch.Tensor, up_qzeros: torch.Tensor,
+                     perm: Optional[torch.Tensor] = None):
     """(s, silu(gate(xn)) * up(xn)) with s = h + delta (h when delta is None) and xn = RMSNorm(s) * norm_weight,
     in ONE launch: the kernel normalises its own input.  Same bits as add_rms_norm followed by llama_mlp_4.
     Decode-sized inputs only (decoder_ops.norm_fusable)."""
@@ -57,7 +58,7 @@ def norm_llama_mlp_4(groupsize: int, h: torch.Tensor, delta: Optional[torch.Tens
     assert (gate_qweight.shape == up_qweight.shape and gate_scales.shape == up_scales.shape
             and gate_qzeros.shape == up_qzeros.shape), "All weights must have the same shape"
     k, n = _check_matmul_args(h, gate_qweight, groupsize)
-    _check_device_tensors(h, gate_qweight, gate_scales, gate_qzeros, up_qweight, up_scales, up_qzeros)
+    _check_device_tensors(h, gate_qweight, gate_scales, gate_qzeros, up_qweight, up_scales, up_qzeros, perm)
     h2, d2, s = check_norm_args(h, delta, norm_weight)
     m = h2.shape[0]
     if not norm_fusable(m, k):
@@ -67,8 +68,8 @@ def norm_llama_mlp_4(groupsize: int, h: torch.Tensor, delta: Optional[torch.Tens
     ws = _lib.workspace(h.device, lib.gptq4_workspace_bytes(_lib.OP_MLP_GATEUP, m, k, n))
     rc = lib.gptq4_norm_mlp_gateup(h2.data_ptr(), _lib.ptr(d2), norm_weight.data_ptr(), float(eps), _lib.ptr(s),
                                    gate_qweight.data_ptr(), gate_qzeros.data_ptr(), gate_scales.data_ptr(),
-                                   up_qweight.data_ptr(), up_qzeros.data_ptr(), up_scales.data_ptr(), c.data_ptr(),
-                                   m, k, n, groupsize, ws.data_ptr(), ws.numel(), _lib.current_stream(h.device))
+                                   up_qweight.data_ptr(), up_qzeros.data_ptr(), up_scales.data_ptr(), _lib.ptr(perm),
+                                   c.data_ptr(), m, k, n, groupsize, ws.data_ptr(), ws.numel(), _lib.current_stream(h.device))
     _lib.check(rc, "gptq4_norm_mlp_gateup")
     return (h if s is None else s.view(h.shape)), c.view(h.shape[:-1] + (n,))
 
@@ -123,13 +124,13 @@ class QuantLlamaMLP(nn.Module):
 
     def norm_fusable(self, rows: int) -> bool:
         from .decoder_ops import norm_fusable
-        return self.g_idx is None and norm_fusable(rows, self.infeatures)
+        return norm_fusable(rows, self.infeatures)
 
     def forward_normed(self, h: torch.Tensor, delta: Optional[torch.Tensor], norm_weight: torch.Tensor, eps: float):
         """(h + delta, forward(RMSNorm(h + delta))): the residual add and the norm run inside the gate/up launch."""
-        s, mid = norm_llama_mlp_4(self.groupsize, h, delta, norm_weight, eps,
-                                  self.gate_proj_qweight, self.gate_proj_scales, self.gate_proj_qzeros,
-                                  self.up_proj_qweight, self.up_proj_scales, self.up_proj_qzeros)
+        gq, uq, perm = self._kernel_weights()
+        s, mid = norm_llama_mlp_4(self.groupsize, h, delta, norm_weight, eps, gq, self.gate_proj_scales, self.gate_proj_qzeros,
+                                  uq, self.up_proj_scales, self.up_proj_qzeros, perm)
         return s, self.down_proj(mid)
 
 

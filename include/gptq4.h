@@ -130,20 +130,20 @@ int gptq4_qkv_rotary(const void *x, const int32_t *qweight, const int32_t *qzero
  *   s = delta ? fp16(x + delta) : x;   if delta: sum_out = s;   xn = norm_weight * fp16(s * rsqrt(mean(s^2) + eps));
  * then gptq4_qkv_rotary / gptq4_mlp_gateup on xn.  x, delta (nullable), sum_out fp16 [M, K], norm_weight
  * fp16 [K]; bit-identical to gptq4_add_rmsnorm (or gptq4_rmsnorm) followed by the plain entry point.
- * Decode-sized calls only: M <= 4, K <= 8192, no act-order permutation (else -GPTQ4_E_SHAPE: run the
- * two calls).  sum_out must not be x or delta: other workgroups of the launch still read them.
+ * Decode-sized calls only: M <= 4, K <= 8192 (else -GPTQ4_E_SHAPE: run the two calls); perm as in the
+ * plain entry points.  sum_out must not be x or delta: other workgroups of the launch still read them.
  * No reference counterpart (the reference runs LlamaRMSNorm as separate torch kernels,
  * src/gptq_triton/__init__.py:32-47). */
 int gptq4_norm_qkv_rotary(const void *x, const void *delta, const void *norm_weight, float eps, void *sum_out,
                           const int32_t *qweight, const int32_t *qzeros, const void *scales,
-                          const int32_t *position_ids, const float *cos_table, const float *sin_table,
-                          int max_pos, void *q, void *k, void *v, int B, int S, int H, int D, int K,
+                          const int32_t *perm, const int32_t *position_ids, const float *cos_table,
+                          const float *sin_table, int max_pos, void *q, void *k, void *v, int B, int S, int H, int D, int K,
                           int groupsize, int kv_capacity, int kv_offset, void *workspace,
                           size_t workspace_bytes, void *stream);
 int gptq4_norm_mlp_gateup(const void *x, const void *delta, const void *norm_weight, float eps, void *sum_out,
                           const int32_t *gate_qweight, const int32_t *gate_qzeros, const void *gate_scales,
                           const int32_t *up_qweight, const int32_t *up_qzeros, const void *up_scales,
-                          void *h, int M, int K, int I, int groupsize, void *workspace,
+                          const int32_t *perm, void *h, int M, int K, int I, int groupsize, void *workspace,
                           size_t workspace_bytes, void *stream);
 
 /* RMSNorm over the last dimension: y = weight * fp16(x * rsqrt(mean(x^2) + eps)), x and y

@@ -136,6 +136,37 @@ def test_norm_in_the_balanced_gemv_equals_two_launches(balanced_gemv, m):
     assert int(ws[:_lib.WS_COUNTER_BYTES].view(torch.int32).abs().sum()) == 0
 
 
+@pytest.mark.parametrize("gemv_mode", [0, 2])
+@pytest.mark.parametrize("m", [1, 3])
+def test_norm_with_act_order_equals_two_launches(gemv_mode, m):
+    """Act-order layers: the kernels gather the permuted activations from the normalised row in LDS."""
+    from gptq_triton_amd import _lib
+    from gptq_triton_amd.decoder_ops import add_rms_norm
+    from test_gpu_baseline_shapes import quant_linear
+    G = gptq()
+    hidden, inter, g = 1024, 768, 128
+    gate = O.make_layer(hidden, inter, g, seed=800, act_order=True)
+    up = O.make_layer(hidden, inter, g, seed=801)
+    up["g_idx"] = gate["g_idx"]
+    down = O.make_layer(inter, hidden, g, seed=802, act_order=True)
+    mlp = G.QuantLlamaMLP(quant_linear(gate, hidden, inter, g, True), quant_linear(down, inter, hidden, g, True),
+                          quant_linear(up, hidden, inter, g, True)).cuda()
+    h, d, w = residual_inputs(m, hidden, seed=m + 37)
+    hd, dd, wd = (torch.from_numpy(t).cuda() for t in (h, d, w))
+    lib = _lib.load()
+    lib.gptq4_set_gemv_tuning(gemv_mode, 0, 0, 0)
+    try:
+        s_ref, x_ref = add_rms_norm(hd, dd, wd, 1e-6)
+        y_ref = mlp(x_ref)
+        s, y = mlp.forward_normed(hd, dd, wd, 1e-6)
+    finally:
+        lib.gptq4_set_gemv_tuning(1, 0, 0, 0)
+    assert torch.equal(s, s_ref) and torch.equal(y, y_ref)
+    ref = O.mlp_gateup_ref(x_ref.cpu().numpy(), (gate["qweight"], gate["qzeros"], gate["scales"], gate["g_idx"]),
+                           (up["qweight"], up["qzeros"], up["scales"], up["g_idx"]), g)
+    assert_close(mlp.gate_up(x_ref).cpu().numpy(), ref, "act-order gate/up on the normalised rows")
+
+
 def test_norm_entry_points_reject_what_they_cannot_take():
     from gptq_triton_amd import _lib
     from gptq_triton_amd.fused_mlp import norm_llama_mlp_4
@@ -156,7 +187,7 @@ def test_norm_entry_points_reject_what_they_cannot_take():
     def call(xp, dp, sp, m):
         return lib.gptq4_norm_mlp_gateup(xp, dp, w.data_ptr(), 1e-6, sp, Dg["qweight"].data_ptr(), Dg["qzeros"].data_ptr(),
                                          Dg["scales"].data_ptr(), Du["qweight"].data_ptr(), Du["qzeros"].data_ptr(),
-                                         Du["scales"].data_ptr(), out.data_ptr(), m, hidden, inter, g, ws.data_ptr(),
+                                         Du["scales"].data_ptr(), None, out.data_ptr(), m, hidden, inter, g, ws.data_ptr(),
                                          ws.numel(), _lib.current_stream(x.device))
 
     s = torch.empty_like(x)
@@ -168,15 +199,15 @@ def test_norm_entry_points_reject_what_they_cannot_take():
     torch.cuda.synchronize()
 
 
-@pytest.mark.parametrize("bsz", [1, 3])
-def test_decoder_with_norm_in_matmul_gives_the_same_tokens(tmp_path, split_k_kernel_only, monkeypatch, bsz):
+@pytest.mark.parametrize("bsz,act_order", [(1, False), (3, False), (2, True)])
+def test_decoder_with_norm_in_matmul_gives_the_same_tokens(tmp_path, split_k_kernel_only, monkeypatch, bsz, act_order):
     """GreedyDecoder takes the 5-launch layer when it can; its tokens (eager and graph-replayed) equal
     those of the 7-launch layer."""
     import gptq_triton_amd as G
     from gptq_triton_amd import decoder_ops
     from gptq_triton_amd.llama import GreedyDecoder
     from test_loader import make_checkpoint
-    cfg = make_checkpoint(tmp_path, 128, seed=21)
+    cfg = make_checkpoint(tmp_path, 128, seed=21, act_order=act_order)
     model = G.load_quant(str(tmp_path), device="cuda", fuse_mlp=True)
     torch.manual_seed(5)
     ids = torch.randint(0, cfg.vocab_size, (bsz, 9)).cuda()
@@ -191,7 +222,7 @@ def test_decoder_with_norm_in_matmul_gives_the_same_tokens(tmp_path, split_k_ker
     fused_eager = model.generate_greedy(ids, 10)
     assert len(calls) > 0, "the decode steps must have taken the fused-norm layer"
     fused_graph = model.generate_greedy(ids, 10, use_graph=True)
-    monkeypatch.setattr(decoder_ops, "norm_fusable", lambda rows, hidden, perm=None: False)
+    monkeypatch.setattr(decoder_ops, "norm_fusable", lambda rows, hidden: False)
     n = len(calls)
     plain = model.generate_greedy(ids, 10)
     assert len(calls) == n, "with the fused norm switched off no call may reach it"
