@@ -14,13 +14,22 @@ from . import _lib
 
 # limits of the matmul kernels that normalise their own input (gptq4_norm_qkv_rotary, gptq4_norm_mlp_gateup)
 NORM_MAX_ROWS, NORM_MAX_HIDDEN = 4, 8192
+# up to how many rows the decoder uses them: one row costs 1.3-1.4 us on top of the plain projection against
+# a 4.7 us norm launch; two rows about as much as the launch, three and four more (every workgroup
+# normalises every row)
+NORM_PAYS_ROWS = 1
 # GPTQ4_NORM_FUSION=0 in the environment keeps the norms as launches of their own (for A/B timing)
 NORM_FUSION = os.environ.get("GPTQ4_NORM_FUSION", "1") != "0"
 
 
 def norm_fusable(rows: int, hidden: int) -> bool:
-    """Whether a projection of `rows` rows can take the residual add + RMSNorm of its input along."""
-    return NORM_FUSION and 0 < rows <= NORM_MAX_ROWS and hidden <= NORM_MAX_HIDDEN and hidden % 8 == 0
+    """Whether a projection of `rows` rows CAN take the residual add + RMSNorm of its input along."""
+    return 0 < rows <= NORM_MAX_ROWS and hidden <= NORM_MAX_HIDDEN and hidden % 8 == 0
+
+
+def norm_fusion_pays(rows: int, hidden: int) -> bool:
+    """Whether it is also the faster way (what the decoder asks)."""
+    return NORM_FUSION and rows <= NORM_PAYS_ROWS and norm_fusable(rows, hidden)
 
 
 def check_norm_args(h: torch.Tensor, delta, weight: torch.Tensor):

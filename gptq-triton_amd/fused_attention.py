@@ -197,8 +197,9 @@ class QuantLlamaAttention(nn.Module):
                           perm=perm, kv_out=kv_out, kv_offset=kv_offset, norm=norm)
 
     def norm_fusable(self, rows: int) -> bool:
-        from .decoder_ops import norm_fusable
-        return norm_fusable(rows, self.hidden_size)
+        """Whether project_qkv(norm=...) is the faster way for this many rows."""
+        from .decoder_ops import norm_fusion_pays
+        return norm_fusion_pays(rows, self.hidden_size)
 
     def forward(
         self,

@@ -123,8 +123,9 @@ class QuantLlamaMLP(nn.Module):
         return self.down_proj(self.gate_up(x))
 
     def norm_fusable(self, rows: int) -> bool:
-        from .decoder_ops import norm_fusable
-        return norm_fusable(rows, self.infeatures)
+        """Whether forward_normed is the faster way for this many rows."""
+        from .decoder_ops import norm_fusion_pays
+        return norm_fusion_pays(rows, self.infeatures)
 
     def forward_normed(self, h: torch.Tensor, delta: Optional[torch.Tensor], norm_weight: torch.Tensor, eps: float):
         """(h + delta, forward(RMSNorm(h + delta))): the residual add and the norm run inside the gate/up launch."""

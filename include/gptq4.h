@@ -131,7 +131,8 @@ int gptq4_qkv_rotary(const void *x, const int32_t *qweight, const int32_t *qzero
  * then gptq4_qkv_rotary / gptq4_mlp_gateup on xn.  x, delta (nullable), sum_out fp16 [M, K], norm_weight
  * fp16 [K]; bit-identical to gptq4_add_rmsnorm (or gptq4_rmsnorm) followed by the plain entry point.
  * Decode-sized calls only: M <= 4, K <= 8192 (else -GPTQ4_E_SHAPE: run the two calls); perm as in the
- * plain entry points.  sum_out must not be x or delta: other workgroups of the launch still read them.
+ * plain entry points.  Every workgroup normalises every row, so it is the faster way for one row (1.3-1.4 us
+ * on top of the plain projection against a 4.7 us norm launch), about even for two, slower beyond.  sum_out must not be x or delta: other workgroups of the launch still read them.
  * No reference counterpart (the reference runs LlamaRMSNorm as separate torch kernels,
  * src/gptq_triton/__init__.py:32-47). */
 int gptq4_norm_qkv_rotary(const void *x, const void *delta, const void *norm_weight, float eps, void *sum_out,

@@ -211,6 +211,7 @@ def test_decoder_with_norm_in_matmul_gives_the_same_tokens(tmp_path, split_k_ker
     model = G.load_quant(str(tmp_path), device="cuda", fuse_mlp=True)
     torch.manual_seed(5)
     ids = torch.randint(0, cfg.vocab_size, (bsz, 9)).cuda()
+    monkeypatch.setattr(decoder_ops, "NORM_PAYS_ROWS", 4)   # by default only one-row steps take the 5-launch layer
     calls = []
     real = model.model.layers[0].mlp.forward_normed.__func__
 
@@ -222,7 +223,7 @@ def test_decoder_with_norm_in_matmul_gives_the_same_tokens(tmp_path, split_k_ker
     fused_eager = model.generate_greedy(ids, 10)
     assert len(calls) > 0, "the decode steps must have taken the fused-norm layer"
     fused_graph = model.generate_greedy(ids, 10, use_graph=True)
-    monkeypatch.setattr(decoder_ops, "norm_fusable", lambda rows, hidden: False)
+    monkeypatch.setattr(decoder_ops, "NORM_PAYS_ROWS", 0)
     n = len(calls)
     plain = model.generate_greedy(ids, 10)
     assert len(calls) == n, "with the fused norm switched off no call may reach it"
