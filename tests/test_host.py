@@ -218,3 +218,22 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     layer = G.QuantLinear(4, 128, 256, 256, bias=False)
     with pytest.raises((_lib.LibraryMissing, RuntimeError, AssertionError)):
         layer(torch.zeros((1, 256), dtype=torch.float16))
+
+
+def test_norm_entry_points_check_their_arguments_on_the_host():
+    lib = _lib.load()
+    fake, ws = 0x1000, 1 << 20
+
+    def gateup(m, k, delta, weight, sums):
+        return lib.gptq4_norm_mlp_gateup(fake, delta, weight, 1e-6, sums, fake, fake, fake, fake, fake, fake, None, fake,
+                                         m, k, 11008, 128, fake, ws, None)
+
+    assert gateup(1, 4096, fake, None, fake) == -1            # no norm weight
+    assert gateup(1, 4096, fake, fake, None) == -1            # a delta but nowhere to put the sums
+    assert gateup(5, 4096, fake, fake, 0x2000) == -2          # more rows than the kernels normalise themselves
+    assert gateup(1, 8192 + 128, fake, fake, 0x2000) == -2    # rows longer than they keep in registers
+    assert gateup(1, 4096, fake, fake, fake) == -2            # sums over the input
+    assert gateup(1, 4096, 0x3000, fake, 0x3000) == -2        # sums over the delta
+    assert gateup(1, 4096, fake + 2, fake, 0x2000) == -5      # misaligned delta
+    args = [fake, None, None, 1e-6, None, fake, fake, fake, None, fake, fake, fake, 2048, fake, fake, fake]
+    assert lib.gptq4_norm_qkv_rotary(*args, 1, 1, 32, 128, 4096, -1, 1, 0, fake, ws, None) == -1   # no norm weight
