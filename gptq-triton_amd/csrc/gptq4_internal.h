@@ -104,11 +104,13 @@ struct KslicePlan {
     int mt;      // 32-row blocks per row tile (1 or 2)
     int splitk;  // workgroups sharing one tile along K, on top of the split inside the workgroup
     int tiles;
+    bool wide;   // plain epilogue: 128-column strips (two blocks per wave tile) instead of 64
     bool ok;     // false: the shape needs another kernel
 };
 struct KsliceTuning {
     int mode;        // 0 never, 1 where it is the faster kernel, 2 wherever it can run
     int mt, splitk;  // 0 = automatic
+    int wide;        // plain epilogue: 1 = 128-column strips, -1 = 64-column strips, 0 = automatic
 };
 extern KsliceTuning g_kslice_tuning;
 KslicePlan kslice_plan(int epi, int M, int N, int K, bool has_perm);

@@ -11,7 +11,7 @@
 // is summed and finished by wave mt.
 //
 // Wave tile: (32*MT) rows x NB blocks of 64 columns.
-//   plain   : NB = 1, one 64-column strip.
+//   plain   : NB = 1, one 64-column strip; or (WIDE, long K and many rows) NB = 2, two adjacent strips.
 //   SiLU*mul: NB = 2, the same 64 columns of the gate and of the up matrix.
 //   rotary  : NB = 2, columns [0, 64) and [64, 128) of one head, so the wave that finishes
 //             a row block holds d and d + 64 itself.
@@ -26,12 +26,15 @@ namespace {
 
 constexpr int BK = 64;
 
-template <int EPI, int MT>
+// WIDE (plain epilogue only): two adjacent 64-column blocks per wave tile, like a rotary head.
+template <int EPI, int MT, bool WIDE>
 __global__ __launch_bounds__(256, 2) void gptq4_kslice_kernel(MatmulArgs p) {
+    static_assert(!WIDE || EPI == EPI_PLAIN, "the other epilogues have two blocks already");
+    constexpr bool ADJ = (EPI == EPI_ROPE) || WIDE;     // the second block is columns + 64 of the same matrix
     constexpr int BM = 32 * MT;
     constexpr int KS = 4;                               // all four waves along K
-    constexpr int NB = (EPI == EPI_PLAIN) ? 1 : 2;      // 64-column blocks of the wave tile
-    constexpr int BN = (EPI == EPI_ROPE) ? 128 : 64;    // output columns of the workgroup
+    constexpr int NB = (EPI == EPI_PLAIN && !WIDE) ? 1 : 2;  // 64-column blocks of the wave tile
+    constexpr int BN = ADJ ? 128 : 64;                  // output columns of the workgroup
     constexpr int NSET = NB;                            // value sets the finishing wave combines
     constexpr int A_HALVES = BM * BK;                   // one wave's K tile of activations
     constexpr int A_UNITS = BM / 8;                     // LDS-direct loads per wave and K tile (8 rows each)
@@ -82,9 +85,9 @@ __global__ __launch_bounds__(256, 2) void gptq4_kslice_kernel(MatmulArgs p) {
         qz_[j] = p.w[j].qzeros + (ncol >> 3);
         sc_[j] = p.w[j].scales + ncol;
     }
-    auto bptr = [&](int j) { return (EPI == EPI_ROPE) ? bptr_[0] + 64 * j : bptr_[j < NPTR ? j : 0]; };
-    auto qz = [&](int j) { return (EPI == EPI_ROPE) ? qz_[0] + 8 * j : qz_[j < NPTR ? j : 0]; };
-    auto sc = [&](int j) { return (EPI == EPI_ROPE) ? sc_[0] + 64 * j : sc_[j < NPTR ? j : 0]; };
+    auto bptr = [&](int j) { return ADJ ? bptr_[0] + 64 * j : bptr_[j < NPTR ? j : 0]; };
+    auto qz = [&](int j) { return ADJ ? qz_[0] + 8 * j : qz_[j < NPTR ? j : 0]; };
+    auto sc = [&](int j) { return ADJ ? sc_[0] + 64 * j : sc_[j < NPTR ? j : 0]; };
     const int tiles_per_group = p.groupsize / BK;
     const int last_group = K / p.groupsize - 1;
 
@@ -338,15 +341,18 @@ __global__ __launch_bounds__(256, 2) void gptq4_kslice_kernel(MatmulArgs p) {
     // ---- epilogue of row block `wave`
     const int row0 = m0 + wave * 32 + 4 * lhi;
     if (EPI == EPI_PLAIN) {
-        h2_t bias2 = {(half_t)0.f, (half_t)0.f};
-        if (p.bias != nullptr) bias2 = as_h2(*reinterpret_cast<const uint32_t *>(p.bias + ncol));
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int row = row0 + 8 * (i >> 2) + (i & 3);
-            if (row < M) {
-                h2_t o = {(half_t)vals[0][0][i], (half_t)vals[0][1][i]};
-                if (p.bias != nullptr) o = o + bias2;
-                *reinterpret_cast<uint32_t *>(p.y + (size_t)row * N + ncol) = as_u32(o);
+        for (int j = 0; j < NSET; ++j) {
+            h2_t bias2 = {(half_t)0.f, (half_t)0.f};
+            if (p.bias != nullptr) bias2 = as_h2(*reinterpret_cast<const uint32_t *>(p.bias + ncol + 64 * j));
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int row = row0 + 8 * (i >> 2) + (i & 3);
+                if (row < M) {
+                    h2_t o = {(half_t)vals[j][0][i], (half_t)vals[j][1][i]};
+                    if (p.bias != nullptr) o = o + bias2;
+                    *reinterpret_cast<uint32_t *>(p.y + (size_t)row * N + ncol + 64 * j) = as_u32(o);
+                }
             }
         }
     } else if (EPI == EPI_SILU_MUL) {
@@ -406,21 +412,23 @@ __global__ __launch_bounds__(256, 2) void gptq4_kslice_kernel(MatmulArgs p) {
     }
 }
 
-template <int EPI, int MT>
+template <int EPI, int MT, bool WIDE>
 int launch_one(const MatmulArgs &a, int tiles, hipStream_t stream) {
     dim3 grid((unsigned)tiles, (unsigned)a.splitk), block(256);
-    hipLaunchKernelGGL((gptq4_kslice_kernel<EPI, MT>), grid, block, 0, stream, a);
+    hipLaunchKernelGGL((gptq4_kslice_kernel<EPI, MT, WIDE>), grid, block, 0, stream, a);
     return (int)hipGetLastError();
 }
 
 template <int EPI>
 int launch_epi(const MatmulArgs &a, const KslicePlan &pl, hipStream_t stream) {
-    return pl.mt == 1 ? launch_one<EPI, 1>(a, pl.tiles, stream) : launch_one<EPI, 2>(a, pl.tiles, stream);
+    if (EPI == EPI_PLAIN && pl.wide)
+        return pl.mt == 1 ? launch_one<EPI_PLAIN, 1, true>(a, pl.tiles, stream) : launch_one<EPI_PLAIN, 2, true>(a, pl.tiles, stream);
+    return pl.mt == 1 ? launch_one<EPI, 1, false>(a, pl.tiles, stream) : launch_one<EPI, 2, false>(a, pl.tiles, stream);
 }
 
 }  // namespace
 
-KsliceTuning g_kslice_tuning = {1, 0, 0};
+KsliceTuning g_kslice_tuning = {1, 0, 0, 0};
 
 // Row tile: 32 rows up to M = 32, else 64 (128-row tiles decode each weight once instead of
 // twice at M = 128, but their 128 KiB of LDS leaves one wave per SIMD and they come out no
@@ -430,7 +438,11 @@ KsliceTuning g_kslice_tuning = {1, 0, 0};
 KslicePlan kslice_plan(int epi, int M, int N, int K, bool has_perm) {
     KslicePlan pl = {};
     const int ks = 4;
-    const int bn = (epi == EPI_ROPE) ? 128 : 64;
+    // plain projections: 128-column strips (half the activation traffic per weight byte, half the tiles) pay
+    // from 256 rows on when K is long (LLaMA-7B down_proj: 39.8 -> 37.3 us at 256 rows, 66.2 -> 61.1 at 512;
+    // o_proj with K = 4096 loses below 512 rows)
+    pl.wide = epi == EPI_PLAIN && (g_kslice_tuning.wide > 0 || (g_kslice_tuning.wide == 0 && M >= 256 && K >= 8192));
+    const int bn = (epi == EPI_ROPE || pl.wide) ? 128 : 64;
     const int nk = K / 64;
     pl.mt = g_kslice_tuning.mt ? g_kslice_tuning.mt : (M <= 32 ? 1 : 2);
     const int bm = 32 * pl.mt;
@@ -439,7 +451,7 @@ KslicePlan kslice_plan(int epi, int M, int N, int K, bool has_perm) {
     if (g_kslice_tuning.splitk > 0) {
         s = g_kslice_tuning.splitk;
     } else {
-        s = ((epi == EPI_PLAIN) ? 512 : 256) / pl.tiles;  // the two-block wave tiles: one workgroup per CU
+        s = ((epi == EPI_PLAIN && !pl.wide) ? 512 : 256) / pl.tiles;  // the two-block wave tiles: one workgroup per CU
         if (s > nk / (4 * ks)) s = nk / (4 * ks);
     }
     if (s > GEMM_MAX_SPLITK) s = GEMM_MAX_SPLITK;
@@ -451,7 +463,7 @@ KslicePlan kslice_plan(int epi, int M, int N, int K, bool has_perm) {
 }
 
 size_t kslice_partial_bytes(int epi, const KslicePlan &pl) {
-    const int nset = (epi == EPI_PLAIN) ? 1 : 2;
+    const int nset = (epi == EPI_PLAIN && !pl.wide) ? 1 : 2;
     return pl.splitk > 1 ? (size_t)pl.tiles * pl.splitk * pl.mt * nset * 32 * 64 * sizeof(float) : 0;
 }
 

@@ -184,8 +184,9 @@ void gptq4_set_gemm_tuning(int mt, int splitk);
 
 /* Same for the mid-M kernel (M > 16 with too few wide tiles for the tiled kernel; K is split
  * across the four waves of a workgroup): mode 0 = never use it, 1 = where it is the faster
- * kernel, 2 = wherever it can run; 32-row blocks per row tile (1, 2) and the split-K
- * factor across workgroups; 0 = automatic. */
+ * kernel, 2 = wherever it can run; 32-row blocks per row tile (1, 2; 10 + that, or 10 alone, also
+ * selects 128-column strips for plain projections, a plain 1 or 2 the 64-column strips) and the
+ * split-K factor across workgroups; 0 = automatic. */
 void gptq4_set_midm_tuning(int mode, int mt, int splitk);
 
 /* Same for the balanced decode GEMV (M <= 4): mode 0 = never use it, 1 = where it is the

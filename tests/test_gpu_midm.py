@@ -13,7 +13,7 @@ from test_gpu_parity import assert_close, gptq
 pytestmark = pytest.mark.gpu
 
 # (32-row blocks per row tile, split-K across workgroups); 0 = automatic
-CONFIGS = [(0, 0), (1, 1), (2, 1), (1, 2), (2, 3)]
+CONFIGS = [(0, 0), (1, 1), (2, 1), (1, 2), (2, 3), (10, 0), (11, 1), (12, 3)]
 
 
 @pytest.fixture(params=CONFIGS, ids=lambda c: "mt%d_s%d" % c)
