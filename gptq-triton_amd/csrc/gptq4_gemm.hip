@@ -572,6 +572,10 @@ GemmPlan gemm_plan(int epi, int M, int N, int K) {
         pl.mt = g_gemm_tuning.mt;
     } else if (wide >= 192) {
         pl.mt = 4;
+        // just over one workgroup per CU (257..384 tiles, e.g. N = 5120 at 2048 rows): a quarter of the CUs
+        // would run two tiles and set the pace; with a long K, three splits fill the chip 3.75 times over
+        // instead (measured: LLaMA-13B down_proj at 2048 rows 337 -> 297 us)
+        if (wide > 256 && wide <= 384 && nk >= 128) s = 3;
     } else if (wide >= 128 && nk >= 32) {
         pl.mt = 4;
         s = 2;
