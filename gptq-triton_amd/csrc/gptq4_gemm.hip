@@ -562,30 +562,54 @@ GemmTuning g_gemm_tuning = {0, 0};
 // CUs out of four a workgroup; from half the CUs on it still wins with K split in two.
 // Below that, 128 x 128 tiles, with K split when even those leave most CUs idle (the
 // M = 17..255 range on narrow layers).
+// How evenly `w` workgroups of equal work fill 256 CUs that hold two of them each: up to 256 every
+// workgroup has a CU to itself, beyond that they run in rounds of 512.  What this captures is the
+// cliff just above a multiple of the CU count (a few CUs run one workgroup more than the rest and
+// set the pace).
+static double fill_efficiency(long w) {
+    if (w <= 256) return (double)w / 256.0;
+    return (double)w / (512.0 * (double)((w + 511) / 512));
+}
+
 GemmPlan gemm_plan(int epi, int M, int N, int K) {
     GemmPlan pl;
     const int bn2 = (epi == EPI_SILU_MUL) ? 64 : 128;  // tile width at MT = 2; twice that at MT = 4
     const int nk = K / 64;
     const long wide = (long)((M + 127) / 128) * (N / (2 * bn2));
     int s = 1;
+    bool scored = false;
     if (g_gemm_tuning.mt) {
         pl.mt = g_gemm_tuning.mt;
-    } else if (wide >= 192) {
+    } else if (wide >= 512) {
         pl.mt = 4;
-        // just over one workgroup per CU (257..384 tiles, e.g. N = 5120 at 2048 rows): a quarter of the CUs
-        // would run two tiles and set the pace; with a long K, three splits fill the chip 3.75 times over
-        // instead (measured: LLaMA-13B down_proj at 2048 rows 337 -> 297 us)
-        if (wide > 256 && wide <= 384 && nk >= 128) s = 3;
-    } else if (wide >= 128 && nk >= 32) {
-        pl.mt = 4;
-        s = 2;
+    } else if (wide >= 96 && nk >= 32) {
+        // Few enough tiles for their count to matter: score (tile, split) candidates by how evenly they fill
+        // the chip, the narrow tile at 0.85 of the wide one's rate, every extra split at 5 % + 20 / (K tiles)
+        // of the time (the exchange of partial sums weighs more on a short K).  Fitted to LLaMA-7B / 13B /
+        // 30B shapes at 896..2048 rows; e.g. 13824 x 5120: 337 -> 297 us at 2048 rows and 193 -> 163 at 1024,
+        // 17920 x 6656 at 1536 rows: 435 -> 367 (three splits each); 4096 x 4096 at 1024 rows: 59 -> 50 us
+        // (256 narrow tiles, no split).
+        const double pen = 0.05 + 20.0 / (double)nk;
+        double best = -1.0;
+        for (int mt = 4; mt >= 2; mt -= 2) {
+            const long tiles = (mt == 4) ? wide : 2 * wide;
+            for (int c = 1; c <= 4 && c <= nk / 8; ++c) {
+                const double score = fill_efficiency(tiles * c) * (mt == 4 ? 1.0 : 0.85) / (1.0 + pen * (c - 1));
+                if (score > best + 1e-9) {
+                    best = score;
+                    pl.mt = mt;
+                    s = c;
+                }
+            }
+        }
+        scored = true;
     } else {
         pl.mt = 2;
     }
     pl.tiles = ((M + 127) / 128) * (N / (pl.mt == 4 ? 2 * bn2 : bn2));
     if (g_gemm_tuning.splitk > 0) {
         s = g_gemm_tuning.splitk;
-    } else if (pl.mt == 2 && pl.tiles < 384) {
+    } else if (pl.mt == 2 && pl.tiles < 384 && !scored) {
         s = (512 + pl.tiles / 2) / pl.tiles;  // aim for ~2 workgroups per CU
         if (s > nk / 8) s = nk / 8;            // keep at least 8 K tiles (512 k) per split
     }
