@@ -108,18 +108,24 @@ int setup_norm(MatmulArgs &a, const void *delta, const void *norm_weight, void *
     return 0;
 }
 
-// M > 16: the mid-M kernel where it is the faster one, else the tiled kernel.
-bool prefer_kslice(const KslicePlan &kp, int epi, int M, int N) {
+// M > 16: the mid-M kernel where it is the faster one, else the tiled kernel.  Measured at LLaMA-7B /
+// 13B / 30B shapes, 256..768 rows: the tiled kernel takes over once it has enough wide tiles (72 for a plain
+// projection, 160 for the gate/up pair, 192 with the rotary epilogue) - with the rotary epilogue not while
+// their number fills the chip badly (just over one per CU with a short K, where splitting does not pay either).
+bool prefer_kslice(const KslicePlan &kp, int epi, int M, int N, int K) {
     if (!kp.ok || g_kslice_tuning.mode == 0) return false;
     if (g_kslice_tuning.mode == 2) return true;
-    // up to 768 rows, while the tiled kernel's wide tiles would leave a quarter of the CUs idle
+    if (M > 768) return false;
     const int wide_bn = (epi == EPI_SILU_MUL) ? 128 : 256;
-    return M <= 768 && (long)((M + 127) / 128) * (N / wide_bn) < 192;
+    const long wide = (long)((M + 127) / 128) * (N / wide_bn);
+    if (epi == EPI_PLAIN) return wide < 72;
+    if (epi == EPI_SILU_MUL) return wide < 160;
+    return wide < 192 || gemm_plan(epi, M, N, K).score < 0.65;
 }
 
 int run_tiled(int epi, MatmulArgs &a, void *workspace, size_t workspace_bytes, hipStream_t s) {
     const KslicePlan kp = kslice_plan(epi, a.M, a.N, a.K, a.perm != nullptr);
-    if (prefer_kslice(kp, epi, a.M, a.N)) {
+    if (prefer_kslice(kp, epi, a.M, a.N, a.K)) {
         a.tiles = kp.tiles;
         a.splitk = kp.splitk;
         const int nk = a.K / 64;

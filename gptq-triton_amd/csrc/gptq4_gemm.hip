@@ -573,6 +573,7 @@ static double fill_efficiency(long w) {
 
 GemmPlan gemm_plan(int epi, int M, int N, int K) {
     GemmPlan pl;
+    pl.score = 1.0;
     const int bn2 = (epi == EPI_SILU_MUL) ? 64 : 128;  // tile width at MT = 2; twice that at MT = 4
     const int nk = K / 64;
     const long wide = (long)((M + 127) / 128) * (N / (2 * bn2));
@@ -598,6 +599,7 @@ GemmPlan gemm_plan(int epi, int M, int N, int K) {
                 if (score > best + 1e-9) {
                     best = score;
                     pl.mt = mt;
+                    pl.score = score;
                     s = c;
                 }
             }

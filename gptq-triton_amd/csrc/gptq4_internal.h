@@ -89,6 +89,7 @@ struct GemmPlan {
     int mt;      // 32-row tiles per wave: 2 = 128 x 128 workgroup tile (2 x 2 waves), 4 = 128 x 256 (1 x 4 waves)
     int splitk;  // workgroups sharing one tile along K
     int tiles;
+    double score;  // expected efficiency of the choice: fill of the chip / cost of the splits (1 where the tile count is large)
 };
 struct GemmTuning {
     int mt, splitk;  // 0 = automatic
