@@ -153,3 +153,48 @@ def test_graph_replays_equal_eager_launches(m):
     ref = O.quant_matmul_ref(x.cpu().numpy(), L["qweight"], L["qzeros"], L["scales"], g)
     ok, max_abs, _ = O.within_tolerance(y.cpu().numpy(), ref)
     assert ok, max_abs
+
+
+@pytest.mark.parametrize("m", [40, 200])
+def test_in_kernel_act_order_gather_with_fused_epilogues(m):
+    """The Python layer permutes tall act-order inputs before the call; a direct caller of the C ABI may pass
+    `perm` instead, and the tiled kernel then gathers the activations itself - also under the SiLU*mul and
+    the rotary epilogue."""
+    from gptq_triton_amd import _lib
+    G = gptq()
+    lib = _lib.load()
+    k, n, g, heads = 1024, 768, 128, 8
+    gate = O.make_layer(k, n, g, seed=90, act_order=True)
+    up = O.make_layer(k, n, g, seed=91)
+    up["g_idx"] = gate["g_idx"]
+    qkv = O.make_layer(k, 3 * k, g, seed=92, act_order=True)
+    x = O.make_x(m, k, seed=93)
+    xd = torch.from_numpy(x).cuda()
+    Dg, Du, Dq = to_dev(gate), to_dev(up), to_dev(qkv)
+    gq, perm = G.prepare_act_order(Dg["qweight"], Dg["g_idx"], g)
+    uq, _ = G.prepare_act_order(Du["qweight"], Dg["g_idx"], g)
+    qq, qperm = G.prepare_act_order(Dq["qweight"], Dq["g_idx"], g)
+    stream = _lib.current_stream(xd.device)
+    h = torch.empty((m, n), dtype=torch.float16, device="cuda")
+    ws = _lib.workspace(xd.device, max(lib.gptq4_workspace_bytes(_lib.OP_MLP_GATEUP, m, k, n),
+                                       lib.gptq4_workspace_bytes(_lib.OP_QKV_ROTARY, m, k, 3 * k)))
+    rc = lib.gptq4_mlp_gateup(xd.data_ptr(), gq.data_ptr(), Dg["qzeros"].data_ptr(), Dg["scales"].data_ptr(),
+                              uq.data_ptr(), Du["qzeros"].data_ptr(), Du["scales"].data_ptr(), perm.data_ptr(),
+                              h.data_ptr(), m, k, n, g, ws.data_ptr(), ws.numel(), stream)
+    assert rc == 0
+    href = O.mlp_gateup_ref(x, (gate["qweight"], gate["qzeros"], gate["scales"], gate["g_idx"]),
+                            (up["qweight"], up["qzeros"], up["scales"], up["g_idx"]), g)
+    assert_close(h.cpu().numpy(), href, f"in-kernel gather, gate/up M={m}")
+    cos, sin = G.RotaryTable(128, 2048).get(torch.device("cuda"), 2048)
+    pos = np.arange(m, dtype=np.int32)[None, :]
+    pd = torch.from_numpy(pos).cuda()
+    q = torch.empty((1, heads, m, 128), dtype=torch.float16, device="cuda")
+    kk, vv = torch.empty_like(q), torch.empty_like(q)
+    rc = lib.gptq4_qkv_rotary(xd.data_ptr(), qq.data_ptr(), Dq["qzeros"].data_ptr(), Dq["scales"].data_ptr(), qperm.data_ptr(),
+                              pd.data_ptr(), cos.data_ptr(), sin.data_ptr(), cos.shape[0], q.data_ptr(), kk.data_ptr(),
+                              vv.data_ptr(), 1, m, heads, 128, k, g, m, 0, ws.data_ptr(), ws.numel(), stream)
+    assert rc == 0
+    qr, kr, vr = O.qkv_rotary_ref(x.reshape(1, m, k), qkv["qweight"], qkv["qzeros"], qkv["scales"], g, pos, heads, 128,
+                                  g_idx=qkv["g_idx"], max_pos=2048)
+    for got, want, name in ((q, qr, "q"), (kk, kr, "k"), (vv, vr, "v")):
+        assert_close(got.cpu().numpy(), want, f"in-kernel gather, {name} M={m}")
