@@ -450,7 +450,10 @@ int launch_norm_variant(const MatmulArgs &a, const GemvPlan &pl, hipStream_t str
 
 template <int EPI>
 int launch_epi(const MatmulArgs &a, const GemvPlan &pl, hipStream_t stream) {
-    if (a.nrm_weight != nullptr) return launch_norm_variant<EPI>(a, pl, stream);
+    if (a.nrm_weight != nullptr) {
+        if (EPI == EPI_PLAIN) return (int)hipErrorInvalidValue;  // no entry point asks a plain projection for it
+        return launch_norm_variant<(EPI == EPI_PLAIN) ? EPI_SILU_MUL : EPI>(a, pl, stream);
+    }
     const int key = pl.waves * 10 + pl.depth;
     switch (key) {
         case 41: return launch_variant<EPI, 1, 4>(a, pl, stream);

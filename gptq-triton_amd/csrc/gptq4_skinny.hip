@@ -526,7 +526,7 @@ int launch_skinny(int epi, const MatmulArgs &a, const SkinnyPlan &pl, hipStream_
         // checked by the caller: automatic plan (8-byte loads, 4 waves), M <= NORM_MAX_M, K <= NORM_MAX_H
         if (epi == EPI_SILU_MUL) return launch_norm_variant<EPI_SILU_MUL, 1>(a, stream);
         if (epi == EPI_ROPE) return launch_norm_variant<EPI_ROPE, 2>(a, stream);
-        return launch_norm_variant<EPI_PLAIN, 2>(a, stream);
+        return (int)hipErrorInvalidValue;  // no entry point asks a plain projection to normalise its input
     }
     switch (epi) {
         case EPI_PLAIN: return launch_epi<EPI_PLAIN>(a, pl, stream);

@@ -13,7 +13,7 @@ from test_gpu_parity import assert_close, gptq
 pytestmark = pytest.mark.gpu
 
 # (units in flight, waves per workgroup, waves per CU); 0 = automatic
-CONFIGS = [(0, 0, 0), (3, 8, 16), (2, 16, 16), (2, 8, 4), (1, 8, 8), (2, 4, 8)]
+CONFIGS = [(0, 0, 0), (3, 8, 16), (2, 16, 16), (2, 8, 4), (1, 8, 8), (2, 4, 8), (3, 4, 8)]
 
 
 @pytest.fixture(params=CONFIGS, ids=lambda c: "d%d_w%d_cu%d" % c)
@@ -67,6 +67,33 @@ def test_gemv_act_order(forced_gemv, m):
     y = layer.cuda()(torch.from_numpy(x).cuda())
     ref = O.quant_matmul_ref(x, L["qweight"], L["qzeros"], L["scales"], g, g_idx=L["g_idx"])
     assert_close(y.cpu().numpy(), ref, f"gemv act-order M={m}")
+
+
+@pytest.mark.parametrize("m", [1, 4])
+def test_gemv_act_order_fused_epilogues(forced_gemv, m):
+    """Act-order under the SiLU*mul and the rotary epilogue: the waves gather their x slices through perm."""
+    G = gptq()
+    k, n, g, heads = 1024, 768, 128, 8
+    gate = O.make_layer(k, n, g, seed=60, act_order=True)
+    up = O.make_layer(k, n, g, seed=61)
+    qkv = O.make_layer(k, 3 * k, g, seed=62)
+    up["g_idx"] = qkv["g_idx"] = gate["g_idx"]
+    Dg, Du, Dq = to_dev(gate), to_dev(up), to_dev(qkv)
+    gq, perm = G.prepare_act_order(Dg["qweight"], Dg["g_idx"], g)
+    uq, _ = G.prepare_act_order(Du["qweight"], Dg["g_idx"], g)
+    qq, _ = G.prepare_act_order(Dq["qweight"], Dg["g_idx"], g)
+    x = O.make_x(m, k, seed=63 + m)
+    xd = torch.from_numpy(x).cuda()
+    h = G.llama_mlp_4(g, xd, gq, Dg["scales"], Dg["qzeros"], uq, Du["scales"], Du["qzeros"], perm=perm)
+    gi = gate["g_idx"]
+    href = O.mlp_gateup_ref(x, (gate["qweight"], gate["qzeros"], gate["scales"], gi), (up["qweight"], up["qzeros"], up["scales"], gi), g)
+    assert_close(h.cpu().numpy(), href, f"gemv act-order gate/up M={m}")
+    cos, sin = G.RotaryTable(128, 2048).get(torch.device("cuda"), 2048)
+    pos = (np.arange(m) * 7 + 3)[:, None].astype(np.int32)
+    q, kk, vv = G.qkv_rotary(g, xd.view(m, 1, k), qq, Dq["scales"], Dq["qzeros"], torch.from_numpy(pos).cuda(), cos, sin, heads, perm=perm)
+    qr, kr, vr = O.qkv_rotary_ref(x.reshape(m, 1, k), qkv["qweight"], qkv["qzeros"], qkv["scales"], g, pos, heads, 128, g_idx=gi, max_pos=2048)
+    for got, want, name in ((q, qr, "q"), (kk, kr, "k"), (vv, vr, "v")):
+        assert_close(got.cpu().numpy(), want, f"gemv act-order {name} M={m}")
 
 
 @pytest.mark.parametrize("g", [-1, 128])

@@ -162,9 +162,68 @@ def test_norm_with_act_order_equals_two_launches(gemv_mode, m):
     finally:
         lib.gptq4_set_gemv_tuning(1, 0, 0, 0)
     assert torch.equal(s, s_ref) and torch.equal(y, y_ref)
+    # the same through the rotary epilogue
+    heads = hidden // 128
+    qkv = O.make_layer(hidden, 3 * hidden, g, seed=803)
+    Dq = to_dev(qkv)
+    qq, perm = G.prepare_act_order(Dq["qweight"], torch.from_numpy(gate["g_idx"]).cuda(), g)
+    cos, sin = G.RotaryTable(128, 2048).get(torch.device("cuda"), 2048)
+    pos = torch.full((m, 1), 9, dtype=torch.int32, device="cuda")
+    lib.gptq4_set_gemv_tuning(gemv_mode, 0, 0, 0)
+    try:
+        q0, k0, v0 = G.qkv_rotary(g, x_ref.view(m, 1, hidden), qq, Dq["scales"], Dq["qzeros"], pos, cos, sin, heads, perm=perm)
+        q, k, v, s3 = G.qkv_rotary(g, hd.view(m, 1, hidden), qq, Dq["scales"], Dq["qzeros"], pos, cos, sin, heads, perm=perm,
+                                   norm=(dd.view(m, 1, hidden), wd, 1e-6))
+    finally:
+        lib.gptq4_set_gemv_tuning(1, 0, 0, 0)
+    assert torch.equal(q, q0) and torch.equal(k, k0) and torch.equal(v, v0) and torch.equal(s3.view(m, hidden), s_ref)
     ref = O.mlp_gateup_ref(x_ref.cpu().numpy(), (gate["qweight"], gate["qzeros"], gate["scales"], gate["g_idx"]),
                            (up["qweight"], up["qzeros"], up["scales"], up["g_idx"]), g)
     assert_close(mlp.gate_up(x_ref).cpu().numpy(), ref, "act-order gate/up on the normalised rows")
+
+
+@pytest.mark.parametrize("gemv_mode", [0, 2])
+@pytest.mark.parametrize("act_order", [False, True])
+@pytest.mark.parametrize("m", [1, 3])
+def test_norm_with_rows_longer_than_4096(gemv_mode, act_order, m):
+    """Hidden size 5120: four chunks per thread cover a row (the variants LLaMA-13B / 30B decoders run)."""
+    from gptq_triton_amd import _lib
+    from gptq_triton_amd.decoder_ops import add_rms_norm
+    from gptq_triton_amd.fused_mlp import norm_llama_mlp_4
+    G = gptq()
+    hidden, inter, heads, g = 5120, 2816, 40, 128
+    gate = O.make_layer(hidden, inter, g, seed=850, act_order=act_order)
+    up = O.make_layer(hidden, inter, g, seed=851)
+    qkv = O.make_layer(hidden, 3 * hidden, g, seed=852)
+    up["g_idx"] = qkv["g_idx"] = gate["g_idx"]
+    Dg, Du, Dq = to_dev(gate), to_dev(up), to_dev(qkv)
+    gq, uq, qq, perm = Dg["qweight"], Du["qweight"], Dq["qweight"], None
+    if act_order:
+        gq, perm = G.prepare_act_order(Dg["qweight"], Dg["g_idx"], g)
+        uq, _ = G.prepare_act_order(Du["qweight"], Dg["g_idx"], g)
+        qq, _ = G.prepare_act_order(Dq["qweight"], Dg["g_idx"], g)
+    h, d, w = residual_inputs(m, hidden, seed=m + 47)
+    hd, dd, wd = (torch.from_numpy(t).cuda() for t in (h, d, w))
+    pos = torch.full((m, 1), 100, dtype=torch.int32, device="cuda")
+    cos, sin = G.RotaryTable(128, 2048).get(torch.device("cuda"), 2048)
+    lib = _lib.load()
+    lib.gptq4_set_gemv_tuning(gemv_mode, 0, 0, 0)
+    try:
+        s_ref, x_ref = add_rms_norm(hd, dd, wd, 1e-6)
+        mid0 = G.llama_mlp_4(g, x_ref, gq, Dg["scales"], Dg["qzeros"], uq, Du["scales"], Du["qzeros"], perm=perm)
+        q0, k0, v0 = G.qkv_rotary(g, x_ref.view(m, 1, hidden), qq, Dq["scales"], Dq["qzeros"], pos, cos, sin, heads, perm=perm)
+        s, mid = norm_llama_mlp_4(g, hd, dd, wd, 1e-6, gq, Dg["scales"], Dg["qzeros"], uq, Du["scales"], Du["qzeros"], perm=perm)
+        q, k, v, s2 = G.qkv_rotary(g, hd.view(m, 1, hidden), qq, Dq["scales"], Dq["qzeros"], pos, cos, sin, heads, perm=perm,
+                                   norm=(dd.view(m, 1, hidden), wd, 1e-6))
+    finally:
+        lib.gptq4_set_gemv_tuning(1, 0, 0, 0)
+    assert torch.equal(s, s_ref) and torch.equal(s2.view(m, hidden), s_ref)
+    assert torch.equal(mid, mid0)
+    assert torch.equal(q, q0) and torch.equal(k, k0) and torch.equal(v, v0)
+    gi = gate["g_idx"]
+    ref = O.mlp_gateup_ref(x_ref.cpu().numpy(), (gate["qweight"], gate["qzeros"], gate["scales"], gi),
+                           (up["qweight"], up["qzeros"], up["scales"], gi), g)
+    assert_close(mid.cpu().numpy(), ref, f"norm + gate/up hidden 5120 M={m}")
 
 
 def test_norm_entry_points_reject_what_they_cannot_take():

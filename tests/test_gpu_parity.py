@@ -384,39 +384,48 @@ def test_empty_inputs_give_empty_outputs():
     assert rc < 0 and b"shape" in lib.gptq4_strerror(rc).lower()
 
 
-@pytest.mark.parametrize("words,depth", [(1, 2), (1, 4), (2, 1), (2, 4), (4, 1), (4, 2)])
+@pytest.mark.parametrize("words,depth", [(1, 2), (1, 4), (2, 1), (2, 2), (2, 4), (4, 1), (4, 2)])
+@pytest.mark.parametrize("act_order", [False, True])
 @pytest.mark.parametrize("m", [1, 7, 16])
-def test_split_k_kernel_launch_shapes(words, depth, m):
+def test_split_k_kernel_launch_shapes(words, depth, act_order, m):
     """Every load width (4, 8, 16 bytes per lane) and ring depth of the split-K decode kernel, all three
-    epilogues and act-order, with the balanced GEMV switched off so that the calls reach it."""
+    epilogues, with and without act-order, with the balanced GEMV switched off so that the calls reach it."""
     from gptq_triton_amd import _lib
     G = gptq()
     lib = _lib.load()
     k, n, g, heads = 1024, 768, 128, 8   # the oracle's rotary path wants hidden = heads * 128
-    L = O.make_layer(k, n, g, seed=40 + words, act_order=True, bias=True)
-    L2 = O.make_layer(k, n, g, seed=41 + words)
-    Lq = O.make_layer(k, 3 * heads * 128, g, seed=42 + words)
+    gate = O.make_layer(k, n, g, seed=40 + words, act_order=act_order, bias=True)
+    up = O.make_layer(k, n, g, seed=41 + words)
+    up["g_idx"] = gate["g_idx"]
+    qkv = O.make_layer(k, 3 * k, g, seed=42 + words)
+    qkv["g_idx"] = gate["g_idx"]
     x = O.make_x(m, k, seed=43 + m)
     xd = torch.from_numpy(x).cuda()
-    D, D2, Dq = to_dev(L), to_dev(L2), to_dev(Lq)
+    Dg, Du, Dq = to_dev(gate), to_dev(up), to_dev(qkv)
+    gq, uq, qq, perm = Dg["qweight"], Du["qweight"], Dq["qweight"], None
+    if act_order:
+        gq, perm = G.prepare_act_order(Dg["qweight"], Dg["g_idx"], g)
+        uq, _ = G.prepare_act_order(Du["qweight"], Dg["g_idx"], g)
+        qq, _ = G.prepare_act_order(Dq["qweight"], Dg["g_idx"], g)
     cos, sin = G.RotaryTable(128, 64).get(torch.device("cuda"), 64)
     pos = (np.arange(m) % 50)[:, None].astype(np.int32)
     lib.gptq4_set_gemv_tuning(0, 0, 0, 0)
     lib.gptq4_set_tuning(words, depth, 0)
     try:
-        qs, perm = G.prepare_act_order(D["qweight"], D["g_idx"], g)
-        y = G.matmul4(g, xd, qs, D["scales"], D["qzeros"], D["bias"], perm=perm)
-        h = G.llama_mlp_4(g, xd, D2["qweight"], D2["scales"], D2["qzeros"], D["qweight"], D["scales"], D["qzeros"])
-        q, kk, vv = G.qkv_rotary(g, xd.view(m, 1, k), Dq["qweight"], Dq["scales"], Dq["qzeros"], torch.from_numpy(pos).cuda(),
-                                 cos, sin, heads)
+        y = G.matmul4(g, xd, gq, Dg["scales"], Dg["qzeros"], Dg["bias"], perm=perm)
+        h = G.llama_mlp_4(g, xd, gq, Dg["scales"], Dg["qzeros"], uq, Du["scales"], Du["qzeros"], perm=perm)
+        q, kk, vv = G.qkv_rotary(g, xd.view(m, 1, k), qq, Dq["scales"], Dq["qzeros"], torch.from_numpy(pos).cuda(),
+                                 cos, sin, heads, perm=perm)
     finally:
         lib.gptq4_set_tuning(0, 0, 0)
         lib.gptq4_set_gemv_tuning(1, 0, 0, 0)
-    ref = O.quant_matmul_ref(x, L["qweight"], L["qzeros"], L["scales"], g, bias=L["bias"], g_idx=L["g_idx"])
+    gi = gate["g_idx"]
+    ref = O.quant_matmul_ref(x, gate["qweight"], gate["qzeros"], gate["scales"], g, bias=gate["bias"], g_idx=gi)
     ok, max_abs, _ = O.within_tolerance(y.cpu().numpy(), ref)
     assert ok, max_abs
-    href = O.mlp_gateup_ref(x, (L2["qweight"], L2["qzeros"], L2["scales"]), (L["qweight"], L["qzeros"], L["scales"]), g)
+    href = O.mlp_gateup_ref(x, (gate["qweight"], gate["qzeros"], gate["scales"], gi), (up["qweight"], up["qzeros"], up["scales"], gi), g)
     assert_close(h.cpu().numpy(), href, f"gate/up words={words} depth={depth} M={m}")
-    qr, kr, vr = O.qkv_rotary_ref(x.reshape(m, 1, k), Lq["qweight"], Lq["qzeros"], Lq["scales"], g, pos, heads, 128, max_pos=64)
+    qr, kr, vr = O.qkv_rotary_ref(x.reshape(m, 1, k), qkv["qweight"], qkv["qzeros"], qkv["scales"], g, pos, heads, 128,
+                                  g_idx=gi, max_pos=64)
     for got, want, name in ((q, qr, "q"), (kk, kr, "k"), (vv, vr, "v")):
         assert_close(got.cpu().numpy(), want, f"{name} words={words} depth={depth} M={m}")

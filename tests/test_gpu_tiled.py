@@ -155,8 +155,9 @@ def test_graph_replays_equal_eager_launches(m):
     assert ok, max_abs
 
 
+@pytest.mark.parametrize("mt", [2, 4])
 @pytest.mark.parametrize("m", [40, 200])
-def test_in_kernel_act_order_gather_with_fused_epilogues(m):
+def test_in_kernel_act_order_gather_with_fused_epilogues(m, mt):
     """The Python layer permutes tall act-order inputs before the call; a direct caller of the C ABI may pass
     `perm` instead, and the tiled kernel then gathers the activations itself - also under the SiLU*mul and
     the rotary epilogue."""
@@ -176,8 +177,22 @@ def test_in_kernel_act_order_gather_with_fused_epilogues(m):
     qq, qperm = G.prepare_act_order(Dq["qweight"], Dq["g_idx"], g)
     stream = _lib.current_stream(xd.device)
     h = torch.empty((m, n), dtype=torch.float16, device="cuda")
+    y = torch.empty((m, n), dtype=torch.float16, device="cuda")
+    lib.gptq4_set_gemm_tuning(mt, 0)
     ws = _lib.workspace(xd.device, max(lib.gptq4_workspace_bytes(_lib.OP_MLP_GATEUP, m, k, n),
                                        lib.gptq4_workspace_bytes(_lib.OP_QKV_ROTARY, m, k, 3 * k)))
+    try:
+        _gather_calls(lib, _lib, G, xd, x, m, k, n, g, heads, gate, up, qkv, Dg, Du, Dq, gq, uq, qq, perm, qperm, h, y, ws, stream)
+    finally:
+        lib.gptq4_set_gemm_tuning(0, 0)
+
+
+def _gather_calls(lib, _lib, G, xd, x, m, k, n, g, heads, gate, up, qkv, Dg, Du, Dq, gq, uq, qq, perm, qperm, h, y, ws, stream):
+    rc = lib.gptq4_matmul(xd.data_ptr(), gq.data_ptr(), Dg["qzeros"].data_ptr(), Dg["scales"].data_ptr(), perm.data_ptr(), None,
+                          y.data_ptr(), m, k, n, g, ws.data_ptr(), ws.numel(), stream)
+    assert rc == 0
+    yref = O.quant_matmul_ref(x, gate["qweight"], gate["qzeros"], gate["scales"], g, g_idx=gate["g_idx"])
+    assert_close(y.cpu().numpy(), yref, f"in-kernel gather, matmul M={m}")
     rc = lib.gptq4_mlp_gateup(xd.data_ptr(), gq.data_ptr(), Dg["qzeros"].data_ptr(), Dg["scales"].data_ptr(),
                               uq.data_ptr(), Du["qzeros"].data_ptr(), Du["scales"].data_ptr(), perm.data_ptr(),
                               h.data_ptr(), m, k, n, g, ws.data_ptr(), ws.numel(), stream)
