@@ -88,9 +88,12 @@ def current_stream(device: torch.device):
     return torch.cuda.current_stream(device).cuda_stream
 
 
-# One workspace per (device, stream): split-K partials + arrival counters.  The counter
-# region must start zeroed; the kernels restore it to zero.
+# One workspace per (device, stream): split-K partials + arrival counters (+ the gathered rows of
+# an act-order call).  The counter region must start zeroed; the kernels restore it to zero.
+# A workspace that has to grow is replaced by one at least twice as large; the old one is kept
+# alive, because captured graphs may still launch kernels that point into it.
 _workspaces: dict = {}
+_outgrown: list = []
 _WS_BYTES = WS_COUNTER_BYTES + 16 * 16 * 2 * 32768 * 4  # splitk 16, M 16, 2 matrices, 32768 columns
 
 
@@ -99,7 +102,9 @@ def workspace(device: torch.device, need: int):
            torch.cuda.current_stream(device).cuda_stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < need:
-        ws = torch.zeros(max(need, _WS_BYTES), dtype=torch.uint8, device=device)
+        if ws is not None:
+            _outgrown.append(ws)
+        ws = torch.zeros(max(need, _WS_BYTES, 2 * ws.numel() if ws is not None else 0), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
 

@@ -42,6 +42,21 @@ int setup_skinny(MatmulArgs &a, const SkinnyPlan &pl, int nmat, void *workspace,
     return 0;
 }
 
+// Act-order: gather the M rows of x into the workspace behind the partial sums (one small launch) and hand
+// the kernel plain activations.  A kernel's own gather reads single 2-byte values, each a cache line to the
+// texture path, and repeats that for every column tile: 3.5 us at one row, twice the time of the whole call
+// at eight rows, +43 % for a 2048-row down_proj.
+int stage_act_order(MatmulArgs &a, size_t partial_bytes_used, void *workspace, size_t workspace_bytes, hipStream_t s) {
+    const size_t off = GPTQ4_WS_COUNTER_BYTES + partial_bytes_used;
+    const size_t bytes = (size_t)a.M * a.K * sizeof(half_t);
+    if (workspace == nullptr || workspace_bytes < off + bytes) return -GPTQ4_E_WORKSPACE;
+    half_t *xg = reinterpret_cast<half_t *>(reinterpret_cast<char *>(workspace) + off);
+    const int rc = launch_gather_cols(a.x, a.perm, xg, a.M, a.K, s);
+    a.x = xg;
+    a.perm = nullptr;
+    return rc;
+}
+
 // M <= 16: the balanced GEMV where its plan says so (by default the one-row gate/up pair),
 // the split-K kernel otherwise.
 int run_small(int epi, MatmulArgs &a, int nmat, void *workspace, size_t workspace_bytes, hipStream_t s) {
@@ -75,6 +90,10 @@ int run_small(int epi, MatmulArgs &a, int nmat, void *workspace, size_t workspac
     const SkinnyPlan pl = skinny_plan(epi, a.N, a.K);
     int rc = setup_skinny(a, pl, nmat, workspace, workspace_bytes);
     if (rc) return rc;
+    if (a.perm != nullptr) {
+        rc = stage_act_order(a, a.splitk > 1 ? partial_bytes(a.splitk, a.M, nmat * a.N) : 0, workspace, workspace_bytes, s);
+        if (rc) return rc;
+    }
     return launch_skinny(epi, a, pl, s);
 }
 
@@ -124,24 +143,35 @@ bool prefer_kslice(const KslicePlan &kp, int epi, int M, int N, int K) {
 }
 
 int run_tiled(int epi, MatmulArgs &a, void *workspace, size_t workspace_bytes, hipStream_t s) {
-    const KslicePlan kp = kslice_plan(epi, a.M, a.N, a.K, a.perm != nullptr);
+    // act-order: staged activations wherever they fit the staging limit (then the mid-M kernel can run too)
+    const bool stage = a.perm != nullptr && !g_gemm_tuning.own_gather &&
+                       (size_t)a.M * a.K * sizeof(half_t) <= ACT_ORDER_STAGE_MAX;
+    const KslicePlan kp = kslice_plan(epi, a.M, a.N, a.K, a.perm != nullptr && !stage);
     if (prefer_kslice(kp, epi, a.M, a.N, a.K)) {
         a.tiles = kp.tiles;
         a.splitk = kp.splitk;
         const int nk = a.K / 64;
         a.slot_q = nk / kp.splitk;
         a.slot_rem = nk % kp.splitk;
+        const size_t partial = kp.splitk > 1 ? kslice_partial_bytes(epi, kp) : 0;
         if (kp.splitk > 1) {
-            if (workspace == nullptr || workspace_bytes < GPTQ4_WS_COUNTER_BYTES + kslice_partial_bytes(epi, kp))
-                return -GPTQ4_E_WORKSPACE;
+            if (workspace == nullptr || workspace_bytes < GPTQ4_WS_COUNTER_BYTES + partial) return -GPTQ4_E_WORKSPACE;
             a.counters = reinterpret_cast<int *>(workspace);
             a.partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_COUNTER_BYTES);
+        }
+        if (stage) {
+            const int rc = stage_act_order(a, partial, workspace, workspace_bytes, s);
+            if (rc) return rc;
         }
         return launch_kslice(epi, a, kp, s);
     }
     const GemmPlan pl = gemm_plan(epi, a.M, a.N, a.K);
-    const int rc = setup_gemm(a, pl, workspace, workspace_bytes);
+    int rc = setup_gemm(a, pl, workspace, workspace_bytes);
     if (rc) return rc;
+    if (stage) {
+        rc = stage_act_order(a, pl.splitk > 1 ? gemm_partial_bytes(pl) : 0, workspace, workspace_bytes, s);
+        if (rc) return rc;
+    }
     return launch_gemm(epi, a, pl, s);
 }
 
@@ -171,6 +201,9 @@ const char *gptq4_strerror(int code) {
 }
 
 void gptq4_set_gemm_tuning(int mt, int splitk) {
+    // 10 + mt: act-order calls use the tiled kernel's own gather (no staging of the activations)
+    g_gemm_tuning.own_gather = (mt >= 10) ? 1 : 0;
+    if (mt >= 10) mt -= 10;
     g_gemm_tuning.mt = (mt == 2 || mt == 4) ? mt : 0;
     g_gemm_tuning.splitk = splitk > 0 ? splitk : 0;
 }
@@ -214,7 +247,7 @@ size_t gptq4_workspace_bytes(int op, int M, int K, int N) {
                 if (pl.ok && gemv_partial_bytes(pl, M, epi) > need) need = gemv_partial_bytes(pl, M, epi);
             }
         }
-        bytes += need;
+        bytes += need + (size_t)M * K * 2;  // + the rows gathered for an act-order call
     } else if ((K % 64) == 0) {
         const int epi = (op == GPTQ4_OP_MLP_GATEUP) ? EPI_SILU_MUL : (op == GPTQ4_OP_QKV_ROTARY ? EPI_ROPE : EPI_PLAIN);
         // whichever kernel the current (automatic or forced) plans pick, with or without act-order
@@ -222,6 +255,8 @@ size_t gptq4_workspace_bytes(int op, int M, int K, int N) {
         const KslicePlan kp = kslice_plan(epi, M, N, K, false);
         if (kp.ok && kslice_partial_bytes(epi, kp) > need) need = kslice_partial_bytes(epi, kp);
         bytes += need;
+        // + the rows gathered for an act-order call
+        if ((size_t)M * K * 2 <= ACT_ORDER_STAGE_MAX) bytes += (size_t)M * K * 2;
     }
     return bytes;
 }

@@ -555,7 +555,7 @@ int launch_epi(const MatmulArgs &a, const GemmPlan &pl, hipStream_t stream) {
 
 }  // namespace
 
-GemmTuning g_gemm_tuning = {0, 0};
+GemmTuning g_gemm_tuning = {0, 0, 0};
 
 // Tile shape and split-K factor of the tiled kernel.  The wide tile (128 x 256, half as
 // wide for SiLU*mul) is the faster one as soon as there are enough of them to give three

@@ -93,6 +93,7 @@ struct GemmPlan {
 };
 struct GemmTuning {
     int mt, splitk;  // 0 = automatic
+    int own_gather;  // 1: act-order calls run the tiled kernel's own gather instead of staging the activations
 };
 extern GemmTuning g_gemm_tuning;
 GemmPlan gemm_plan(int epi, int M, int N, int K);
@@ -123,6 +124,8 @@ int launch_dequant(const uint32_t *qweight, const uint32_t *qzeros, const half_t
                    hipStream_t stream);
 int launch_sort_rows(const uint32_t *qweight, const int32_t *perm, uint32_t *out, int K, int N,
                      hipStream_t stream);
+// out[m][j] = x[m][perm[j]] for M rows of K values.
+int launch_gather_cols(const half_t *x, const int32_t *perm, half_t *out, int M, int K, hipStream_t stream);
 int launch_rope_table(float *cos_out, float *sin_out, int max_pos, int D, float base,
                       hipStream_t stream);
 // Decoder-side operators (gptq4_decoder.hip).
@@ -135,4 +138,6 @@ int launch_attn_decode(const half_t *q, const half_t *kc, const half_t *vc, cons
 // arrival counters sit one per 128-byte line: atomics on one line are served one after
 // the other by the memory side
 enum { COUNTER_STRIDE = 32 };
+// act-order: activations up to this many bytes are gathered into the workspace ahead of the kernel
+constexpr size_t ACT_ORDER_STAGE_MAX = (size_t)1 << 30;
 enum { GEMV_MAX_M = 4, SKINNY_MAX_M = 16, SKINNY_MAX_SPLITK = 16, SKINNY_MAX_TILES = 4096, GEMM_MAX_SPLITK = 16 };

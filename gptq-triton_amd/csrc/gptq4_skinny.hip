@@ -75,9 +75,12 @@ struct Batch {
 // all M rows into LDS (gptq4_norm.h; the workgroup of tile 0, split 0 also writes the sums out)
 // and takes its A operand from there instead of from memory.
 // NORM = chunks of 8 values per thread that cover a row (2: K <= 4096, 4: K <= 8192), 0 = off.
+// PERM (with NORM only): act-order - the rows in LDS are then put into the order of the sorted weight
+// rows, xs[j] <- xs[perm[j]].  Without NORM the caller passes activations that are gathered already.
 template <int EPI, int W, int DEPTH, bool PERM, int NW, int NORM>
 __global__ __launch_bounds__(64 * NW) void gptq4_skinny_kernel(MatmulArgs p) {
     static_assert(!NORM || NW == 4, "the fused norm is written for 256 threads");
+    static_assert(!PERM || NORM, "act-order inside the kernel needs the rows in LDS");
     constexpr int NV = (EPI == EPI_PLAIN) ? 1 : 2;  // strips loaded per K step
     constexpr int SW = 16 * W;                      // strip width in columns
     constexpr int TILE_COLS = SW * NV;              // columns of the LDS tile
@@ -163,32 +166,10 @@ __global__ __launch_bounds__(64 * NW) void gptq4_skinny_kernel(MatmulArgs p) {
             for (int i = 0; i < 4; ++i) B.w[v][i] = *reinterpret_cast<const wvec_t *>(base + (size_t)(4 * i) * N);
         }
         B.b = b;
+        if (!NORM) {
+            // NORM takes the A operand from LDS at compute time
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int k = b * 128 + 32 * i + 8 * lrow;
-            uint4 a;
-            if (NORM) {
-                // the A operand comes from LDS at compute time; act-order: keep the 8 source
-                // positions (below 8192, two per word)
-                if (!PERM) break;
-                const int4 i0 = *reinterpret_cast<const int4 *>(p.perm + k);
-                const int4 i1 = *reinterpret_cast<const int4 *>(p.perm + k + 4);
-                a.x = (uint32_t)i0.x | ((uint32_t)i0.y << 16);
-                a.y = (uint32_t)i0.z | ((uint32_t)i0.w << 16);
-                a.z = (uint32_t)i1.x | ((uint32_t)i1.y << 16);
-                a.w = (uint32_t)i1.z | ((uint32_t)i1.w << 16);
-            } else if (!PERM) {
-                a = *reinterpret_cast<const uint4 *>(xrow + k);
-            } else {
-                const int4 i0 = *reinterpret_cast<const int4 *>(p.perm + k);
-                const int4 i1 = *reinterpret_cast<const int4 *>(p.perm + k + 4);
-                const uint16_t *xs = reinterpret_cast<const uint16_t *>(xrow);
-                a.x = (uint32_t)xs[i0.x] | ((uint32_t)xs[i0.y] << 16);
-                a.y = (uint32_t)xs[i0.z] | ((uint32_t)xs[i0.w] << 16);
-                a.z = (uint32_t)xs[i1.x] | ((uint32_t)xs[i1.y] << 16);
-                a.w = (uint32_t)xs[i1.z] | ((uint32_t)xs[i1.w] << 16);
-            }
-            B.a[i] = a;
+            for (int i = 0; i < 4; ++i) B.a[i] = *reinterpret_cast<const uint4 *>(xrow + b * 128 + 32 * i + 8 * lrow);
         }
         B.group = ld_group;
         if (--ld_left == 0) {
@@ -225,16 +206,7 @@ __global__ __launch_bounds__(64 * NW) void gptq4_skinny_kernel(MatmulArgs p) {
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            uint4 av = B.a[i];
-            if (NORM && !PERM) av = xs[xs_row + B.b * 16 + 4 * i + lrow];
-            if (NORM && PERM) {
-                const uint16_t *xh = reinterpret_cast<const uint16_t *>(xs + xs_row);
-                const uint32_t ix[4] = {av.x, av.y, av.z, av.w};
-                uint32_t o[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) o[e] = (uint32_t)xh[ix[e] & 0xFFFFu] | ((uint32_t)xh[ix[e] >> 16] << 16);
-                av = make_uint4(o[0], o[1], o[2], o[3]);
-            }
+            const uint4 av = NORM ? xs[xs_row + B.b * 16 + 4 * i + lrow] : B.a[i];
             const h8_t a = pair_order_a(av);
 #pragma unroll
             for (int v = 0; v < NV; ++v) {
@@ -273,6 +245,36 @@ __global__ __launch_bounds__(64 * NW) void gptq4_skinny_kernel(MatmulArgs p) {
                 norm_rows_to_lds<true>(p.x, p.nrm_delta, p.nrm_weight, sums, xs, norm_part, M, K, p.nrm_eps, tid, nl);
             else
                 norm_rows_to_lds<false>(p.x, p.x, p.nrm_weight, nullptr, xs, norm_part, M, K, p.nrm_eps, tid, nl);
+        }
+        if (NORM && PERM) {
+            // act-order: put each row into the order of the sorted weight rows, xs[j] <- xs[perm[j]], in
+            // place: every thread gathers its chunks into registers, all wait, then the chunks go back.  (The
+            // source positions are only asked for here, in registers that the norm has just given up: held
+            // from before the weight loads they would cost a wave per SIMD.)
+            int4 src[NORM ? NORM : 1][2];
+#pragma unroll
+            for (int c = 0; c < NORM; ++c) {
+                const int chunk = min(tid + 256 * c, (K >> 3) - 1);
+                src[c][0] = *reinterpret_cast<const int4 *>(p.perm + 8 * chunk);
+                src[c][1] = *reinterpret_cast<const int4 *>(p.perm + 8 * chunk + 4);
+            }
+            for (int m = 0; m < M; ++m) {
+                const uint16_t *xh = reinterpret_cast<const uint16_t *>(xs + m * (K >> 3));
+                uint4 g[NORM ? NORM : 1];
+#pragma unroll
+                for (int c = 0; c < NORM; ++c) {
+                    const int4 i0 = src[c][0], i1 = src[c][1];
+                    g[c].x = (uint32_t)xh[i0.x] | ((uint32_t)xh[i0.y] << 16);
+                    g[c].y = (uint32_t)xh[i0.z] | ((uint32_t)xh[i0.w] << 16);
+                    g[c].z = (uint32_t)xh[i1.x] | ((uint32_t)xh[i1.y] << 16);
+                    g[c].w = (uint32_t)xh[i1.z] | ((uint32_t)xh[i1.w] << 16);
+                }
+                __syncthreads();
+#pragma unroll
+                for (int c = 0; c < NORM; ++c)
+                    if (tid + 256 * c < (K >> 3)) xs[m * (K >> 3) + tid + 256 * c] = g[c];
+            }
+            __syncthreads();
         }
         for (int b = b0; b < b1; b += DEPTH) {
 #pragma unroll
@@ -433,10 +435,9 @@ int launch_variant(const MatmulArgs &a, hipStream_t stream) {
     const int per_xcd = 8 * LINE_TILES;
     const int groups = (a.tiles + per_xcd - 1) / per_xcd;
     dim3 grid((unsigned)(groups * per_xcd), (unsigned)a.splitk), block(64 * NW);
-    if (a.perm == nullptr)
-        hipLaunchKernelGGL((gptq4_skinny_kernel<EPI, W, DEPTH, false, NW, 0>), grid, block, 0, stream, a);
-    else
-        hipLaunchKernelGGL((gptq4_skinny_kernel<EPI, W, DEPTH, true, NW, 0>), grid, block, 0, stream, a);
+    // act-order: the caller hands over the activations already gathered (launch_gather_cols)
+    if (a.perm != nullptr) return (int)hipErrorInvalidValue;
+    hipLaunchKernelGGL((gptq4_skinny_kernel<EPI, W, DEPTH, false, NW, 0>), grid, block, 0, stream, a);
     return (int)hipGetLastError();
 }
 

@@ -61,6 +61,48 @@ __global__ __launch_bounds__(256) void gptq4_sort_rows_kernel(const uint32_t *__
     out[(size_t)r * N + n] = w;
 }
 
+// out[m][j] = x[m][perm[j]]: the activations in the order of the sorted weight rows.  One thread
+// makes 8 neighbouring outputs of one row (K % 8 == 0, perm 16-byte aligned).
+__global__ __launch_bounds__(256) void gptq4_gather_cols_kernel(const half_t *__restrict__ x,
+                                                                const int32_t *__restrict__ perm,
+                                                                half_t *__restrict__ out, int K) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (8 * c >= K) return;
+    const int4 i0 = *reinterpret_cast<const int4 *>(perm + 8 * c);
+    const int4 i1 = *reinterpret_cast<const int4 *>(perm + 8 * c + 4);
+    const uint16_t *row = reinterpret_cast<const uint16_t *>(x) + (size_t)blockIdx.y * K;
+    uint4 o;
+    o.x = (uint32_t)row[i0.x] | ((uint32_t)row[i0.y] << 16);
+    o.y = (uint32_t)row[i0.z] | ((uint32_t)row[i0.w] << 16);
+    o.z = (uint32_t)row[i1.x] | ((uint32_t)row[i1.y] << 16);
+    o.w = (uint32_t)row[i1.z] | ((uint32_t)row[i1.w] << 16);
+    *reinterpret_cast<uint4 *>(out + (size_t)blockIdx.y * K + 8 * c) = o;
+}
+
+// The same for many rows: one workgroup per row first copies the row into LDS (whole 16-byte chunks), then
+// gathers from there - single 2-byte reads of global memory cost a cache line each.
+__global__ __launch_bounds__(256) void gptq4_gather_cols_lds_kernel(const half_t *__restrict__ x,
+                                                                    const int32_t *__restrict__ perm,
+                                                                    half_t *__restrict__ out, int K) {
+    extern __shared__ uint4 row_chunks[];  // K / 8
+    const int chunks = K >> 3;
+    const uint4 *src = reinterpret_cast<const uint4 *>(x + (size_t)blockIdx.x * K);
+    for (int c = threadIdx.x; c < chunks; c += 256) row_chunks[c] = src[c];
+    __syncthreads();
+    const uint16_t *row = reinterpret_cast<const uint16_t *>(row_chunks);
+    uint4 *dst = reinterpret_cast<uint4 *>(out + (size_t)blockIdx.x * K);
+    for (int c = threadIdx.x; c < chunks; c += 256) {
+        const int4 i0 = *reinterpret_cast<const int4 *>(perm + 8 * c);
+        const int4 i1 = *reinterpret_cast<const int4 *>(perm + 8 * c + 4);
+        uint4 o;
+        o.x = (uint32_t)row[i0.x] | ((uint32_t)row[i0.y] << 16);
+        o.y = (uint32_t)row[i0.z] | ((uint32_t)row[i0.w] << 16);
+        o.z = (uint32_t)row[i1.x] | ((uint32_t)row[i1.y] << 16);
+        o.w = (uint32_t)row[i1.z] | ((uint32_t)row[i1.w] << 16);
+        dst[c] = o;
+    }
+}
+
 __global__ __launch_bounds__(256) void gptq4_rope_table_kernel(float *__restrict__ cos_out,
                                                                float *__restrict__ sin_out, int max_pos,
                                                                int half_dim, float base) {
@@ -92,6 +134,18 @@ int launch_sort_rows(const uint32_t *qweight, const int32_t *perm, uint32_t *out
                      hipStream_t stream) {
     dim3 grid((unsigned)((N + 255) / 256), (unsigned)(K / 8)), block(256);
     hipLaunchKernelGGL(gptq4_sort_rows_kernel, grid, block, 0, stream, qweight, perm, out, K, N);
+    return (int)hipGetLastError();
+}
+
+int launch_gather_cols(const half_t *x, const int32_t *perm, half_t *out, int M, int K, hipStream_t stream) {
+    if (M > 16 && (size_t)K * sizeof(half_t) <= 65536) {
+        hipLaunchKernelGGL(gptq4_gather_cols_lds_kernel, dim3((unsigned)M), dim3(256), (size_t)K * sizeof(half_t), stream, x,
+                           perm, out, K);
+        return (int)hipGetLastError();
+    }
+    const int threads = (K / 8 >= 256) ? 256 : 64;
+    dim3 grid((unsigned)((K / 8 + threads - 1) / threads), (unsigned)M), block(threads);
+    hipLaunchKernelGGL(gptq4_gather_cols_kernel, grid, block, 0, stream, x, perm, out, K);
     return (int)hipGetLastError();
 }
 

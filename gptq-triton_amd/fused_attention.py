@@ -18,7 +18,7 @@ import torch
 import torch.nn as nn
 
 from . import _lib
-from .quant_linear import QuantLinear, _check_device_tensors, _check_matmul_args, gather_act_order
+from .quant_linear import QuantLinear, _check_device_tensors, _check_matmul_args
 
 
 @dataclass
@@ -116,7 +116,7 @@ def qkv_rotary(groupsize: int, hidden_states: torch.Tensor, qweight: torch.Tenso
     lib = _lib.load()
     need = lib.gptq4_workspace_bytes(_lib.OP_QKV_ROTARY, bsz * q_len, k_in, n)
     ws = _lib.workspace(dev, need)
-    x2d, perm = gather_act_order(hidden_states.view(-1, k_in), perm)
+    x2d = hidden_states.view(-1, k_in)
     rc = lib.gptq4_qkv_rotary(x2d.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(),
                               _lib.ptr(perm), pos.data_ptr(), cos.data_ptr(), sin.data_ptr(), cos.shape[0],
                               q.data_ptr(), kk.data_ptr(), vv.data_ptr(), bsz, q_len, num_heads, head_dim, k_in,

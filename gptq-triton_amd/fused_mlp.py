@@ -13,7 +13,7 @@ import torch
 import torch.nn as nn
 
 from . import _lib
-from .quant_linear import QuantLinear, _check_device_tensors, _check_matmul_args, gather_act_order
+from .quant_linear import QuantLinear, _check_device_tensors, _check_matmul_args
 
 
 def llama_mlp_4(groupsize: int, a: torch.Tensor,
@@ -33,7 +33,6 @@ def llama_mlp_4(groupsize: int, a: torch.Tensor,
     c = torch.empty((m, n), device=a.device, dtype=torch.float16)
     if m == 0:
         return c.view(a.shape[:-1] + (n,))
-    x, perm = gather_act_order(x, perm)
     need = lib.gptq4_workspace_bytes(_lib.OP_MLP_GATEUP, m, k, n)
     ws = _lib.workspace(a.device, need)
     rc = lib.gptq4_mlp_gateup(x.data_ptr(), gate_qweight.data_ptr(), gate_qzeros.data_ptr(), gate_scales.data_ptr(),

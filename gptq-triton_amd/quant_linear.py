@@ -43,19 +43,6 @@ def _check_device_tensors(a, *tensors):
             raise RuntimeError("quantised tensors must be contiguous")
 
 
-# With more rows than this, gathering the activations once (x[:, perm], one pass over x)
-# beats gathering them inside the kernel, where every column tile repeats the gather.
-ACT_ORDER_GATHER_ROWS = 16
-
-
-def gather_act_order(x2d: torch.Tensor, perm: Optional[torch.Tensor]):
-    """(x, perm) as the kernels should see them: for a tall x the permutation is applied
-    here and the kernel runs its plain path."""
-    if perm is not None and x2d.shape[0] > ACT_ORDER_GATHER_ROWS:
-        return x2d.index_select(1, perm), None
-    return x2d, perm
-
-
 def matmul4(groupsize: int, a: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor,
             qzeros: torch.Tensor, bias: Optional[torch.Tensor] = None,
             perm: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -74,7 +61,6 @@ def matmul4(groupsize: int, a: torch.Tensor, qweight: torch.Tensor, scales: torc
     c = torch.empty((m, n), device=a.device, dtype=torch.float16)
     if m == 0:
         return c.view(a.shape[:-1] + (n,))
-    x, perm = gather_act_order(x, perm)
     need = lib.gptq4_workspace_bytes(_lib.OP_MATMUL, m, k, n)
     ws = _lib.workspace(a.device, need)
     rc = lib.gptq4_matmul(x.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(),

@@ -23,8 +23,11 @@
  *    N % 256 == 0 (what the reference accepts: quant_linear.py:244-257).
  *  - `perm` (nullable) is the act-order row permutation made by
  *    gptq4_actorder_sort_rows(): logical weight row j multiplies x[:, perm[j]] and
- *    belongs to group j / groupsize.
- *  - `workspace` holds split-K partial sums and arrival counters.  Size it with
+ *    belongs to group j / groupsize.  The calls gather the rows of x into the workspace
+ *    with one small launch of their own and multiply from there (up to 1 GiB of rows; the
+ *    tiled kernel gathers by itself beyond that).
+ *  - `workspace` holds split-K partial sums, arrival counters and, for a call with
+ *    `perm`, the gathered activations (M * K * 2 bytes).  Size it with
  *    gptq4_workspace_bytes(); its first GPTQ4_WS_COUNTER_BYTES bytes must be zero
  *    before the FIRST call that uses it (each call leaves them zero again).  One
  *    workspace may be shared by all calls on one stream; calls that run
@@ -179,7 +182,9 @@ int gptq4_decode_attention(const void *q, const void *k_cache, const void *v_cac
 void gptq4_set_tuning(int words, int depth, int splitk);
 
 /* Same for the tiled (M > 16) kernel: workgroup tile (mt = 2: 128 x 128, mt = 4: 128 x 256
- * outputs; half as wide for the fused gate/up) and the split-K factor; 0 = automatic. */
+ * outputs; half as wide for the fused gate/up) and the split-K factor; 0 = automatic.
+ * mt = 10, 12 or 14: the same tile choice, and act-order calls use the tiled kernel's own
+ * gather of the activations instead of the copy staged in the workspace. */
 void gptq4_set_gemm_tuning(int mt, int splitk);
 
 /* Same for the mid-M kernel (M > 16 with too few wide tiles for the tiled kernel; K is split

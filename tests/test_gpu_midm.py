@@ -145,9 +145,10 @@ def test_midm_and_tiled_kernels_agree_within_rounding():
     assert bool(((y0 - y1).abs() <= ulp + 1e-4).all())
 
 
-def test_act_order_inputs_take_the_tiled_kernel():
-    """The mid-M kernel has no act-order gather: with a permutation the call must still give
-    the right answer (through the tiled kernel), also when the mid-M kernel is forced."""
+def test_act_order_inputs_reach_the_mid_m_kernel_through_the_staged_copy():
+    """The mid-M kernel has no act-order gather of its own: the call gathers the rows into the
+    workspace first, so a permutation gives the right answer with the mid-M kernel forced too -
+    and a workspace without room for that copy is refused."""
     from gptq_triton_amd import _lib
     lib = _lib.load()
     k, n, g, m = 2048, 512, 128, 48
@@ -168,3 +169,9 @@ def test_act_order_inputs_take_the_tiled_kernel():
     assert rc == 0
     ref = O.quant_matmul_ref(x, L["qweight"], L["qzeros"], L["scales"], g, g_idx=L["g_idx"])
     assert_close(y.cpu().numpy(), ref, "act-order through the C ABI, M=48")
+    need = lib.gptq4_workspace_bytes(_lib.OP_MATMUL, m, k, n)
+    assert need >= _lib.WS_COUNTER_BYTES + m * k * 2
+    rc = lib.gptq4_matmul(xd.data_ptr(), Wq.data_ptr(), D["qzeros"].data_ptr(), D["scales"].data_ptr(), perm.data_ptr(), None,
+                          y.data_ptr(), m, k, n, g, ws.data_ptr(), _lib.WS_COUNTER_BYTES + m * k * 2 - 16,
+                          _lib.current_stream(xd.device))
+    assert rc < 0 and b"workspace" in lib.gptq4_strerror(rc).lower()

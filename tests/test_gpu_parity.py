@@ -336,9 +336,10 @@ def test_fused_qkv_equals_three_projections():
                 assert d <= 2 ** -7
 
 
-def test_tiled_kernel_gathers_act_order_rows_itself_when_asked():
-    """The Python layer applies the permutation to tall inputs before the call; the C entry
-    point still accepts `perm` for any M (the tiled kernel then gathers in its A staging)."""
+@pytest.mark.parametrize("own_gather", [False, True])
+def test_act_order_above_16_rows_staged_or_gathered_by_the_tiled_kernel(own_gather):
+    """With `perm` the call gathers the rows of x into its workspace and runs the plain kernels; asked to
+    (tile selector + 10), the tiled kernel gathers in its own A staging instead.  Same result either way."""
     from gptq_triton_amd import _lib
     k, n, g, m = 1024, 512, 128, 40
     L = O.make_layer(k, n, g, seed=31, act_order=True)
@@ -350,11 +351,18 @@ def test_tiled_kernel_gathers_act_order_rows_itself_when_asked():
     y = torch.empty((m, n), dtype=torch.float16, device="cuda")
     lib = _lib.load()
     ws = _lib.workspace(xd.device, lib.gptq4_workspace_bytes(_lib.OP_MATMUL, m, k, n))
-    rc = lib.gptq4_matmul(xd.data_ptr(), qs.data_ptr(), D["qzeros"].data_ptr(), D["scales"].data_ptr(), perm.data_ptr(), None,
-                          y.data_ptr(), m, k, n, g, ws.data_ptr(), ws.numel(), _lib.current_stream(xd.device))
+    if own_gather:
+        lib.gptq4_set_midm_tuning(0, 0, 0)
+        lib.gptq4_set_gemm_tuning(10, 0)
+    try:
+        rc = lib.gptq4_matmul(xd.data_ptr(), qs.data_ptr(), D["qzeros"].data_ptr(), D["scales"].data_ptr(), perm.data_ptr(),
+                              None, y.data_ptr(), m, k, n, g, ws.data_ptr(), ws.numel(), _lib.current_stream(xd.device))
+    finally:
+        lib.gptq4_set_gemm_tuning(0, 0)
+        lib.gptq4_set_midm_tuning(1, 0, 0)
     assert rc == 0
     ref = O.quant_matmul_ref(x, L["qweight"], L["qzeros"], L["scales"], g, g_idx=L["g_idx"])
-    assert_close(y.cpu().numpy(), ref, "tiled kernel, in-kernel act-order gather")
+    assert_close(y.cpu().numpy(), ref, f"act-order, M={m}, own gather {own_gather}")
 
 
 def test_empty_inputs_give_empty_outputs():

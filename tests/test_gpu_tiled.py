@@ -158,9 +158,9 @@ def test_graph_replays_equal_eager_launches(m):
 @pytest.mark.parametrize("mt", [2, 4])
 @pytest.mark.parametrize("m", [40, 200])
 def test_in_kernel_act_order_gather_with_fused_epilogues(m, mt):
-    """The Python layer permutes tall act-order inputs before the call; a direct caller of the C ABI may pass
-    `perm` instead, and the tiled kernel then gathers the activations itself - also under the SiLU*mul and
-    the rotary epilogue."""
+    """Act-order calls normally run on a gathered copy of the activations; with the tile selector + 10 the tiled
+    kernel gathers them itself (what a call does whose copy would pass the staging limit) - also under the
+    SiLU*mul and the rotary epilogue."""
     from gptq_triton_amd import _lib
     G = gptq()
     lib = _lib.load()
@@ -178,13 +178,15 @@ def test_in_kernel_act_order_gather_with_fused_epilogues(m, mt):
     stream = _lib.current_stream(xd.device)
     h = torch.empty((m, n), dtype=torch.float16, device="cuda")
     y = torch.empty((m, n), dtype=torch.float16, device="cuda")
-    lib.gptq4_set_gemm_tuning(mt, 0)
+    lib.gptq4_set_midm_tuning(0, 0, 0)
+    lib.gptq4_set_gemm_tuning(10 + mt, 0)
     ws = _lib.workspace(xd.device, max(lib.gptq4_workspace_bytes(_lib.OP_MLP_GATEUP, m, k, n),
                                        lib.gptq4_workspace_bytes(_lib.OP_QKV_ROTARY, m, k, 3 * k)))
     try:
         _gather_calls(lib, _lib, G, xd, x, m, k, n, g, heads, gate, up, qkv, Dg, Du, Dq, gq, uq, qq, perm, qperm, h, y, ws, stream)
     finally:
         lib.gptq4_set_gemm_tuning(0, 0)
+        lib.gptq4_set_midm_tuning(1, 0, 0)
 
 
 def _gather_calls(lib, _lib, G, xd, x, m, k, n, g, heads, gate, up, qkv, Dg, Du, Dq, gq, uq, qq, perm, qperm, h, y, ws, stream):
