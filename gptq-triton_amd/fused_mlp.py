@@ -13,7 +13,7 @@ import torch
 import torch.nn as nn
 
 from . import _lib
-from .quant_linear import QuantLinear, _check_device_tensors, _check_matmul_args
+from .quant_linear import QuantLinear, _check_device_tensors, _check_matmul_args, matmul4
 
 
 def llama_mlp_4(groupsize: int, a: torch.Tensor,
@@ -73,6 +73,17 @@ def norm_llama_mlp_4(groupsize: int, h: torch.Tensor, delta: Optional[torch.Tens
     return (h if s is None else s.view(h.shape)), c.view(h.shape[:-1] + (n,))
 
 
+def _move_zero_columns(qzeros: torch.Tensor, cols: torch.Tensor) -> torch.Tensor:
+    """qzeros [G, N/8] (eight 4-bit stored zeros per word, column 8c+t in bits [4t, 4t+4)) with its
+    columns gathered: column j of the result = column cols[j] of the input."""
+    shifts = torch.arange(0, 32, 4, device=qzeros.device, dtype=torch.int64)
+    z = ((qzeros.to(torch.int64) & 0xFFFFFFFF).unsqueeze(-1) >> shifts) & 0xF   # [G, N/8, 8]
+    z = z.reshape(qzeros.shape[0], -1).index_select(1, cols).reshape(qzeros.shape[0], -1, 8)
+    packed = (z << shifts).sum(-1)
+    packed = torch.where(packed >= 2 ** 31, packed - 2 ** 32, packed)
+    return packed.to(torch.int32).contiguous()
+
+
 class QuantLlamaMLP(nn.Module):
     """forward(x) = down_proj(silu(gate(x)) * up(x)).  Holds the six gate/up tensors as its
     own buffers under the reference's names and keeps down_proj as a submodule
@@ -101,6 +112,7 @@ class QuantLlamaMLP(nn.Module):
         else:
             self.g_idx = None
         self._sorted = None
+        self._chained = None
 
     def _kernel_weights(self):
         if self.g_idx is None:
@@ -118,8 +130,41 @@ class QuantLlamaMLP(nn.Module):
         return llama_mlp_4(self.groupsize, x, gq, self.gate_proj_scales, self.gate_proj_qzeros,
                            uq, self.up_proj_scales, self.up_proj_qzeros, perm)
 
+    def _chained_weights(self):
+        """The tensors forward() multiplies with: (gate/up set, input permutation, down_proj's sorted qweight).
+
+        With an act-order down_proj the OUTPUT columns of gate and up are laid out once in the order of
+        down_proj's sorted rows (column j of the copies = column perm_down[j] of the originals: a
+        column only moves, its values do not change).  The intermediate then comes out of the gate/up
+        launch already in the order down_proj's kernel reads, and down_proj runs without a gather."""
+        down_q, down_perm = self.down_proj.kernel_weights()
+        if down_perm is None:
+            gq, uq, perm = self._kernel_weights()
+            return (gq, self.gate_proj_scales, self.gate_proj_qzeros, uq, self.up_proj_scales, self.up_proj_qzeros), perm, down_q
+        key = (self.gate_proj_qweight.data_ptr(), self.up_proj_qweight.data_ptr(), down_perm.data_ptr(),
+               None if self.g_idx is None else self.g_idx.data_ptr())
+        if self._chained is None or self._chained[0] != key:
+            cols = down_perm.long()
+            if self.g_idx is None:
+                gq, uq, perm = self.gate_proj_qweight, self.up_proj_qweight, None
+            else:
+                from .quant_linear import prepare_act_order
+                gq, perm = prepare_act_order(self.gate_proj_qweight, self.g_idx, self.groupsize)
+                uq, _ = prepare_act_order(self.up_proj_qweight, self.g_idx, self.groupsize)
+            tensors = (gq.index_select(1, cols).contiguous(), self.gate_proj_scales.index_select(1, cols).contiguous(),
+                       _move_zero_columns(self.gate_proj_qzeros, cols),
+                       uq.index_select(1, cols).contiguous(), self.up_proj_scales.index_select(1, cols).contiguous(),
+                       _move_zero_columns(self.up_proj_qzeros, cols))
+            self._chained = (key, tensors, perm)
+        return self._chained[1], self._chained[2], down_q
+
+    def _down(self, mid: torch.Tensor, down_q: torch.Tensor) -> torch.Tensor:
+        d = self.down_proj
+        return matmul4(d.groupsize, mid, down_q, d.scales, d.qzeros, d.bias, None)
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return self.down_proj(self.gate_up(x))
+        w, perm, down_q = self._chained_weights()
+        return self._down(llama_mlp_4(self.groupsize, x, *w, perm), down_q)
 
     def norm_fusable(self, rows: int) -> bool:
         """Whether forward_normed is the faster way for this many rows."""
@@ -128,10 +173,9 @@ class QuantLlamaMLP(nn.Module):
 
     def forward_normed(self, h: torch.Tensor, delta: Optional[torch.Tensor], norm_weight: torch.Tensor, eps: float):
         """(h + delta, forward(RMSNorm(h + delta))): the residual add and the norm run inside the gate/up launch."""
-        gq, uq, perm = self._kernel_weights()
-        s, mid = norm_llama_mlp_4(self.groupsize, h, delta, norm_weight, eps, gq, self.gate_proj_scales, self.gate_proj_qzeros,
-                                  uq, self.up_proj_scales, self.up_proj_qzeros, perm)
-        return s, self.down_proj(mid)
+        w, perm, down_q = self._chained_weights()
+        s, mid = norm_llama_mlp_4(self.groupsize, h, delta, norm_weight, eps, *w, perm)
+        return s, self._down(mid, down_q)
 
 
 def _is_llama_mlp(m: nn.Module) -> bool:

@@ -173,6 +173,34 @@ def test_13b_act_order_mlp_gateup(m):
     assert_close(h[rows].cpu().numpy(), ref, f"13B act-order gate/up M={m}")
 
 
+@pytest.mark.parametrize("gate_act_order", [True, False])
+@pytest.mark.parametrize("m", [1, 8, 48, 300])
+def test_act_order_mlp_forward_chains_into_down_proj_without_a_gather(m, gate_act_order):
+    """forward() lays the gate/up output columns out in the order of down_proj's sorted rows: the result must be
+    the very bits of down_proj(gate_up(x)), which gathers the intermediate, and meet the oracle's bar."""
+    k, n, g = 1024, 2560, 128
+    gate = O.make_layer(k, n, g, seed=1330, act_order=gate_act_order)
+    up = O.make_layer(k, n, g, seed=1331)
+    up["g_idx"] = gate["g_idx"]
+    down = O.make_layer(n, k, g, seed=1332, act_order=True)
+    mlp = gptq().QuantLlamaMLP(quant_linear(gate, k, n, g, gate_act_order), quant_linear(down, n, k, g, True),
+                               quant_linear(up, k, n, g, gate_act_order)).cuda()
+    x = O.make_x(m, k, seed=1333 + m)
+    xd = torch.from_numpy(x).cuda()
+    mid = mlp.gate_up(xd)
+    two_step = mlp.down_proj(mid)
+    y = mlp(xd)
+    assert torch.equal(y, two_step)
+    ref = O.quant_matmul_ref(mid.cpu().numpy(), down["qweight"], down["qzeros"], down["scales"], g, g_idx=down["g_idx"])
+    assert_close(y.cpu().numpy(), ref, f"act-order MLP forward M={m}")
+    if m <= 4:
+        w = torch.from_numpy(np.random.default_rng(5).standard_normal(k).astype(np.float16)).cuda()
+        delta = torch.from_numpy(O.make_x(m, k, seed=77)).cuda()
+        s, y2 = mlp.forward_normed(xd, delta, w, 1e-6)
+        s_ref, normed = gptq().add_rms_norm(xd, delta, w, 1e-6)
+        assert torch.equal(s, s_ref) and torch.equal(y2, mlp(normed))
+
+
 def test_13b_act_order_qkv_rotary():
     hidden, H, Dh, g, S = 5120, 40, 128, 128, 2048
     L = O.make_layer(hidden, 3 * hidden, g, seed=1320, act_order=True)
