@@ -462,7 +462,7 @@ int gptq4_add_rmsnorm(const void *x, const void *delta, const void *weight, void
 }
 
 int gptq4_decode_attention(const void *q, const void *k_cache, const void *v_cache, const int32_t *positions, void *out,
-                           int B, int H, int D, int kv_capacity, float scale, void *workspace, size_t workspace_bytes,
+                           const int32_t *out_index, int B, int H, int D, int kv_capacity, float scale, void *workspace, size_t workspace_bytes,
                            void *stream) {
     if (!q || !k_cache || !v_cache || !positions || !out) return -GPTQ4_E_NULL;
     if (B < 1 || H < 1 || D != 128 || kv_capacity < 1 || (long)B * H > SKINNY_MAX_TILES) return -GPTQ4_E_SHAPE;
@@ -471,7 +471,7 @@ int gptq4_decode_attention(const void *q, const void *k_cache, const void *v_cac
         return -GPTQ4_E_WORKSPACE;
     float *partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_COUNTER_BYTES);
     return launch_attn_decode(reinterpret_cast<const half_t *>(q), reinterpret_cast<const half_t *>(k_cache),
-                              reinterpret_cast<const half_t *>(v_cache), positions, reinterpret_cast<half_t *>(out), B, H,
+                              reinterpret_cast<const half_t *>(v_cache), positions, reinterpret_cast<half_t *>(out), out_index, B, H,
                               kv_capacity, scale, reinterpret_cast<int *>(workspace), partials,
                               reinterpret_cast<hipStream_t>(stream));
 }

@@ -53,12 +53,14 @@ __global__ __launch_bounds__(256) void gptq4_rmsnorm_kernel(const half_t *x, con
 // LDS and the partial [max, sum, acc[128]] goes to the workspace.  The splits of one (b, h)
 // meet through an arrival counter (agent-scope stores, completion wait, atomic count, as
 // in the matmul kernels); the last one merges the partials in split order and writes
-// out[b, h*128 + d].
+// out[b, h*128 + d] - or, with out_index, out[b, out_index[h*128 + d]]: the order in which an act-order
+// o_proj reads its input, so that it needs no gather.
 constexpr int ATT_PART = 130;  // floats per partial: max, sum, 128 accumulators
 
 __global__ __launch_bounds__(256) void gptq4_attn_decode_kernel(const half_t *__restrict__ q, const half_t *__restrict__ kc,
                                                                 const half_t *__restrict__ vc, const int *__restrict__ positions,
-                                                                float *part, int *counters, half_t *__restrict__ out, int H,
+                                                                float *part, int *counters, half_t *__restrict__ out,
+                                                                const int32_t *__restrict__ out_index, int H,
                                                                 int capacity, int chunk, float scale) {
     __shared__ float s_m[16], s_l[16];
     __shared__ float s_acc[16][128];
@@ -180,7 +182,11 @@ __global__ __launch_bounds__(256) void gptq4_attn_decode_kernel(const half_t *__
             }
         }
     }
-    if (tid < 128) out[(size_t)bh * 128 + tid] = (half_t)(a / lw);
+    if (tid < 128) {
+        const int b = bh / H;
+        const int col = (bh - b * H) * 128 + tid;
+        out[(size_t)b * H * 128 + (out_index ? out_index[col] : col)] = (half_t)(a / lw);
+    }
 }
 
 }  // namespace
@@ -207,13 +213,13 @@ size_t attn_decode_partial_bytes(int BH, int capacity) {
     return (size_t)BH * attn_decode_splits(BH, capacity) * ATT_PART * sizeof(float);
 }
 
-int launch_attn_decode(const half_t *q, const half_t *kc, const half_t *vc, const int *positions, half_t *out, int B,
-                       int H, int capacity, float scale, int *counters, float *partials, hipStream_t stream) {
+int launch_attn_decode(const half_t *q, const half_t *kc, const half_t *vc, const int *positions, half_t *out,
+                       const int32_t *out_index, int B, int H, int capacity, float scale, int *counters, float *partials, hipStream_t stream) {
     const int BH = B * H;
     const int nsplit = attn_decode_splits(BH, capacity);
     int chunk = (capacity + nsplit - 1) / nsplit;
     chunk = (chunk + 15) & ~15;
     hipLaunchKernelGGL(gptq4_attn_decode_kernel, dim3((unsigned)nsplit, (unsigned)BH), dim3(256), 0, stream, q, kc, vc,
-                       positions, partials, counters, out, H, capacity, chunk, scale);
+                       positions, partials, counters, out, out_index, H, capacity, chunk, scale);
     return (int)hipGetLastError();
 }

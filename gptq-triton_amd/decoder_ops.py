@@ -90,9 +90,11 @@ def add_rms_norm(x: torch.Tensor, delta: torch.Tensor, weight: torch.Tensor, eps
     return s.reshape(x.shape), y.reshape(x.shape)
 
 
-def decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
+def decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, positions: torch.Tensor,
+                     out_index: torch.Tensor = None) -> torch.Tensor:
     """q fp16 [B, H, 1, 128]; caches fp16 [B, H, capacity, 128]; positions int32 [B] or [B, 1]:
-    sequence b attends to cache rows 0..positions[b].  Returns fp16 [B, 1, H*128]."""
+    sequence b attends to cache rows 0..positions[b].  Returns fp16 [B, 1, H*128]; with out_index
+    (int32 [H*128], a permutation) feature f of a row is stored at position out_index[f]."""
     for t, name in ((q, "q"), (k_cache, "k_cache"), (v_cache, "v_cache"), (positions, "positions")):
         _lib.require_cuda(t, name)
     bsz, heads, q_len, hd = q.shape
@@ -108,12 +110,16 @@ def decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
         pos = pos.to(torch.int32).contiguous()
         if pos.numel() != bsz:
             raise ValueError("one position per sequence")
+    if out_index is not None:
+        _lib.require_cuda(out_index, "out_index")
+        if out_index.dtype != torch.int32 or out_index.shape != (heads * hd,) or not out_index.is_contiguous():
+            raise ValueError("out_index must be a contiguous int32 tensor of H*128 positions")
     cap = k_cache.shape[2]
     out = torch.empty((bsz, 1, heads * hd), dtype=torch.float16, device=q.device)
     lib = _lib.load()
     ws = _lib.workspace(q.device, lib.gptq4_workspace_bytes(_lib.OP_DECODE_ATTENTION, bsz * heads, cap, 0))
     rc = lib.gptq4_decode_attention(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), pos.data_ptr(), out.data_ptr(),
-                                    bsz, heads, hd, cap, 1.0 / math.sqrt(hd), ws.data_ptr(), ws.numel(),
+                                    _lib.ptr(out_index), bsz, heads, hd, cap, 1.0 / math.sqrt(hd), ws.data_ptr(), ws.numel(),
                                     _lib.current_stream(q.device))
     _lib.check(rc, "gptq4_decode_attention")
     return out

@@ -18,7 +18,7 @@ import torch
 import torch.nn as nn
 
 from . import _lib
-from .quant_linear import QuantLinear, _check_device_tensors, _check_matmul_args
+from .quant_linear import QuantLinear, _check_device_tensors, _check_matmul_args, matmul4
 
 
 @dataclass
@@ -185,6 +185,7 @@ class QuantLlamaAttention(nn.Module):
         self.rotary_emb = rotary_emb
         self.rope = RotaryTable(self.head_dim, self.max_position_embeddings,
                                 float(getattr(config, 'rope_theta', 10000.0)))
+        self._context_order = None
 
     def project_qkv(self, hidden_states: torch.Tensor, position_ids: torch.Tensor,
                     kv_out=None, kv_offset: int = 0, norm=None):
@@ -195,6 +196,27 @@ class QuantLlamaAttention(nn.Module):
         return qkv_rotary(self.qkv_proj.groupsize, hidden_states, qweight, self.qkv_proj.scales,
                           self.qkv_proj.qzeros, position_ids, cos, sin, self.num_heads, self.head_dim,
                           perm=perm, kv_out=kv_out, kv_offset=kv_offset, norm=norm)
+
+    def context_order(self):
+        """Where each feature of the attention output should be stored so that an act-order o_proj reads
+        it in the order of its sorted rows (int32 [hidden], the inverse of o_proj's permutation), or
+        None without act-order.  decode_attention(out_index=...) writes in that order."""
+        _, perm = self.o_proj.kernel_weights()
+        if perm is None:
+            return None
+        if self._context_order is None or self._context_order[0] != perm.data_ptr():
+            inv = torch.empty_like(perm)
+            inv[perm.long()] = torch.arange(perm.numel(), device=perm.device, dtype=perm.dtype)
+            self._context_order = (perm.data_ptr(), inv)
+        return self._context_order[1]
+
+    def project_out(self, context: torch.Tensor, ordered: bool = False) -> torch.Tensor:
+        """o_proj(context); ordered: the context already is in the order of context_order()."""
+        if not ordered:
+            return self.o_proj(context)
+        o = self.o_proj
+        qweight, _ = o.kernel_weights()
+        return matmul4(o.groupsize, context, qweight, o.scales, o.qzeros, o.bias, None)
 
     def norm_fusable(self, rows: int) -> bool:
         """Whether project_qkv(norm=...) is the faster way for this many rows."""

@@ -187,7 +187,8 @@ class GreedyDecoder:
             attn = layer.self_attn
             q, _, _ = attn.project_qkv(x, position_ids, kv_out=(kc, vc), kv_offset=kv_offset)
             norm = layer.post_attention_layernorm
-            h, x = add_rms_norm(h, attn.o_proj(attend(q, kc, vc)), norm.weight, norm.variance_epsilon)  # attend -> [B, S, hidden]
+            # attend -> ([B, S, hidden], whether in attn.context_order())
+            h, x = add_rms_norm(h, attn.project_out(*attend(q, kc, vc, attn)), norm.weight, norm.variance_epsilon)
             norm = layers[i + 1].input_layernorm if i + 1 < len(layers) else self.model.model.norm
             h, x = add_rms_norm(h, layer.mlp(x), norm.weight, norm.variance_epsilon)
         return self.model.lm_head(x[:, -1:, :]).argmax(-1)
@@ -202,7 +203,7 @@ class GreedyDecoder:
             attn, n1, n2 = layer.self_attn, layer.input_layernorm, layer.post_attention_layernorm
             q, _, _, h = attn.project_qkv(h, position_ids, kv_out=(kc, vc), kv_offset=kv_offset,
                                           norm=(delta, n1.weight, n1.variance_epsilon))
-            h, delta = layer.mlp.forward_normed(h, attn.o_proj(attend(q, kc, vc)), n2.weight, n2.variance_epsilon)
+            h, delta = layer.mlp.forward_normed(h, attn.project_out(*attend(q, kc, vc, attn)), n2.weight, n2.variance_epsilon)
         norm = self.model.model.norm
         h, x = add_rms_norm(h, delta, norm.weight, norm.variance_epsilon)
         return self.model.lm_head(x[:, -1:, :]).argmax(-1)
@@ -217,9 +218,9 @@ class GreedyDecoder:
         position_ids = torch.arange(prompt, device=dev, dtype=torch.int32).unsqueeze(0).expand(bsz, prompt).contiguous()
         sdpa = torch.nn.functional.scaled_dot_product_attention
 
-        def attend(q, kc, vc):
+        def attend(q, kc, vc, attn):
             o = sdpa(q, kc[:, :, :prompt], vc[:, :, :prompt], is_causal=prompt > 1)
-            return o.transpose(1, 2).reshape(bsz, prompt, self.model.config.hidden_size)
+            return o.transpose(1, 2).reshape(bsz, prompt, self.model.config.hidden_size), False
 
         nxt = self._layers(self.model.model.embed_tokens(input_ids), position_ids, 0, attend)
         self.tokens.copy_(nxt)
@@ -230,8 +231,9 @@ class GreedyDecoder:
         """One decode token from the static buffers: reads tokens/position, writes them back."""
         from .fused_attention import KV_AT_POSITION
 
-        def attend(q, kc, vc):  # rows 0..position of the cache, one HIP launch pair
-            return decode_attention(q, kc, vc, self.position)
+        def attend(q, kc, vc, attn):  # rows 0..position of the cache; act-order o_proj: written in the order it reads
+            order = attn.context_order()
+            return decode_attention(q, kc, vc, self.position, out_index=order), order is not None
 
         nxt = self._layers(self.model.model.embed_tokens(self.tokens), self.position, KV_AT_POSITION, attend)
         self.tokens.copy_(nxt)

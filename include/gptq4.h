@@ -166,11 +166,15 @@ int gptq4_add_rmsnorm(const void *x, const void *delta, const void *weight, void
  * softmax(q . K[0..positions[b]]^T * scale) . V[0..positions[b]], in fp32, written as fp16
  * out [B, H*D] (the layout o_proj consumes).  q fp16 [B, H, 1, D]; k_cache, v_cache fp16
  * [B, H, kv_capacity, D]; positions int32 [B] (clamped into [0, kv_capacity)); D must be
- * 128; B * H <= 4096.  workspace as for the matmuls (zeroed head, gptq4_workspace_bytes with
+ * 128; B * H <= 4096.  out_index (nullable) int32 [H*D], a permutation of 0..H*D-1: feature f of
+ * a row is then stored at out[b, out_index[f]] - with the inverse of an act-order o_proj's `perm`
+ * the context comes out in the order of that projection's sorted rows, and o_proj is called
+ * without `perm`.  workspace as for the matmuls (zeroed head, gptq4_workspace_bytes with
  * GPTQ4_OP_DECODE_ATTENTION).  Replaces the attention core of QuantLlamaAttention.forward for q_len == 1
  * (fused_attention.py:118-148: scores, mask, fp32 softmax, weighted sum, transpose). */
 int gptq4_decode_attention(const void *q, const void *k_cache, const void *v_cache,
-                           const int32_t *positions, void *out, int B, int H, int D,
+                           const int32_t *positions, void *out, const int32_t *out_index,
+                           int B, int H, int D,
                            int kv_capacity, float scale, void *workspace,
                            size_t workspace_bytes, void *stream);
 

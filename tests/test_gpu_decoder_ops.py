@@ -75,6 +75,13 @@ def test_decode_attention(bsz, heads, cap, positions):
     err = np.abs(out.cpu().numpy().astype(np.float64) - ref)
     assert (err <= 2e-3 + 1e-2 * np.abs(ref)).all(), err.max()
     assert err.max() < 2e-3  # fp32 softmax of fp16 inputs, one fp16 rounding of the result
+    # with an output order, feature f of every row lands at position order[f]: same values, moved
+    order = torch.from_numpy(np.random.default_rng(1).permutation(heads * 128).astype(np.int32)).cuda()
+    moved = gptq().decode_attention(torch.from_numpy(q).cuda(), torch.from_numpy(k).cuda(), torch.from_numpy(v).cuda(),
+                                    torch.from_numpy(pos).cuda(), out_index=order)
+    want = torch.empty_like(out)
+    want[..., order.long()] = out
+    assert torch.equal(moved, want)
 
 
 def test_decode_attention_peaked_scores_do_not_overflow():

@@ -189,6 +189,13 @@ def test_graph_replayed_decode_equals_eager_decode(tmp_path, groupsize, act_orde
         rest = dec.decode(10, use_graph=True)
         want = model.generate_greedy(ids2, 11)
         assert torch.equal(torch.cat([ids2, first, rest], dim=1), want)
+    # and the decoder's tokens are those of the module-by-module forward over the growing sequence (which has
+    # neither the decoder's cache placement by position nor its attention output in o_proj's row order)
+    cur = ids
+    for _ in range(12):
+        lg, _ = model(cur)
+        cur = torch.cat([cur, lg[:, -1:].argmax(-1)], dim=1)
+    assert (eager == cur).float().mean() > 0.9
 
 
 @pytest.mark.gpu
