@@ -15,6 +15,7 @@ LIB_PATH = Path(__file__).resolve().parent / "csrc" / "libgptq4.so"
 ABI_VERSION = 1
 WS_COUNTER_BYTES = 524288
 OP_MATMUL, OP_MLP_GATEUP, OP_QKV_ROTARY, OP_DECODE_ATTENTION = 0, 1, 2, 3
+OP_WITH_PERM = 0x100  # or-ed to a matmul selector in gptq4_workspace_bytes: the call passes `perm`
 
 # every symbol include/gptq4.h declares: (restype, argtypes)
 SIGNATURES = {
@@ -78,6 +79,11 @@ class Gptq4Error(RuntimeError):
 def check(code: int, where: str) -> None:
     if code != 0:
         raise Gptq4Error(code, where)
+
+
+def op_for(op: int, perm) -> int:
+    """Selector for gptq4_workspace_bytes: calls that pass `perm` need room for the gathered rows."""
+    return op | OP_WITH_PERM if perm is not None else op
 
 
 def ptr(t: torch.Tensor | None):

@@ -234,6 +234,8 @@ void gptq4_set_tuning(int words, int depth, int splitk) {
 
 size_t gptq4_workspace_bytes(int op, int M, int K, int N) {
     size_t bytes = GPTQ4_WS_COUNTER_BYTES;
+    const bool with_perm = (op & GPTQ4_OP_WITH_PERM) != 0;
+    op &= ~GPTQ4_OP_WITH_PERM;
     if (op == GPTQ4_OP_DECODE_ATTENTION) return (M < 1 || K < 1) ? bytes : bytes + attn_decode_partial_bytes(M, K);
     if (M < 1 || N <= 0 || K <= 0) return bytes;
     if (M <= SKINNY_MAX_M) {
@@ -247,7 +249,7 @@ size_t gptq4_workspace_bytes(int op, int M, int K, int N) {
                 if (pl.ok && gemv_partial_bytes(pl, M, epi) > need) need = gemv_partial_bytes(pl, M, epi);
             }
         }
-        bytes += need + (size_t)M * K * 2;  // + the rows gathered for an act-order call
+        bytes += need + (with_perm ? (size_t)M * K * 2 : 0);  // + the rows gathered for an act-order call
     } else if ((K % 64) == 0) {
         const int epi = (op == GPTQ4_OP_MLP_GATEUP) ? EPI_SILU_MUL : (op == GPTQ4_OP_QKV_ROTARY ? EPI_ROPE : EPI_PLAIN);
         // whichever kernel the current (automatic or forced) plans pick, with or without act-order
@@ -256,7 +258,7 @@ size_t gptq4_workspace_bytes(int op, int M, int K, int N) {
         if (kp.ok && kslice_partial_bytes(epi, kp) > need) need = kslice_partial_bytes(epi, kp);
         bytes += need;
         // + the rows gathered for an act-order call
-        if ((size_t)M * K * 2 <= ACT_ORDER_STAGE_MAX) bytes += (size_t)M * K * 2;
+        if (with_perm && (size_t)M * K * 2 <= ACT_ORDER_STAGE_MAX) bytes += (size_t)M * K * 2;
     }
     return bytes;
 }

@@ -114,7 +114,7 @@ def qkv_rotary(groupsize: int, hidden_states: torch.Tensor, qweight: torch.Tenso
     if bsz * q_len == 0:
         return q, kk, vv
     lib = _lib.load()
-    need = lib.gptq4_workspace_bytes(_lib.OP_QKV_ROTARY, bsz * q_len, k_in, n)
+    need = lib.gptq4_workspace_bytes(_lib.op_for(_lib.OP_QKV_ROTARY, perm), bsz * q_len, k_in, n)
     ws = _lib.workspace(dev, need)
     x2d = hidden_states.view(-1, k_in)
     rc = lib.gptq4_qkv_rotary(x2d.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(),

@@ -33,7 +33,7 @@ def llama_mlp_4(groupsize: int, a: torch.Tensor,
     c = torch.empty((m, n), device=a.device, dtype=torch.float16)
     if m == 0:
         return c.view(a.shape[:-1] + (n,))
-    need = lib.gptq4_workspace_bytes(_lib.OP_MLP_GATEUP, m, k, n)
+    need = lib.gptq4_workspace_bytes(_lib.op_for(_lib.OP_MLP_GATEUP, perm), m, k, n)
     ws = _lib.workspace(a.device, need)
     rc = lib.gptq4_mlp_gateup(x.data_ptr(), gate_qweight.data_ptr(), gate_qzeros.data_ptr(), gate_scales.data_ptr(),
                               up_qweight.data_ptr(), up_qzeros.data_ptr(), up_scales.data_ptr(), _lib.ptr(perm),

@@ -61,7 +61,7 @@ def matmul4(groupsize: int, a: torch.Tensor, qweight: torch.Tensor, scales: torc
     c = torch.empty((m, n), device=a.device, dtype=torch.float16)
     if m == 0:
         return c.view(a.shape[:-1] + (n,))
-    need = lib.gptq4_workspace_bytes(_lib.OP_MATMUL, m, k, n)
+    need = lib.gptq4_workspace_bytes(_lib.op_for(_lib.OP_MATMUL, perm), m, k, n)
     ws = _lib.workspace(a.device, need)
     rc = lib.gptq4_matmul(x.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(),
                           _lib.ptr(perm), _lib.ptr(bias), c.data_ptr(), m, k, n, groupsize,

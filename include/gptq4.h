@@ -28,7 +28,7 @@
  *    tiled kernel gathers by itself beyond that).
  *  - `workspace` holds split-K partial sums, arrival counters and, for a call with
  *    `perm`, the gathered activations (M * K * 2 bytes).  Size it with
- *    gptq4_workspace_bytes(); its first GPTQ4_WS_COUNTER_BYTES bytes must be zero
+ *    gptq4_workspace_bytes() (selector | GPTQ4_OP_WITH_PERM for such calls); its first GPTQ4_WS_COUNTER_BYTES bytes must be zero
  *    before the FIRST call that uses it (each call leaves them zero again).  One
  *    workspace may be shared by all calls on one stream; calls that run
  *    concurrently on different streams need a workspace each.
@@ -60,12 +60,14 @@ extern "C" {
 #define GPTQ4_OP_MLP_GATEUP 1
 #define GPTQ4_OP_QKV_ROTARY 2
 #define GPTQ4_OP_DECODE_ATTENTION 3 /* M = B * H, K = kv_capacity, N unused */
+#define GPTQ4_OP_WITH_PERM 0x100    /* or-ed to a matmul selector: the call will pass `perm` */
 
 int gptq4_abi_version(void);
 const char *gptq4_strerror(int code);
 
 /* Bytes of workspace an operation needs for M rows and N output columns
- * (N = I for MLP_GATEUP, N = 3*H*D for QKV_ROTARY).  No reference counterpart: the
+ * (N = I for MLP_GATEUP, N = 3*H*D for QKV_ROTARY; or GPTQ4_OP_WITH_PERM to the selector for
+ * calls that pass `perm`: room for the gathered rows).  No reference counterpart: the
  * Triton kernels own a whole K loop per output tile; split-K across workgroups is
  * what fills 256 CUs on GEMV-sized problems. */
 size_t gptq4_workspace_bytes(int op, int M, int K, int N);

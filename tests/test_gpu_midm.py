@@ -159,7 +159,7 @@ def test_act_order_inputs_reach_the_mid_m_kernel_through_the_staged_copy():
     D = to_dev(L)
     xd = torch.from_numpy(x).cuda()
     y = torch.empty((m, n), dtype=torch.float16, device="cuda")
-    ws = _lib.workspace(xd.device, lib.gptq4_workspace_bytes(_lib.OP_MATMUL, m, k, n))
+    ws = _lib.workspace(xd.device, lib.gptq4_workspace_bytes(_lib.OP_MATMUL | _lib.OP_WITH_PERM, m, k, n))
     try:
         lib.gptq4_set_midm_tuning(2, 0, 0)
         rc = lib.gptq4_matmul(xd.data_ptr(), Wq.data_ptr(), D["qzeros"].data_ptr(), D["scales"].data_ptr(), perm.data_ptr(), None,
@@ -169,7 +169,7 @@ def test_act_order_inputs_reach_the_mid_m_kernel_through_the_staged_copy():
     assert rc == 0
     ref = O.quant_matmul_ref(x, L["qweight"], L["qzeros"], L["scales"], g, g_idx=L["g_idx"])
     assert_close(y.cpu().numpy(), ref, "act-order through the C ABI, M=48")
-    need = lib.gptq4_workspace_bytes(_lib.OP_MATMUL, m, k, n)
+    need = lib.gptq4_workspace_bytes(_lib.OP_MATMUL | _lib.OP_WITH_PERM, m, k, n)
     assert need >= _lib.WS_COUNTER_BYTES + m * k * 2
     rc = lib.gptq4_matmul(xd.data_ptr(), Wq.data_ptr(), D["qzeros"].data_ptr(), D["scales"].data_ptr(), perm.data_ptr(), None,
                           y.data_ptr(), m, k, n, g, ws.data_ptr(), _lib.WS_COUNTER_BYTES + m * k * 2 - 16,

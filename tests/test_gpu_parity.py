@@ -350,7 +350,7 @@ def test_act_order_above_16_rows_staged_or_gathered_by_the_tiled_kernel(own_gath
     xd = torch.from_numpy(x).cuda()
     y = torch.empty((m, n), dtype=torch.float16, device="cuda")
     lib = _lib.load()
-    ws = _lib.workspace(xd.device, lib.gptq4_workspace_bytes(_lib.OP_MATMUL, m, k, n))
+    ws = _lib.workspace(xd.device, lib.gptq4_workspace_bytes(_lib.OP_MATMUL | _lib.OP_WITH_PERM, m, k, n))
     if own_gather:
         lib.gptq4_set_midm_tuning(0, 0, 0)
         lib.gptq4_set_gemm_tuning(10, 0)

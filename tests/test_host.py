@@ -62,19 +62,17 @@ def test_error_codes_are_returned_before_any_launch():
 def test_workspace_query():
     lib = _lib.load()
     base = _lib.WS_COUNTER_BYTES
-
-    def rows(m, k):  # room for the gathered activations of an act-order call
-        return m * k * 2
-
-    # enough tiles: no split-K, only the counters and the rows
-    assert lib.gptq4_workspace_bytes(_lib.OP_MATMUL, 4096, 4096, 12288) == base + rows(4096, 4096)
+    assert lib.gptq4_workspace_bytes(_lib.OP_MATMUL, 4096, 4096, 12288) == base   # enough tiles: no split-K, only the counters
     one = lib.gptq4_workspace_bytes(_lib.OP_MATMUL, 1, 4096, 4096)
-    assert one >= base + 16 * 1 * 4096 * 4 + rows(1, 4096)    # 16 split-K slots at least; the decode GEMV may want more
-    assert lib.gptq4_workspace_bytes(_lib.OP_MLP_GATEUP, 16, 4096, 11008) == base + 16 * 16 * 2 * 11008 * 4 + rows(16, 4096)
+    assert one >= base + 16 * 1 * 4096 * 4                    # 16 split-K slots at least; the decode GEMV may want more
+    assert lib.gptq4_workspace_bytes(_lib.OP_MLP_GATEUP, 16, 4096, 11008) == base + 16 * 16 * 2 * 11008 * 4
     # mid-M on a narrow layer: 32 tiles of 128x128, split 8 ways, 64 KiB of fp32 per tile and split
-    assert lib.gptq4_workspace_bytes(_lib.OP_MATMUL, 128, 4096, 4096) == base + 32 * 8 * 65536 + rows(128, 4096)
-    # rows beyond the staging limit (1 GiB) are gathered by the tiled kernel itself: no room asked for
-    assert lib.gptq4_workspace_bytes(_lib.OP_MATMUL, 32768, 17920, 6656) == base
+    assert lib.gptq4_workspace_bytes(_lib.OP_MATMUL, 128, 4096, 4096) == base + 32 * 8 * 65536
+    # a call that will pass `perm` also needs room for its gathered rows (M * K fp16 values) ...
+    for op, m, k, n in ((_lib.OP_MATMUL, 4096, 4096, 12288), (_lib.OP_MLP_GATEUP, 16, 4096, 11008), (_lib.OP_QKV_ROTARY, 128, 4096, 12288)):
+        assert lib.gptq4_workspace_bytes(op | _lib.OP_WITH_PERM, m, k, n) == lib.gptq4_workspace_bytes(op, m, k, n) + m * k * 2
+    # ... unless they pass the staging limit (1 GiB): the tiled kernel gathers such rows itself
+    assert lib.gptq4_workspace_bytes(_lib.OP_MATMUL | _lib.OP_WITH_PERM, 32768, 17920, 6656) == base
 
 
 def test_quant_linear_layout_and_errors():
