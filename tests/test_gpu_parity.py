@@ -365,6 +365,45 @@ def test_act_order_above_16_rows_staged_or_gathered_by_the_tiled_kernel(own_gath
     assert_close(y.cpu().numpy(), ref, f"act-order, M={m}, own gather {own_gather}")
 
 
+@pytest.mark.parametrize("k,n", [(128, 256), (640, 768), (1408, 512), (3072, 1024)])
+@pytest.mark.parametrize("m", [1, 3, 16, 17, 77, 300, 600])
+def test_a_call_with_perm_equals_the_call_on_gathered_rows(k, n, m):
+    """Whatever kernel the row count selects, passing `perm` must give the very bits of the same call on
+    x[:, perm]: the call only gathers the rows (for the decode GEMV: inside its LDS copy) and then does what it
+    does without a permutation.  Odd K included (K/128 = 1, 5, 11, 24)."""
+    G = gptq()
+    gen = torch.Generator(device="cuda"); gen.manual_seed(k + n + m)
+    g = 128
+    W = [(torch.randint(-2**31, 2**31 - 1, (k // 8, n), dtype=torch.int32, device="cuda", generator=gen),
+          torch.randint(-2**31, 2**31 - 1, (k // g, n // 8), dtype=torch.int32, device="cuda", generator=gen),
+          (0.002 + 0.02 * torch.rand((k // g, n), device="cuda", generator=gen)).half()) for _ in range(2)]
+    perm = torch.randperm(k, device="cuda", generator=gen).int()
+    x = torch.randn((m, k), device="cuda", generator=gen).half()
+    xg = x[:, perm.long()].contiguous()
+    (q0, z0, s0), (q1, z1, s1) = W
+    assert torch.equal(G.matmul4(g, x, q0, s0, z0, perm=perm), G.matmul4(g, xg, q0, s0, z0))
+    assert torch.equal(G.llama_mlp_4(g, x, q0, s0, z0, q1, s1, z1, perm=perm), G.llama_mlp_4(g, xg, q0, s0, z0, q1, s1, z1))
+
+
+@pytest.mark.parametrize("heads", [2, 6, 10])
+@pytest.mark.parametrize("m", [1, 3, 16, 17, 77, 300, 600])
+def test_qkv_rotary_with_perm_equals_the_call_on_gathered_rows(heads, m):
+    G = gptq()
+    gen = torch.Generator(device="cuda"); gen.manual_seed(heads + m)
+    k, g = heads * 128, 128
+    qw = torch.randint(-2**31, 2**31 - 1, (k // 8, 3 * k), dtype=torch.int32, device="cuda", generator=gen)
+    qz = torch.randint(-2**31, 2**31 - 1, (k // g, 3 * k // 8), dtype=torch.int32, device="cuda", generator=gen)
+    sc = (0.002 + 0.02 * torch.rand((k // g, 3 * k), device="cuda", generator=gen)).half()
+    perm = torch.randperm(k, device="cuda", generator=gen).int()
+    x = torch.randn((1, m, k), device="cuda", generator=gen).half()
+    xg = x[..., perm.long()].contiguous()
+    cos, sin = G.RotaryTable(128, 1024).get(torch.device("cuda"), 1024)
+    pos = torch.arange(m, device="cuda", dtype=torch.int32)[None]
+    a = G.qkv_rotary(g, x, qw, sc, qz, pos, cos, sin, heads, perm=perm)
+    b = G.qkv_rotary(g, xg, qw, sc, qz, pos, cos, sin, heads)
+    assert all(torch.equal(u, v) for u, v in zip(a, b))
+
+
 def test_empty_inputs_give_empty_outputs():
     """Zero rows: every functional returns a tensor of the right shape and launches nothing;
     the C entry points themselves reject M < 1."""
