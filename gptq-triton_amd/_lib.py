@@ -31,8 +31,8 @@ SIGNATURES = {
     "gptq4_norm_qkv_rotary": (c_int, [c_void_p] * 3 + [c_float] + [c_void_p] * 8 + [c_int] + [c_void_p] * 3 + [c_int] * 8
                               + [c_void_p, c_size_t, c_void_p]),
     "gptq4_norm_mlp_gateup": (c_int, [c_void_p] * 3 + [c_float] + [c_void_p] * 9 + [c_int] * 4 + [c_void_p, c_size_t, c_void_p]),
-    "gptq4_rmsnorm": (c_int, [c_void_p] * 3 + [c_int, c_int, c_float, c_void_p]),
-    "gptq4_add_rmsnorm": (c_int, [c_void_p] * 5 + [c_int, c_int, c_float, c_void_p]),
+    "gptq4_rmsnorm": (c_int, [c_void_p] * 4 + [c_int, c_int, c_float, c_void_p]),
+    "gptq4_add_rmsnorm": (c_int, [c_void_p] * 6 + [c_int, c_int, c_float, c_void_p]),
     "gptq4_decode_attention": (c_int, [c_void_p] * 6 + [c_int] * 4 + [c_float, c_void_p, c_size_t, c_void_p]),
     "gptq4_set_tuning": (None, [c_int, c_int, c_int]),
     "gptq4_set_gemm_tuning": (None, [c_int, c_int]),

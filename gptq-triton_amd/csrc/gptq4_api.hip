@@ -444,23 +444,26 @@ int gptq4_norm_qkv_rotary(const void *x, const void *delta, const void *norm_wei
                            workspace_bytes, stream, true);
 }
 
-int gptq4_rmsnorm(const void *x, const void *weight, void *y, int M, int H, float eps, void *stream) {
+int gptq4_rmsnorm(const void *x, const void *weight, void *y, const int32_t *y_index, int M, int H, float eps, void *stream) {
     if (!x || !weight || !y) return -GPTQ4_E_NULL;
     if (M < 1 || H < 8 || (H % 8) != 0 || !(eps >= 0.f)) return -GPTQ4_E_SHAPE;
-    if (misaligned16(x) || misaligned16(weight) || misaligned16(y)) return -GPTQ4_E_ALIGN;
+    if (y_index && y == x) return -GPTQ4_E_SHAPE;  // the moved values would overwrite input still to be read
+    if (misaligned16(x) || misaligned16(weight) || misaligned16(y) || (y_index && misaligned16(y_index))) return -GPTQ4_E_ALIGN;
     return launch_rmsnorm(reinterpret_cast<const half_t *>(x), nullptr, reinterpret_cast<const half_t *>(weight), nullptr,
-                          reinterpret_cast<half_t *>(y), M, H, eps, reinterpret_cast<hipStream_t>(stream));
+                          reinterpret_cast<half_t *>(y), y_index, M, H, eps, reinterpret_cast<hipStream_t>(stream));
 }
 
-int gptq4_add_rmsnorm(const void *x, const void *delta, const void *weight, void *sum_out, void *y, int M, int H, float eps,
-                      void *stream) {
+int gptq4_add_rmsnorm(const void *x, const void *delta, const void *weight, void *sum_out, void *y, const int32_t *y_index,
+                      int M, int H, float eps, void *stream) {
     if (!x || !delta || !weight || !sum_out || !y) return -GPTQ4_E_NULL;
     if (M < 1 || H < 8 || (H % 8) != 0 || !(eps >= 0.f)) return -GPTQ4_E_SHAPE;
-    if (misaligned16(x) || misaligned16(delta) || misaligned16(weight) || misaligned16(sum_out) || misaligned16(y))
+    if (y_index && (y == x || y == delta || y == sum_out)) return -GPTQ4_E_SHAPE;
+    if (misaligned16(x) || misaligned16(delta) || misaligned16(weight) || misaligned16(sum_out) || misaligned16(y) ||
+        (y_index && misaligned16(y_index)))
         return -GPTQ4_E_ALIGN;
     return launch_rmsnorm(reinterpret_cast<const half_t *>(x), reinterpret_cast<const half_t *>(delta),
                           reinterpret_cast<const half_t *>(weight), reinterpret_cast<half_t *>(sum_out),
-                          reinterpret_cast<half_t *>(y), M, H, eps, reinterpret_cast<hipStream_t>(stream));
+                          reinterpret_cast<half_t *>(y), y_index, M, H, eps, reinterpret_cast<hipStream_t>(stream));
 }
 
 int gptq4_decode_attention(const void *q, const void *k_cache, const void *v_cache, const int32_t *positions, void *out,

@@ -12,9 +12,12 @@ namespace {
 // fp16, then an fp16 multiply by the weight - the rounding order of the LLaMA RMSNorm
 // module.  One workgroup per row, H % 8 == 0; sum_out may alias x.  The arithmetic lives in
 // gptq4_norm.h, shared with the matmul kernels that normalise their own input.
+// y_index (nullable): value f of a row is stored at y[row][y_index[f]] - the order in which an
+// act-order projection reads its input, so that it needs no gather.
 template <bool ADD>
 __global__ __launch_bounds__(256) void gptq4_rmsnorm_kernel(const half_t *x, const half_t *delta, const half_t *__restrict__ w,
-                                                            half_t *sum_out, half_t *__restrict__ y, int H, float eps) {
+                                                            half_t *sum_out, half_t *__restrict__ y,
+                                                            const int32_t *__restrict__ y_index, int H, float eps) {
     __shared__ float part[4];
     const int tid = threadIdx.x;
     const size_t row = (size_t)blockIdx.x * H;
@@ -38,7 +41,20 @@ __global__ __launch_bounds__(256) void gptq4_rmsnorm_kernel(const half_t *x, con
         if (tid + 256 * n < chunks) held[n] = take(tid + 256 * n);
     for (int c = tid + 256 * KEEP; c < chunks; c += 256) take(c);
     const float inv = norm_inv_rms(ss, part, tid, H, eps);
-    auto put = [&](int c, uint4 v) { yr[c] = norm_put(v, wr[c], inv); };
+    uint16_t *yh = reinterpret_cast<uint16_t *>(y + row);
+    auto put = [&](int c, uint4 v) {
+        const uint4 o = norm_put(v, wr[c], inv);
+        if (y_index == nullptr) {
+            yr[c] = o;
+            return;
+        }
+        const int4 i0 = *reinterpret_cast<const int4 *>(y_index + 8 * c);
+        const int4 i1 = *reinterpret_cast<const int4 *>(y_index + 8 * c + 4);
+        yh[i0.x] = (uint16_t)o.x, yh[i0.y] = (uint16_t)(o.x >> 16);
+        yh[i0.z] = (uint16_t)o.y, yh[i0.w] = (uint16_t)(o.y >> 16);
+        yh[i1.x] = (uint16_t)o.z, yh[i1.y] = (uint16_t)(o.z >> 16);
+        yh[i1.z] = (uint16_t)o.w, yh[i1.w] = (uint16_t)(o.w >> 16);
+    };
 #pragma unroll
     for (int n = 0; n < KEEP; ++n)
         if (tid + 256 * n < chunks) put(tid + 256 * n, held[n]);
@@ -191,12 +207,13 @@ __global__ __launch_bounds__(256) void gptq4_attn_decode_kernel(const half_t *__
 
 }  // namespace
 
-int launch_rmsnorm(const half_t *x, const half_t *delta, const half_t *w, half_t *sum_out, half_t *y, int M, int H, float eps,
-                   hipStream_t stream) {
+int launch_rmsnorm(const half_t *x, const half_t *delta, const half_t *w, half_t *sum_out, half_t *y, const int32_t *y_index,
+                   int M, int H, float eps, hipStream_t stream) {
     if (delta != nullptr)
-        hipLaunchKernelGGL(gptq4_rmsnorm_kernel<true>, dim3((unsigned)M), dim3(256), 0, stream, x, delta, w, sum_out, y, H, eps);
+        hipLaunchKernelGGL(gptq4_rmsnorm_kernel<true>, dim3((unsigned)M), dim3(256), 0, stream, x, delta, w, sum_out, y, y_index, H,
+                           eps);
     else
-        hipLaunchKernelGGL(gptq4_rmsnorm_kernel<false>, dim3((unsigned)M), dim3(256), 0, stream, x, x, w, y, y, H, eps);
+        hipLaunchKernelGGL(gptq4_rmsnorm_kernel<false>, dim3((unsigned)M), dim3(256), 0, stream, x, x, w, y, y, y_index, H, eps);
     return (int)hipGetLastError();
 }
 

@@ -49,8 +49,16 @@ def check_norm_args(h: torch.Tensor, delta, weight: torch.Tensor):
     return h2, d2, s
 
 
-def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
-    """y = weight * fp16(x * rsqrt(mean(x^2, -1) + eps)) for fp16 x [..., H] on the GPU."""
+def _check_out_index(out_index, h: int) -> None:
+    if out_index is not None:
+        _lib.require_cuda(out_index, "out_index")
+        if out_index.dtype != torch.int32 or out_index.shape != (h,) or not out_index.is_contiguous():
+            raise ValueError(f"out_index must be a contiguous int32 tensor of {h} positions")
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, out_index: torch.Tensor = None) -> torch.Tensor:
+    """y = weight * fp16(x * rsqrt(mean(x^2, -1) + eps)) for fp16 x [..., H] on the GPU.  With out_index (int32
+    [H], a permutation) value f of a row is stored at position out_index[f]."""
     _lib.require_cuda(x, "x")
     _lib.require_cuda(weight, "weight")
     if x.dtype != torch.float16 or weight.dtype != torch.float16:
@@ -58,20 +66,22 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     h = x.shape[-1]
     if weight.shape != (h,) or h % 8 != 0:
         raise ValueError(f"weight must be [{h}] and the hidden size a multiple of 8")
+    _check_out_index(out_index, h)
     x2 = x.reshape(-1, h)
     if not x2.is_contiguous():
         x2 = x2.contiguous()
     y = torch.empty_like(x2)
     if x2.shape[0] == 0:
         return y.reshape(x.shape)
-    rc = _lib.load().gptq4_rmsnorm(x2.data_ptr(), weight.data_ptr(), y.data_ptr(), x2.shape[0], h, float(eps),
-                                   _lib.current_stream(x.device))
+    rc = _lib.load().gptq4_rmsnorm(x2.data_ptr(), weight.data_ptr(), y.data_ptr(), _lib.ptr(out_index), x2.shape[0], h,
+                                   float(eps), _lib.current_stream(x.device))
     _lib.check(rc, "gptq4_rmsnorm")
     return y.reshape(x.shape)
 
 
-def add_rms_norm(x: torch.Tensor, delta: torch.Tensor, weight: torch.Tensor, eps: float):
-    """(x + delta, RMSNorm(x + delta)) in one launch; fp16 GPU tensors of equal shape [..., H]."""
+def add_rms_norm(x: torch.Tensor, delta: torch.Tensor, weight: torch.Tensor, eps: float, out_index: torch.Tensor = None):
+    """(x + delta, RMSNorm(x + delta)) in one launch; fp16 GPU tensors of equal shape [..., H].  out_index as in
+    rms_norm (the sum keeps its order)."""
     for t, name in ((x, "x"), (delta, "delta"), (weight, "weight")):
         _lib.require_cuda(t, name)
         if t.dtype != torch.float16:
@@ -79,13 +89,14 @@ def add_rms_norm(x: torch.Tensor, delta: torch.Tensor, weight: torch.Tensor, eps
     h = x.shape[-1]
     if delta.shape != x.shape or weight.shape != (h,) or h % 8 != 0:
         raise ValueError("x and delta must have one shape [..., H], weight [H], H a multiple of 8")
+    _check_out_index(out_index, h)
     x2 = x.reshape(-1, h).contiguous()
     d2 = delta.reshape(-1, h).contiguous()
     s = torch.empty_like(x2)
     y = torch.empty_like(x2)
     if x2.shape[0]:
         rc = _lib.load().gptq4_add_rmsnorm(x2.data_ptr(), d2.data_ptr(), weight.data_ptr(), s.data_ptr(), y.data_ptr(),
-                                           x2.shape[0], h, float(eps), _lib.current_stream(x.device))
+                                           _lib.ptr(out_index), x2.shape[0], h, float(eps), _lib.current_stream(x.device))
         _lib.check(rc, "gptq4_add_rmsnorm")
     return s.reshape(x.shape), y.reshape(x.shape)
 
@@ -110,10 +121,7 @@ def decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
         pos = pos.to(torch.int32).contiguous()
         if pos.numel() != bsz:
             raise ValueError("one position per sequence")
-    if out_index is not None:
-        _lib.require_cuda(out_index, "out_index")
-        if out_index.dtype != torch.int32 or out_index.shape != (heads * hd,) or not out_index.is_contiguous():
-            raise ValueError("out_index must be a contiguous int32 tensor of H*128 positions")
+    _check_out_index(out_index, heads * hd)
     cap = k_cache.shape[2]
     out = torch.empty((bsz, 1, heads * hd), dtype=torch.float16, device=q.device)
     lib = _lib.load()

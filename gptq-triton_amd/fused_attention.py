@@ -18,7 +18,7 @@ import torch
 import torch.nn as nn
 
 from . import _lib
-from .quant_linear import QuantLinear, _check_device_tensors, _check_matmul_args, matmul4
+from .quant_linear import QuantLinear, _check_device_tensors, _check_matmul_args, inverse_permutation, matmul4
 
 
 @dataclass
@@ -186,16 +186,18 @@ class QuantLlamaAttention(nn.Module):
         self.rope = RotaryTable(self.head_dim, self.max_position_embeddings,
                                 float(getattr(config, 'rope_theta', 10000.0)))
         self._context_order = None
+        self._input_order = None
 
     def project_qkv(self, hidden_states: torch.Tensor, position_ids: torch.Tensor,
-                    kv_out=None, kv_offset: int = 0, norm=None):
-        """norm = (delta or None, norm_weight, eps): see qkv_rotary."""
+                    kv_out=None, kv_offset: int = 0, norm=None, ordered: bool = False):
+        """norm = (delta or None, norm_weight, eps): see qkv_rotary.  ordered: hidden_states already are in the
+        order of input_order()."""
         need = max(kv_offset, 0) + hidden_states.shape[1]
         cos, sin = self.rope.get(hidden_states.device, max(need, self.max_position_embeddings))
         qweight, perm = self.qkv_proj.kernel_weights()
         return qkv_rotary(self.qkv_proj.groupsize, hidden_states, qweight, self.qkv_proj.scales,
                           self.qkv_proj.qzeros, position_ids, cos, sin, self.num_heads, self.head_dim,
-                          perm=perm, kv_out=kv_out, kv_offset=kv_offset, norm=norm)
+                          perm=None if ordered else perm, kv_out=kv_out, kv_offset=kv_offset, norm=norm)
 
     def context_order(self):
         """Where each feature of the attention output should be stored so that an act-order o_proj reads
@@ -205,10 +207,18 @@ class QuantLlamaAttention(nn.Module):
         if perm is None:
             return None
         if self._context_order is None or self._context_order[0] != perm.data_ptr():
-            inv = torch.empty_like(perm)
-            inv[perm.long()] = torch.arange(perm.numel(), device=perm.device, dtype=perm.dtype)
-            self._context_order = (perm.data_ptr(), inv)
+            self._context_order = (perm.data_ptr(), inverse_permutation(perm))
         return self._context_order[1]
+
+    def input_order(self):
+        """The same for the input of the fused QKV projection: rms_norm / add_rms_norm(out_index=...) write in
+        that order, and project_qkv(ordered=True) then runs without a gather.  None without act-order."""
+        _, perm = self.qkv_proj.kernel_weights()
+        if perm is None:
+            return None
+        if self._input_order is None or self._input_order[0] != perm.data_ptr():
+            self._input_order = (perm.data_ptr(), inverse_permutation(perm))
+        return self._input_order[1]
 
     def project_out(self, context: torch.Tensor, ordered: bool = False) -> torch.Tensor:
         """o_proj(context); ordered: the context already is in the order of context_order()."""

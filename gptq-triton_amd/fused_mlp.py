@@ -113,6 +113,7 @@ class QuantLlamaMLP(nn.Module):
             self.g_idx = None
         self._sorted = None
         self._chained = None
+        self._input_order = None
 
     def _kernel_weights(self):
         if self.g_idx is None:
@@ -162,9 +163,22 @@ class QuantLlamaMLP(nn.Module):
         d = self.down_proj
         return matmul4(d.groupsize, mid, down_q, d.scales, d.qzeros, d.bias, None)
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
+    def input_order(self):
+        """Where a producer should store each input feature so that x arrives in the order gate and up read it
+        (int32 [infeatures], the inverse of their shared permutation; None without act-order):
+        rms_norm / add_rms_norm(out_index=...) write in that order and forward(x, ordered=True) runs
+        without a gather."""
+        perm = self._chained_weights()[1]
+        if perm is None:
+            return None
+        if self._input_order is None or self._input_order[0] != perm.data_ptr():
+            from .quant_linear import inverse_permutation
+            self._input_order = (perm.data_ptr(), inverse_permutation(perm))
+        return self._input_order[1]
+
+    def forward(self, x: torch.Tensor, ordered: bool = False) -> torch.Tensor:
         w, perm, down_q = self._chained_weights()
-        return self._down(llama_mlp_4(self.groupsize, x, *w, perm), down_q)
+        return self._down(llama_mlp_4(self.groupsize, x, *w, None if ordered else perm), down_q)
 
     def norm_fusable(self, rows: int) -> bool:
         """Whether forward_normed is the faster way for this many rows."""

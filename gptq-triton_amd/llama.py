@@ -20,6 +20,9 @@ import torch.nn as nn
 from .decoder_ops import add_rms_norm, decode_attention, rms_norm
 from .fused_attention import LlamaConfigLite
 
+# up to this many rows the decoder's norms write act-order inputs in their consumer's order
+ORDERED_NORM_ROWS = 16
+
 
 def config_from_json(path) -> LlamaConfigLite:
     """Read the fields this path needs from an HF-style config.json."""
@@ -182,15 +185,28 @@ class GreedyDecoder:
         if all(getattr(l.self_attn, "norm_fusable", lambda r: False)(rows) and getattr(l.mlp, "norm_fusable", lambda r: False)(rows)
                for l in layers):
             return self._layers_norm_in_matmul(h, position_ids, kv_offset, attend)
-        x = layers[0].input_layernorm(h)
+        # act-order and a handful of rows: every norm writes in the order its consumer's sorted rows read, so the
+        # consumer needs no gather launch (tall inputs leave the gather to the consumer: there the norm's
+        # scattered 2-byte stores would cost more than the copy)
+        def order_of(block):
+            fn = getattr(block, "input_order", None)
+            return fn() if fn is not None and rows <= ORDERED_NORM_ROWS else None
+
+        n0 = layers[0].input_layernorm
+        oq = order_of(layers[0].self_attn)
+        x = rms_norm(h, n0.weight, n0.variance_epsilon, out_index=oq)
         for i, (layer, (kc, vc)) in enumerate(zip(layers, self.caches)):
             attn = layer.self_attn
-            q, _, _ = attn.project_qkv(x, position_ids, kv_out=(kc, vc), kv_offset=kv_offset)
+            q, _, _ = attn.project_qkv(x, position_ids, kv_out=(kc, vc), kv_offset=kv_offset, ordered=oq is not None)
             norm = layer.post_attention_layernorm
+            om = order_of(layer.mlp)
             # attend -> ([B, S, hidden], whether in attn.context_order())
-            h, x = add_rms_norm(h, attn.project_out(*attend(q, kc, vc, attn)), norm.weight, norm.variance_epsilon)
-            norm = layers[i + 1].input_layernorm if i + 1 < len(layers) else self.model.model.norm
-            h, x = add_rms_norm(h, layer.mlp(x), norm.weight, norm.variance_epsilon)
+            h, x = add_rms_norm(h, attn.project_out(*attend(q, kc, vc, attn)), norm.weight, norm.variance_epsilon, out_index=om)
+            last = i + 1 == len(layers)
+            norm = self.model.model.norm if last else layers[i + 1].input_layernorm
+            oq = None if last else order_of(layers[i + 1].self_attn)
+            y = layer.mlp(x, ordered=True) if om is not None else layer.mlp(x)
+            h, x = add_rms_norm(h, y, norm.weight, norm.variance_epsilon, out_index=oq)
         return self.model.lm_head(x[:, -1:, :]).argmax(-1)
 
     def _layers_norm_in_matmul(self, h, position_ids, kv_offset, attend):

@@ -87,6 +87,14 @@ def dequantize(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor
     return out
 
 
+def inverse_permutation(perm: torch.Tensor) -> torch.Tensor:
+    """inv with inv[perm[j]] = j: where a producer must store feature f (at inv[f]) so that its output is in the
+    order x[:, perm] an act-order projection reads."""
+    inv = torch.empty_like(perm)
+    inv[perm.long()] = torch.arange(perm.numel(), device=perm.device, dtype=perm.dtype)
+    return inv
+
+
 def prepare_act_order(qweight: torch.Tensor, g_idx: torch.Tensor, groupsize: int):
     """Load-time re-layout for act-order checkpoints.
 

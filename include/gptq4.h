@@ -155,14 +155,20 @@ int gptq4_norm_mlp_gateup(const void *x, const void *delta, const void *norm_wei
 /* RMSNorm over the last dimension: y = weight * fp16(x * rsqrt(mean(x^2) + eps)), x and y
  * fp16 [M, H], weight fp16 [H], H a multiple of 8; statistics in fp32.  Stands in for the
  * LlamaRMSNorm modules of the model the reference builds and runs between its fused blocks
- * (src/gptq_triton/__init__.py:32-47; the quantised linears are the only modules it swaps). */
-int gptq4_rmsnorm(const void *x, const void *weight, void *y, int M, int H, float eps, void *stream);
+ * (src/gptq_triton/__init__.py:32-47; the quantised linears are the only modules it swaps).
+ * y_index (nullable) int32 [H], a permutation of 0..H-1: value f of a row is then stored at
+ * y[m, y_index[f]] (y must not alias an input) - with the inverse of an act-order projection's
+ * `perm`, y comes out in the order of that projection's sorted rows and the projection is called
+ * without `perm`. */
+int gptq4_rmsnorm(const void *x, const void *weight, void *y, const int32_t *y_index, int M, int H,
+                  float eps, void *stream);
 
 /* The residual add that precedes every RMSNorm of a decoder layer, fused with it:
- * sum_out = fp16(x + delta) (may alias x), y = RMSNorm(sum_out).  Same shapes as above.  In
- * the reference these are two torch ops of the HF decoder layer around its patched blocks. */
+ * sum_out = fp16(x + delta) (may alias x), y = RMSNorm(sum_out).  Same shapes and y_index as
+ * above.  In the reference these are two torch ops of the HF decoder layer around its patched
+ * blocks. */
 int gptq4_add_rmsnorm(const void *x, const void *delta, const void *weight, void *sum_out, void *y,
-                      int M, int H, float eps, void *stream);
+                      const int32_t *y_index, int M, int H, float eps, void *stream);
 
 /* Attention of ONE query token per sequence over a preallocated KV cache: for each (b, h)
  * softmax(q . K[0..positions[b]]^T * scale) . V[0..positions[b]], in fp32, written as fp16

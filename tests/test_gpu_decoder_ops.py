@@ -45,6 +45,36 @@ def test_add_rmsnorm(m, h):
     assert torch.equal(y, y2)
 
 
+@pytest.mark.parametrize("m,h", [(1, 4096), (8, 5120), (16, 13824), (40, 6656), (2, 8200)])
+def test_norms_store_in_a_given_order(m, h):
+    """With out_index, value f of every row lands at position out_index[f]: the same bits, moved (rows longer
+    than the 8192 values held in registers included); the sum keeps its order."""
+    G = gptq()
+    gen = torch.Generator(device="cuda"); gen.manual_seed(m + h)
+    x = (3 * torch.randn((m, h), device="cuda", generator=gen)).half()
+    d = torch.randn((m, h), device="cuda", generator=gen).half()
+    w = (1 + 0.1 * torch.randn(h, device="cuda", generator=gen)).half()
+    order = torch.randperm(h, device="cuda", generator=gen).int()
+    y = G.rms_norm(x, w, 1e-6)
+    moved = G.rms_norm(x, w, 1e-6, out_index=order)
+    want = torch.empty_like(y)
+    want[:, order.long()] = y
+    assert torch.equal(moved, want)
+    s, y = G.add_rms_norm(x, d, w, 1e-6)
+    s2, moved = G.add_rms_norm(x, d, w, 1e-6, out_index=order)
+    want[:, order.long()] = y
+    assert torch.equal(s, s2) and torch.equal(moved, want)
+    # the moved values may not land in a tensor that is still being read
+    from gptq_triton_amd import _lib
+    lib = _lib.load()
+    stream = _lib.current_stream(x.device)
+    rc = lib.gptq4_rmsnorm(x.data_ptr(), w.data_ptr(), x.data_ptr(), order.data_ptr(), m, h, 1e-6, stream)
+    assert rc < 0 and b"shape" in lib.gptq4_strerror(rc).lower()
+    rc = lib.gptq4_add_rmsnorm(x.data_ptr(), d.data_ptr(), w.data_ptr(), s.data_ptr(), d.data_ptr(), order.data_ptr(), m, h, 1e-6,
+                               stream)
+    assert rc < 0
+
+
 def test_rmsnorm_keeps_batch_dims_and_rejects_host_tensors():
     x = torch.randn(2, 3, 256).half()
     w = torch.ones(256).half()
