@@ -143,9 +143,17 @@ bool prefer_kslice(const KslicePlan &kp, int epi, int M, int N, int K) {
 }
 
 int run_tiled(int epi, MatmulArgs &a, void *workspace, size_t workspace_bytes, hipStream_t s) {
-    // act-order: staged activations wherever they fit the staging limit (then the mid-M kernel can run too)
-    const bool stage = a.perm != nullptr && !g_gemm_tuning.own_gather &&
-                       (size_t)a.M * a.K * sizeof(half_t) <= ACT_ORDER_STAGE_MAX;
+    // act-order: staged activations wherever they fit the staging limit and the workspace (then the mid-M
+    // kernel can run too); else the tiled kernel gathers by itself
+    const size_t rows_bytes = (size_t)a.M * a.K * sizeof(half_t);
+    bool stage = a.perm != nullptr && !g_gemm_tuning.own_gather && rows_bytes <= ACT_ORDER_STAGE_MAX;
+    const GemmPlan pl = gemm_plan(epi, a.M, a.N, a.K);
+    if (stage) {
+        const KslicePlan kp = kslice_plan(epi, a.M, a.N, a.K, false);
+        const size_t partial = prefer_kslice(kp, epi, a.M, a.N, a.K) ? (kp.splitk > 1 ? kslice_partial_bytes(epi, kp) : 0)
+                                                                       : (pl.splitk > 1 ? gemm_partial_bytes(pl) : 0);
+        if (workspace == nullptr || workspace_bytes < GPTQ4_WS_COUNTER_BYTES + partial + rows_bytes) stage = false;
+    }
     const KslicePlan kp = kslice_plan(epi, a.M, a.N, a.K, a.perm != nullptr && !stage);
     if (prefer_kslice(kp, epi, a.M, a.N, a.K)) {
         a.tiles = kp.tiles;
@@ -165,7 +173,6 @@ int run_tiled(int epi, MatmulArgs &a, void *workspace, size_t workspace_bytes, h
         }
         return launch_kslice(epi, a, kp, s);
     }
-    const GemmPlan pl = gemm_plan(epi, a.M, a.N, a.K);
     int rc = setup_gemm(a, pl, workspace, workspace_bytes);
     if (rc) return rc;
     if (stage) {

@@ -24,8 +24,9 @@
  *  - `perm` (nullable) is the act-order row permutation made by
  *    gptq4_actorder_sort_rows(): logical weight row j multiplies x[:, perm[j]] and
  *    belongs to group j / groupsize.  The calls gather the rows of x into the workspace
- *    with one small launch of their own and multiply from there (up to 1 GiB of rows; the
- *    tiled kernel gathers by itself beyond that).
+ *    with one small launch of their own and multiply from there (up to 1 GiB of rows; beyond
+ *    that, or with more than 16 rows and a workspace without room for them, the tiled kernel
+ *    gathers by itself, which is slower).
  *  - `workspace` holds split-K partial sums, arrival counters and, for a call with
  *    `perm`, the gathered activations (M * K * 2 bytes).  Size it with
  *    gptq4_workspace_bytes() (selector | GPTQ4_OP_WITH_PERM for such calls); its first GPTQ4_WS_COUNTER_BYTES bytes must be zero
