@@ -517,7 +517,9 @@ GemvPlan gemv_plan(int epi, int M, int N, int K, bool norm) {
     if (lds < want) lds = want;
     pl.lds_bytes = lds;
     // waves touching one tile: its NB units are owned by consecutive waves of >= q units
-    pl.max_contrib = (pl.q > 0) ? (pl.nb + pl.q - 1) / pl.q + 1 : 1;
+    // (fewer units than waves: every unit has a wave of its own, a tile as many contributors as batches)
+    pl.max_contrib = (pl.q > 0) ? (pl.nb + pl.q - 1) / pl.q + 1 : pl.nb;
+    if (pl.max_contrib > pl.nb) pl.max_contrib = pl.nb;
     return pl;
 }
 

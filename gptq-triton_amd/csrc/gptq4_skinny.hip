@@ -452,10 +452,22 @@ int launch_norm_variant(const MatmulArgs &a, hipStream_t stream) {
         hipLaunchKernelGGL((gptq4_skinny_kernel<EPI, 2, DEPTH, false, 4, 2>), grid, block, lds, stream, a);
     else if (a.K <= 4096)
         hipLaunchKernelGGL((gptq4_skinny_kernel<EPI, 2, DEPTH, true, 4, 2>), grid, block, lds, stream, a);
-    else if (!perm)
-        hipLaunchKernelGGL((gptq4_skinny_kernel<EPI, 2, DEPTH, false, 4, 4>), grid, block, lds, stream, a);
-    else
-        hipLaunchKernelGGL((gptq4_skinny_kernel<EPI, 2, DEPTH, true, 4, 4>), grid, block, lds, stream, a);
+    else {
+        // rows of more than 4096 values: up to 64 KiB of rows on top of the 16 KiB reduction buffer - more than
+        // the 64 KiB a launch may ask for unless the kernel is marked for it (once per variant)
+        static bool allowed[2] = {false, false};
+        if (!allowed[perm]) {
+            const void *fn = perm ? reinterpret_cast<const void *>(&gptq4_skinny_kernel<EPI, 2, DEPTH, true, 4, 4>)
+                                  : reinterpret_cast<const void *>(&gptq4_skinny_kernel<EPI, 2, DEPTH, false, 4, 4>);
+            const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, NORM_MAX_M * NORM_MAX_H * (int)sizeof(half_t));
+            if (e != hipSuccess) return (int)e;
+            allowed[perm] = true;
+        }
+        if (!perm)
+            hipLaunchKernelGGL((gptq4_skinny_kernel<EPI, 2, DEPTH, false, 4, 4>), grid, block, lds, stream, a);
+        else
+            hipLaunchKernelGGL((gptq4_skinny_kernel<EPI, 2, DEPTH, true, 4, 4>), grid, block, lds, stream, a);
+    }
     return (int)hipGetLastError();
 }
 

@@ -144,6 +144,7 @@ int launch_gather_cols(const half_t *x, const int32_t *perm, half_t *out, int M,
         return (int)hipGetLastError();
     }
     const int threads = (K / 8 >= 256) ? 256 : 64;
+    if (M > 65535) return (int)hipErrorInvalidConfiguration;  // rows ride in grid.y here; callers reject this on the host first
     dim3 grid((unsigned)((K / 8 + threads - 1) / threads), (unsigned)M), block(threads);
     hipLaunchKernelGGL(gptq4_gather_cols_kernel, grid, block, 0, stream, x, perm, out, K);
     return (int)hipGetLastError();

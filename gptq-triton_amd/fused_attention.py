@@ -18,7 +18,8 @@ import torch
 import torch.nn as nn
 
 from . import _lib
-from .quant_linear import QuantLinear, _check_device_tensors, _check_matmul_args, inverse_permutation, matmul4
+from .quant_linear import (QuantLinear, _check_device_tensors, _check_matmul_args, inverse_permutation, matmul4,
+                           tensor_key)
 
 
 @dataclass
@@ -192,7 +193,12 @@ class QuantLlamaAttention(nn.Module):
                     kv_out=None, kv_offset: int = 0, norm=None, ordered: bool = False):
         """norm = (delta or None, norm_weight, eps): see qkv_rotary.  ordered: hidden_states already are in the
         order of input_order()."""
-        need = max(kv_offset, 0) + hidden_states.shape[1]
+        # rows of the cos/sin table: with KV_AT_POSITION the positions come from the device and can be anything the
+        # cache has room for, so the table covers the whole cache (the kernels clamp positions to the table)
+        if kv_offset < 0 and kv_out is not None:
+            need = kv_out[0].shape[2]
+        else:
+            need = max(kv_offset, 0) + hidden_states.shape[1]
         cos, sin = self.rope.get(hidden_states.device, max(need, self.max_position_embeddings))
         qweight, perm = self.qkv_proj.kernel_weights()
         return qkv_rotary(self.qkv_proj.groupsize, hidden_states, qweight, self.qkv_proj.scales,
@@ -206,8 +212,8 @@ class QuantLlamaAttention(nn.Module):
         _, perm = self.o_proj.kernel_weights()
         if perm is None:
             return None
-        if self._context_order is None or self._context_order[0] != perm.data_ptr():
-            self._context_order = (perm.data_ptr(), inverse_permutation(perm))
+        if self._context_order is None or self._context_order[0] != tensor_key(perm):
+            self._context_order = (tensor_key(perm), inverse_permutation(perm))
         return self._context_order[1]
 
     def input_order(self):
@@ -216,8 +222,8 @@ class QuantLlamaAttention(nn.Module):
         _, perm = self.qkv_proj.kernel_weights()
         if perm is None:
             return None
-        if self._input_order is None or self._input_order[0] != perm.data_ptr():
-            self._input_order = (perm.data_ptr(), inverse_permutation(perm))
+        if self._input_order is None or self._input_order[0] != tensor_key(perm):
+            self._input_order = (tensor_key(perm), inverse_permutation(perm))
         return self._input_order[1]
 
     def project_out(self, context: torch.Tensor, ordered: bool = False) -> torch.Tensor:

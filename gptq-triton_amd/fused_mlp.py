@@ -13,7 +13,7 @@ import torch
 import torch.nn as nn
 
 from . import _lib
-from .quant_linear import QuantLinear, _check_device_tensors, _check_matmul_args, matmul4
+from .quant_linear import QuantLinear, _check_device_tensors, _check_matmul_args, matmul4, tensor_key
 
 
 def llama_mlp_4(groupsize: int, a: torch.Tensor,
@@ -118,7 +118,7 @@ class QuantLlamaMLP(nn.Module):
     def _kernel_weights(self):
         if self.g_idx is None:
             return self.gate_proj_qweight, self.up_proj_qweight, None
-        key = (self.gate_proj_qweight.data_ptr(), self.up_proj_qweight.data_ptr(), self.g_idx.data_ptr())
+        key = tensor_key(self.gate_proj_qweight, self.up_proj_qweight, self.g_idx)
         if self._sorted is None or self._sorted[0] != key:
             from .quant_linear import prepare_act_order
             gq, perm = prepare_act_order(self.gate_proj_qweight, self.g_idx, self.groupsize)
@@ -142,8 +142,8 @@ class QuantLlamaMLP(nn.Module):
         if down_perm is None:
             gq, uq, perm = self._kernel_weights()
             return (gq, self.gate_proj_scales, self.gate_proj_qzeros, uq, self.up_proj_scales, self.up_proj_qzeros), perm, down_q
-        key = (self.gate_proj_qweight.data_ptr(), self.up_proj_qweight.data_ptr(), down_perm.data_ptr(),
-               None if self.g_idx is None else self.g_idx.data_ptr())
+        key = tensor_key(self.gate_proj_qweight, self.up_proj_qweight, self.gate_proj_scales, self.up_proj_scales,
+                         self.gate_proj_qzeros, self.up_proj_qzeros, down_perm, self.g_idx)
         if self._chained is None or self._chained[0] != key:
             cols = down_perm.long()
             if self.g_idx is None:
@@ -171,9 +171,9 @@ class QuantLlamaMLP(nn.Module):
         perm = self._chained_weights()[1]
         if perm is None:
             return None
-        if self._input_order is None or self._input_order[0] != perm.data_ptr():
+        if self._input_order is None or self._input_order[0] != tensor_key(perm):
             from .quant_linear import inverse_permutation
-            self._input_order = (perm.data_ptr(), inverse_permutation(perm))
+            self._input_order = (tensor_key(perm), inverse_permutation(perm))
         return self._input_order[1]
 
     def forward(self, x: torch.Tensor, ordered: bool = False) -> torch.Tensor:

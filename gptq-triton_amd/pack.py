@@ -9,8 +9,8 @@ quantiser (the GPTQ paper's baseline, what the reference's `dumbquant` applies,
 quantize.py:294-329): per output channel and group, scale = (max - min) / 15 with the
 range widened to include 0, zero = round(-min / scale).
 CPU-side, load-time code; not on the inference path.  The bit layout is pinned by round trips
-through the unpackers; the rounding of the computed quotients is parity unpinned (the
-reference holds no vectors for it).
+through the unpackers; the quantiser's scales, zero points and rounding are pinned by vectors written from
+the reference's `Quantizer.find_params` / `quantize` (gptq.py:174-178,205-286; tests/golden/rtn_vectors.npz).
 """
 from __future__ import annotations
 
@@ -20,8 +20,14 @@ from .quant_linear import QuantLinear
 
 
 @torch.no_grad()
-def quantize_rtn(weight: torch.Tensor, groupsize: int = -1, bits: int = 4):
-    """weight [out, in] -> (dequantised weight [out, in], scale [out, G], zero [out, G])."""
+def quantize_rtn(weight: torch.Tensor, groupsize: int = -1, bits: int = 4, packable: bool = True):
+    """weight [out, in] -> (dequantised weight [out, in], scale [out, G], zero [out, G]).
+
+    packable=False is the reference's formula as it stands (gptq.py:205-286): a group without a negative weight
+    gets zero point 0, which the checkpoint format cannot hold - it stores zero - 1 in four bits
+    (quantize.py:276), and the reference's packer then spills into the neighbouring nibbles.  packable=True
+    (default) gives such a group the range [-max/14, max] instead: zero point 1, scale max/14, the largest
+    weight still on the grid; every other group is quantised exactly as by the reference."""
     w = weight.detach().float().cpu()
     out_f, in_f = w.shape
     gs = in_f if groupsize == -1 else groupsize
@@ -34,6 +40,11 @@ def quantize_rtn(weight: torch.Tensor, groupsize: int = -1, bits: int = 4):
     wmax = torch.where(flat, torch.full_like(wmax, 1.0), wmax)
     scale = (wmax - wmin) / maxq
     zero = torch.round(-wmin / scale)
+    if packable:
+        low = zero < 1
+        wmin = torch.where(low, -wmax / (maxq - 1), wmin)
+        scale = torch.where(low, (wmax - wmin) / maxq, scale)
+        zero = torch.where(low, torch.ones_like(zero), zero)
     q = torch.clamp(torch.round(groups / scale[..., None]) + zero[..., None], 0, maxq)
     deq = (scale[..., None] * (q - zero[..., None])).reshape(out_f, in_f)
     return deq, scale, zero

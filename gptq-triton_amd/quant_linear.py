@@ -87,6 +87,12 @@ def dequantize(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor
     return out
 
 
+def tensor_key(*tensors):
+    """Cache key of derived copies: storage address AND in-place version of every source tensor, so that
+    load_state_dict / copy_ into an existing buffer invalidates what was derived from the old contents."""
+    return tuple(None if t is None else (t.data_ptr(), t._version, t.device) for t in tensors)
+
+
 def inverse_permutation(perm: torch.Tensor) -> torch.Tensor:
     """inv with inv[perm[j]] = j: where a producer must store feature f (at inv[f]) so that its output is in the
     order x[:, perm] an act-order projection reads."""
@@ -150,7 +156,7 @@ class QuantLinear(nn.Module):
         self._sorted = None  # (key, qweight_sorted, perm), built at first use
 
     def _act_order(self):
-        key = (self.qweight.data_ptr(), self.g_idx.data_ptr(), self.qweight.device)
+        key = tensor_key(self.qweight, self.g_idx)
         if self._sorted is None or self._sorted[0] != key:
             qs, perm = prepare_act_order(self.qweight, self.g_idx, self.groupsize)
             self._sorted = (key, qs, perm)

@@ -4,6 +4,11 @@ dequantised weights.  TEST INFRASTRUCTURE ONLY (same rule as the rest of oracle/
 Layer structure as the reference drives it through HF's decoder layer
 (fused_attention.py:79-153 for attention, fused_mlp.py:78-79 for the MLP):
 x + attn(rmsnorm(x)), then h + mlp(rmsnorm(h)); rotary by the closed form in gptq_oracle.
+
+Pinned by tests/test_oracle_transformers.py: logits equal transformers' LlamaForCausalLM (float32, the
+oracle's dequantised weights loaded into its nn.Linear modules) within 1e-4; causality (logits at t do not
+move when later tokens change); a model whose o_proj and down_proj decode to zero returns
+lm_head(norm(embedding)).
 """
 from __future__ import annotations
 

@@ -213,8 +213,9 @@ def mlp_ref(x, gate, up, down, groupsize) -> np.ndarray:
 
 
 # --------------------------------------------------------------------------- rotary
-def rotary_tables(max_pos: int, head_dim: int = 128, base: float = 10000.0):
-    """cos, sin float32 [max_pos, head_dim/2].
+def rotary_tables(max_pos: int, head_dim: int = 128, base: float = 10000.0, inv_freq=None):
+    """cos, sin float32 [max_pos, head_dim/2].  inv_freq (float32 [head_dim/2]) replaces the computed frequencies
+    (the transformers pin passes the library's own, which its float32 pow leaves up to one ulp away).
 
     inv_freq[i] = float32(base^(-2i/D)), theta[p, i] = float32(p) * inv_freq[i] (a
     float32 product), cos/sin evaluated on that float32 angle and rounded to float32.  (Third-party: transformers'
@@ -225,7 +226,9 @@ def rotary_tables(max_pos: int, head_dim: int = 128, base: float = 10000.0):
     # inv_freq is the float32 nearest to the real number base^(-2i/D) (evaluated in
     # float64, rounded once); a float32 pow differs from it by at most one ulp.
     expo = np.arange(0, head_dim, 2, dtype=np.float64) / float(head_dim)
-    inv_freq = (1.0 / np.power(float(base), expo)).astype(np.float32)
+    if inv_freq is None:
+        inv_freq = (1.0 / np.power(float(base), expo)).astype(np.float32)
+    inv_freq = np.asarray(inv_freq, dtype=np.float32)
     pos = np.arange(max_pos, dtype=np.float32)
     theta = (pos[:, None] * inv_freq[None, :]).astype(np.float32)
     # evaluate the trig functions in float64 on the float32 angle, then round

@@ -184,14 +184,16 @@ def test_norm_with_act_order_equals_two_launches(gemv_mode, m):
 
 @pytest.mark.parametrize("gemv_mode", [0, 2])
 @pytest.mark.parametrize("act_order", [False, True])
-@pytest.mark.parametrize("m", [1, 3])
-def test_norm_with_rows_longer_than_4096(gemv_mode, act_order, m):
-    """Hidden size 5120: four chunks per thread cover a row (the variants LLaMA-13B / 30B decoders run)."""
+@pytest.mark.parametrize("hidden,m", [(5120, 1), (5120, 3), (6656, 4), (8192, 4)])
+def test_norm_with_rows_longer_than_4096(gemv_mode, act_order, hidden, m):
+    """Hidden sizes above 4096: four chunks per thread cover a row (the variants LLaMA-13B / 30B decoders run).
+    Four rows of 6656 or 8192 values are the largest calls the entry points accept: 52 and 64 KiB of normalised
+    rows in LDS on top of the kernel's 16 KiB reduction buffer."""
     from gptq_triton_amd import _lib
     from gptq_triton_amd.decoder_ops import add_rms_norm
     from gptq_triton_amd.fused_mlp import norm_llama_mlp_4
     G = gptq()
-    hidden, inter, heads, g = 5120, 2816, 40, 128
+    inter, heads, g = 2816, hidden // 128, 128
     gate = O.make_layer(hidden, inter, g, seed=850, act_order=act_order)
     up = O.make_layer(hidden, inter, g, seed=851)
     qkv = O.make_layer(hidden, 3 * hidden, g, seed=852)
@@ -223,7 +225,7 @@ def test_norm_with_rows_longer_than_4096(gemv_mode, act_order, m):
     gi = gate["g_idx"]
     ref = O.mlp_gateup_ref(x_ref.cpu().numpy(), (gate["qweight"], gate["qzeros"], gate["scales"], gi),
                            (up["qweight"], up["qzeros"], up["scales"], gi), g)
-    assert_close(mid.cpu().numpy(), ref, f"norm + gate/up hidden 5120 M={m}")
+    assert_close(mid.cpu().numpy(), ref, f"norm + gate/up hidden {hidden} M={m}")
 
 
 def test_norm_entry_points_reject_what_they_cannot_take():

@@ -224,3 +224,28 @@ def test_qkv_rotary_places_kv_by_position():
             untouched = torch.ones(cap, dtype=torch.bool)
             untouched[pos[b]] = False
             assert bool((kc[b][:, untouched] == 7.0).all()) and bool((vc[b][:, untouched] == 7.0).all())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("use_graph", [False, True])
+def test_decode_past_max_position_embeddings_keeps_rotating(tmp_path, use_graph):
+    """A decode step places K/V by the position buffer on the device; the rotary table it reads must cover the
+    whole cache, not just config.max_position_embeddings (positions beyond the table are clamped to its last
+    row, which silently freezes the rotation).  The cache rows written by 11 decode steps past the 16 positions
+    of the config equal those of one forward pass over the whole sequence."""
+    from gptq_triton_amd.llama import GreedyDecoder
+    torch.manual_seed(13)
+    cfg = make_checkpoint(tmp_path, 128, seed=13)
+    model = G.load_quant(str(tmp_path), device="cuda", fuse_mlp=True)
+    for layer in model.model.layers:          # a table of 16 rows unless the call asks for more
+        layer.self_attn.max_position_embeddings = 16
+        layer.self_attn.rope = G.RotaryTable(layer.self_attn.head_dim, 16)
+    ids = torch.randint(0, cfg.vocab_size, (2, 9)).cuda()
+    dec = GreedyDecoder(model, 2, 9 + 12)
+    first = dec.prefill(ids)
+    rest = dec.decode(11, use_graph=use_graph)
+    seq = torch.cat([ids, first, rest], dim=1)            # 21 tokens; the cache holds the first 20
+    _, past = model(seq[:, :20], use_cache=True)
+    for (kc, vc), (k_full, v_full) in zip(dec.caches, past):
+        assert (kc[:, :, :20].float() - k_full.float()).abs().max().item() < 0.03 * k_full.float().abs().max().item()
+        assert (vc[:, :, :20].float() - v_full.float()).abs().max().item() < 0.03 * v_full.float().abs().max().item()
