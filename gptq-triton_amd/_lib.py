@@ -14,6 +14,7 @@ import torch
 LIB_PATH = Path(__file__).resolve().parent / "csrc" / "libgptq4.so"
 ABI_VERSION = 1
 WS_COUNTER_BYTES = 524288
+STATIC_SCRATCH_BYTES = WS_COUNTER_BYTES + (8 << 20)  # GPTQ4_STATIC_SCRATCH_BYTES: what gptq4_matmul_static holds per GPU
 OP_MATMUL, OP_MLP_GATEUP, OP_QKV_ROTARY, OP_DECODE_ATTENTION = 0, 1, 2, 3
 OP_WITH_PERM = 0x100  # or-ed to a matmul selector in gptq4_workspace_bytes: the call passes `perm`
 
@@ -25,6 +26,7 @@ SIGNATURES = {
     "gptq4_dequant": (c_int, [c_void_p] * 5 + [c_int, c_int, c_int, c_void_p]),
     "gptq4_actorder_sort_rows": (c_int, [c_void_p] * 3 + [c_int, c_int, c_void_p]),
     "gptq4_matmul": (c_int, [c_void_p] * 7 + [c_int] * 4 + [c_void_p, c_size_t, c_void_p]),
+    "gptq4_matmul_static": (c_int, [c_void_p] * 6 + [c_int] * 4 + [c_void_p]),
     "gptq4_mlp_gateup": (c_int, [c_void_p] * 9 + [c_int] * 4 + [c_void_p, c_size_t, c_void_p]),
     "gptq4_rope_table": (c_int, [c_void_p, c_void_p, c_int, c_int, c_float, c_void_p]),
     "gptq4_qkv_rotary": (c_int, [c_void_p] * 8 + [c_int] + [c_void_p] * 3 + [c_int] * 8 + [c_void_p, c_size_t, c_void_p]),

@@ -6,6 +6,13 @@
 #include "gptq4_internal.h"
 #include "gptq4_norm.h"
 
+#include <mutex>
+
+// Scratch memory of gptq4_matmul_static: arrival counters, then split-K partial sums, laid out like a
+// caller's workspace.  Zero when the module is loaded; every launch leaves the counters zero again.
+// In host code this name is only a handle for hipGetSymbolAddress: the kernels get the device address.
+static __device__ __align__(256) unsigned char scratch[GPTQ4_STATIC_SCRATCH_BYTES];
+
 namespace {
 
 inline bool misaligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) != 0; }
@@ -50,6 +57,8 @@ int stage_act_order(MatmulArgs &a, size_t partial_bytes_used, void *workspace, s
     const size_t off = GPTQ4_WS_COUNTER_BYTES + partial_bytes_used;
     const size_t bytes = (size_t)a.M * a.K * sizeof(half_t);
     if (workspace == nullptr || workspace_bytes < off + bytes) return -GPTQ4_E_WORKSPACE;
+    // rows longer than 32768 values are gathered with the row index in grid.y, which ends at 65535
+    if (a.M > 65535 && a.K > 32768) return -GPTQ4_E_SHAPE;
     half_t *xg = reinterpret_cast<half_t *>(reinterpret_cast<char *>(workspace) + off);
     const int rc = launch_gather_cols(a.x, a.perm, xg, a.M, a.K, s);
     a.x = xg;
@@ -202,6 +211,8 @@ const char *gptq4_strerror(int code) {
             return "workspace is NULL or too small (see gptq4_workspace_bytes)";
         case GPTQ4_E_ALIGN:
             return "a pointer is not 16-byte aligned";
+        case GPTQ4_E_STATIC_LIMIT:
+            return "the call needs more scratch memory than gptq4_matmul_static holds (GPTQ4_STATIC_SCRATCH_BYTES): use gptq4_matmul with a workspace";
         default:
             return "unknown gptq4 error";
     }
@@ -315,6 +326,42 @@ int gptq4_matmul(const void *x, const int32_t *qweight, const int32_t *qzeros, c
         return run_small(EPI_PLAIN, a, 1, workspace, workspace_bytes, s);
     }
     return run_tiled(EPI_PLAIN, a, workspace, workspace_bytes, s);
+}
+
+// The device address of `scratch` on the current device; looked up once per device.
+static int static_scratch(void **out) {
+    enum { MAX_DEVICES = 64 };
+    static void *ptrs[MAX_DEVICES];
+    static std::mutex lock;
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= MAX_DEVICES) return (int)hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> guard(lock);
+    if (ptrs[dev] == nullptr) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (p == nullptr) return (int)hipErrorInvalidSymbol;
+        ptrs[dev] = p;
+    }
+    *out = ptrs[dev];
+    return 0;
+}
+
+int gptq4_matmul_static(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
+                        const void *bias, void *y, int M, int K, int N, int groupsize, void *stream) {
+    if (!x || !qweight || !qzeros || !scales || !y) return -GPTQ4_E_NULL;
+    if (M < 1) return -GPTQ4_E_SHAPE;
+    int g = groupsize;
+    int rc = check_dims(K, N, &g);
+    if (rc) return rc;
+    // what the same call would ask of a caller's workspace has to fit the static array
+    if (gptq4_workspace_bytes(GPTQ4_OP_MATMUL, M, K, N) > (size_t)GPTQ4_STATIC_SCRATCH_BYTES) return -GPTQ4_E_STATIC_LIMIT;
+    void *ws = nullptr;
+    rc = static_scratch(&ws);
+    if (rc) return rc;
+    return gptq4_matmul(x, qweight, qzeros, scales, nullptr, bias, y, M, K, N, groupsize, ws, GPTQ4_STATIC_SCRATCH_BYTES, stream);
 }
 
 static int mlp_gateup_impl(const void *x, const void *delta, const void *norm_weight, void *sum_out, float eps,

@@ -52,9 +52,12 @@ extern "C" {
 #define GPTQ4_E_GROUPSIZE 3  /* groupsize does not divide K / not a multiple of 128 */
 #define GPTQ4_E_WORKSPACE 4  /* workspace NULL or smaller than required          */
 #define GPTQ4_E_ALIGN 5      /* a pointer is not 16-byte aligned                 */
+#define GPTQ4_E_STATIC_LIMIT 6 /* gptq4_matmul_static: the call needs more scratch than the library holds */
 
 #define GPTQ4_WS_COUNTER_BYTES 524288
 #define GPTQ4_KV_AT_POSITION (-1)
+/* scratch memory inside the library for gptq4_matmul_static: the counters plus 8 MiB of partial sums */
+#define GPTQ4_STATIC_SCRATCH_BYTES (GPTQ4_WS_COUNTER_BYTES + (8u << 20))
 
 /* operation selector for gptq4_workspace_bytes */
 #define GPTQ4_OP_MATMUL 0
@@ -95,6 +98,21 @@ int gptq4_matmul(const void *x, const int32_t *qweight, const int32_t *qzeros,
                  const void *scales, const int32_t *perm, const void *bias, void *y,
                  int M, int K, int N, int groupsize, void *workspace,
                  size_t workspace_bytes, void *stream);
+
+/* gptq4_matmul for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): no workspace argument - the arrival counters and split-K partial
+ * sums live in a fixed array inside the library (GPTQ4_STATIC_SCRATCH_BYTES = 8.5 MiB per GPU, held until the
+ * process ends), and the call itself allocates and frees nothing.  No reference counterpart.
+ * Same kernels and results as gptq4_matmul without `perm` (act-order calls need room for the gathered
+ * rows: use gptq4_matmul).  Calls whose workspace requirement - gptq4_workspace_bytes(GPTQ4_OP_MATMUL, M, K, N) -
+ * exceeds the array return -GPTQ4_E_STATIC_LIMIT and launch nothing; decode-sized calls fit up to
+ * M * N <= 131072 (16 rows of 8192 columns, 8 of 16384).  Every call on one GPU shares that GPU's array:
+ * calls that overlap in time on one GPU (different streams or threads) race; calls on one stream do not.
+ * The first call on a device looks the array's address up (hipGetSymbolAddress); make that call outside
+ * stream capture. */
+int gptq4_matmul_static(const void *x, const int32_t *qweight, const int32_t *qzeros,
+                        const void *scales, const void *bias, void *y, int M, int K, int N,
+                        int groupsize, void *stream);
 
 /* h fp16 [M, I] = silu(x @ Wgate) * (x @ Wup); SiLU and the product are taken on the
  * fp32 accumulators, one rounding to fp16.

@@ -55,7 +55,11 @@ def test_error_codes_are_returned_before_any_launch():
     assert lib.gptq4_qkv_rotary(*args, 2048, fake, fake, fake, 1, 1, 32, 64, 4096, -1, 1, 0, fake, ws, None) == -2
     assert lib.gptq4_qkv_rotary(*args, 2048, fake, fake, fake, 1, 4, 32, 128, 4096, -1, 3, 0, fake, ws, None) == -2
     assert lib.gptq4_mlp_gateup(fake, fake, fake, fake, None, fake, fake, None, fake, 1, 4096, 11008, -1, fake, ws, None) == -1
-    for code in (0, -1, -2, -3, -4, -5):
+    # the entry point with its own scratch memory: argument errors first, then its size limit - all before any GPU call
+    assert lib.gptq4_matmul_static(None, fake, fake, fake, None, fake, 1, 4096, 4096, -1, None) == -1
+    assert lib.gptq4_matmul_static(fake, fake, fake, fake, None, fake, 1, 4096, 4096, 96, None) == -3
+    assert lib.gptq4_matmul_static(fake, fake, fake, fake, None, fake, 16, 4096, 32768, -1, None) == -6
+    for code in (0, -1, -2, -3, -4, -5, -6):
         assert len(lib.gptq4_strerror(code)) > 0
 
 
