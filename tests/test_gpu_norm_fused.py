@@ -182,9 +182,10 @@ def test_norm_with_act_order_equals_two_launches(gemv_mode, m):
     assert_close(mlp.gate_up(x_ref).cpu().numpy(), ref, "act-order gate/up on the normalised rows")
 
 
-@pytest.mark.parametrize("gemv_mode", [0, 2])
+# (four rows of 6656 or 8192 values leave the balanced GEMV no room in its 64 KiB of LDS: the self-normalising call
+# then runs the split-K kernel whatever the mode, so only mode 0 compares like with like)
 @pytest.mark.parametrize("act_order", [False, True])
-@pytest.mark.parametrize("hidden,m", [(5120, 1), (5120, 3), (6656, 4), (8192, 4)])
+@pytest.mark.parametrize("hidden,m,gemv_mode", [(5120, 1, 0), (5120, 1, 2), (5120, 3, 0), (5120, 3, 2), (6656, 4, 0), (8192, 4, 0)])
 def test_norm_with_rows_longer_than_4096(gemv_mode, act_order, hidden, m):
     """Hidden sizes above 4096: four chunks per thread cover a row (the variants LLaMA-13B / 30B decoders run).
     Four rows of 6656 or 8192 values are the largest calls the entry points accept: 52 and 64 KiB of normalised
