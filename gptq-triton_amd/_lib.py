@@ -6,7 +6,7 @@ operator that needs it raises with it.  There is no CPU fallback.
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_char_p, c_float, c_int, c_size_t, c_void_p
+from ctypes import POINTER, Structure, c_char_p, c_float, c_int, c_size_t, c_uint, c_void_p
 from pathlib import Path
 
 import torch
@@ -17,6 +17,20 @@ WS_COUNTER_BYTES = 524288
 STATIC_SCRATCH_BYTES = WS_COUNTER_BYTES + (8 << 20)  # GPTQ4_STATIC_SCRATCH_BYTES: what gptq4_matmul_static holds per GPU
 OP_MATMUL, OP_MLP_GATEUP, OP_QKV_ROTARY, OP_DECODE_ATTENTION = 0, 1, 2, 3
 OP_WITH_PERM = 0x100  # or-ed to a matmul selector in gptq4_workspace_bytes: the call passes `perm`
+
+IN_ROWS, IN_NORM_ROWS, IN_PREV, IN_NORM_PREV = 0, 1, 2, 3     # gptq4_phase_t.input
+OUT_NONE, OUT_ROWS, OUT_ROPE = 0, 1, 2                        # gptq4_phase_t.output
+CHAIN_MAX_PHASES, CHAIN_MAX_M, CHAIN_ERROR_OFFSET = 8, 4, 4
+
+
+class Phase(Structure):
+    """gptq4_phase_t of include/gptq4.h: one projection of a chained decode launch."""
+    _fields_ = [(n, c_void_p) for n in ("qweight", "qzeros", "scales", "up_qweight", "up_qzeros", "up_scales", "perm",
+                                        "x", "delta", "norm_weight", "sum_out", "y", "bias", "position_ids",
+                                        "cos_table", "sin_table", "q", "k", "v")] + \
+               [(n, c_int) for n in ("K", "N", "groupsize", "input", "output")] + [("eps", c_float)] + \
+               [(n, c_int) for n in ("H", "max_pos", "kv_capacity", "kv_offset")]
+
 
 # every symbol include/gptq4.h declares: (restype, argtypes)
 SIGNATURES = {
@@ -36,6 +50,9 @@ SIGNATURES = {
     "gptq4_rmsnorm": (c_int, [c_void_p] * 4 + [c_int, c_int, c_float, c_void_p]),
     "gptq4_add_rmsnorm": (c_int, [c_void_p] * 6 + [c_int, c_int, c_float, c_void_p]),
     "gptq4_decode_attention": (c_int, [c_void_p] * 6 + [c_int] * 4 + [c_float, c_void_p, c_size_t, c_void_p]),
+    "gptq4_chain_workspace_bytes": (c_size_t, [POINTER(Phase), c_int, c_int]),
+    "gptq4_decode_chain": (c_int, [POINTER(Phase), c_int, c_int, c_void_p, c_size_t, c_void_p]),
+    "gptq4_set_chain_tuning": (None, [c_int, c_int, c_uint, c_int]),
     "gptq4_set_tuning": (None, [c_int, c_int, c_int]),
     "gptq4_set_gemm_tuning": (None, [c_int, c_int]),
     "gptq4_set_midm_tuning": (None, [c_int, c_int, c_int]),

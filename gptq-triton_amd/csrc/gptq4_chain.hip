@@ -1,0 +1,838 @@
+// Chained decode launch for gfx950: several small-M (1..4 rows) quantised projections in ONE persistent
+// launch, e.g. o_proj -> residual add + RMSNorm -> gate/up + SiLU*mul -> down_proj.
+//
+// Why: a decode GEMV streams 9..47 MB in 6..15 us, of which about 6 us are a serial chain per launch (launch
+// floor, prologue, first-load latency, partial-sum exchange) during which HBM idles.  Weights do not depend on
+// activations, so here ONE grid (one workgroup per CU, resident for the whole launch) streams the weights of
+// all phases as one sequence: every wave keeps DEPTH units of loads in flight at all times, and the loads of
+// the next phase's first units are already under way while the phase before it is being reduced, handed over
+// and normalised.
+//
+// Work decomposition (per phase)
+//   unit   = (tile, 128-k batch): 2 strips of 32 columns x 128 k = 4 KiB of packed weights.  The two strips
+//            are adjacent columns (plain projection), the same columns of gate and up (SiLU*mul), or head
+//            columns d and d + 64 (rotary).  Lane l loads row l/16 of each 4-row K step and 2 adjacent words:
+//            a word is the complete B operand of one v_mfma_f32_16x16x32_f16.
+//   The units of a phase are one flat range dealt to workgroups (q or q+1 each) and inside a workgroup to
+//   waves (contiguous sub-ranges), so every CU streams the same number of bytes +-1 unit whatever the tile
+//   count.  A wave's range lies in one tile or crosses into the next.
+//   x      = the M rows the phase multiplies with, staged once per workgroup in LDS in the k order the
+//            decoded weights come out in ("pair order"); the A operand of every wave is read from there.
+//   hand-over: the waves of a workgroup add their accumulators per tile through LDS (wave order), the
+//            workgroup stores one partial tile per touched tile in its slot of the workspace (slot = its rank
+//            among the workgroups sharing the tile), waits for the stores to complete and raises its
+//            completion flag to the phase's epoch.  A consumer polls the flags of all workgroups (one wave,
+//            bounded), then adds the partial tiles it needs in rank order - every consumer the same order, so
+//            results are deterministic - and applies what lies between the two projections itself: rounding
+//            to fp16, bias, residual add, RMSNorm, SiLU*mul.
+//   Outputs that must exist in memory (y, q/k/v with rotary) are written by all workgroups, a slice each,
+//   at the next point where the launch waits anyway (or at its end).
+//
+// Ordering across workgroups is by completion, as in the other decode kernels: partial sums, sums and flags are
+// written with agent-scope (sc1) stores and read with agent-scope loads, which go around the per-XCD L2s; a
+// workgroup waits for the acknowledgement of its data stores (s_waitcnt vmcnt(0)) before it stores its flag.
+// Every wait is bounded: a workgroup that gives up records CHAIN_ERR_TIMEOUT in the state and returns, which
+// makes every other workgroup give up in turn; the error is sticky until the host clears the workspace.
+#include "gptq4_chain.h"
+
+#include "../../include/gptq4.h"
+#include "gptq4_norm.h"
+
+#include <mutex>
+
+namespace {
+
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+constexpr uint32_t OFF_RANGE = 0x80000000u;  // a lane offset beyond any buffer: the load returns zeros, untouched memory
+constexpr int AUX_SC1 = 16;                  // cache policy of buffer loads / stores: agent scope
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *p, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ int div_magic(int n, int d, uint32_t magic) { return d == 1 ? n : (int)__umulhi((unsigned)n, magic); }
+
+typedef const __attribute__((address_space(4))) ChainPhase *PhasePtr;
+
+struct UnitRegs {
+    u32x2_t w[2][4];    // packed weights: [strip][K step], 2 adjacent columns per lane
+    uint32_t raw_s[2];  // the 2 fp16 scales of the lane's columns
+    uint32_t raw_z[2];  // the zero-point word holding the lane's columns
+};
+
+// tile -> first column of strip 0; second strip: `strip1` columns further (in w1)
+__device__ __forceinline__ int tile_col0(int epi, int tile) {
+    return epi == EPI_PLAIN ? tile * 64 : (epi == EPI_SILU_MUL ? tile * 32 : (tile >> 1) * 128 + (tile & 1) * 32);
+}
+
+// first unit and unit count of a workgroup / of one of its waves
+__device__ __forceinline__ void wg_range(PhasePtr P, int wg, int &u0, int &n) {
+    u0 = wg * P->q + min(wg, P->r);
+    n = P->q + (wg < P->r ? 1 : 0);
+}
+template <int NW>
+__device__ __forceinline__ void wave_range(PhasePtr P, int wg, int wave, int &u0, int &n) {
+    int U0, nw;
+    wg_range(P, wg, U0, nw);
+    const int wq = nw / NW, wr = nw % NW;
+    u0 = U0 + wave * wq + min(wave, wr);
+    n = wq + (wave < wr ? 1 : 0);
+}
+// the workgroup that owns unit u
+__device__ __forceinline__ int wg_of_unit(PhasePtr P, int u) {
+    const int big = P->r * (P->q + 1);
+    return u < big ? div_magic(u, P->q + 1, P->q1_magic) : P->r + div_magic(u - big, P->q, P->q_magic);
+}
+
+__device__ __forceinline__ float f_of(uint32_t u) { return __builtin_bit_cast(float, u); }
+
+// Sum of the partial tiles of 8 adjacent columns (two 16-byte loads per contributing workgroup, all issued
+// before the first add), in rank order.  `base` = float offset of (tile, rank 0, row m, column) in the partial
+// region, `stride` = floats between ranks.
+__device__ __forceinline__ void sum_partials8(const __amdgpu_buffer_rsrc_t &rs, uint32_t base, uint32_t stride, int nc, float out[8]) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) out[i] = 0.f;
+    for (int r0 = 0; r0 < nc; r0 += 4) {
+        u32x4_t a[4], b[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t off = (r0 + j < nc) ? (base + (uint32_t)(r0 + j) * stride) * 4u : OFF_RANGE;
+            a[j] = __builtin_amdgcn_raw_buffer_load_b128(rs, off, 0, AUX_SC1);
+            b[j] = __builtin_amdgcn_raw_buffer_load_b128(rs, off + 16u, 0, AUX_SC1);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (r0 + j < nc) {
+                out[0] += f_of(a[j].x), out[1] += f_of(a[j].y), out[2] += f_of(a[j].z), out[3] += f_of(a[j].w);
+                out[4] += f_of(b[j].x), out[5] += f_of(b[j].y), out[6] += f_of(b[j].z), out[7] += f_of(b[j].w);
+            }
+        }
+    }
+}
+
+__device__ __forceinline__ uint4 pack_h8(const half_t h[8]) {
+    uint4 r;
+    r.x = as_u32((h2_t){h[0], h[1]});
+    r.y = as_u32((h2_t){h[2], h[3]});
+    r.z = as_u32((h2_t){h[4], h[5]});
+    r.w = as_u32((h2_t){h[6], h[7]});
+    return r;
+}
+
+// 8 adjacent output values of phase P (row m, columns n0 .. n0+7, n0 % 8 == 0) from its partial tiles, as the
+// next consumer sees them: fp16(sum) (+ bias) of a plain phase, fp16(silu(gate) * up) of a pair.
+__device__ __forceinline__ uint4 phase_output8(PhasePtr P, const __amdgpu_buffer_rsrc_t &rs, int M, int m, int n0) {
+    const int tile = (P->epi == EPI_PLAIN) ? (n0 >> 6) : (n0 >> 5);
+    const int col = (P->epi == EPI_PLAIN) ? (n0 & 63) : (n0 & 31);
+    const int first = wg_of_unit(P, tile * P->nb);
+    const int nc = wg_of_unit(P, tile * P->nb + P->nb - 1) - first + 1;
+    const uint32_t stride = (uint32_t)M * 64u;
+    const uint32_t base = P->partial_off + ((uint32_t)tile * P->max_contrib * M + m) * 64u + col;
+    float s[8];
+    half_t h[8];
+    sum_partials8(rs, base, stride, nc, s);
+    if (P->epi == EPI_PLAIN) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) h[i] = (half_t)s[i];
+        if (P->bias != nullptr) {
+            const uint4 bv = *reinterpret_cast<const uint4 *>(P->bias + n0);
+            const h2_t b2[4] = {as_h2(bv.x), as_h2(bv.y), as_h2(bv.z), as_h2(bv.w)};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) h[2 * i] = h[2 * i] + b2[i].x, h[2 * i + 1] = h[2 * i + 1] + b2[i].y;
+        }
+    } else {
+        float u[8];
+        sum_partials8(rs, base + 32u, stride, nc, u);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) h[i] = (half_t)(silu_f32(s[i]) * u[i]);
+    }
+    return pack_h8(h);
+}
+
+template <int NW, int DEPTH>
+__global__ __launch_bounds__(64 * NW) void gptq4_chain_kernel(const ChainArgs args_by_value) {
+    // The arguments are read where the launch put them, in the kernel-argument segment (constant memory, scalar
+    // loads with a dynamic phase index); touching the by-value copy would make the compiler spill the whole
+    // table to scratch memory to index it.
+    const __attribute__((address_space(4))) ChainArgs *const A =
+        (const __attribute__((address_space(4))) ChainArgs *)__builtin_amdgcn_kernarg_segment_ptr();
+    constexpr int T = 64 * NW;
+    extern __shared__ uint4 smem[];
+    __shared__ int s_ft[NW], s_lt[NW];
+    __shared__ float s_part[CHAIN_MAX_M * 4];
+    __shared__ uint32_t s_ctl[2];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lrow = lane >> 4;
+    const int lcol = lane & 15;
+    const int wg = blockIdx.x;
+    const int G = gridDim.x;
+    const int M = A->M;
+    const int P = A->nphases;
+
+    uint4 *const xs = smem;
+    float *const red = reinterpret_cast<float *>(smem + A->red_off);
+    const int xs_stride = A->xs_stride;
+
+    ChainState *const st = A->state;
+    if (tid == 0) {
+        s_ctl[0] = __hip_atomic_load(&st->epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_ctl[1] = (uint32_t)__hip_atomic_load(&st->error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    const uint32_t epoch = s_ctl[0];
+    if (s_ctl[1] != 0) return;  // an earlier launch on this workspace gave up: the state is not trustworthy
+    __syncthreads();
+
+    const __amdgpu_buffer_rsrc_t rs_part = make_rsrc(A->partials, A->partial_bytes);
+    const __amdgpu_buffer_rsrc_t rs_flags = make_rsrc(st->flags, (uint32_t)G * 4u);
+
+    // ------------------------------------------------------------------ the weight stream
+    // Per wave the units of all phases are ONE sequence: for every phase with units for this wave, its units
+    // padded to a multiple of DEPTH with switched-off loads, so that unit i of a phase always sits in ring slot
+    // i % DEPTH.  The load cursor (lp, li) runs DEPTH entries ahead of the compute cursor.
+    __amdgpu_buffer_rsrc_t rs_w0, rs_w1, rs_s0, rs_s1, rs_z0, rs_z1;
+    int l_epi = 0, l_N = 0, l_nb = 1, l_strip1 = 0, l_u0 = 0, l_n = 0, l_pad = 0, l_bpg = 1;
+    uint32_t l_nb_magic = 0, l_group_magic = 0;
+    int lp = -1, li = 0;
+    auto next_stream_phase = [&]() {
+        for (;;) {
+            ++lp;
+            if (lp >= P) {
+                l_n = 0;
+                l_pad = 0x7fffffff;
+                li = 0;
+                return;
+            }
+            const PhasePtr Q = A->ph + lp;
+            wave_range<NW>(Q, wg, wave, l_u0, l_n);
+            if (l_n == 0) continue;
+            l_pad = (l_n + DEPTH - 1) / DEPTH * DEPTH;
+            li = 0;
+            l_epi = Q->epi, l_N = Q->N, l_nb = Q->nb, l_nb_magic = Q->nb_magic, l_bpg = Q->bpg, l_group_magic = Q->group_magic;
+            l_strip1 = (Q->epi == EPI_PLAIN) ? 32 : (Q->epi == EPI_ROPE ? 64 : 0);
+            const int m1 = (Q->epi == EPI_SILU_MUL) ? 1 : 0;
+            const uint32_t wbytes = (uint32_t)(Q->K >> 3) * Q->N * 4u;
+            rs_w0 = make_rsrc(Q->w[0].qweight, wbytes);
+            rs_w1 = make_rsrc(Q->w[m1].qweight, wbytes);
+            rs_s0 = make_rsrc(Q->w[0].scales, (uint32_t)Q->groups * Q->N * 2u);
+            rs_s1 = make_rsrc(Q->w[m1].scales, (uint32_t)Q->groups * Q->N * 2u);
+            rs_z0 = make_rsrc(Q->w[0].qzeros, (uint32_t)Q->groups * (Q->N >> 3) * 4u);
+            rs_z1 = make_rsrc(Q->w[m1].qzeros, (uint32_t)Q->groups * (Q->N >> 3) * 4u);
+            return;
+        }
+    };
+    {
+        // descriptors must be valid even for a wave without any unit: point them at phase 0
+        const PhasePtr Q = A->ph;
+        rs_w0 = rs_w1 = make_rsrc(Q->w[0].qweight, 16u);
+        rs_s0 = rs_s1 = make_rsrc(Q->w[0].scales, 16u);
+        rs_z0 = rs_z1 = make_rsrc(Q->w[0].qzeros, 16u);
+    }
+    next_stream_phase();
+
+    auto issue_load = [&](UnitRegs &U) {
+        if (li >= l_pad) next_stream_phase();
+        const uint32_t dead = (li < l_n) ? 0u : OFF_RANGE;
+        const int u = l_u0 + max(min(li, l_n - 1), 0);
+        ++li;
+        const int tile = div_magic(u, l_nb, l_nb_magic);
+        const int b = u - tile * l_nb;
+        const int col0 = tile_col0(l_epi, tile);
+        const uint32_t N = (uint32_t)l_N;
+        const uint32_t vw = (((uint32_t)lrow * N + 2u * lcol) * 4u) | dead;
+        const uint32_t vs = ((uint32_t)(2 * lcol) * 2u) | dead;
+        const uint32_t vz = ((uint32_t)((2 * lcol) >> 3) * 4u) | dead;
+        const uint32_t sw = ((uint32_t)(b * 16) * N + col0) * 4u;
+        const uint32_t kstep = 16u * N;
+        const uint32_t s1 = (uint32_t)l_strip1;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            U.w[0][k] = __builtin_amdgcn_raw_buffer_load_b64(rs_w0, vw, sw + k * kstep, 0);
+            U.w[1][k] = __builtin_amdgcn_raw_buffer_load_b64(rs_w1, vw + s1 * 4u, sw + k * kstep, 0);
+        }
+        const int g = div_magic(b, l_bpg, l_group_magic);
+        const uint32_t ss = ((uint32_t)g * N + col0) * 2u;
+        const uint32_t sz = ((uint32_t)g * (N >> 3) + (col0 >> 3)) * 4u;
+        U.raw_s[0] = __builtin_amdgcn_raw_buffer_load_b32(rs_s0, vs, ss, 0);
+        U.raw_z[0] = __builtin_amdgcn_raw_buffer_load_b32(rs_z0, vz, sz, 0);
+        U.raw_s[1] = __builtin_amdgcn_raw_buffer_load_b32(rs_s1, vs + s1 * 2u, ss, 0);
+        U.raw_z[1] = __builtin_amdgcn_raw_buffer_load_b32(rs_z1, vz + (s1 >> 3) * 4u, sz, 0);
+    };
+
+    UnitRegs ring[DEPTH];
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) issue_load(ring[d]);
+
+    // ------------------------------------------------------------------ waiting for a phase to be complete everywhere
+    // One wave polls the completion flags of all workgroups (16-byte agent-scope loads, 256 flags per pass);
+    // bounded by A->spin_limit polls.  Returns false (to every thread) when the workgroup gives up.
+    auto wait_done = [&](int p) -> bool {
+        const uint32_t target = epoch + (uint32_t)p + 1u;
+        if (wave == 0) {
+            bool ok = false;
+            for (uint32_t spin = 0; spin < A->spin_limit; ++spin) {
+                bool all = true;
+                for (int base = 0; base < G; base += 256) {
+                    const int i0 = base + 4 * lane;
+                    const u32x4_t f = __builtin_amdgcn_raw_buffer_load_b128(rs_flags, (uint32_t)i0 * 4u, 0, AUX_SC1);
+                    const uint32_t fv[4] = {f.x, f.y, f.z, f.w};
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        if (i0 + j < G && (int32_t)(fv[j] - target) < 0) all = false;
+                }
+                if (__builtin_amdgcn_ballot_w64(!all) == 0) {
+                    ok = true;
+                    break;
+                }
+                if ((spin & 15u) == 15u &&
+                    __hip_atomic_load(&st->error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)
+                    break;  // somebody else gave up already
+                __builtin_amdgcn_s_sleep(2);
+            }
+            if (lane == 0) {
+                s_ctl[0] = ok ? 1u : 0u;
+                if (!ok) __hip_atomic_store(&st->error, (int32_t)CHAIN_ERR_TIMEOUT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        __syncthreads();
+        const bool ok = s_ctl[0] != 0;
+        __syncthreads();
+        return ok;
+    };
+
+    // ------------------------------------------------------------------ outputs that must exist in memory
+    auto write_outputs = [&](int p) {
+        const PhasePtr C = A->ph + p;
+        if (C->out_kind == CHAIN_OUT_ROWS) {
+            const int row_chunks = C->N >> 3;
+            const int total = M * row_chunks;
+            for (int i = wg * T + tid; i < total; i += G * T) {
+                const int m = i / row_chunks, c = i - m * row_chunks;
+                *reinterpret_cast<uint4 *>(C->y + (size_t)m * C->N + 8 * c) = phase_output8(C, rs_part, M, m, 8 * c);
+            }
+        } else if (C->out_kind == CHAIN_OUT_ROPE) {
+            // item = (row, tile, 8 head dimensions d and their partners d + 64)
+            const __attribute__((address_space(4))) RopeArgs *r = &C->rope;
+            const int total = M * C->tiles * 4;
+            for (int i = wg * T + tid; i < total; i += G * T) {
+                const int cc = i & 3;
+                const int rest = i >> 2;
+                const int m = rest / C->tiles, tile = rest - m * C->tiles;
+                const int first = wg_of_unit(C, tile * C->nb);
+                const int nc = wg_of_unit(C, tile * C->nb + C->nb - 1) - first + 1;
+                const uint32_t stride = (uint32_t)M * 64u;
+                const uint32_t base = C->partial_off + ((uint32_t)tile * C->max_contrib * M + m) * 64u + 8 * cc;
+                float x1[8], x2[8];
+                sum_partials8(rs_part, base, stride, nc, x1);
+                sum_partials8(rs_part, base + 32u, stride, nc, x2);
+                const int head_col = tile >> 1;
+                const int d = (tile & 1) * 32 + 8 * cc;
+                const int which = head_col / r->H;
+                const int head = head_col - which * r->H;
+                const int pid = r->position_ids[m];
+                half_t o1[8], o2[8];
+                if (which < 2) {
+                    const int pos = min(max(pid, 0), r->max_pos - 1);
+                    const float *ct = r->cos_table + (size_t)pos * 64 + d;
+                    const float *sn = r->sin_table + (size_t)pos * 64 + d;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const float cs = ct[j], sv = sn[j];
+                        o1[j] = (half_t)(x1[j] * cs - x2[j] * sv);
+                        o2[j] = (half_t)(x2[j] * cs + x1[j] * sv);
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) o1[j] = (half_t)x1[j], o2[j] = (half_t)x2[j];
+                }
+                half_t *dst;
+                size_t off;
+                if (which == 0) {
+                    dst = r->q;
+                    off = ((size_t)m * r->H + head) * 128;  // one token per sequence: [B, H, 1, D]
+                } else {
+                    dst = (which == 1) ? r->k : r->v;
+                    const int crow = r->kv_offset >= 0 ? r->kv_offset : min(max(pid, 0), r->kv_capacity - 1);
+                    off = (((size_t)m * r->H + head) * r->kv_capacity + crow) * 128;
+                }
+                *reinterpret_cast<uint4 *>(dst + off + d) = pack_h8(o1);
+                *reinterpret_cast<uint4 *>(dst + off + 64 + d) = pack_h8(o2);
+            }
+        }
+    };
+
+    uint32_t pending = 0;  // phases whose outputs are still to be written
+    auto flush_outputs = [&](int upto) {
+        for (int p = 0; p <= upto; ++p)
+            if (pending & (1u << p)) write_outputs(p);
+        pending &= ~((2u << upto) - 1u);
+    };
+
+    // ------------------------------------------------------------------ the phases
+    // (p == P is the end of the launch: outputs still to be written, and the epoch moves on)
+    for (int p = 0; p <= P; ++p) {
+        const PhasePtr C = A->ph + min(p, P - 1);
+        const bool wait_here = (p == P) ? (pending != 0 || wg == 0) : (C->in_kind >= CHAIN_IN_PREV);
+        if (wait_here) {
+            if (!wait_done(p - 1)) return;
+            flush_outputs(p - 1);
+        }
+        if (p == P) {
+            // every workgroup has read `epoch` long ago (it completed P phases since): move it on for the next launch
+            if (wg == 0 && tid == 0) __hip_atomic_store(&st->epoch, epoch + (uint32_t)P, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
+        }
+        int U0, nwg;
+        wg_range(C, wg, U0, nwg);
+        const int nb = C->nb;
+
+        // ---- the rows this phase multiplies with -> LDS, pair order
+        // staged batches: all of them (slot = batch) or the workgroup's own, starting at batch st_b0
+        const int st_b0 = C->stage_full ? 0 : U0 - div_magic(U0, nb, C->nb_magic) * nb;
+        const int st_n = C->stage_full ? nb : min(nwg, nb);
+        if (C->in_kind == CHAIN_IN_ROWS || C->in_kind == CHAIN_IN_PREV) {
+            const PhasePtr Pv = A->ph + (p > 0 ? p - 1 : 0);
+            for (int m = 0; m < M; ++m) {
+                for (int i = tid; i < st_n * 16; i += T) {
+                    int b = st_b0 + (i >> 4);
+                    if (b >= nb) b -= nb;
+                    const int k0 = b * 128 + (i & 15) * 8;
+                    uint4 v;
+                    if (C->in_kind == CHAIN_IN_ROWS)
+                        v = *reinterpret_cast<const uint4 *>(C->x + (size_t)m * C->K + k0);
+                    else
+                        v = phase_output8(Pv, rs_part, M, m, k0);
+                    xs[m * xs_stride + i] = pair_order_u4(v);
+                }
+            }
+            __syncthreads();
+        } else {
+            // residual add + RMSNorm of whole rows.  The sum of squares is taken by threads 0..255 over the chunks
+            // tid, tid + 256, ... and combined as the stand-alone kernel combines it: same bits.
+            const PhasePtr Pv = A->ph + (p > 0 ? p - 1 : 0);
+            const int chunks = C->K >> 3;
+            const bool writer = (wg == p % G) && C->sum_out != nullptr;
+            const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(C->x, (uint32_t)M * C->K * 2u);
+            const __amdgpu_buffer_rsrc_t rs_sum = make_rsrc(C->sum_out != nullptr ? C->sum_out : const_cast<half_t *>(C->x), (uint32_t)M * C->K * 2u);
+            for (int m = 0; m < M; ++m) {
+                for (int c = tid; c < chunks; c += T) {
+                    const uint32_t off = ((uint32_t)m * C->K + 8u * c) * 2u;
+                    uint4 v = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rs_x, off, 0, AUX_SC1));
+                    bool added = false;
+                    uint4 d = v;
+                    if (C->in_kind == CHAIN_IN_NORM_PREV) {
+                        d = phase_output8(Pv, rs_part, M, m, 8 * c);
+                        added = true;
+                    } else if (C->delta != nullptr) {
+                        d = *reinterpret_cast<const uint4 *>(C->delta + (size_t)m * C->K + 8 * c);
+                        added = true;
+                    }
+                    if (added) {
+                        float unused = 0.f;
+                        v = norm_take<true>(v, d, unused);
+                        if (writer) __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, v), rs_sum, off, 0, AUX_SC1);
+                    }
+                    xs[m * xs_stride + c] = v;
+                }
+            }
+            __syncthreads();
+            if (tid < 256) {
+                for (int m = 0; m < M; ++m) {
+                    float ss = 0.f;
+                    for (int c = tid; c < chunks; c += 256) {
+                        const uint4 v = xs[m * xs_stride + c];
+                        norm_take<false>(v, v, ss);
+                    }
+                    ss = norm_wave_sum(ss);
+                    if (lane == 0) s_part[4 * m + wave] = ss;
+                }
+            }
+            __syncthreads();
+            for (int m = 0; m < M; ++m) {
+                const float inv = rsqrtf((s_part[4 * m] + s_part[4 * m + 1] + s_part[4 * m + 2] + s_part[4 * m + 3]) / (float)C->K + C->eps);
+                for (int c = tid; c < chunks; c += T) {
+                    const uint4 g = *reinterpret_cast<const uint4 *>(C->norm_w + 8 * c);
+                    xs[m * xs_stride + c] = pair_order_u4(norm_put(xs[m * xs_stride + c], g, inv));
+                }
+            }
+            __syncthreads();
+        }
+
+        // ---- this wave's units
+        int u0, n;
+        wave_range<NW>(C, wg, wave, u0, n);
+        const int T0 = div_magic(U0, nb, C->nb_magic);  // first tile of the workgroup
+        f4_t acc[2][2];
+#pragma unroll
+        for (int v = 0; v < 2; ++v)
+#pragma unroll
+            for (int t = 0; t < 2; ++t) acc[v][t] = (f4_t){0.f, 0.f, 0.f, 0.f};
+        int cur_tile = div_magic(u0, nb, C->nb_magic);
+        if (lane == 0) {
+            s_ft[wave] = n > 0 ? cur_tile : 0x7fffffff;
+            s_lt[wave] = n > 0 ? div_magic(u0 + n - 1, nb, C->nb_magic) : -1;
+        }
+        // accumulators of one tile -> this wave's slot of the reduction area (rows 0..3 live in lanes 0..15)
+        auto flush_tile = [&](int tile) {
+            float *dst = red + ((size_t)((tile - T0) * NW + wave) * M) * 64;
+            if (lane < 16) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (e < M) {
+#pragma unroll
+                        for (int v = 0; v < 2; ++v)
+#pragma unroll
+                            for (int t = 0; t < 2; ++t) dst[e * 64 + v * 32 + 2 * lcol + t] = acc[v][t][e];
+                    }
+            }
+        };
+        const uint4 *xa = xs + min(lcol, M - 1) * xs_stride + lrow;
+        auto compute_unit = [&](const UnitRegs &U, int b) {
+            int slot = b - st_b0;
+            if (slot < 0) slot += nb;
+            const uint4 *ap = xa + slot * 16;
+            h8_t a[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) a[k] = __builtin_bit_cast(h8_t, ap[4 * k]);
+            ColDecode cd[2][2];
+#pragma unroll
+            for (int v = 0; v < 2; ++v) {
+                const uint32_t zs = U.raw_z[v] >> (((2 * lcol) & 7) * 4);
+#pragma unroll
+                for (int t = 0; t < 2; ++t) cd[v][t] = make_col_decode((zs >> (4 * t)) & 0xFu, U.raw_s[v] >> (16 * t));
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+#pragma unroll
+                for (int v = 0; v < 2; ++v)
+#pragma unroll
+                    for (int t = 0; t < 2; ++t)
+                        acc[v][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[k], decode_word_h8(t == 0 ? U.w[v][k].x : U.w[v][k].y, cd[v][t]), acc[v][t], 0, 0, 0);
+        };
+        const int n_pad = (n + DEPTH - 1) / DEPTH * DEPTH;
+        for (int i = 0; i < n_pad; i += DEPTH) {
+#pragma unroll
+            for (int d = 0; d < DEPTH; ++d) {
+                if (i + d < n) {
+                    const int u = u0 + i + d;
+                    const int tile = div_magic(u, nb, C->nb_magic);
+                    if (tile != cur_tile) {
+                        flush_tile(cur_tile);
+#pragma unroll
+                        for (int v = 0; v < 2; ++v)
+#pragma unroll
+                            for (int t = 0; t < 2; ++t) acc[v][t] = (f4_t){0.f, 0.f, 0.f, 0.f};
+                        cur_tile = tile;
+                    }
+                    compute_unit(ring[d], u - tile * nb);
+                }
+                issue_load(ring[d]);
+            }
+        }
+        if (n > 0) flush_tile(cur_tile);
+        __syncthreads();
+
+        // ---- the workgroup's partial tiles -> its slots in the workspace, then the completion flag
+        if (nwg > 0) {
+            const int T1 = div_magic(U0 + nwg - 1, nb, C->nb_magic);
+            const int per_tile = M * 64;
+            const int total = (T1 - T0 + 1) * per_tile;
+            for (int e = tid; e < total; e += T) {
+                const int tl = e / per_tile;
+                const int rem = e - tl * per_tile;
+                const int tile = T0 + tl;
+                float s = 0.f;
+#pragma unroll
+                for (int w = 0; w < NW; ++w)
+                    if (s_ft[w] <= tile && tile <= s_lt[w]) s += red[(size_t)(tl * NW + w) * per_tile + rem];
+                const int rank = wg - wg_of_unit(C, tile * nb);
+                const uint32_t off = C->partial_off + ((uint32_t)tile * C->max_contrib + rank) * per_tile + rem;
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, s), rs_part, off * 4u, 0, AUX_SC1);
+            }
+        }
+        // completion, not fences, orders the hand-over: the stores above (and this phase's sum_out) are acknowledged
+        // by the memory side before the flag is raised
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0 && wg != A->skip_flag_wg)
+            __hip_atomic_store(&st->flags[wg], epoch + (uint32_t)p + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (C->out_kind != CHAIN_OUT_NONE) pending |= 1u << p;
+    }
+
+}
+
+// ---------------------------------------------------------------------------------------------- host side
+struct ChainTuning {
+    int waves;   // waves per workgroup: 8 or 16 (0 = automatic)
+    int depth;   // units of loads in flight per wave: 1..3 (0 = automatic)
+    uint32_t spin_limit;
+    int skip_flag_wg;
+};
+ChainTuning g_chain_tuning = {0, 0, 0, -1};
+
+uint32_t magic_of(int d) { return d > 1 ? (uint32_t)(0x100000000ull / (unsigned)d + 1) : 0u; }
+
+struct DeviceInfo {
+    int cus;
+    size_t lds_per_wg;
+    bool known;
+};
+// number of CUs and the LDS a workgroup may use, asked once per device
+int device_info(DeviceInfo *out) {
+    enum { MAX_DEVICES = 64 };
+    static DeviceInfo info[MAX_DEVICES];
+    static std::mutex lock;
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= MAX_DEVICES) return (int)hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> guard(lock);
+    if (!info[dev].known) {
+        hipDeviceProp_t prop;
+        e = hipGetDeviceProperties(&prop, dev);
+        if (e != hipSuccess) return (int)e;
+        info[dev].cus = prop.multiProcessorCount;
+        info[dev].lds_per_wg = prop.sharedMemPerBlock;
+        info[dev].known = true;
+    }
+    *out = info[dev];
+    return 0;
+}
+
+template <int NW, int DEPTH>
+int launch_variant(const ChainArgs &a, int grid, size_t lds, hipStream_t stream) {
+    static bool prepared = false;
+    static std::mutex lock;
+    {
+        std::lock_guard<std::mutex> guard(lock);
+        if (!prepared) {
+            const void *fn = reinterpret_cast<const void *>(&gptq4_chain_kernel<NW, DEPTH>);
+            hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 2048);
+            if (e != hipSuccess) return (int)e;
+            prepared = true;
+        }
+    }
+    // the grid must be resident as a whole (workgroups wait for each other): one workgroup per CU
+    int per_cu = 0;
+    hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gptq4_chain_kernel<NW, DEPTH>, 64 * NW, lds);
+    if (e != hipSuccess) return (int)e;
+    if (per_cu < 1) return (int)hipErrorLaunchOutOfResources;
+    hipLaunchKernelGGL((gptq4_chain_kernel<NW, DEPTH>), dim3((unsigned)grid), dim3(64 * NW), lds, stream, a);
+    return (int)hipGetLastError();
+}
+
+struct ChainPlan {
+    ChainArgs a;
+    int grid;
+    int waves, depth;
+    size_t lds_bytes;
+    size_t partial_bytes;
+    int rc;  // 0 or a negative GPTQ4_E_* code
+};
+
+int epi_of(const gptq4_phase_t &ph) {
+    if (ph.up_qweight != nullptr) return EPI_SILU_MUL;
+    return ph.output == GPTQ4_OUT_ROPE ? EPI_ROPE : EPI_PLAIN;
+}
+
+// Validates the phase list and lays the launch out.  `grid` = number of CUs (0: do not ask the device, plan for 256).
+ChainPlan plan_chain(const gptq4_phase_t *phases, int nphases, int M, int grid) {
+    ChainPlan pl = {};
+    pl.rc = -GPTQ4_E_SHAPE;
+    if (phases == nullptr) {
+        pl.rc = -GPTQ4_E_NULL;
+        return pl;
+    }
+    if (nphases < 1 || nphases > CHAIN_MAX_PHASES || M < 1 || M > CHAIN_MAX_M) return pl;
+    if (grid <= 0) grid = 256;
+    if (grid > CHAIN_MAX_GRID) grid = CHAIN_MAX_GRID;
+    pl.grid = grid;
+    pl.waves = (g_chain_tuning.waves == 8 || g_chain_tuning.waves == 16) ? g_chain_tuning.waves : 8;
+    pl.depth = (g_chain_tuning.depth >= 1 && g_chain_tuning.depth <= 3) ? g_chain_tuning.depth : 2;
+    ChainArgs &a = pl.a;
+    a.nphases = nphases;
+    a.M = M;
+    a.spin_limit = g_chain_tuning.spin_limit ? g_chain_tuning.spin_limit : (4u << 20);
+    a.skip_flag_wg = g_chain_tuning.skip_flag_wg;
+    size_t partial_floats = 0;
+    int stage_chunks = 16, red_tiles = 1;
+    for (int p = 0; p < nphases; ++p) {
+        const gptq4_phase_t &ph = phases[p];
+        ChainPhase &c = a.ph[p];
+        if (!ph.qweight || !ph.qzeros || !ph.scales) {
+            pl.rc = -GPTQ4_E_NULL;
+            return pl;
+        }
+        const bool pair = ph.up_qweight != nullptr;
+        if (pair && (!ph.up_qzeros || !ph.up_scales)) {
+            pl.rc = -GPTQ4_E_NULL;
+            return pl;
+        }
+        int g = ph.groupsize;
+        const int K = ph.K, N = ph.N;
+        if (K <= 0 || N <= 0 || (K % 128) != 0 || (N % 256) != 0) return pl;
+        if (g == -1) g = K;
+        if (g <= 0 || (g % 128) != 0 || (K % g) != 0) {
+            pl.rc = -GPTQ4_E_GROUPSIZE;
+            return pl;
+        }
+        if ((uint64_t)K * N / 2 >= (1ull << 31) || (uint64_t)M * K * 2 >= (1ull << 31)) return pl;
+        if (ph.perm != nullptr) return pl;  // act-order inputs are not taken by the chained launch
+        c.epi = epi_of(ph);
+        if (pair && ph.output == GPTQ4_OUT_ROPE) return pl;
+        c.w[0] = QMat{reinterpret_cast<const uint32_t *>(ph.qweight), reinterpret_cast<const uint32_t *>(ph.qzeros),
+                      reinterpret_cast<const half_t *>(ph.scales)};
+        c.w[1] = pair ? QMat{reinterpret_cast<const uint32_t *>(ph.up_qweight), reinterpret_cast<const uint32_t *>(ph.up_qzeros),
+                             reinterpret_cast<const half_t *>(ph.up_scales)}
+                      : c.w[0];
+        c.K = K, c.N = N, c.nb = K / 128;
+        c.tiles = pair ? N / 32 : N / 64;
+        c.bpg = g / 128, c.groups = K / g;
+        c.group_magic = magic_of(c.bpg), c.nb_magic = magic_of(c.nb);
+        const long units = (long)c.tiles * c.nb;
+        if (units >= (1L << 24)) return pl;
+        c.q = (int)(units / grid), c.r = (int)(units % grid);
+        c.q_magic = magic_of(c.q), c.q1_magic = magic_of(c.q + 1);
+        c.max_contrib = c.q > 0 ? (c.nb + c.q - 1) / c.q + 1 : c.nb;
+        if (c.max_contrib > c.nb) c.max_contrib = c.nb;
+        if (c.max_contrib > grid) c.max_contrib = grid;
+        // ---- input
+        c.in_kind = ph.input;
+        c.eps = ph.eps;
+        c.x = reinterpret_cast<const half_t *>(ph.x);
+        c.delta = reinterpret_cast<const half_t *>(ph.delta);
+        c.norm_w = reinterpret_cast<const half_t *>(ph.norm_weight);
+        c.sum_out = reinterpret_cast<half_t *>(ph.sum_out);
+        c.bias = reinterpret_cast<const half_t *>(ph.bias);
+        const bool norm = ph.input == GPTQ4_IN_NORM_ROWS || ph.input == GPTQ4_IN_NORM_PREV;
+        const bool from_prev = ph.input == GPTQ4_IN_PREV || ph.input == GPTQ4_IN_NORM_PREV;
+        if (ph.input < GPTQ4_IN_ROWS || ph.input > GPTQ4_IN_NORM_PREV) return pl;
+        if (from_prev) {
+            if (p == 0) return pl;
+            const gptq4_phase_t &pv = phases[p - 1];
+            if (pv.N != K || pv.output == GPTQ4_OUT_ROPE) return pl;             // the previous output is this phase's input row
+            if (ph.input == GPTQ4_IN_NORM_PREV && pv.up_qweight != nullptr) return pl;  // a residual add takes a plain projection
+        }
+        if (ph.input != GPTQ4_IN_PREV && !ph.x) {
+            pl.rc = -GPTQ4_E_NULL;
+            return pl;
+        }
+        if (norm) {
+            if (!ph.norm_weight) {
+                pl.rc = -GPTQ4_E_NULL;
+                return pl;
+            }
+            if (K > 8192 || !(ph.eps >= 0.f)) return pl;
+            if (ph.sum_out != nullptr && (ph.sum_out == ph.x || ph.sum_out == ph.delta)) return pl;  // other workgroups still read them
+            // the residual rows may be the sums an earlier phase of this launch wrote
+            for (int e = 0; e < p; ++e)
+                if (phases[e].sum_out != nullptr && phases[e].sum_out == ph.x) c.x_in_launch = 1;
+        }
+        c.stage_full = norm ? 1 : 0;
+        const int per_wg = c.q + (c.r ? 1 : 0);
+        const int staged = (norm || per_wg >= c.nb) ? c.nb : per_wg;
+        if (staged * 16 > stage_chunks) stage_chunks = staged * 16;
+        const int touched = (per_wg + c.nb - 1) / c.nb + 1;
+        if (touched > red_tiles) red_tiles = touched;
+        // ---- output
+        c.out_kind = ph.output;
+        if (ph.output < GPTQ4_OUT_NONE || ph.output > GPTQ4_OUT_ROPE) return pl;
+        if (ph.output == GPTQ4_OUT_ROWS) {
+            if (!ph.y) {
+                pl.rc = -GPTQ4_E_NULL;
+                return pl;
+            }
+            c.y = reinterpret_cast<half_t *>(ph.y);
+        } else if (ph.output == GPTQ4_OUT_ROPE) {
+            if (!ph.position_ids || !ph.cos_table || !ph.sin_table || !ph.q || !ph.k || !ph.v) {
+                pl.rc = -GPTQ4_E_NULL;
+                return pl;
+            }
+            if (ph.H < 1 || N != 3 * ph.H * 128 || ph.max_pos < 1 || ph.kv_capacity < 1 || ph.kv_offset < GPTQ4_KV_AT_POSITION ||
+                (ph.kv_offset >= 0 && ph.kv_capacity < ph.kv_offset + 1))
+                return pl;
+            c.rope.position_ids = ph.position_ids;
+            c.rope.cos_table = ph.cos_table, c.rope.sin_table = ph.sin_table;
+            c.rope.q = reinterpret_cast<half_t *>(ph.q), c.rope.k = reinterpret_cast<half_t *>(ph.k), c.rope.v = reinterpret_cast<half_t *>(ph.v);
+            c.rope.S = 1, c.rope.H = ph.H, c.rope.kv_capacity = ph.kv_capacity, c.rope.kv_offset = ph.kv_offset, c.rope.max_pos = ph.max_pos;
+        } else if (p + 1 == nphases || (phases[p + 1].input != GPTQ4_IN_PREV && phases[p + 1].input != GPTQ4_IN_NORM_PREV)) {
+            return pl;  // a phase nobody reads and that leaves nothing in memory
+        }
+        if (ph.bias != nullptr && pair) return pl;
+        c.partial_off = (uint32_t)partial_floats;
+        partial_floats += (size_t)c.tiles * c.max_contrib * M * 64;
+        if (partial_floats * 4 >= (1ull << 31)) return pl;
+    }
+    pl.partial_bytes = partial_floats * 4;
+    a.partial_bytes = (uint32_t)pl.partial_bytes;
+    // LDS: [M rows of staged activations][reduction area]; rows 64 bytes apart modulo 128 so that two rows'
+    // A-operand reads fall into different banks
+    int stride = stage_chunks;
+    if ((stride & 7) != 4) stride += (4 - (stride & 7) + 8) & 7;
+    a.xs_stride = stride;
+    a.red_off = M * stride;
+    a.red_tiles = red_tiles;
+    const size_t red_bytes = (size_t)red_tiles * pl.waves * M * 64 * sizeof(float);
+    pl.lds_bytes = (size_t)a.red_off * 16 + red_bytes;
+    if (pl.lds_bytes > 150 * 1024) return pl;
+    // more than half of a CU's 160 KiB: no CU can take two workgroups, so the grid spreads over all CUs
+    if (pl.lds_bytes < 84 * 1024) pl.lds_bytes = 84 * 1024;
+    pl.rc = 0;
+    return pl;
+}
+
+}  // namespace
+
+extern "C" {
+
+void gptq4_set_chain_tuning(int waves, int depth, unsigned spin_limit, int skip_flag_wg) {
+    g_chain_tuning.waves = (waves == 8 || waves == 16) ? waves : 0;
+    g_chain_tuning.depth = (depth >= 1 && depth <= 3) ? depth : 0;
+    g_chain_tuning.spin_limit = spin_limit;
+    g_chain_tuning.skip_flag_wg = skip_flag_wg;
+}
+
+size_t gptq4_chain_workspace_bytes(const gptq4_phase_t *phases, int nphases, int M) {
+    DeviceInfo di = {};
+    const int grid = device_info(&di) == 0 ? di.cus : 0;
+    const ChainPlan pl = plan_chain(phases, nphases, M, grid);
+    if (pl.rc != 0) return 0;
+    return (size_t)CHAIN_STATE_BYTES + pl.partial_bytes;
+}
+
+int gptq4_decode_chain(const gptq4_phase_t *phases, int nphases, int M, void *workspace, size_t workspace_bytes, void *stream) {
+    // argument errors first: they need no device
+    ChainPlan pl = plan_chain(phases, nphases, M, 0);
+    if (pl.rc != 0) return pl.rc;
+    DeviceInfo di = {};
+    int rc = device_info(&di);
+    if (rc) return rc;
+    pl = plan_chain(phases, nphases, M, di.cus);
+    if (pl.rc != 0) return pl.rc;
+    if (workspace == nullptr || workspace_bytes < (size_t)CHAIN_STATE_BYTES + pl.partial_bytes) return -GPTQ4_E_WORKSPACE;
+    if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return -GPTQ4_E_ALIGN;
+    for (int p = 0; p < nphases; ++p) {
+        const gptq4_phase_t &ph = phases[p];
+        const void *ptrs[] = {ph.qweight, ph.scales, ph.up_qweight, ph.up_scales, ph.x, ph.delta, ph.norm_weight, ph.sum_out,
+                              ph.y, ph.bias, ph.q, ph.k, ph.v, ph.cos_table, ph.sin_table};
+        for (const void *q : ptrs)
+            if (q != nullptr && (reinterpret_cast<uintptr_t>(q) & 15u) != 0) return -GPTQ4_E_ALIGN;
+    }
+    pl.a.state = reinterpret_cast<ChainState *>(workspace);
+    pl.a.partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + CHAIN_STATE_BYTES);
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const int key = pl.waves * 10 + pl.depth;
+    switch (key) {
+        case 81: return launch_variant<8, 1>(pl.a, pl.grid, pl.lds_bytes, s);
+        case 83: return launch_variant<8, 3>(pl.a, pl.grid, pl.lds_bytes, s);
+        case 161: return launch_variant<16, 1>(pl.a, pl.grid, pl.lds_bytes, s);
+        case 162: return launch_variant<16, 2>(pl.a, pl.grid, pl.lds_bytes, s);
+        default: return launch_variant<8, 2>(pl.a, pl.grid, pl.lds_bytes, s);
+    }
+}
+
+}  // extern "C"

@@ -205,6 +205,79 @@ int gptq4_decode_attention(const void *q, const void *k_cache, const void *v_cac
                            int kv_capacity, float scale, void *workspace,
                            size_t workspace_bytes, void *stream);
 
+/* ---- Chained decode launch: several decode-sized projections in ONE persistent launch ----------------------
+ * A decode step is a chain of small projections, each streaming its weights once; launched one by one, about
+ * 6 us of every 6-15 us launch are launch floor, prologue, first-load latency and partial-sum exchange, during
+ * which HBM idles.  gptq4_decode_chain runs a list of up to 8 "phases" on one resident grid (one workgroup per
+ * CU) that streams the weights of all phases as one sequence: the loads of the next phase are in flight while
+ * the one before is handed over.  No reference counterpart: the reference launches one Triton kernel per
+ * projection (quant_linear.py:264-274, fused_mlp.py:286-297) with the torch ops of the decoder layer between
+ * them.
+ *
+ * A phase is a 4-bit projection (or a gate/up pair: up_* set) of M <= 4 rows.  `input` says what it multiplies:
+ *   GPTQ4_IN_ROWS       x fp16 [M, K], in memory before the launch
+ *   GPTQ4_IN_NORM_ROWS  norm_weight * rmsnorm(x (+ delta)), x and delta in memory before the launch; the sums
+ *                       x + delta go to sum_out (nullable)
+ *   GPTQ4_IN_PREV       the output of the phase before it: fp16(sums) (+ bias) of a projection,
+ *                       fp16(silu(gate) * up) of a pair; its N is this phase's K
+ *   GPTQ4_IN_NORM_PREV  norm_weight * rmsnorm(x + previous output): x fp16 [M, K] is the residual stream (in
+ *                       memory before the launch, or the sum_out of an earlier phase); sums to sum_out (nullable)
+ * (the rounding order of gptq4_add_rmsnorm / gptq4_matmul / gptq4_mlp_gateup run one after the other; only the
+ * order in which fp32 partial sums are added differs, fixed for a given shape and GPU).  `output`:
+ *   GPTQ4_OUT_NONE      only the next phase reads it (which must then be IN_PREV / IN_NORM_PREV)
+ *   GPTQ4_OUT_ROWS      y fp16 [M, N] is written as well (a pair writes silu(gate) * up)
+ *   GPTQ4_OUT_ROPE      N = 3 * H * 128 columns q, k, v: rotary + head-major stores as gptq4_qkv_rotary with one
+ *                       token per sequence (B = M, S = 1); nothing can read it as IN_PREV
+ * K % 128 == 0, N % 256 == 0, groupsize as elsewhere; norm inputs need K <= 8192; `perm` must be NULL (act-order
+ * inputs are not taken).  sum_out must not be x or delta.
+ *
+ * Workspace: gptq4_chain_workspace_bytes() bytes, 256-byte aligned, ZERO before the first launch; it carries
+ * state from launch to launch (do not clear it between launches, do not share it with the other entry points,
+ * one per stream).  All waits inside the launch are bounded: if a workgroup ever gives up (the grid was not
+ * resident as a whole, e.g. because another stream's kernel held CUs for seconds), every workgroup returns,
+ * outputs are undefined and the int32 at byte offset 4 of the workspace is set to 1 - later launches on that
+ * workspace then return at once until the caller clears it (hipMemsetAsync the whole workspace, outside a graph).
+ * Launch nothing else on other streams that needs the whole GPU for long while a chain runs. */
+#define GPTQ4_IN_ROWS 0
+#define GPTQ4_IN_NORM_ROWS 1
+#define GPTQ4_IN_PREV 2
+#define GPTQ4_IN_NORM_PREV 3
+#define GPTQ4_OUT_NONE 0
+#define GPTQ4_OUT_ROWS 1
+#define GPTQ4_OUT_ROPE 2
+#define GPTQ4_CHAIN_MAX_PHASES 8
+#define GPTQ4_CHAIN_MAX_M 4
+#define GPTQ4_CHAIN_ERROR_OFFSET 4
+
+typedef struct gptq4_phase {
+    const int32_t *qweight, *qzeros;
+    const void *scales;
+    const int32_t *up_qweight, *up_qzeros; /* all three set: qweight.. is gate, this is up */
+    const void *up_scales;
+    const int32_t *perm; /* must be NULL */
+    const void *x, *delta, *norm_weight;
+    void *sum_out;
+    void *y;
+    const void *bias;
+    /* GPTQ4_OUT_ROPE */
+    const int32_t *position_ids; /* [M] */
+    const float *cos_table, *sin_table;
+    void *q, *k, *v;
+    int K, N, groupsize;
+    int input, output;
+    float eps;
+    int H, max_pos, kv_capacity, kv_offset;
+} gptq4_phase_t;
+
+/* 0 if the list is not one gptq4_decode_chain accepts */
+size_t gptq4_chain_workspace_bytes(const gptq4_phase_t *phases, int nphases, int M);
+int gptq4_decode_chain(const gptq4_phase_t *phases, int nphases, int M, void *workspace,
+                       size_t workspace_bytes, void *stream);
+/* Measurement and test knobs of the chained launch: waves per workgroup (8, 16), units of loads in flight per
+ * wave (1..3), polls before a wait gives up (0 = default, about seconds), and a workgroup that never reports
+ * completion (-1 = none; lets a test see the bounded waits give up with every kernel exiting normally). */
+void gptq4_set_chain_tuning(int waves, int depth, unsigned spin_limit, int skip_flag_wg);
+
 /* Host-side launch tuning of the small-M kernels, for measurements: words per lane and
  * load (1, 2 or 4: strips of 16, 32 or 64 columns), batches of loads in flight per
  * wave (1..4) and the split-K factor; 0 = automatic for each.  Process-wide; not

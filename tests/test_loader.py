@@ -140,10 +140,17 @@ def test_loaded_model_matches_cpu_reference(tmp_path, groupsize, act_order):
     ref = decoder_ref.forward(state, cfg, groupsize, ids)
     logits, _ = model(ids.cuda())
     got = logits.float().cpu()
-    # fp16 activations through 2 layers against a float32 reference
+    # fp16 activations through 2 layers against a float32 reference.  Measured over 9 such checkpoints (3 seeds x
+    # 3 configurations): logits up to 4.5 in magnitude, largest error 0.0021-0.0026, mean error 4.0e-4 - about two
+    # fp16 roundings of the hidden state.  The bound is 2.3 times the largest error seen; where the reference's
+    # best logit leads by more than twice the bound, the greedy token must be the same.
+    bound = 0.006
     err = (got - ref).abs()
-    assert err.max() < 0.05 * ref.abs().max() and err.mean() < 0.01 * ref.abs().mean() + 1e-3
-    assert (got.argmax(-1) == ref.argmax(-1)).float().mean() > 0.9
+    assert err.max().item() < bound and err.mean().item() < 1e-3, (err.max().item(), err.mean().item())
+    top2 = ref.topk(2, dim=-1).values
+    clear = (top2[..., 0] - top2[..., 1]) > 2 * bound
+    assert clear.float().mean() > 0.8, "the check needs positions with a clear winner"
+    assert torch.equal(got.argmax(-1)[clear], ref.argmax(-1)[clear])
 
     # incremental decoding with the KV cache equals the full forward
     full, _ = model(ids.cuda())
