@@ -29,7 +29,8 @@ struct ChainPhase {
     float eps;
     int epi;                 // EPI_PLAIN, EPI_SILU_MUL, EPI_ROPE: which strips make a tile
     int in_kind, out_kind;
-    int x_in_launch;         // IN_NORM_PREV: x was written by an earlier phase of this launch (read it around the L2)
+    int x_in_launch;         // IN_NORM_PREV: x is the sum_out of the last norm phase before this one: taken from the copy in LDS
+    int keep_sums;           // IN_NORM_*: a later phase reads this phase's sums as its x: keep them in LDS
     int K, N;                // N: columns of one matrix
     int nb;                  // K / 128
     int tiles;               // plain: N / 64; pair: N / 32 (32 of gate + the same 32 of up); rotary: N / 64 (32 of d + 32 of d + 64)
@@ -40,15 +41,15 @@ struct ChainPhase {
     uint32_t q_magic, q1_magic;
     int max_contrib;         // workgroups that can share one tile
     int stage_full;          // 1: the whole row is staged in LDS (slot = batch), 0: only the workgroup's batches
-    uint32_t partial_off;    // this phase's partial sums: float offset into the partial region
+    uint32_t partial_off;    // this phase's partial sums: element offset ({fp32 bits, tag} pairs) into the partial region
 };
 
 // Persistent state in the chain workspace (zero before the first launch; launches maintain it).
 struct ChainState {
-    uint32_t epoch;   // phases completed by all earlier launches: phase p of a launch completes at epoch + p + 1
-    int32_t error;    // 0, or CHAIN_ERR_* of the first launch that gave up (sticky: later launches return at once)
+    uint32_t launches;  // launches completed on this workspace (informational)
+    int32_t error;      // 0, or CHAIN_ERR_* of the first launch that gave up (sticky: later launches return at once)
     uint32_t pad[30];
-    uint32_t flags[CHAIN_MAX_GRID];  // per workgroup: the last phase epoch it completed
+    uint32_t wg_epoch[CHAIN_MAX_GRID];  // per workgroup: phases of all earlier launches; phase p of a launch tags its sums epoch + p + 1
 };
 enum { CHAIN_ERR_TIMEOUT = 1 };
 
@@ -60,10 +61,11 @@ struct ChainArgs {
     int nphases;
     int M;
     int xs_stride;     // 16-byte chunks per staged row (LDS)
+    int keep_off;      // LDS offset (chunks) of the residual sums kept for a later phase
     int red_off;       // LDS offset (chunks) of the reduction area
     int red_tiles;     // tiles a workgroup can touch in one phase
-    uint32_t spin_limit;  // polls of the completion flags before a workgroup gives up
-    int skip_flag_wg;     // test hook: this workgroup never reports completion (-1: none)
+    uint32_t spin_limit;  // polls of a partial tile before a thread gives up
+    int skip_flag_wg;     // test hook: this workgroup never stores its partial sums (-1: none)
 };
 
 static_assert(sizeof(ChainState) <= CHAIN_STATE_BYTES, "state region");

@@ -18,27 +18,40 @@
 //   count.  A wave's range lies in one tile or crosses into the next.
 //   x      = the M rows the phase multiplies with, staged once per workgroup in LDS in the k order the
 //            decoded weights come out in ("pair order"); the A operand of every wave is read from there.
-//   hand-over: the waves of a workgroup add their accumulators per tile through LDS (wave order), the
+//   hand-over: the waves of a workgroup add their accumulators per tile through LDS (wave order) and the
 //            workgroup stores one partial tile per touched tile in its slot of the workspace (slot = its rank
-//            among the workgroups sharing the tile), waits for the stores to complete and raises its
-//            completion flag to the phase's epoch.  A consumer polls the flags of all workgroups (one wave,
-//            bounded), then adds the partial tiles it needs in rank order - every consumer the same order, so
-//            results are deterministic - and applies what lies between the two projections itself: rounding
-//            to fp16, bias, residual add, RMSNorm, SiLU*mul.
+//            among the workgroups sharing the tile), every value as an 8-byte element {fp32 bits, tag}, tag =
+//            the phase's number in the life of the workspace.  Nothing waits on the producer side.  A consumer
+//            reads the partial tiles it needs, polls until all of them carry the tag it expects (bounded), adds
+//            them in rank order - every consumer the same order, so results are deterministic - and applies
+//            what lies between the two projections itself: rounding to fp16, bias, residual add, RMSNorm,
+//            SiLU*mul.  There is no grid-wide barrier: a consumer waits for exactly the tiles it reads.
 //   Outputs that must exist in memory (y, q/k/v with rotary) are written by all workgroups, a slice each,
-//   at the next point where the launch waits anyway (or at its end).
+//   where the launch reads the previous phase anyway (or at its end).
 //
-// Ordering across workgroups is by completion, as in the other decode kernels: partial sums, sums and flags are
-// written with agent-scope (sc1) stores and read with agent-scope loads, which go around the per-XCD L2s; a
-// workgroup waits for the acknowledgement of its data stores (s_waitcnt vmcnt(0)) before it stores its flag.
-// Every wait is bounded: a workgroup that gives up records CHAIN_ERR_TIMEOUT in the state and returns, which
-// makes every other workgroup give up in turn; the error is sticky until the host clears the workspace.
+// Visibility across workgroups: partial sums are written with agent-scope (sc1) 8-byte stores and read with
+// agent-scope loads, which go around the per-XCD L2s; an aligned 8-byte store is never seen half-written, so a
+// value next to the expected tag is the value that was stored with it.  Every poll is bounded: a thread that
+// gives up records CHAIN_ERR_TIMEOUT in the state, its workgroup returns at the next barrier, and the
+// workgroups that depend on it give up in turn; the error is sticky until the host clears the workspace.
 #include "gptq4_chain.h"
 
 #include "../../include/gptq4.h"
 #include "gptq4_norm.h"
 
 #include <mutex>
+
+// Development aid, compiled out of the product build: per-workgroup 100 MHz clock stamps at the stage boundaries
+// of every phase, written behind the partial sums (the workspace is then 1 MiB larger).
+#ifdef GPTQ4_CHAIN_TIMERS
+#define CHAIN_STAMP(i)                                                                                                   \
+    do {                                                                                                                 \
+        if (ht == 0)                                                                                                     \
+            reinterpret_cast<unsigned long long *>(reinterpret_cast<char *>(A->partials) + A->partial_bytes)[wg * 64 + (i)] = wall_clock64(); \
+    } while (0)
+#else
+#define CHAIN_STAMP(i)
+#endif
 
 namespace {
 
@@ -87,28 +100,40 @@ __device__ __forceinline__ int wg_of_unit(PhasePtr P, int u) {
 
 __device__ __forceinline__ float f_of(uint32_t u) { return __builtin_bit_cast(float, u); }
 
-// Sum of the partial tiles of 8 adjacent columns (two 16-byte loads per contributing workgroup, all issued
-// before the first add), in rank order.  `base` = float offset of (tile, rank 0, row m, column) in the partial
-// region, `stride` = floats between ranks.
-__device__ __forceinline__ void sum_partials8(const __amdgpu_buffer_rsrc_t &rs, uint32_t base, uint32_t stride, int nc, float out[8]) {
+// Partial sums travel as 8-byte elements {fp32 bits, tag}: an aligned 8-byte store becomes visible as a whole,
+// so a consumer that reads the tag it expects next to a value knows the value is this launch's, this phase's -
+// no separate flag, no wait for store acknowledgements on the producer side, no grid-wide barrier.  The tag of
+// phase p is the workgroup's launch-to-launch epoch + p + 1; the workspace starts zeroed and tags only grow.
+//
+// Sum over the contributing workgroups (rank order) of 8 adjacent columns; `base` = element offset of (tile,
+// rank 0, row m, column) in the partial region, `stride` = elements between ranks.  Returns false if any element
+// does not carry `tag` yet (the caller polls).
+__device__ __forceinline__ bool sum_partials8(const __amdgpu_buffer_rsrc_t &rs, uint32_t base, uint32_t stride, int nc, uint32_t tag,
+                                              float out[8]) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) out[i] = 0.f;
-    for (int r0 = 0; r0 < nc; r0 += 4) {
-        u32x4_t a[4], b[4];
+    bool valid = true;
+    for (int r0 = 0; r0 < nc; r0 += 2) {
+        u32x4_t a[2][4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const uint32_t off = (r0 + j < nc) ? (base + (uint32_t)(r0 + j) * stride) * 4u : OFF_RANGE;
-            a[j] = __builtin_amdgcn_raw_buffer_load_b128(rs, off, 0, AUX_SC1);
-            b[j] = __builtin_amdgcn_raw_buffer_load_b128(rs, off + 16u, 0, AUX_SC1);
+        for (int j = 0; j < 2; ++j) {
+            const uint32_t off = (base + (uint32_t)min(r0 + j, nc - 1) * stride) * 8u;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) a[j][q] = __builtin_amdgcn_raw_buffer_load_b128(rs, off + 16u * q, 0, AUX_SC1);
         }
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < 2; ++j) {
             if (r0 + j < nc) {
-                out[0] += f_of(a[j].x), out[1] += f_of(a[j].y), out[2] += f_of(a[j].z), out[3] += f_of(a[j].w);
-                out[4] += f_of(b[j].x), out[5] += f_of(b[j].y), out[6] += f_of(b[j].z), out[7] += f_of(b[j].w);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    valid = valid && a[j][q].y == tag && a[j][q].w == tag;
+                    out[2 * q] += f_of(a[j][q].x);
+                    out[2 * q + 1] += f_of(a[j][q].z);
+                }
             }
         }
     }
+    return valid;
 }
 
 __device__ __forceinline__ uint4 pack_h8(const half_t h[8]) {
@@ -120,18 +145,37 @@ __device__ __forceinline__ uint4 pack_h8(const half_t h[8]) {
     return r;
 }
 
+// What a bounded poll needs: the limit, where to report giving up.
+struct PollCtx {
+    uint32_t limit;
+    int32_t *error;      // global error word
+    uint32_t *abort_lds; // workgroup flag: somebody gave up
+};
+
 // 8 adjacent output values of phase P (row m, columns n0 .. n0+7, n0 % 8 == 0) from its partial tiles, as the
-// next consumer sees them: fp16(sum) (+ bias) of a plain phase, fp16(silu(gate) * up) of a pair.
-__device__ __forceinline__ uint4 phase_output8(PhasePtr P, const __amdgpu_buffer_rsrc_t &rs, int M, int m, int n0) {
+// next consumer sees them: fp16(sum) (+ bias) of a plain phase, fp16(silu(gate) * up) of a pair.  Polls until the
+// partial tiles carry `tag` (bounded: gives up after ctx.limit polls, reports it and returns what it has).
+__device__ __forceinline__ uint4 phase_output8(PhasePtr P, const __amdgpu_buffer_rsrc_t &rs, int M, int m, int n0, uint32_t tag,
+                                               const PollCtx &ctx) {
     const int tile = (P->epi == EPI_PLAIN) ? (n0 >> 6) : (n0 >> 5);
     const int col = (P->epi == EPI_PLAIN) ? (n0 & 63) : (n0 & 31);
     const int first = wg_of_unit(P, tile * P->nb);
     const int nc = wg_of_unit(P, tile * P->nb + P->nb - 1) - first + 1;
     const uint32_t stride = (uint32_t)M * 64u;
     const uint32_t base = P->partial_off + ((uint32_t)tile * P->max_contrib * M + m) * 64u + col;
-    float s[8];
+    float s[8], u[8];
+    for (uint32_t spin = 0;; ++spin) {
+        bool ok = sum_partials8(rs, base, stride, nc, tag, s);
+        if (P->epi != EPI_PLAIN) ok = sum_partials8(rs, base + 32u, stride, nc, tag, u) && ok;
+        if (ok) break;
+        if (spin >= ctx.limit || ((spin & 63u) == 63u && *ctx.abort_lds != 0)) {
+            __hip_atomic_store(ctx.error, (int32_t)CHAIN_ERR_TIMEOUT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            *ctx.abort_lds = 1u;
+            break;
+        }
+        __builtin_amdgcn_s_sleep(1);
+    }
     half_t h[8];
-    sum_partials8(rs, base, stride, nc, s);
     if (P->epi == EPI_PLAIN) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) h[i] = (half_t)s[i];
@@ -142,30 +186,41 @@ __device__ __forceinline__ uint4 phase_output8(PhasePtr P, const __amdgpu_buffer
             for (int i = 0; i < 4; ++i) h[2 * i] = h[2 * i] + b2[i].x, h[2 * i + 1] = h[2 * i + 1] + b2[i].y;
         }
     } else {
-        float u[8];
-        sum_partials8(rs, base + 32u, stride, nc, u);
 #pragma unroll
         for (int i = 0; i < 8; ++i) h[i] = (half_t)(silu_f32(s[i]) * u[i]);
     }
     return pack_h8(h);
 }
 
-template <int NW, int DEPTH>
-__global__ __launch_bounds__(64 * NW) void gptq4_chain_kernel(const ChainArgs args_by_value) {
+// Waves of a workgroup have two roles.  NS streaming waves own the weight stream and the matrix-core work: their
+// memory queue holds nothing but weight loads, DEPTH units deep, and stays full while a phase is handed over.
+// CHAIN_NH helper waves do everything that is latency-critical and small - polling and adding partial tiles,
+// residual add / RMSNorm / SiLU*mul into LDS, the workgroup's partial stores, the outputs - so that none of
+// those loads ever queues behind a wave's own weight prefetch (a wave's loads return in order).
+// The roles meet at workgroup barriers only; both execute the same barrier sequence.
+constexpr int CHAIN_NH = 4;
+
+template <int NS, int DEPTH>
+__global__ __launch_bounds__(64 * (NS + CHAIN_NH)) void gptq4_chain_kernel(const ChainArgs args_by_value) {
     // The arguments are read where the launch put them, in the kernel-argument segment (constant memory, scalar
     // loads with a dynamic phase index); touching the by-value copy would make the compiler spill the whole
     // table to scratch memory to index it.
     const __attribute__((address_space(4))) ChainArgs *const A =
         (const __attribute__((address_space(4))) ChainArgs *)__builtin_amdgcn_kernarg_segment_ptr();
-    constexpr int T = 64 * NW;
+    constexpr int NH = CHAIN_NH;
+    constexpr int TH = 64 * NH;  // helper threads
+    static_assert(TH == 256, "the RMSNorm statistics follow the stand-alone kernel's 256-thread order");
     extern __shared__ uint4 smem[];
-    __shared__ int s_ft[NW], s_lt[NW];
+    __shared__ int s_ft[NS], s_lt[NS];
     __shared__ float s_part[CHAIN_MAX_M * 4];
-    __shared__ uint32_t s_ctl[2];
+    __shared__ uint32_t s_ctl[4];  // epoch, error word at the start, "somebody gave up"
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const bool helper = wave >= NS;
+    const int ht = tid - 64 * NS;  // index among the helper threads (negative in streaming waves)
+    const int hw = wave - NS;
     const int lrow = lane >> 4;
     const int lcol = lane & 15;
     const int wg = blockIdx.x;
@@ -175,22 +230,26 @@ __global__ __launch_bounds__(64 * NW) void gptq4_chain_kernel(const ChainArgs ar
 
     uint4 *const xs = smem;
     float *const red = reinterpret_cast<float *>(smem + A->red_off);
+    uint4 *const keep = smem + A->keep_off;  // the last residual sums, for a later phase of this launch
     const int xs_stride = A->xs_stride;
 
     ChainState *const st = A->state;
-    if (tid == 0) {
-        s_ctl[0] = __hip_atomic_load(&st->epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (ht == 0) {
+        // the workgroup's own epoch: every launch on this workspace moves every workgroup's on by its phase count
+        s_ctl[0] = __hip_atomic_load(&st->wg_epoch[wg], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         s_ctl[1] = (uint32_t)__hip_atomic_load(&st->error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_ctl[2] = 0u;
     }
-    __syncthreads();
-    const uint32_t epoch = s_ctl[0];
-    if (s_ctl[1] != 0) return;  // an earlier launch on this workspace gave up: the state is not trustworthy
-    __syncthreads();
+    uint32_t epoch = 0;  // read from s_ctl behind the first barrier
+    CHAIN_STAMP(0);
 
     const __amdgpu_buffer_rsrc_t rs_part = make_rsrc(A->partials, A->partial_bytes);
-    const __amdgpu_buffer_rsrc_t rs_flags = make_rsrc(st->flags, (uint32_t)G * 4u);
+    PollCtx poll;
+    poll.limit = A->spin_limit;
+    poll.error = &st->error;
+    poll.abort_lds = &s_ctl[2];
 
-    // ------------------------------------------------------------------ the weight stream
+    // ------------------------------------------------------------------ the weight stream (streaming waves)
     // Per wave the units of all phases are ONE sequence: for every phase with units for this wave, its units
     // padded to a multiple of DEPTH with switched-off loads, so that unit i of a phase always sits in ring slot
     // i % DEPTH.  The load cursor (lp, li) runs DEPTH entries ahead of the compute cursor.
@@ -208,7 +267,7 @@ __global__ __launch_bounds__(64 * NW) void gptq4_chain_kernel(const ChainArgs ar
                 return;
             }
             const PhasePtr Q = A->ph + lp;
-            wave_range<NW>(Q, wg, wave, l_u0, l_n);
+            wave_range<NS>(Q, wg, wave, l_u0, l_n);
             if (l_n == 0) continue;
             l_pad = (l_n + DEPTH - 1) / DEPTH * DEPTH;
             li = 0;
@@ -232,7 +291,6 @@ __global__ __launch_bounds__(64 * NW) void gptq4_chain_kernel(const ChainArgs ar
         rs_s0 = rs_s1 = make_rsrc(Q->w[0].scales, 16u);
         rs_z0 = rs_z1 = make_rsrc(Q->w[0].qzeros, 16u);
     }
-    next_stream_phase();
 
     auto issue_load = [&](UnitRegs &U) {
         if (li >= l_pad) next_stream_phase();
@@ -264,61 +322,29 @@ __global__ __launch_bounds__(64 * NW) void gptq4_chain_kernel(const ChainArgs ar
     };
 
     UnitRegs ring[DEPTH];
+    if (!helper) {
+        next_stream_phase();
 #pragma unroll
-    for (int d = 0; d < DEPTH; ++d) issue_load(ring[d]);
+        for (int d = 0; d < DEPTH; ++d) issue_load(ring[d]);
+    }
+    CHAIN_STAMP(1);
 
-    // ------------------------------------------------------------------ waiting for a phase to be complete everywhere
-    // One wave polls the completion flags of all workgroups (16-byte agent-scope loads, 256 flags per pass);
-    // bounded by A->spin_limit polls.  Returns false (to every thread) when the workgroup gives up.
-    auto wait_done = [&](int p) -> bool {
-        const uint32_t target = epoch + (uint32_t)p + 1u;
-        if (wave == 0) {
-            bool ok = false;
-            for (uint32_t spin = 0; spin < A->spin_limit; ++spin) {
-                bool all = true;
-                for (int base = 0; base < G; base += 256) {
-                    const int i0 = base + 4 * lane;
-                    const u32x4_t f = __builtin_amdgcn_raw_buffer_load_b128(rs_flags, (uint32_t)i0 * 4u, 0, AUX_SC1);
-                    const uint32_t fv[4] = {f.x, f.y, f.z, f.w};
-#pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                        if (i0 + j < G && (int32_t)(fv[j] - target) < 0) all = false;
-                }
-                if (__builtin_amdgcn_ballot_w64(!all) == 0) {
-                    ok = true;
-                    break;
-                }
-                if ((spin & 15u) == 15u &&
-                    __hip_atomic_load(&st->error, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)
-                    break;  // somebody else gave up already
-                __builtin_amdgcn_s_sleep(2);
-            }
-            if (lane == 0) {
-                s_ctl[0] = ok ? 1u : 0u;
-                if (!ok) __hip_atomic_store(&st->error, (int32_t)CHAIN_ERR_TIMEOUT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-        }
-        __syncthreads();
-        const bool ok = s_ctl[0] != 0;
-        __syncthreads();
-        return ok;
-    };
-
-    // ------------------------------------------------------------------ outputs that must exist in memory
+    // ------------------------------------------------------------------ outputs that must exist in memory (helper threads)
     auto write_outputs = [&](int p) {
         const PhasePtr C = A->ph + p;
+        const uint32_t tag = epoch + (uint32_t)p + 1u;
         if (C->out_kind == CHAIN_OUT_ROWS) {
             const int row_chunks = C->N >> 3;
             const int total = M * row_chunks;
-            for (int i = wg * T + tid; i < total; i += G * T) {
+            for (int i = wg * TH + ht; i < total; i += G * TH) {
                 const int m = i / row_chunks, c = i - m * row_chunks;
-                *reinterpret_cast<uint4 *>(C->y + (size_t)m * C->N + 8 * c) = phase_output8(C, rs_part, M, m, 8 * c);
+                *reinterpret_cast<uint4 *>(C->y + (size_t)m * C->N + 8 * c) = phase_output8(C, rs_part, M, m, 8 * c, tag, poll);
             }
         } else if (C->out_kind == CHAIN_OUT_ROPE) {
             // item = (row, tile, 8 head dimensions d and their partners d + 64)
             const __attribute__((address_space(4))) RopeArgs *r = &C->rope;
             const int total = M * C->tiles * 4;
-            for (int i = wg * T + tid; i < total; i += G * T) {
+            for (int i = wg * TH + ht; i < total; i += G * TH) {
                 const int cc = i & 3;
                 const int rest = i >> 2;
                 const int m = rest / C->tiles, tile = rest - m * C->tiles;
@@ -327,8 +353,17 @@ __global__ __launch_bounds__(64 * NW) void gptq4_chain_kernel(const ChainArgs ar
                 const uint32_t stride = (uint32_t)M * 64u;
                 const uint32_t base = C->partial_off + ((uint32_t)tile * C->max_contrib * M + m) * 64u + 8 * cc;
                 float x1[8], x2[8];
-                sum_partials8(rs_part, base, stride, nc, x1);
-                sum_partials8(rs_part, base + 32u, stride, nc, x2);
+                for (uint32_t spin = 0;; ++spin) {
+                    bool ok = sum_partials8(rs_part, base, stride, nc, tag, x1);
+                    ok = sum_partials8(rs_part, base + 32u, stride, nc, tag, x2) && ok;
+                    if (ok) break;
+                    if (spin >= poll.limit || ((spin & 63u) == 63u && s_ctl[2] != 0)) {
+                        __hip_atomic_store(&st->error, (int32_t)CHAIN_ERR_TIMEOUT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        s_ctl[2] = 1u;
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep(1);
+                }
                 const int head_col = tile >> 1;
                 const int d = (tile & 1) * 32 + 8 * cc;
                 const int which = head_col / r->H;
@@ -365,10 +400,11 @@ __global__ __launch_bounds__(64 * NW) void gptq4_chain_kernel(const ChainArgs ar
         }
     };
 
-    uint32_t pending = 0;  // phases whose outputs are still to be written
+    uint32_t pending = 0;  // phases whose outputs are still to be written (kept by every thread alike)
     auto flush_outputs = [&](int upto) {
-        for (int p = 0; p <= upto; ++p)
-            if (pending & (1u << p)) write_outputs(p);
+        if (helper)
+            for (int p = 0; p <= upto; ++p)
+                if (pending & (1u << p)) write_outputs(p);
         pending &= ~((2u << upto) - 1u);
     };
 
@@ -376,199 +412,214 @@ __global__ __launch_bounds__(64 * NW) void gptq4_chain_kernel(const ChainArgs ar
     // (p == P is the end of the launch: outputs still to be written, and the epoch moves on)
     for (int p = 0; p <= P; ++p) {
         const PhasePtr C = A->ph + min(p, P - 1);
-        const bool wait_here = (p == P) ? (pending != 0 || wg == 0) : (C->in_kind >= CHAIN_IN_PREV);
-        if (wait_here) {
-            if (!wait_done(p - 1)) return;
-            flush_outputs(p - 1);
-        }
+        const bool flush_here = (p == P) || (C->in_kind >= CHAIN_IN_PREV);
+        CHAIN_STAMP(2 + 7 * p);
+        if (flush_here && p > 0) flush_outputs(p - 1);  // (the helper threads are about to poll phase p - 1 anyway)
+        CHAIN_STAMP(4 + 7 * p);
         if (p == P) {
-            // every workgroup has read `epoch` long ago (it completed P phases since): move it on for the next launch
-            if (wg == 0 && tid == 0) __hip_atomic_store(&st->epoch, epoch + (uint32_t)P, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (ht == 0 && s_ctl[2] == 0)
+                __hip_atomic_store(&st->wg_epoch[wg], epoch + (uint32_t)P, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (wg == 0 && ht == 0) __hip_atomic_fetch_add(&st->launches, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             break;
         }
         int U0, nwg;
         wg_range(C, wg, U0, nwg);
         const int nb = C->nb;
+        if (p == 0) {
+            // the first barrier: the epoch and the error word are in LDS now
+            __syncthreads();
+            epoch = s_ctl[0];
+            if (s_ctl[1] != 0) return;  // an earlier launch on this workspace gave up: its state is not trustworthy
+        }
+        const uint32_t prev_tag = epoch + (uint32_t)p;  // the tag of phase p - 1
 
-        // ---- the rows this phase multiplies with -> LDS, pair order
+        // ---- the rows this phase multiplies with -> LDS, pair order (helper threads)
         // staged batches: all of them (slot = batch) or the workgroup's own, starting at batch st_b0
         const int st_b0 = C->stage_full ? 0 : U0 - div_magic(U0, nb, C->nb_magic) * nb;
         const int st_n = C->stage_full ? nb : min(nwg, nb);
+        const PhasePtr Pv = A->ph + (p > 0 ? p - 1 : 0);
         if (C->in_kind == CHAIN_IN_ROWS || C->in_kind == CHAIN_IN_PREV) {
-            const PhasePtr Pv = A->ph + (p > 0 ? p - 1 : 0);
-            for (int m = 0; m < M; ++m) {
-                for (int i = tid; i < st_n * 16; i += T) {
-                    int b = st_b0 + (i >> 4);
-                    if (b >= nb) b -= nb;
-                    const int k0 = b * 128 + (i & 15) * 8;
-                    uint4 v;
-                    if (C->in_kind == CHAIN_IN_ROWS)
-                        v = *reinterpret_cast<const uint4 *>(C->x + (size_t)m * C->K + k0);
-                    else
-                        v = phase_output8(Pv, rs_part, M, m, k0);
-                    xs[m * xs_stride + i] = pair_order_u4(v);
+            if (helper) {
+                for (int m = 0; m < M; ++m) {
+                    for (int i = ht; i < st_n * 16; i += TH) {
+                        int b = st_b0 + (i >> 4);
+                        if (b >= nb) b -= nb;
+                        const int k0 = b * 128 + (i & 15) * 8;
+                        uint4 v;
+                        if (C->in_kind == CHAIN_IN_ROWS)
+                            v = *reinterpret_cast<const uint4 *>(C->x + (size_t)m * C->K + k0);
+                        else
+                            v = phase_output8(Pv, rs_part, M, m, k0, prev_tag, poll);
+                        xs[m * xs_stride + i] = pair_order_u4(v);
+                    }
                 }
             }
             __syncthreads();
         } else {
-            // residual add + RMSNorm of whole rows.  The sum of squares is taken by threads 0..255 over the chunks
-            // tid, tid + 256, ... and combined as the stand-alone kernel combines it: same bits.
-            const PhasePtr Pv = A->ph + (p > 0 ? p - 1 : 0);
+            // residual add + RMSNorm of whole rows.  The sum of squares is taken by the 256 helper threads over the
+            // chunks t, t + 256, ... and combined as the stand-alone kernel combines it: same bits.
             const int chunks = C->K >> 3;
-            const bool writer = (wg == p % G) && C->sum_out != nullptr;
-            const __amdgpu_buffer_rsrc_t rs_x = make_rsrc(C->x, (uint32_t)M * C->K * 2u);
-            const __amdgpu_buffer_rsrc_t rs_sum = make_rsrc(C->sum_out != nullptr ? C->sum_out : const_cast<half_t *>(C->x), (uint32_t)M * C->K * 2u);
-            for (int m = 0; m < M; ++m) {
-                for (int c = tid; c < chunks; c += T) {
-                    const uint32_t off = ((uint32_t)m * C->K + 8u * c) * 2u;
-                    uint4 v = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rs_x, off, 0, AUX_SC1));
-                    bool added = false;
-                    uint4 d = v;
-                    if (C->in_kind == CHAIN_IN_NORM_PREV) {
-                        d = phase_output8(Pv, rs_part, M, m, 8 * c);
-                        added = true;
-                    } else if (C->delta != nullptr) {
-                        d = *reinterpret_cast<const uint4 *>(C->delta + (size_t)m * C->K + 8 * c);
-                        added = true;
+            if (helper) {
+                const bool writer = (wg == p % G) && C->sum_out != nullptr;
+                for (int m = 0; m < M; ++m) {
+                    for (int c = ht; c < chunks; c += TH) {
+                        // the residual rows: from memory, or the sums an earlier phase of this launch left in LDS
+                        uint4 v = C->x_in_launch ? keep[m * chunks + c] : *reinterpret_cast<const uint4 *>(C->x + (size_t)m * C->K + 8 * c);
+                        bool added = false;
+                        uint4 d = v;
+                        if (C->in_kind == CHAIN_IN_NORM_PREV) {
+                            d = phase_output8(Pv, rs_part, M, m, 8 * c, prev_tag, poll);
+                            added = true;
+                        } else if (C->delta != nullptr) {
+                            d = *reinterpret_cast<const uint4 *>(C->delta + (size_t)m * C->K + 8 * c);
+                            added = true;
+                        }
+                        if (added) {
+                            float unused = 0.f;
+                            v = norm_take<true>(v, d, unused);
+                            if (writer) *reinterpret_cast<uint4 *>(C->sum_out + (size_t)m * C->K + 8 * c) = v;
+                        }
+                        if (C->keep_sums) keep[m * chunks + c] = v;
+                        xs[m * xs_stride + c] = v;
                     }
-                    if (added) {
-                        float unused = 0.f;
-                        v = norm_take<true>(v, d, unused);
-                        if (writer) __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, v), rs_sum, off, 0, AUX_SC1);
-                    }
-                    xs[m * xs_stride + c] = v;
                 }
             }
             __syncthreads();
-            if (tid < 256) {
+            if (helper) {
                 for (int m = 0; m < M; ++m) {
                     float ss = 0.f;
-                    for (int c = tid; c < chunks; c += 256) {
+                    for (int c = ht; c < chunks; c += TH) {
                         const uint4 v = xs[m * xs_stride + c];
                         norm_take<false>(v, v, ss);
                     }
                     ss = norm_wave_sum(ss);
-                    if (lane == 0) s_part[4 * m + wave] = ss;
+                    if (lane == 0) s_part[4 * m + hw] = ss;
                 }
             }
             __syncthreads();
-            for (int m = 0; m < M; ++m) {
-                const float inv = rsqrtf((s_part[4 * m] + s_part[4 * m + 1] + s_part[4 * m + 2] + s_part[4 * m + 3]) / (float)C->K + C->eps);
-                for (int c = tid; c < chunks; c += T) {
-                    const uint4 g = *reinterpret_cast<const uint4 *>(C->norm_w + 8 * c);
-                    xs[m * xs_stride + c] = pair_order_u4(norm_put(xs[m * xs_stride + c], g, inv));
+            if (helper) {
+                for (int m = 0; m < M; ++m) {
+                    const float inv = rsqrtf((s_part[4 * m] + s_part[4 * m + 1] + s_part[4 * m + 2] + s_part[4 * m + 3]) / (float)C->K + C->eps);
+                    for (int c = ht; c < chunks; c += TH) {
+                        const uint4 g = *reinterpret_cast<const uint4 *>(C->norm_w + 8 * c);
+                        xs[m * xs_stride + c] = pair_order_u4(norm_put(xs[m * xs_stride + c], g, inv));
+                    }
                 }
             }
             __syncthreads();
         }
+        if (s_ctl[2] != 0) return;  // a poll gave up (here or in another wave): every thread of the workgroup leaves
+        CHAIN_STAMP(5 + 7 * p);
 
-        // ---- this wave's units
-        int u0, n;
-        wave_range<NW>(C, wg, wave, u0, n);
+        // ---- the streaming waves' units
         const int T0 = div_magic(U0, nb, C->nb_magic);  // first tile of the workgroup
-        f4_t acc[2][2];
+        if (!helper) {
+            int u0, n;
+            wave_range<NS>(C, wg, wave, u0, n);
+            f4_t acc[2][2];
 #pragma unroll
-        for (int v = 0; v < 2; ++v)
+            for (int v = 0; v < 2; ++v)
 #pragma unroll
-            for (int t = 0; t < 2; ++t) acc[v][t] = (f4_t){0.f, 0.f, 0.f, 0.f};
-        int cur_tile = div_magic(u0, nb, C->nb_magic);
-        if (lane == 0) {
-            s_ft[wave] = n > 0 ? cur_tile : 0x7fffffff;
-            s_lt[wave] = n > 0 ? div_magic(u0 + n - 1, nb, C->nb_magic) : -1;
-        }
-        // accumulators of one tile -> this wave's slot of the reduction area (rows 0..3 live in lanes 0..15)
-        auto flush_tile = [&](int tile) {
-            float *dst = red + ((size_t)((tile - T0) * NW + wave) * M) * 64;
-            if (lane < 16) {
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    if (e < M) {
-#pragma unroll
-                        for (int v = 0; v < 2; ++v)
-#pragma unroll
-                            for (int t = 0; t < 2; ++t) dst[e * 64 + v * 32 + 2 * lcol + t] = acc[v][t][e];
-                    }
+                for (int t = 0; t < 2; ++t) acc[v][t] = (f4_t){0.f, 0.f, 0.f, 0.f};
+            int cur_tile = div_magic(u0, nb, C->nb_magic);
+            if (lane == 0) {
+                s_ft[wave] = n > 0 ? cur_tile : 0x7fffffff;
+                s_lt[wave] = n > 0 ? div_magic(u0 + n - 1, nb, C->nb_magic) : -1;
             }
-        };
-        const uint4 *xa = xs + min(lcol, M - 1) * xs_stride + lrow;
-        auto compute_unit = [&](const UnitRegs &U, int b) {
-            int slot = b - st_b0;
-            if (slot < 0) slot += nb;
-            const uint4 *ap = xa + slot * 16;
-            h8_t a[4];
+            // accumulators of one tile -> this wave's slot of the reduction area (rows 0..3 live in lanes 0..15)
+            auto flush_tile = [&](int tile) {
+                float *dst = red + ((size_t)((tile - T0) * NS + wave) * M) * 64;
+                if (lane < 16) {
 #pragma unroll
-            for (int k = 0; k < 4; ++k) a[k] = __builtin_bit_cast(h8_t, ap[4 * k]);
-            ColDecode cd[2][2];
+                    for (int e = 0; e < 4; ++e)
+                        if (e < M) {
 #pragma unroll
-            for (int v = 0; v < 2; ++v) {
-                const uint32_t zs = U.raw_z[v] >> (((2 * lcol) & 7) * 4);
+                            for (int v = 0; v < 2; ++v)
 #pragma unroll
-                for (int t = 0; t < 2; ++t) cd[v][t] = make_col_decode((zs >> (4 * t)) & 0xFu, U.raw_s[v] >> (16 * t));
-            }
-#pragma unroll
-            for (int k = 0; k < 4; ++k)
-#pragma unroll
-                for (int v = 0; v < 2; ++v)
-#pragma unroll
-                    for (int t = 0; t < 2; ++t)
-                        acc[v][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[k], decode_word_h8(t == 0 ? U.w[v][k].x : U.w[v][k].y, cd[v][t]), acc[v][t], 0, 0, 0);
-        };
-        const int n_pad = (n + DEPTH - 1) / DEPTH * DEPTH;
-        for (int i = 0; i < n_pad; i += DEPTH) {
-#pragma unroll
-            for (int d = 0; d < DEPTH; ++d) {
-                if (i + d < n) {
-                    const int u = u0 + i + d;
-                    const int tile = div_magic(u, nb, C->nb_magic);
-                    if (tile != cur_tile) {
-                        flush_tile(cur_tile);
-#pragma unroll
-                        for (int v = 0; v < 2; ++v)
-#pragma unroll
-                            for (int t = 0; t < 2; ++t) acc[v][t] = (f4_t){0.f, 0.f, 0.f, 0.f};
-                        cur_tile = tile;
-                    }
-                    compute_unit(ring[d], u - tile * nb);
+                                for (int t = 0; t < 2; ++t) dst[e * 64 + v * 32 + 2 * lcol + t] = acc[v][t][e];
+                        }
                 }
-                issue_load(ring[d]);
+            };
+            const uint4 *xa = xs + min(lcol, M - 1) * xs_stride + lrow;
+            auto compute_unit = [&](const UnitRegs &U, int b) {
+                int slot = b - st_b0;
+                if (slot < 0) slot += nb;
+                const uint4 *ap = xa + slot * 16;
+                h8_t a[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) a[k] = __builtin_bit_cast(h8_t, ap[4 * k]);
+                ColDecode cd[2][2];
+#pragma unroll
+                for (int v = 0; v < 2; ++v) {
+                    const uint32_t zs = U.raw_z[v] >> (((2 * lcol) & 7) * 4);
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) cd[v][t] = make_col_decode((zs >> (4 * t)) & 0xFu, U.raw_s[v] >> (16 * t));
+                }
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+#pragma unroll
+                    for (int v = 0; v < 2; ++v)
+#pragma unroll
+                        for (int t = 0; t < 2; ++t)
+                            acc[v][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[k], decode_word_h8(t == 0 ? U.w[v][k].x : U.w[v][k].y, cd[v][t]), acc[v][t], 0, 0, 0);
+            };
+            const int n_pad = (n + DEPTH - 1) / DEPTH * DEPTH;
+            for (int i = 0; i < n_pad; i += DEPTH) {
+#pragma unroll
+                for (int d = 0; d < DEPTH; ++d) {
+                    if (i + d < n) {
+                        const int u = u0 + i + d;
+                        const int tile = div_magic(u, nb, C->nb_magic);
+                        if (tile != cur_tile) {
+                            flush_tile(cur_tile);
+#pragma unroll
+                            for (int v = 0; v < 2; ++v)
+#pragma unroll
+                                for (int t = 0; t < 2; ++t) acc[v][t] = (f4_t){0.f, 0.f, 0.f, 0.f};
+                            cur_tile = tile;
+                        }
+                        compute_unit(ring[d], u - tile * nb);
+                    }
+                    issue_load(ring[d]);
+                }
             }
+            if (n > 0) flush_tile(cur_tile);
         }
-        if (n > 0) flush_tile(cur_tile);
+        CHAIN_STAMP(6 + 7 * p);
         __syncthreads();
+        CHAIN_STAMP(7 + 7 * p);
 
-        // ---- the workgroup's partial tiles -> its slots in the workspace, then the completion flag
-        if (nwg > 0) {
+        // ---- the workgroup's partial tiles -> its slots in the workspace, each value with the phase's tag (helper
+        //      threads; nothing waits for these stores)
+        if (helper && nwg > 0 && wg != A->skip_flag_wg) {
+            const uint32_t tag = epoch + (uint32_t)p + 1u;
             const int T1 = div_magic(U0 + nwg - 1, nb, C->nb_magic);
             const int per_tile = M * 64;
             const int total = (T1 - T0 + 1) * per_tile;
-            for (int e = tid; e < total; e += T) {
+            for (int e = ht; e < total; e += TH) {
                 const int tl = e / per_tile;
                 const int rem = e - tl * per_tile;
                 const int tile = T0 + tl;
                 float s = 0.f;
 #pragma unroll
-                for (int w = 0; w < NW; ++w)
-                    if (s_ft[w] <= tile && tile <= s_lt[w]) s += red[(size_t)(tl * NW + w) * per_tile + rem];
+                for (int w = 0; w < NS; ++w)
+                    if (s_ft[w] <= tile && tile <= s_lt[w]) s += red[(size_t)(tl * NS + w) * per_tile + rem];
                 const int rank = wg - wg_of_unit(C, tile * nb);
                 const uint32_t off = C->partial_off + ((uint32_t)tile * C->max_contrib + rank) * per_tile + rem;
-                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, s), rs_part, off * 4u, 0, AUX_SC1);
+                const u32x2_t val = {__builtin_bit_cast(uint32_t, s), tag};
+                __builtin_amdgcn_raw_buffer_store_b64(val, rs_part, off * 8u, 0, AUX_SC1);
             }
         }
-        // completion, not fences, orders the hand-over: the stores above (and this phase's sum_out) are acknowledged
-        // by the memory side before the flag is raised
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        if (tid == 0 && wg != A->skip_flag_wg)
-            __hip_atomic_store(&st->flags[wg], epoch + (uint32_t)p + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        CHAIN_STAMP(8 + 7 * p);
+        __syncthreads();  // the reduction area and s_ft / s_lt are free again
         if (C->out_kind != CHAIN_OUT_NONE) pending |= 1u << p;
     }
-
 }
 
 // ---------------------------------------------------------------------------------------------- host side
 struct ChainTuning {
-    int waves;   // waves per workgroup: 8 or 16 (0 = automatic)
-    int depth;   // units of loads in flight per wave: 1..3 (0 = automatic)
+    int waves;   // streaming waves per workgroup: 8 or 12 (0 = automatic)
+    int depth;   // units of loads in flight per streaming wave: 1..4 (0 = automatic)
     uint32_t spin_limit;
     int skip_flag_wg;
 };
@@ -618,10 +669,10 @@ int launch_variant(const ChainArgs &a, int grid, size_t lds, hipStream_t stream)
     }
     // the grid must be resident as a whole (workgroups wait for each other): one workgroup per CU
     int per_cu = 0;
-    hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gptq4_chain_kernel<NW, DEPTH>, 64 * NW, lds);
+    hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gptq4_chain_kernel<NW, DEPTH>, 64 * (NW + CHAIN_NH), lds);
     if (e != hipSuccess) return (int)e;
     if (per_cu < 1) return (int)hipErrorLaunchOutOfResources;
-    hipLaunchKernelGGL((gptq4_chain_kernel<NW, DEPTH>), dim3((unsigned)grid), dim3(64 * NW), lds, stream, a);
+    hipLaunchKernelGGL((gptq4_chain_kernel<NW, DEPTH>), dim3((unsigned)grid), dim3(64 * (NW + CHAIN_NH)), lds, stream, a);
     return (int)hipGetLastError();
 }
 
@@ -651,15 +702,15 @@ ChainPlan plan_chain(const gptq4_phase_t *phases, int nphases, int M, int grid) 
     if (grid <= 0) grid = 256;
     if (grid > CHAIN_MAX_GRID) grid = CHAIN_MAX_GRID;
     pl.grid = grid;
-    pl.waves = (g_chain_tuning.waves == 8 || g_chain_tuning.waves == 16) ? g_chain_tuning.waves : 8;
-    pl.depth = (g_chain_tuning.depth >= 1 && g_chain_tuning.depth <= 3) ? g_chain_tuning.depth : 2;
+    pl.waves = (g_chain_tuning.waves == 8 || g_chain_tuning.waves == 12) ? g_chain_tuning.waves : 8;
+    pl.depth = (g_chain_tuning.depth >= 1 && g_chain_tuning.depth <= 4) ? g_chain_tuning.depth : 3;
     ChainArgs &a = pl.a;
     a.nphases = nphases;
     a.M = M;
     a.spin_limit = g_chain_tuning.spin_limit ? g_chain_tuning.spin_limit : (4u << 20);
     a.skip_flag_wg = g_chain_tuning.skip_flag_wg;
-    size_t partial_floats = 0;
-    int stage_chunks = 16, red_tiles = 1;
+    size_t partial_elems = 0;
+    int stage_chunks = 16, red_tiles = 1, keep_chunks = 0;
     for (int p = 0; p < nphases; ++p) {
         const gptq4_phase_t &ph = phases[p];
         ChainPhase &c = a.ph[p];
@@ -728,9 +779,20 @@ ChainPlan plan_chain(const gptq4_phase_t *phases, int nphases, int M, int grid) 
             }
             if (K > 8192 || !(ph.eps >= 0.f)) return pl;
             if (ph.sum_out != nullptr && (ph.sum_out == ph.x || ph.sum_out == ph.delta)) return pl;  // other workgroups still read them
-            // the residual rows may be the sums an earlier phase of this launch wrote
-            for (int e = 0; e < p; ++e)
-                if (phases[e].sum_out != nullptr && phases[e].sum_out == ph.x) c.x_in_launch = 1;
+            // the residual rows may be the sums an earlier phase of this launch wrote: only the latest such sums are
+            // at hand (every workgroup keeps them in LDS; the copy in memory is not complete before the launch ends)
+            int last_norm = -1;
+            for (int e = 0; e < p; ++e) {
+                const bool e_norm = phases[e].input == GPTQ4_IN_NORM_ROWS || phases[e].input == GPTQ4_IN_NORM_PREV;
+                if (e_norm) last_norm = e;
+            }
+            for (int e = 0; e < p; ++e) {
+                if (phases[e].sum_out == nullptr || phases[e].sum_out != ph.x) continue;
+                if (e != last_norm || phases[e].K != K) return pl;
+                c.x_in_launch = 1;
+                a.ph[e].keep_sums = 1;
+                if (K / 8 > keep_chunks) keep_chunks = K / 8;
+            }
         }
         c.stage_full = norm ? 1 : 0;
         const int per_wg = c.q + (c.r ? 1 : 0);
@@ -763,18 +825,19 @@ ChainPlan plan_chain(const gptq4_phase_t *phases, int nphases, int M, int grid) 
             return pl;  // a phase nobody reads and that leaves nothing in memory
         }
         if (ph.bias != nullptr && pair) return pl;
-        c.partial_off = (uint32_t)partial_floats;
-        partial_floats += (size_t)c.tiles * c.max_contrib * M * 64;
-        if (partial_floats * 4 >= (1ull << 31)) return pl;
+        c.partial_off = (uint32_t)partial_elems;
+        partial_elems += (size_t)c.tiles * c.max_contrib * M * 64;
+        if (partial_elems * 8 >= (1ull << 31)) return pl;
     }
-    pl.partial_bytes = partial_floats * 4;
+    pl.partial_bytes = partial_elems * 8;  // {fp32 bits, tag} per value
     a.partial_bytes = (uint32_t)pl.partial_bytes;
-    // LDS: [M rows of staged activations][reduction area]; rows 64 bytes apart modulo 128 so that two rows'
+    // LDS: [M rows of staged activations][kept residual sums][reduction area]; rows 64 bytes apart modulo 128 so that two rows'
     // A-operand reads fall into different banks
     int stride = stage_chunks;
     if ((stride & 7) != 4) stride += (4 - (stride & 7) + 8) & 7;
     a.xs_stride = stride;
-    a.red_off = M * stride;
+    a.keep_off = M * stride;
+    a.red_off = a.keep_off + M * keep_chunks;
     a.red_tiles = red_tiles;
     const size_t red_bytes = (size_t)red_tiles * pl.waves * M * 64 * sizeof(float);
     pl.lds_bytes = (size_t)a.red_off * 16 + red_bytes;
@@ -790,8 +853,8 @@ ChainPlan plan_chain(const gptq4_phase_t *phases, int nphases, int M, int grid) 
 extern "C" {
 
 void gptq4_set_chain_tuning(int waves, int depth, unsigned spin_limit, int skip_flag_wg) {
-    g_chain_tuning.waves = (waves == 8 || waves == 16) ? waves : 0;
-    g_chain_tuning.depth = (depth >= 1 && depth <= 3) ? depth : 0;
+    g_chain_tuning.waves = (waves == 8 || waves == 12) ? waves : 0;
+    g_chain_tuning.depth = (depth >= 1 && depth <= 4) ? depth : 0;
     g_chain_tuning.spin_limit = spin_limit;
     g_chain_tuning.skip_flag_wg = skip_flag_wg;
 }
@@ -801,7 +864,11 @@ size_t gptq4_chain_workspace_bytes(const gptq4_phase_t *phases, int nphases, int
     const int grid = device_info(&di) == 0 ? di.cus : 0;
     const ChainPlan pl = plan_chain(phases, nphases, M, grid);
     if (pl.rc != 0) return 0;
+#ifdef GPTQ4_CHAIN_TIMERS
+    return (size_t)CHAIN_STATE_BYTES + pl.partial_bytes + (1u << 20);
+#else
     return (size_t)CHAIN_STATE_BYTES + pl.partial_bytes;
+#endif
 }
 
 int gptq4_decode_chain(const gptq4_phase_t *phases, int nphases, int M, void *workspace, size_t workspace_bytes, void *stream) {
@@ -828,10 +895,11 @@ int gptq4_decode_chain(const gptq4_phase_t *phases, int nphases, int M, void *wo
     const int key = pl.waves * 10 + pl.depth;
     switch (key) {
         case 81: return launch_variant<8, 1>(pl.a, pl.grid, pl.lds_bytes, s);
-        case 83: return launch_variant<8, 3>(pl.a, pl.grid, pl.lds_bytes, s);
-        case 161: return launch_variant<16, 1>(pl.a, pl.grid, pl.lds_bytes, s);
-        case 162: return launch_variant<16, 2>(pl.a, pl.grid, pl.lds_bytes, s);
-        default: return launch_variant<8, 2>(pl.a, pl.grid, pl.lds_bytes, s);
+        case 82: return launch_variant<8, 2>(pl.a, pl.grid, pl.lds_bytes, s);
+        case 84: return launch_variant<8, 4>(pl.a, pl.grid, pl.lds_bytes, s);
+        case 122: return launch_variant<12, 2>(pl.a, pl.grid, pl.lds_bytes, s);
+        case 123: return launch_variant<12, 3>(pl.a, pl.grid, pl.lds_bytes, s);
+        default: return launch_variant<8, 3>(pl.a, pl.grid, pl.lds_bytes, s);
     }
 }
 

@@ -273,8 +273,8 @@ typedef struct gptq4_phase {
 size_t gptq4_chain_workspace_bytes(const gptq4_phase_t *phases, int nphases, int M);
 int gptq4_decode_chain(const gptq4_phase_t *phases, int nphases, int M, void *workspace,
                        size_t workspace_bytes, void *stream);
-/* Measurement and test knobs of the chained launch: waves per workgroup (8, 16), units of loads in flight per
- * wave (1..3), polls before a wait gives up (0 = default, about seconds), and a workgroup that never reports
+/* Measurement and test knobs of the chained launch: streaming waves per workgroup (8, 12), units of loads in
+ * flight per streaming wave (1..4), polls before a wait gives up (0 = default, about seconds), and a workgroup that never reports
  * completion (-1 = none; lets a test see the bounded waits give up with every kernel exiting normally). */
 void gptq4_set_chain_tuning(int waves, int depth, unsigned spin_limit, int skip_flag_wg);
 
