@@ -67,8 +67,11 @@ DECODERS = {
 }
 
 
-def run_decoder(args):
-    """Full-decoder workload: prefill + graph-replayed greedy decode on a random-init model."""
+def decoder_figures(workload, bsz, prompt, new):
+    """Full-decoder workload: prefill + graph-replayed greedy decode on a random-init model.  Returns the result
+    record (the JSON line of `--workload llamaNNb`)."""
+    import gc
+
     import torch
 
     torch.set_grad_enabled(False)
@@ -82,15 +85,14 @@ def run_decoder(args):
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    layers, hidden, inter, heads, groupsize, act_order = DECODERS[args.workload]
-    bsz, prompt, new = args.batch, args.prompt, args.new_tokens
+    layers, hidden, inter, heads, groupsize, act_order = DECODERS[workload]
     cfg = LlamaConfigLite()
     cfg.hidden_size, cfg.intermediate_size, cfg.num_attention_heads, cfg.num_hidden_layers = hidden, inter, heads, layers
     cfg.vocab_size, cfg.max_position_embeddings = 32000, max(2048, prompt + new)
     gen = torch.Generator(device=dev)
     gen.manual_seed(1234)
 
-    log(f"building a random-init {args.workload} decoder ({layers} layers, groupsize {groupsize}, act-order {act_order}) ...")
+    log(f"building a random-init {workload} decoder ({layers} layers, groupsize {groupsize}, act-order {act_order}) ...")
     dtype0 = torch.get_default_dtype()
     torch.set_default_dtype(torch.half)
     try:
@@ -161,10 +163,10 @@ def run_decoder(args):
     log(f"decode: {step_s * 1e3:.3f} ms/step graph-replayed ({bsz / step_s:.1f} tok/s), {eager_s * 1e3:.3f} ms/step eager; "
         f"{step_bytes / 1e9:.2f} GB per step -> {gbs:.0f} GB/s")
     result = {
-        "metric": f"{args.workload}-shape 4-bit greedy decode tok/s (full decoder)", "value": round(bsz / step_s, 2),
+        "metric": f"{workload}-shape 4-bit greedy decode tok/s (full decoder)", "value": round(bsz / step_s, 2),
         "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": eager_steps + 2, "ms_per_step": round(step_s * 1e3, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp16", "data": "synthetic",
-        "config": {"workload": f"random-init {args.workload}-shape decoder, batch {bsz}, {prompt}-token prompt prefill then "
+        "config": {"workload": f"random-init {workload}-shape decoder, batch {bsz}, {prompt}-token prompt prefill then "
                                f"{new} greedy tokens, 4-bit groupsize {groupsize}{' act-order' if act_order else ''}, "
                                "fp16 lm_head, one HIP-graph replay per token",
                    "layers": layers, "hidden": hidden, "intermediate": inter, "heads": heads, "batch": bsz,
@@ -178,7 +180,14 @@ def run_decoder(args):
                   "prefill_frac_of_fp16_mfma_peak": round(prefill_tf / MFMA_FP16_PEAK_TFLOPS, 4),
                   "eager_decode_ms_per_step": round(eager_s * 1e3, 3), "last_tokens": toks[0, -4:].tolist()},
     }
-    print(json.dumps(result), flush=True)
+    del dec, model, toks, ids
+    gc.collect()
+    torch.cuda.empty_cache()
+    return result
+
+
+def run_decoder(args):
+    print(json.dumps(decoder_figures(args.workload, args.batch, args.prompt, args.new_tokens)), flush=True)
 
 
 def main():
@@ -188,6 +197,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the per-operator / prefill extras")
+    ap.add_argument("--no-decoders", action="store_true", help="skip the full-decoder workloads (C4 / C5) in the extras")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="for rocprofv3 --pmc runs: a 256 MiB device copy (calibration) followed by plain launches of "
                          "each decode operator on distinct weights; prints no JSON")
@@ -218,8 +228,8 @@ def main():
     gen = torch.Generator(device=dev)
     gen.manual_seed(1234)
 
-    def make(k, n):
-        groups = k // GROUPSIZE
+    def make(k, n, g=GROUPSIZE):
+        groups = 1 if g == -1 else k // g
         qw = torch.randint(-2**31, 2**31 - 1, (k // 8, n), dtype=torch.int32, device=dev, generator=gen)
         qz = torch.randint(-2**31, 2**31 - 1, (groups, n // 8), dtype=torch.int32, device=dev, generator=gen)
         sc = (0.002 + 0.018 * torch.rand((groups, n), device=dev, generator=gen)).half()
@@ -340,6 +350,9 @@ def main():
                 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
                 # `bench.py --traffic-probe`, scaled by a 256 MiB copy (x2.000 / x1.000)
                 "traffic": 50_601_000 + 1_286_000,
+                "traffic_source": "constant: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this kernel, profiles/decode_gemv_llama7b_m1.md",
+                "step_frac": round(LAYERS * layer_bytes / ms_per_step / 1e6 / HBM_PEAK_GBS, 4),
+                "step_GBps": round(LAYERS * layer_bytes / ms_per_step / 1e6, 1),
                 "kernel": "gptq4_gemv_kernel<SILU_MUL> (gate/up GEMV, M=1, K=4096, I=11008, g=128)",
                 "bytes_per_launch": gu_bytes, "avg_launch_us": round(gu_us, 2)}
     log(f"gate/up GEMV: {gu_us:.2f} us/launch, {gu_gbs:.0f} GB/s = {100 * gu_gbs / HBM_PEAK_GBS:.1f}% of HBM peak")
@@ -387,6 +400,49 @@ def main():
                    2 * m * HIDDEN * INTER, nsets=ns, reps=5)
             per_op(f"M={m} o_proj (4096x4096)", lambda L: o_op(xm, L), wo + 4 * m * HIDDEN, 2 * m * HIDDEN * HIDDEN,
                    nsets=ns, reps=5)
+        # ---- the BASELINE.json configurations exactly as stated, each with its own roofline fraction
+        rows = []
+
+        def config_row(cfg, op, m, fn, sets, nbytes, flops, reps=10):
+            g, _ = capture(lambda: [fn(w) for w in sets])
+            us = statistics.median(time_graph(g, reps)) * 1e3 / len(sets)
+            del g
+            gbs, tf = nbytes / us / 1e3, flops / us / 1e6
+            hbm, mfma = gbs / HBM_PEAK_GBS, tf / MFMA_FP16_PEAK_TFLOPS
+            # what binds: memory up to 16 rows, the matrix cores beyond (ridge: 312 flop per byte)
+            bound = "hbm" if flops / nbytes < MFMA_FP16_PEAK_TFLOPS * 1e3 / HBM_PEAK_GBS else "mfma"
+            rows.append({"config": cfg, "op": op, "M": m, "us": round(us, 2), "bytes": nbytes, "flops": flops, "GBps": round(gbs, 1),
+                         "TFLOPs": round(tf, 2), "bound": bound, "frac": round(hbm if bound == "hbm" else mfma, 4),
+                         "frac_hbm": round(hbm, 4), "frac_mfma": round(mfma, 4)})
+            log(f"  {cfg} {op:28s} M={m:<5d} {us:9.2f} us  {gbs:8.0f} GB/s  {tf:8.1f} TFLOP/s  {bound} {rows[-1]['frac']:.3f}")
+
+        # C1: one QuantLinear 4096 -> 4096, one group (groupsize -1), M in {1, 128}; 40 weight sets = 336 MB
+        c1 = [make(HIDDEN, HIDDEN, -1) for _ in range(40)]
+        w1 = weight_bytes(HIDDEN, HIDDEN, HIDDEN)
+        for m in (1, 128):
+            xm = torch.randn((m, HIDDEN), device=dev, generator=gen).half()
+            config_row("C1", "QuantLinear 4096x4096 g=-1", m, lambda w: G.matmul4(HIDDEN, xm, w[0], w[2], w[1]), c1,
+                       w1 + 4 * m * HIDDEN, 2 * m * HIDDEN * HIDDEN)
+        del c1
+        # C2: the fused MLP module, gate/up + SiLU*mul then down, groupsize 128, M in {1, 16, 512}
+        for m in (1, 16, 512):
+            xm = torch.randn((m, HIDDEN), device=dev, generator=gen).half()
+            config_row("C2", "MLP gate/up+silu*mul, down g=128", m, lambda L: down_op(gateup_op(xm, L), L), layers,
+                       2 * wg + wd + 4 * m * HIDDEN + 4 * m * INTER, 6 * m * HIDDEN * INTER, reps=5)
+        # C3: fused QKV + rotary 4096 -> 12288, one group, M = 1 at position 2047 and a 2048-token prefill
+        c3 = [make(HIDDEN, 3 * HIDDEN, -1) for _ in range(12)]
+        w3 = weight_bytes(HIDDEN, 3 * HIDDEN, HIDDEN)
+        pos2047 = torch.tensor([[2047]], device=dev, dtype=torch.int32)
+        x1r = torch.randn((1, 1, HIDDEN), device=dev, generator=gen).half()
+        config_row("C3", "QKV+rotary 4096x12288 g=-1", 1, lambda w: G.qkv_rotary(HIDDEN, x1r, w[0], w[2], w[1], pos2047, cos, sin, HEADS), c3,
+                   w3 + 2 * HIDDEN + 6 * HIDDEN, 2 * HIDDEN * 3 * HIDDEN)
+        xp = torch.randn((1, 2048, HIDDEN), device=dev, generator=gen).half()
+        posp = torch.arange(2048, device=dev, dtype=torch.int32).unsqueeze(0)
+        config_row("C3", "QKV+rotary 4096x12288 g=-1", 2048, lambda w: G.qkv_rotary(HIDDEN, xp, w[0], w[2], w[1], posp, cos, sin, HEADS), c3[:4],
+                   w3 + 2 * 2048 * HIDDEN + 6 * 2048 * HIDDEN, 2 * 2048 * HIDDEN * 3 * HIDDEN, reps=5)
+        del c3, xp
+        extra["baseline_configs"] = rows
+
         # Yardstick: the vendor library's DENSE fp16 GEMM (torch.matmul) on the same M = 2048
         # shapes, weights already dequantised.  It does no 4-bit decode and reads 4x the
         # weight bytes; it shows what fraction of the nominal MFMA peak a tuned kernel
@@ -414,32 +470,76 @@ def main():
         extra["prefill_best_TFLOPs"] = best_prefill
         extra["prefill_frac_of_fp16_mfma_peak"] = round(best_prefill / MFMA_FP16_PEAK_TFLOPS, 4)
 
+    L0 = None if args.no_cpu else {k: tuple(t.cpu() for t in v) for k, v in layers[0].items()}
+    # ------------------------------------------------- C4 / C5: the full decoders (prefill + greedy decode)
+    if not args.no_extra and not args.no_decoders:
+        del layers, step_graph, gu_graph
+        import gc
+        gc.collect()
+        torch.cuda.empty_cache()
+        decs = {}
+        for name, bsz in (("llama7b", 1), ("llama13b", 1), ("llama30b", 1), ("llama30b", 8)):
+            try:
+                r = decoder_figures(name, bsz, 2048, 128 if name != "llama30b" else 256)
+            except Exception as e:  # report, do not lose the line
+                decs[f"{name}_b{bsz}"] = {"error": repr(e)}
+                continue
+            decs[f"{name}_b{bsz}"] = {"tok_s": r["value"], "ms_per_step": r["ms_per_step"], "prefill_ms": r["extra"]["prefill_ms"],
+                                      "prefill_linear_TFLOPs": r["extra"]["prefill_linear_TFLOPs"],
+                                      "step_GBps": r["roofline"]["achieved"], "step_frac_hbm": r["roofline"]["frac"],
+                                      "workload": r["config"]["workload"]}
+        extra["decoders"] = decs
+
     # --------------------------------------------------------------------- CPU baseline
     cpu_baseline = None
     if not args.no_cpu:
         from oracle import torch_cpu as T
-        L0 = {k: tuple(t.cpu() for t in v) for k, v in layers[0].items()}
         xc = x1.cpu().view(1, HIDDEN)
         torch.set_grad_enabled(False)
+        REPS = 5
 
+        def median_s(fn):
+            fn()
+            ts = []
+            for _ in range(REPS):
+                t0 = time.perf_counter()
+                fn()
+                ts.append(time.perf_counter() - t0)
+            return statistics.median(ts)
+
+        # (a) what the reference-style path costs per call: dequantise, then a float32 matmul
         def cpu_layer():
             T.quant_matmul(xc, *L0["qkv"], GROUPSIZE)
             T.quant_matmul(xc, *L0["o"], GROUPSIZE)
             T.mlp(xc, L0["gate"], L0["up"], L0["down"], GROUPSIZE)
 
-        cpu_layer()
-        ts = []
-        for _ in range(3):
-            t0 = time.perf_counter()
-            cpu_layer()
-            ts.append(time.perf_counter() - t0)
-        t_layer = statistics.median(ts)
+        t_layer = median_s(cpu_layer)
+        # (b) the matmuls alone, on weights dequantised beforehand
+        W = {k: T.dequant_fp16(*v, GROUPSIZE).float() for k, v in L0.items()}
+        xf = xc.float()
+
+        def cpu_layer_matmul_only():
+            xf @ W["qkv"]
+            xf @ W["o"]
+            h = (torch.nn.functional.silu(xf @ W["gate"]) * (xf @ W["up"])).half().float()
+            h @ W["down"]
+
+        t_mm = median_s(cpu_layer_matmul_only)
+        # C1 as stated: one 4096 x 4096 layer, M = 1 and 128 (the o_proj tensors have that shape)
+        c1 = {}
+        for m in (1, 128):
+            xm = torch.randn((m, HIDDEN)).half()
+            c1[f"M={m}"] = {"dequant+matmul_ms": round(median_s(lambda: T.quant_matmul(xm, *L0["o"], GROUPSIZE)) * 1e3, 2),
+                            "matmul_only_ms": round(median_s(lambda: xm.float() @ W["o"]) * 1e3, 3)}
+        del W
         cpu_baseline = {"value": round(1.0 / (t_layer * LAYERS), 4), "unit": "tok/s", "cores": torch.get_num_threads(),
                         "kind": "port",
                         "sample": f"1 of {LAYERS} layers (qkv, o_proj, gate/up+silu*mul, down at M=1; dequantise + fp32 "
-                                  f"matmul per call), median of 3 runs = {t_layer:.3f} s, extrapolated x{LAYERS}; "
-                                  f"host has {os.cpu_count()} logical CPUs"}
-        log(f"cpu baseline: {t_layer:.3f} s per layer on {torch.get_num_threads()} threads")
+                                  f"matmul per call), median of {REPS} runs = {t_layer:.3f} s, extrapolated x{LAYERS}; "
+                                  f"torch threads {torch.get_num_threads()}, host has {os.cpu_count()} logical CPUs",
+                        "matmul_only_value": round(1.0 / (t_mm * LAYERS), 3), "matmul_only_layer_s": round(t_mm, 4),
+                        "quantlinear_4096x4096": c1}
+        log(f"cpu baseline: {t_layer:.3f} s per layer dequantise + matmul, {t_mm:.4f} s matmul alone, on {torch.get_num_threads()} threads")
 
     result = {
         "metric": "LLaMA-7B-shape 4-bit decode tok/s", "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1,

@@ -33,7 +33,7 @@ struct ChainPhase {
     int keep_sums;           // IN_NORM_*: a later phase reads this phase's sums as its x: keep them in LDS
     int K, N;                // N: columns of one matrix
     int nb;                  // K / 128
-    int tiles;               // plain: N / 64; pair: N / 32 (32 of gate + the same 32 of up); rotary: N / 64 (32 of d + 32 of d + 64)
+    int tiles;               // plain: N / 128; pair: N / 64 (64 columns of gate + the same 64 of up); rotary: N / 128 (one head: d and d + 64)
     int bpg, groups;         // batches per group, groups
     uint32_t group_magic, nb_magic;
     // units (tile, batch) dealt to workgroups: q each, the first r one more
@@ -42,6 +42,8 @@ struct ChainPhase {
     int max_contrib;         // workgroups that can share one tile
     int stage_full;          // 1: the whole row is staged in LDS (slot = batch), 0: only the workgroup's batches
     uint32_t partial_off;    // this phase's partial sums: element offset ({fp32 bits, tag} pairs) into the partial region
+    uint32_t final_off;      // its finished values for the next phase: element offset ({2 fp16, tag}), M * N / 2 elements
+    int feeds_next;          // the next phase reads this one's output
 };
 
 // Persistent state in the chain workspace (zero before the first launch; launches maintain it).
@@ -63,6 +65,8 @@ struct ChainArgs {
     int xs_stride;     // 16-byte chunks per staged row (LDS)
     int keep_off;      // LDS offset (chunks) of the residual sums kept for a later phase
     int red_off;       // LDS offset (chunks) of the reduction area
+    int ring_off;      // LDS offset (chunks) of the streaming waves' unit ring
+    int ring_slots;    // units per streaming wave in that ring (>= 2)
     int red_tiles;     // tiles a workgroup can touch in one phase
     uint32_t spin_limit;  // polls of a partial tile before a thread gives up
     int skip_flag_wg;     // test hook: this workgroup never stores its partial sums (-1: none)

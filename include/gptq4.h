@@ -273,10 +273,10 @@ typedef struct gptq4_phase {
 size_t gptq4_chain_workspace_bytes(const gptq4_phase_t *phases, int nphases, int M);
 int gptq4_decode_chain(const gptq4_phase_t *phases, int nphases, int M, void *workspace,
                        size_t workspace_bytes, void *stream);
-/* Measurement and test knobs of the chained launch: streaming waves per workgroup (8, 12), units of loads in
- * flight per streaming wave (1..4), polls before a wait gives up (0 = default, about seconds), and a workgroup that never reports
- * completion (-1 = none; lets a test see the bounded waits give up with every kernel exiting normally). */
-void gptq4_set_chain_tuning(int waves, int depth, unsigned spin_limit, int skip_flag_wg);
+/* Measurement and test knobs of the chained launch: units of LDS ring per streaming wave (2..4, 0 = as many as
+ * fit), a reserved value, polls before a wait gives up (0 = default, about seconds), and a workgroup that never
+ * stores its partial sums (-1 = none; lets a test see the bounded waits give up with every kernel exiting normally). */
+void gptq4_set_chain_tuning(int ring_slots, int reserved, unsigned spin_limit, int skip_flag_wg);
 
 /* Host-side launch tuning of the small-M kernels, for measurements: words per lane and
  * load (1, 2 or 4: strips of 16, 32 or 64 columns), batches of loads in flight per
