@@ -190,6 +190,112 @@ def run_decoder(args):
     print(json.dumps(decoder_figures(args.workload, args.batch, args.prompt, args.new_tokens)), flush=True)
 
 
+def chain_probe(args):
+    """Chained decode launch (gptq4_decode_chain) against the separate launches on LLaMA-7B shapes, us per layer
+    under graph replay; with a timing build of the library (python gptq-triton_amd/build.py -DGPTQ4_CHAIN_TIMERS)
+    also the in-kernel timeline of one o_proj -> add+RMSNorm -> gate/up -> down_proj launch.  Prints text, no JSON."""
+    import numpy as np
+    import torch
+
+    import gptq_triton_amd as G
+    from gptq_triton_amd import _lib
+    from gptq_triton_amd import chain as C
+    from gptq_triton_amd.decoder_ops import add_rms_norm
+
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(1)
+    m, gs = args.batch, GROUPSIZE
+
+    def make(k, n):
+        g = k // gs
+        return (torch.randint(-2**31, 2**31 - 1, (k // 8, n), dtype=torch.int32, device=dev, generator=gen),
+                torch.randint(-2**31, 2**31 - 1, (g, n // 8), dtype=torch.int32, device=dev, generator=gen),
+                ((0.002 + 0.018 * torch.rand((g, n), device=dev, generator=gen)) * (6.0 / k ** 0.5)).half())
+
+    layers = [dict(qkv=make(HIDDEN, 3 * HIDDEN), o=make(HIDDEN, HIDDEN), gate=make(HIDDEN, INTER), up=make(HIDDEN, INTER),
+                   down=make(INTER, HIDDEN)) for _ in range(LAYERS)]
+    cos, sin = G.RotaryTable(128, 2048).get(dev, 2048)
+    x = torch.randn((m, HIDDEN), device=dev, generator=gen).half()
+    h = torch.randn((m, HIDDEN), device=dev, generator=gen).half()
+    w = torch.ones(HIDDEN, device=dev).half()
+    pos = torch.full((m,), 2047, dtype=torch.int32, device=dev)
+    q = torch.empty((m, HEADS, 1, 128), device=dev).half()
+    kk, vv = torch.empty_like(q), torch.empty_like(q)
+    s, y = torch.empty((m, HIDDEN), device=dev).half(), torch.empty((m, HIDDEN), device=dev).half()
+
+    def graph_us(fn, reps=20):
+        st = torch.cuda.Stream()
+        st.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(st):
+            fn()
+        torch.cuda.current_stream().wait_stream(st)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=st):
+            fn()
+        for _ in range(3):
+            g.replay()
+        torch.cuda.synchronize()
+        ts = []
+        for _ in range(reps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            g.replay()
+            e1.record()
+            e1.synchronize()
+            ts.append(e0.elapsed_time(e1))
+        return statistics.median(ts) * 1e3 / LAYERS
+
+    p_o = lambda L: C.projection(*L["o"], gs, x=x)
+    p_gu = lambda L: C.projection(*L["gate"], gs, up=L["up"], input=C.IN_NORM_PREV, x=h, norm_weight=w, eps=1e-6, sum_out=s)
+    p_dn = lambda L: C.projection(*L["down"], gs, input=C.IN_PREV, output=C.OUT_ROWS, y=y)
+    rope = dict(position_ids=pos, cos=cos, sin=sin, q=q, k=kk, v=vv, heads=HEADS)
+    p_qkv = lambda L: C.projection(*L["qkv"], gs, x=x, output=C.OUT_ROPE, rope=rope)
+
+    def separate(with_qkv):
+        def run():
+            for L in layers:
+                if with_qkv:
+                    G.qkv_rotary(gs, x.view(m, 1, HIDDEN), L["qkv"][0], L["qkv"][2], L["qkv"][1], pos.view(m, 1), cos, sin, HEADS)
+                o = G.matmul4(gs, x, L["o"][0], L["o"][2], L["o"][1])
+                _, xn = add_rms_norm(h, o, w, 1e-6)
+                a = G.llama_mlp_4(gs, xn, L["gate"][0], L["gate"][2], L["gate"][1], L["up"][0], L["up"][2], L["up"][1])
+                G.matmul4(gs, a, L["down"][0], L["down"][2], L["down"][1])
+        return run
+
+    def chained(phases_of):
+        def run():
+            for L in layers:
+                C.decode_chain(phases_of(L), m, dev)
+        return run
+
+    print(f"LLaMA-7B shapes, M = {m}, groupsize {gs}, {LAYERS} layers of distinct weights, us per layer (graph replay)")
+    print(f"  separate launches, with QKV + rotary (5 launches)     {graph_us(separate(True)):7.2f}")
+    print(f"  separate launches, o_proj .. down_proj (4 launches)   {graph_us(separate(False)):7.2f}")
+    print(f"  chain o_proj -> norm -> gate/up -> down (1 launch)    {graph_us(chained(lambda L: [p_o(L), p_gu(L), p_dn(L)])):7.2f}")
+    print(f"  chain with QKV + rotary in front (1 launch)           {graph_us(chained(lambda L: [p_qkv(L), p_o(L), p_gu(L), p_dn(L)])):7.2f}")
+    if not args.chain_timeline:
+        return
+    # the in-kernel timeline: needs the library built with the stamps (its workspace is then 1 MiB larger)
+    ph = [p_o(layers[0]), p_gu(layers[0]), p_dn(layers[0])]
+    arr = (_lib.Phase * 3)(*ph)
+    need = lib.gptq4_chain_workspace_bytes(arr, 3, m)
+    ws = torch.zeros(need, dtype=torch.uint8, device=dev)
+    for L in layers[:4]:
+        C.decode_chain([p_o(L), p_gu(L), p_dn(L)], m, dev, ws=ws)
+    torch.cuda.synchronize()
+    stamps = ws[need - (1 << 20):need - (1 << 20) + 256 * 64 * 8].view(torch.int64).cpu().numpy().reshape(256, 64).astype(np.float64) / 100.0
+    t0 = stamps[:, 0].min()
+    print("  timeline of one chained launch, us from the first stamp: min / median / max over the workgroups")
+    for p, name in enumerate(("o_proj", "gate/up", "down_proj")):
+        for j, what in ((3, "rows staged in LDS"), (5, "all streaming waves through"), (6, "partial tiles stored"), (1, "slice of finished values stored")):
+            col = stamps[:, 2 + 7 * p + j] - t0
+            print(f"    {name:10s} {what:34s} {col.min():7.2f} {np.median(col):7.2f} {col.max():7.2f}")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -201,6 +307,10 @@ def main():
     ap.add_argument("--traffic-probe", action="store_true",
                     help="for rocprofv3 --pmc runs: a 256 MiB device copy (calibration) followed by plain launches of "
                          "each decode operator on distinct weights; prints no JSON")
+    ap.add_argument("--chain-probe", action="store_true",
+                    help="time gptq4_decode_chain against the separate launches (7B shapes, --batch rows); prints text, no JSON")
+    ap.add_argument("--chain-timeline", action="store_true",
+                    help="with --chain-probe: also print the in-kernel timeline (needs the library built with -DGPTQ4_CHAIN_TIMERS)")
     ap.add_argument("--workload", default="linears7b", choices=["linears7b"] + sorted(DECODERS),
                     help="linears7b (default): the quantised-linear hot path of one 7B decode token; llamaNNb: a full "
                          "random-init decoder of that shape, prefill + greedy decode")
@@ -213,6 +323,8 @@ def main():
               file=sys.stderr)
         sys.exit(2)
 
+    if args.chain_probe:
+        return chain_probe(args)
     if args.workload != "linears7b":
         return run_decoder(args)
 
