@@ -146,9 +146,10 @@ bool prefer_kslice(const KslicePlan &kp, int epi, int M, int N, int K) {
     if (M > 768) return false;
     const int wide_bn = (epi == EPI_SILU_MUL) ? 128 : 256;
     const long wide = (long)((M + 127) / 128) * (N / wide_bn);
-    if (epi == EPI_PLAIN) return wide < 72;
-    if (epi == EPI_SILU_MUL) return wide < 160;
-    return wide < 192 || gemm_plan(epi, M, N, K).score < 0.65;
+    const long cus = device_shape().cus;  // the crossovers were measured on 256 CUs: 72, 160 and 192 wide tiles
+    if (epi == EPI_PLAIN) return wide < 9 * cus / 32;
+    if (epi == EPI_SILU_MUL) return wide < 5 * cus / 8;
+    return wide < 3 * cus / 4 || gemm_plan(epi, M, N, K).score < 0.65;
 }
 
 int run_tiled(int epi, MatmulArgs &a, void *workspace, size_t workspace_bytes, hipStream_t s) {

@@ -219,7 +219,8 @@ int launch_rmsnorm(const half_t *x, const half_t *delta, const half_t *w, half_t
 
 // Rows per split: enough workgroups to cover the chip (~2 per CU), at least 64 rows each.
 int attn_decode_splits(int BH, int capacity) {
-    int nsplit = (512 + BH - 1) / BH;
+    const int want = 2 * device_shape().cus;  // 512 workgroups on MI355X
+    int nsplit = (want + BH - 1) / BH;
     const int max_split = (capacity + 63) / 64;
     if (nsplit > max_split) nsplit = max_split;
     if (nsplit < 1) nsplit = 1;

@@ -562,13 +562,14 @@ GemmTuning g_gemm_tuning = {0, 0, 0};
 // CUs out of four a workgroup; from half the CUs on it still wins with K split in two.
 // Below that, 128 x 128 tiles, with K split when even those leave most CUs idle (the
 // M = 17..255 range on narrow layers).
-// How evenly `w` workgroups of equal work fill 256 CUs that hold two of them each: up to 256 every
-// workgroup has a CU to itself, beyond that they run in rounds of 512.  What this captures is the
+// How evenly `w` workgroups of equal work fill the device's CUs (256 on MI355X) that hold two of them each: up to
+// one per CU every workgroup has a CU to itself, beyond that they run in rounds of two per CU.  What this captures is the
 // cliff just above a multiple of the CU count (a few CUs run one workgroup more than the rest and
 // set the pace).
 static double fill_efficiency(long w) {
-    if (w <= 256) return (double)w / 256.0;
-    return (double)w / (512.0 * (double)((w + 511) / 512));
+    const long cus = device_shape().cus;
+    if (w <= cus) return (double)w / (double)cus;
+    return (double)w / ((double)(2 * cus) * (double)((w + 2 * cus - 1) / (2 * cus)));
 }
 
 GemmPlan gemm_plan(int epi, int M, int N, int K) {
@@ -579,11 +580,12 @@ GemmPlan gemm_plan(int epi, int M, int N, int K) {
     const long wide = (long)((M + 127) / 128) * (N / (2 * bn2));
     int s = 1;
     bool scored = false;
+    const long cus = device_shape().cus;  // the thresholds below are 512, 96 and 384 workgroups on MI355X's 256 CUs
     if (g_gemm_tuning.mt) {
         pl.mt = g_gemm_tuning.mt;
-    } else if (wide >= 512) {
+    } else if (wide >= 2 * cus) {
         pl.mt = 4;
-    } else if (wide >= 96 && nk >= 32) {
+    } else if (wide >= 3 * cus / 8 && nk >= 32) {
         // Few enough tiles for their count to matter: score (tile, split) candidates by how evenly they fill
         // the chip, the narrow tile at 0.85 of the wide one's rate, every extra split at 5 % + 20 / (K tiles)
         // of the time (the exchange of partial sums weighs more on a short K).  Fitted to LLaMA-7B / 13B /
@@ -611,8 +613,8 @@ GemmPlan gemm_plan(int epi, int M, int N, int K) {
     pl.tiles = ((M + 127) / 128) * (N / (pl.mt == 4 ? 2 * bn2 : bn2));
     if (g_gemm_tuning.splitk > 0) {
         s = g_gemm_tuning.splitk;
-    } else if (pl.mt == 2 && pl.tiles < 384 && !scored) {
-        s = (512 + pl.tiles / 2) / pl.tiles;  // aim for ~2 workgroups per CU
+    } else if (pl.mt == 2 && pl.tiles < 3 * cus / 2 && !scored) {
+        s = (int)((2 * cus + pl.tiles / 2) / pl.tiles);  // aim for ~2 workgroups per CU
         if (s > nk / 8) s = nk / 8;            // keep at least 8 K tiles (512 k) per split
     }
     if (s > GEMM_MAX_SPLITK) s = GEMM_MAX_SPLITK;

@@ -473,7 +473,7 @@ uint32_t magic_of(int d) { return d > 1 ? (uint32_t)(0x100000000ull / (unsigned)
 
 GemvTuning g_gemv_tuning = {1, 0, 0, 0};
 
-// Launch shape: the grid holds `waves_per_cu` waves per CU on all 256 CUs (or fewer
+// Launch shape: the grid holds `waves_per_cu` waves per CU on all CUs of the device (or fewer
 // waves when there are fewer units than that), each wave owning q or q+1 units.
 GemvPlan gemv_plan(int epi, int M, int N, int K, bool norm) {
     GemvPlan pl = {};
@@ -487,7 +487,7 @@ GemvPlan gemv_plan(int epi, int M, int N, int K, bool norm) {
     pl.tiles = (epi == EPI_ROPE) ? (N / 128) * (64 / sw) : N / sw;
     pl.nb = K / 128;
     const long units = (long)pl.tiles * pl.nb;
-    long total_waves = 256L * waves_per_cu;
+    long total_waves = (long)device_shape().cus * waves_per_cu;
     if (total_waves > units) total_waves = units;
     pl.workgroups = (int)((total_waves + pl.waves - 1) / pl.waves);
     total_waves = (long)pl.workgroups * pl.waves;

@@ -135,6 +135,14 @@ size_t attn_decode_partial_bytes(int BH, int capacity);
 int launch_attn_decode(const half_t *q, const half_t *kc, const half_t *vc, const int *positions, half_t *out,
                        const int32_t *out_index, int B, int H, int capacity, float scale, int *counters, float *partials, hipStream_t stream);
 
+// Compute units and XCDs of the current device, asked once per device (hipDeviceProp_t / hipDeviceAttributeNumberOfXccs).
+// Launch plans size their grids from it.  Where no device can be asked (plans made on a machine without a GPU, e.g.
+// gptq4_workspace_bytes in a host-only test) it answers with MI355X's 256 CUs in 8 XCDs.
+struct DeviceShape {
+    int cus, xcds;
+};
+DeviceShape device_shape();
+
 // arrival counters sit one per 128-byte line: atomics on one line are served one after
 // the other by the memory side
 enum { COUNTER_STRIDE = 32 };

@@ -455,11 +455,12 @@ KslicePlan kslice_plan(int epi, int M, int N, int K, bool has_perm) {
         // tiles per wave.  Fitted to sweeps at LLaMA-7B / 13B / 30B shapes, 32..256 rows: on average 1 % off
         // the best split (a fixed target of 512 workgroups: 2.3 %, worst case 17 %).
         const double pen = 0.04 + 15.0 / (double)nk;
+        const long cus = device_shape().cus;  // 256 on MI355X
         double best = -1.0;
         for (int c = 1; c <= 8 && c <= nk / (4 * ks); ++c) {
             const long w = (long)pl.tiles * c;
-            double e = (w <= 256) ? (double)w / 256.0 : (double)w / (512.0 * (double)((w + 511) / 512));
-            if (w >= 512 && e < 0.8) e = 0.8;
+            double e = (w <= cus) ? (double)w / (double)cus : (double)w / ((double)(2 * cus) * (double)((w + 2 * cus - 1) / (2 * cus)));
+            if (w >= 2 * cus && e < 0.8) e = 0.8;
             const double score = e / (1.0 + pen * (c - 1));
             if (score > best + 1e-9) {
                 best = score;

@@ -497,7 +497,8 @@ SkinnyTuning g_skinny_tuning = {0, 0, 0, 0};
 // workgroups: then those are 10-18 % faster (13B / 30B down_proj and gate/up; never at 7B shapes, where the
 // split is capped first).  The rotary epilogue keeps 8-byte loads (two strips per head either way).
 static int split_for(int tiles, int k_batches, int waves) {
-    int s = (1024 + tiles - 1) / tiles;
+    const int want = 4 * device_shape().cus;  // 1024 workgroups on MI355X
+    int s = (want + tiles - 1) / tiles;
     if (s > k_batches / (2 * waves)) s = k_batches / (2 * waves);
     if (s > SKINNY_MAX_SPLITK) s = SKINNY_MAX_SPLITK;
     return s < 1 ? 1 : s;

@@ -122,6 +122,26 @@ __global__ __launch_bounds__(256) void gptq4_rope_table_kernel(float *__restrict
 
 }  // namespace
 
+DeviceShape device_shape() {
+    enum { MAX_DEVICES = 64 };
+    static DeviceShape known[MAX_DEVICES];  // cus == 0: not asked yet
+    const DeviceShape fallback = {256, 8};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+        (void)hipGetLastError();
+        return fallback;
+    }
+    if (known[dev].cus == 0) {  // (a race between two first callers writes the same values twice)
+        DeviceShape d = fallback;
+        int v = 0;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) d.cus = v;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeNumberOfXccs, dev) == hipSuccess && v > 0) d.xcds = v;
+        (void)hipGetLastError();
+        known[dev] = d;
+    }
+    return known[dev];
+}
+
 int launch_dequant(const uint32_t *qweight, const uint32_t *qzeros, const half_t *scales,
                    const int32_t *g_idx, half_t *out, int K, int N, int groupsize, hipStream_t stream) {
     dim3 grid((unsigned)((N + 255) / 256), (unsigned)(K / 8)), block(256);
