@@ -157,6 +157,10 @@ class QuantLlamaMLP(nn.Module):
                        uq.index_select(1, cols).contiguous(), self.up_proj_scales.index_select(1, cols).contiguous(),
                        _move_zero_columns(self.up_proj_qzeros, cols))
             self._chained = (key, tensors, perm)
+            # the row-sorted copies were only a step on the way: beside the checkpoint tensors (which state_dict
+            # needs) the module keeps ONE derived copy of gate and up; gate_up() rebuilds the sorted pair if asked
+            self._sorted = None
+            del gq, uq
         return self._chained[1], self._chained[2], down_q
 
     def _down(self, mid: torch.Tensor, down_q: torch.Tensor) -> torch.Tensor:

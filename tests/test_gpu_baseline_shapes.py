@@ -282,3 +282,40 @@ def test_one_hot_rows_at_full_size():
     D = to_dev(L)
     y = gptq().matmul4(g, torch.from_numpy(x).cuda(), D["qweight"], D["scales"], D["qzeros"])
     assert (bits(y.cpu().numpy()) == bits(W[sel])).all()
+
+
+# ------------------------------------------------- derived copies follow in-place updates of the checkpoint tensors
+def test_act_order_copies_follow_in_place_updates():
+    """The sorted / column-ordered copies an act-order module derives at first use are keyed on the tensors'
+    versions as well as their addresses: reloading weights into the existing buffers (load_state_dict, copy_)
+    after a first forward must not keep serving the copies made from the old contents."""
+    G = gptq()
+    k, inter, g, m = 512, 768, 128, 3
+    x = torch.from_numpy(O.make_x(m, k, seed=5)).cuda()
+
+    def layers(seed):
+        gate = O.make_layer(k, inter, g, seed=seed, act_order=True)
+        up = O.make_layer(k, inter, g, seed=seed + 1)
+        up["g_idx"] = gate["g_idx"]
+        down = O.make_layer(inter, k, g, seed=seed + 2, act_order=True)
+        return gate, up, down
+
+    def build(seed):
+        gate, up, down = layers(seed)
+        return G.QuantLlamaMLP(quant_linear(gate, k, inter, g, True), quant_linear(down, inter, k, g, True),
+                               quant_linear(up, k, inter, g, True)).cuda()
+
+    old, new = build(100), build(200)
+    y_old = old(x)
+    want = new(x)
+    assert not torch.equal(y_old, want)
+    # the new weights into the OLD module's buffers, in place: same addresses, other contents
+    old.load_state_dict(new.state_dict())
+    assert torch.equal(old(x), want), "stale act-order copies served after an in-place reload"
+    # a single QuantLinear likewise
+    L1, L2 = O.make_layer(k, k, g, seed=300, act_order=True), O.make_layer(k, k, g, seed=301, act_order=True)
+    a, b = quant_linear(L1, k, k, g, True).cuda(), quant_linear(L2, k, k, g, True).cuda()
+    a(x)
+    for name in ("qweight", "qzeros", "scales", "g_idx"):
+        getattr(a, name).copy_(getattr(b, name))
+    assert torch.equal(a(x), b(x))
