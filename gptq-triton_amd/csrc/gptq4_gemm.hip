@@ -124,6 +124,48 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
 
     const half_t *a_base = p.x + (size_t)m0 * K;
 
+    // Rotary epilogue of the wide tile: the cos / sin rows of the tile's 128 tokens come through LDS, a block of
+    // 32 tokens (8 KiB per table) at a time in two buffers, filled by LDS-direct loads that all four waves share
+    // (they need the same values: both heads of the tile, and d and d + 64 of a head, turn by the same angles).
+    // Blocks 0 and 1 are asked for here, ahead of the K loop; 2 and 3 follow in the epilogue as the buffers
+    // become free.  Read from memory per lane instead (16 tokens x 2 tables in registers, after the positions
+    // they depend on, once per block of 32 rows), the epilogue is four round trips to memory long with the
+    // matrix cores idle: the two workgroups of a CU start together and so reach it together.
+    constexpr bool ROPE_TAB = (EPI == EPI_ROPE) && (MT == 4);
+    extern __shared__ __attribute__((aligned(16))) float rope_tab[];  // ROPE_TAB: [2 buffers][cos, sin][32 tokens][64]
+    bool need_tab = false;
+    int tab_voff[4][2];  // per block and unit of 4 tokens: byte offset of the lane's 16-byte chunk in the tables
+    __amdgpu_buffer_rsrc_t cos_rsrc, sin_rsrc;
+    if constexpr (ROPE_TAB) {
+        const RopeArgs &r = p.rope;
+        need_tab = (n0 >> 7) / r.H < 2;  // the tile's first head is of q or k (else both are heads of v)
+        if (need_tab) {
+#pragma unroll
+            for (int blk = 0; blk < 4; ++blk)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int row = min(m0 + 32 * blk + 4 * (2 * wave + j) + (lane >> 4), M - 1);
+                    const int tp = min(max(r.position_ids[row], 0), r.max_pos - 1);
+                    tab_voff[blk][j] = tp * 256 + (lane & 15) * 16;
+                }
+        }
+        cos_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)r.cos_table, 0, (int)((uint32_t)r.max_pos * 256u), 0x00020000);
+        sin_rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)r.sin_table, 0, (int)((uint32_t)r.max_pos * 256u), 0x00020000);
+    }
+    // wave w brings tokens 8w .. 8w + 7 of the block: one load = 4 table rows of 256 bytes = 1 KiB of LDS
+    auto dma_table = [&](int blk, int buf) {
+        if constexpr (ROPE_TAB) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                float *const dst = rope_tab + buf * (2 * 32 * 64) + (2 * wave + j) * 256;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(cos_rsrc, (__attribute__((address_space(3))) void *)dst, 16, tab_voff[blk][j], 0, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(sin_rsrc, (__attribute__((address_space(3))) void *)(dst + 32 * 64), 16,
+                                                         tab_voff[blk][j], 0, 0, 0);
+            }
+            asm volatile("" ::: "memory");
+        }
+    };
+
     // K tiles [k_begin, nk) of this split (host-side quotient / remainder, no division here
     // except the one that finds the first group)
     const int split = blockIdx.y;
@@ -197,6 +239,10 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
         bf[0] = decode_word_h8(bw[0].x, cd[0]);
         bf[1] = decode_word_h8(bw[0].y, cd[1]);
         load_b_step(min(k_begin + 1, nk - 1), 0);
+        if (need_tab) {
+            dma_table(0, 0);
+            dma_table(1, 1);
+        }
 
         for (int kt = k_begin; kt < nk; ++kt) {
             const int buf = kt & 1;
@@ -348,6 +394,12 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
                 bf[1] = decode_word_natural(nw.y, cn[1]);
             }
         };
+        // the first two blocks of the rotary tables: older than every load the waits below count, so landed
+        // long before the epilogue
+        if (need_tab) {
+            dma_table(0, 0);
+            dma_table(1, 1);
+        }
         // pairs of tiles without a branch between them (a join there would make the compiler
         // move packed words that are still in flight, and wait for them), then the odd one
         int kt = k_begin;
@@ -482,6 +534,60 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
         const size_t seq_stride = (size_t)r.H * cap * 128;
         const bool at_position = (which != 0) && r.kv_offset < 0;  // cache row = the token's position
         const int row_shift = (which == 0 || r.kv_offset < 0) ? 0 : r.kv_offset;
+        if constexpr (ROPE_TAB) {
+            if (PERM) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // table blocks 0 and 1 (the plain path has waited already)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                if (need_tab) {
+                    // the block of this step was asked for a step ago: wait for this wave's share of it before
+                    // the barrier, and before asking for the next one
+                    if (mt >= 2) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                    __syncthreads();  // the step before is finished: its exchange regions and table buffer are free
+                    if (mt >= 1 && mt + 1 < MT) dma_table(mt + 1, (mt + 1) & 1);
+                    if (which < 2) {
+#pragma unroll
+                        for (int t = 0; t < 2; ++t)
+#pragma unroll
+                            for (int i = 0; i < 16; ++i) mine[(t * 16 + i) * 64 + lane] = acc[mt][t][i];
+                    }
+                    __syncthreads();
+                }
+                int pos[16];
+                if (at_position) {
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const int row = min(wrow0 + mt * 32 + 8 * (i >> 2) + 4 * lhi + (i & 3), M - 1);
+                        pos[i] = max(r.position_ids[row], 0);
+                    }
+                }
+                const float *const tcos = rope_tab + (mt & 1) * (2 * 32 * 64) + (4 * lhi) * 64 + 2 * l32;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int row = wrow0 + mt * 32 + 8 * (i >> 2) + 4 * lhi + (i & 3);
+                    float o0 = acc[mt][0][i], o1 = acc[mt][1][i];
+                    if (which < 2) {
+                        const float2 cs = *reinterpret_cast<const float2 *>(tcos + (8 * (i >> 2) + (i & 3)) * 64);
+                        const float2 sn = *reinterpret_cast<const float2 *>(tcos + 32 * 64 + (8 * (i >> 2) + (i & 3)) * 64);
+                        const float p0 = theirs[(0 * 16 + i) * 64 + lane], p1 = theirs[(1 * 16 + i) * 64 + lane];
+                        if (wn_odd == 0) {
+                            o0 = o0 * cs.x - p0 * sn.x;
+                            o1 = o1 * cs.y - p1 * sn.y;
+                        } else {
+                            o0 = o0 * cs.x + p0 * sn.x;
+                            o1 = o1 * cs.y + p1 * sn.y;
+                        }
+                    }
+                    if (row < M) {
+                        int bb, srow;
+                        split_row(r, row, bb, srow);
+                        const int crow = at_position ? min(pos[i], r.kv_capacity - 1) : srow + row_shift;
+                        const h2_t o = {(half_t)o0, (half_t)o1};
+                        *reinterpret_cast<uint32_t *>(dst + (size_t)bb * seq_stride + (size_t)crow * 128) = as_u32(o);
+                    }
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             if (which < 2) {
@@ -541,10 +647,24 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
 template <int EPI, int MT>
 int launch_one(const MatmulArgs &a, int tiles, hipStream_t stream) {
     dim3 grid((unsigned)tiles, (unsigned)a.splitk), block(256);
-    if (a.perm == nullptr)
-        hipLaunchKernelGGL((gptq4_gemm_kernel<EPI, MT, false>), grid, block, 0, stream, a);
+    const bool perm = a.perm != nullptr;
+    // the wide rotary tile stages its cos / sin rows in 32 KiB of LDS on top of the activation tiles: more than
+    // the 64 KiB a launch may ask for unless the kernel is marked for it (once per variant)
+    const size_t lds = (EPI == EPI_ROPE && MT == 4) ? 2 * 2 * 32 * 64 * sizeof(float) : 0;
+    if (lds) {
+        static bool allowed[2] = {false, false};
+        if (!allowed[perm]) {
+            const void *fn = perm ? reinterpret_cast<const void *>(&gptq4_gemm_kernel<EPI, MT, true>)
+                                  : reinterpret_cast<const void *>(&gptq4_gemm_kernel<EPI, MT, false>);
+            const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return (int)e;
+            allowed[perm] = true;
+        }
+    }
+    if (!perm)
+        hipLaunchKernelGGL((gptq4_gemm_kernel<EPI, MT, false>), grid, block, lds, stream, a);
     else
-        hipLaunchKernelGGL((gptq4_gemm_kernel<EPI, MT, true>), grid, block, 0, stream, a);
+        hipLaunchKernelGGL((gptq4_gemm_kernel<EPI, MT, true>), grid, block, lds, stream, a);
     return (int)hipGetLastError();
 }
 

@@ -75,6 +75,40 @@ def test_tiled_qkv_rotary(forced_tiled, b, s, pos0, g):
         assert_close(got.cpu().numpy(), ref, f"tiled {name} b={b} s={s} g={g}")
 
 
+def test_tiled_rotary_by_position_with_positions_outside_the_table(forced_tiled):
+    """Cache rows placed by position id (kv_offset = KV_AT_POSITION) in the tiled kernel, with position ids below 0
+    and past the end of the cos / sin tables: the angle is that of the nearest table row, the cache row is the
+    position clamped into the cache.  150 tokens per sequence: a ragged last row tile."""
+    from gptq_triton_amd.fused_attention import KV_AT_POSITION
+    H, Dh, hidden, g = 8, 128, 1024, 128
+    L = O.make_layer(hidden, 3 * hidden, g, seed=520)
+    D = to_dev(L)
+    G = gptq()
+    max_pos, cap, b, s = 96, 256, 2, 150
+    cos, sin = G.RotaryTable(Dh, max_pos).get(torch.device("cuda"), max_pos)
+    cos, sin = cos[:max_pos].contiguous(), sin[:max_pos].contiguous()
+    rng = np.random.default_rng(521)
+    pos = np.stack([1 + rng.permutation(cap - 1)[:s] for _ in range(b)]).astype(np.int64)   # distinct cache rows, none 0
+    pos[0, 7], pos[1, 140] = -3, -1                                                          # these go to row 0
+    x = O.make_x(b * s, hidden, seed=522).reshape(b, s, hidden)
+    kc = torch.full((b, H, cap, Dh), 7.0, dtype=torch.float16, device="cuda")
+    vc = torch.full((b, H, cap, Dh), 7.0, dtype=torch.float16, device="cuda")
+    xd, pd = torch.from_numpy(x).cuda(), torch.from_numpy(pos).cuda()
+    q, _, _ = G.qkv_rotary(g, xd, D["qweight"], D["scales"], D["qzeros"], pd, cos, sin, H, Dh,
+                           kv_out=(kc, vc), kv_offset=KV_AT_POSITION)
+    angle_row = np.clip(pos, 0, max_pos - 1)
+    qr, kr, vr = O.qkv_rotary_ref(x, L["qweight"], L["qzeros"], L["scales"], g, angle_row, H, Dh, max_pos=max_pos)
+    assert_close(q.cpu().numpy(), qr, "q by position")
+    cache_row = np.clip(pos, 0, cap - 1)
+    for bi in range(b):
+        rows = torch.from_numpy(cache_row[bi]).cuda()
+        assert_close(kc[bi][:, rows].cpu().numpy(), kr[bi], f"k rows of sequence {bi}")
+        assert_close(vc[bi][:, rows].cpu().numpy(), vr[bi], f"v rows of sequence {bi}")
+        untouched = torch.ones(cap, dtype=torch.bool)
+        untouched[cache_row[bi]] = False
+        assert bool((kc[bi][:, untouched] == 7.0).all()) and bool((vc[bi][:, untouched] == 7.0).all())
+
+
 def test_prefill_sized_call_takes_the_wide_tiles_by_itself():
     """2048 rows x 3072 columns = 192 wide tiles: the automatic plan picks the 128 x 256 tile
     without any forcing; K is small so that the oracle finishes in seconds."""
