@@ -12,9 +12,11 @@ from pathlib import Path
 import torch
 
 LIB_PATH = Path(__file__).resolve().parent / "csrc" / "libgptq4.so"
-ABI_VERSION = 1
-WS_COUNTER_BYTES = 524288
-STATIC_SCRATCH_BYTES = WS_COUNTER_BYTES + (8 << 20)  # GPTQ4_STATIC_SCRATCH_BYTES: what gptq4_matmul_static holds per GPU
+ABI_VERSION = 2
+WS_COUNTER_BYTES = 524288            # arrival counters
+WS_HEAD_BYTES = WS_COUNTER_BYTES + (16 << 20)  # GPTQ4_WS_HEAD_BYTES: counters + marked partial sums, zero between calls
+WS_ERROR_WORD = 1                     # GPTQ4_WS_ERROR_WORD
+STATIC_SCRATCH_BYTES = WS_HEAD_BYTES + (8 << 20)  # GPTQ4_STATIC_SCRATCH_BYTES: what gptq4_matmul_static holds per GPU
 OP_MATMUL, OP_MLP_GATEUP, OP_QKV_ROTARY, OP_DECODE_ATTENTION = 0, 1, 2, 3
 OP_WITH_PERM = 0x100  # or-ed to a matmul selector in gptq4_workspace_bytes: the call passes `perm`
 
@@ -57,6 +59,7 @@ SIGNATURES = {
     "gptq4_set_gemm_tuning": (None, [c_int, c_int]),
     "gptq4_set_midm_tuning": (None, [c_int, c_int, c_int]),
     "gptq4_set_gemv_tuning": (None, [c_int, c_int, c_int, c_int]),
+    "gptq4_set_exchange_spin_limit": (None, [ctypes.c_uint]),
 }
 
 
@@ -119,7 +122,7 @@ def current_stream(device: torch.device):
 # alive, because captured graphs may still launch kernels that point into it.
 _workspaces: dict = {}
 _outgrown: list = []
-_WS_BYTES = WS_COUNTER_BYTES + 16 * 16 * 2 * 32768 * 4  # splitk 16, M 16, 2 matrices, 32768 columns
+_WS_BYTES = WS_HEAD_BYTES + 16 * 16 * 2 * 32768 * 4  # splitk 16, M 16, 2 matrices, 32768 columns
 
 
 def workspace(device: torch.device, need: int):

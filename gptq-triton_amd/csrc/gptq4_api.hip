@@ -41,11 +41,24 @@ int setup_skinny(MatmulArgs &a, const SkinnyPlan &pl, int nmat, void *workspace,
     a.slot_rem = nbatches % slots;
     a.batches_per_group = a.groupsize / 128;
     if (a.tiles > SKINNY_MAX_TILES) return -GPTQ4_E_SHAPE;
-    if (workspace == nullptr || workspace_bytes < GPTQ4_WS_COUNTER_BYTES) return -GPTQ4_E_WORKSPACE;
-    if (a.splitk > 1 && workspace_bytes < GPTQ4_WS_COUNTER_BYTES + partial_bytes(a.splitk, a.M, nmat * a.N))
+    if (workspace == nullptr || workspace_bytes < GPTQ4_WS_HEAD_BYTES) return -GPTQ4_E_WORKSPACE;
+    if (a.splitk > 1 && workspace_bytes < GPTQ4_WS_HEAD_BYTES + partial_bytes(a.splitk, a.M, nmat * a.N))
         return -GPTQ4_E_WORKSPACE;
     a.counters = reinterpret_cast<int *>(workspace);
-    a.partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_COUNTER_BYTES);
+    a.partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_HEAD_BYTES);
+    // The exchange through marked 8-byte values where it is the faster one - up to 4 rows, and few enough splits
+    // for the finishing workgroup to poll them all in one round (16 loads per thread: 8, 4 or 2 splits by the
+    // values a thread holds) - and the values fit their region of the head; else arrival counters and plain
+    // partial sums.  Measured at LLaMA-7B / 30B shapes: QKV 11.5 -> 10.9 / 24.4 -> 21.8 us at one row, o_proj and
+    // down_proj 0.1 - 0.2 us ahead, but behind the counters from 8 rows on (gate/up 18.5 -> 19.4 us) and with 15
+    // splits to poll (30B down_proj 18.9 -> 19.8 us).
+    a.tagged = nullptr;
+    const int per_thread = pl.words * nmat * (nmat == 1 && a.rope.q != nullptr ? 2 : 1);  // values a finishing thread holds per row block
+    const int round = per_thread >= 8 ? 2 : (per_thread >= 4 ? 4 : 8);
+    const bool marked = g_skinny_tuning.exchange == 2 || (g_skinny_tuning.exchange == 0 && a.M <= 4 && a.splitk - 1 <= round);
+    if (a.splitk > 1 && marked && 2 * partial_bytes(a.splitk, a.M, nmat * a.N) <= GPTQ4_WS_TAGGED_BYTES)
+        a.tagged = reinterpret_cast<uint64_t *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_COUNTER_BYTES);
+    a.spin_limit = g_gemv_tuning.spin_limit ? g_gemv_tuning.spin_limit : (1u << 22);
     return 0;
 }
 
@@ -54,7 +67,7 @@ int setup_skinny(MatmulArgs &a, const SkinnyPlan &pl, int nmat, void *workspace,
 // texture path, and repeats that for every column tile: 3.5 us at one row, twice the time of the whole call
 // at eight rows, +43 % for a 2048-row down_proj.
 int stage_act_order(MatmulArgs &a, size_t partial_bytes_used, void *workspace, size_t workspace_bytes, hipStream_t s) {
-    const size_t off = GPTQ4_WS_COUNTER_BYTES + partial_bytes_used;
+    const size_t off = GPTQ4_WS_HEAD_BYTES + partial_bytes_used;
     const size_t bytes = (size_t)a.M * a.K * sizeof(half_t);
     if (workspace == nullptr || workspace_bytes < off + bytes) return -GPTQ4_E_WORKSPACE;
     // rows longer than 32768 values are gathered with the row index in grid.y, which ends at 65535
@@ -74,10 +87,9 @@ int run_small(int epi, MatmulArgs &a, int nmat, void *workspace, size_t workspac
         if (a.M <= GEMV_MAX_M) {
             const GemvPlan gp = gemv_plan(epi, a.M, a.N, a.K, true);
             if (gp.ok) {
-                if (workspace == nullptr || workspace_bytes < GPTQ4_WS_COUNTER_BYTES + gemv_partial_bytes(gp, a.M, epi))
-                    return -GPTQ4_E_WORKSPACE;
+                if (workspace == nullptr || workspace_bytes < GPTQ4_WS_HEAD_BYTES) return -GPTQ4_E_WORKSPACE;
                 a.counters = reinterpret_cast<int *>(workspace);
-                a.partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_COUNTER_BYTES);
+                a.tagged = reinterpret_cast<uint64_t *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_COUNTER_BYTES);
                 return launch_gemv(epi, a, gp, s);
             }
         }
@@ -89,10 +101,9 @@ int run_small(int epi, MatmulArgs &a, int nmat, void *workspace, size_t workspac
     if (a.M <= GEMV_MAX_M) {
         const GemvPlan pl = gemv_plan(epi, a.M, a.N, a.K);
         if (pl.ok) {
-            if (workspace == nullptr || workspace_bytes < GPTQ4_WS_COUNTER_BYTES + gemv_partial_bytes(pl, a.M, epi))
-                return -GPTQ4_E_WORKSPACE;
+            if (workspace == nullptr || workspace_bytes < GPTQ4_WS_HEAD_BYTES) return -GPTQ4_E_WORKSPACE;
             a.counters = reinterpret_cast<int *>(workspace);
-            a.partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_COUNTER_BYTES);
+            a.tagged = reinterpret_cast<uint64_t *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_COUNTER_BYTES);
             return launch_gemv(epi, a, pl, s);
         }
     }
@@ -114,10 +125,10 @@ int setup_gemm(MatmulArgs &a, const GemmPlan &pl, void *workspace, size_t worksp
     a.slot_q = nk / pl.splitk;
     a.slot_rem = nk % pl.splitk;
     if (pl.splitk > 1) {
-        if (workspace == nullptr || workspace_bytes < GPTQ4_WS_COUNTER_BYTES + gemm_partial_bytes(pl))
+        if (workspace == nullptr || workspace_bytes < GPTQ4_WS_HEAD_BYTES + gemm_partial_bytes(pl))
             return -GPTQ4_E_WORKSPACE;
         a.counters = reinterpret_cast<int *>(workspace);
-        a.partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_COUNTER_BYTES);
+        a.partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_HEAD_BYTES);
     }
     return 0;
 }
@@ -162,7 +173,7 @@ int run_tiled(int epi, MatmulArgs &a, void *workspace, size_t workspace_bytes, h
         const KslicePlan kp = kslice_plan(epi, a.M, a.N, a.K, false);
         const size_t partial = prefer_kslice(kp, epi, a.M, a.N, a.K) ? (kp.splitk > 1 ? kslice_partial_bytes(epi, kp) : 0)
                                                                        : (pl.splitk > 1 ? gemm_partial_bytes(pl) : 0);
-        if (workspace == nullptr || workspace_bytes < GPTQ4_WS_COUNTER_BYTES + partial + rows_bytes) stage = false;
+        if (workspace == nullptr || workspace_bytes < GPTQ4_WS_HEAD_BYTES + partial + rows_bytes) stage = false;
     }
     const KslicePlan kp = kslice_plan(epi, a.M, a.N, a.K, a.perm != nullptr && !stage);
     if (prefer_kslice(kp, epi, a.M, a.N, a.K)) {
@@ -173,9 +184,9 @@ int run_tiled(int epi, MatmulArgs &a, void *workspace, size_t workspace_bytes, h
         a.slot_rem = nk % kp.splitk;
         const size_t partial = kp.splitk > 1 ? kslice_partial_bytes(epi, kp) : 0;
         if (kp.splitk > 1) {
-            if (workspace == nullptr || workspace_bytes < GPTQ4_WS_COUNTER_BYTES + partial) return -GPTQ4_E_WORKSPACE;
+            if (workspace == nullptr || workspace_bytes < GPTQ4_WS_HEAD_BYTES + partial) return -GPTQ4_E_WORKSPACE;
             a.counters = reinterpret_cast<int *>(workspace);
-            a.partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_COUNTER_BYTES);
+            a.partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_HEAD_BYTES);
         }
         if (stage) {
             const int rc = stage_act_order(a, partial, workspace, workspace_bytes, s);
@@ -242,9 +253,14 @@ void gptq4_set_gemv_tuning(int mode, int depth, int waves, int waves_per_cu) {
     g_gemv_tuning.waves = (waves == 4 || waves == 8 || waves == 16) ? waves : 0;
     g_gemv_tuning.waves_per_cu = (waves_per_cu >= 4 && waves_per_cu <= 32) ? waves_per_cu : 0;
 }
+void gptq4_set_exchange_spin_limit(unsigned polls) { g_gemv_tuning.spin_limit = polls; }
+
 static_assert(GPTQ4_WS_COUNTER_BYTES == SKINNY_MAX_TILES * COUNTER_STRIDE * 4, "one counter line per tile");
 
 void gptq4_set_tuning(int words, int depth, int splitk) {
+    // 10 + words: exchange the split-K partial sums through arrival counters; 20 + words: through marked values wherever they fit
+    g_skinny_tuning.exchange = (words >= 20) ? 2 : (words >= 10) ? 1 : 0;
+    words %= 10;
     g_skinny_tuning.waves = 0;
     g_skinny_tuning.words = (words == 1 || words == 2 || words == 4) ? words : 0;
     g_skinny_tuning.depth = (depth >= 1 && depth <= 4) ? depth : 0;
@@ -252,7 +268,7 @@ void gptq4_set_tuning(int words, int depth, int splitk) {
 }
 
 size_t gptq4_workspace_bytes(int op, int M, int K, int N) {
-    size_t bytes = GPTQ4_WS_COUNTER_BYTES;
+    size_t bytes = GPTQ4_WS_HEAD_BYTES;
     const bool with_perm = (op & GPTQ4_OP_WITH_PERM) != 0;
     op &= ~GPTQ4_OP_WITH_PERM;
     if (op == GPTQ4_OP_DECODE_ATTENTION) return (M < 1 || K < 1) ? bytes : bytes + attn_decode_partial_bytes(M, K);
@@ -260,14 +276,6 @@ size_t gptq4_workspace_bytes(int op, int M, int K, int N) {
     if (M <= SKINNY_MAX_M) {
         const int cols = (op == GPTQ4_OP_MLP_GATEUP) ? 2 * N : N;
         size_t need = partial_bytes(SKINNY_MAX_SPLITK, M, cols);
-        if (M <= GEMV_MAX_M && (K % 128) == 0 && (N % 256) == 0) {
-            const int epi = (op == GPTQ4_OP_MLP_GATEUP) ? EPI_SILU_MUL : (op == GPTQ4_OP_QKV_ROTARY ? EPI_ROPE : EPI_PLAIN);
-            // whichever launch shape runs: the tuned one, or the automatic one of the self-normalising variant
-            for (int norm = 0; norm < 2; ++norm) {
-                const GemvPlan pl = gemv_plan(epi, M, N, K, norm != 0);
-                if (pl.ok && gemv_partial_bytes(pl, M, epi) > need) need = gemv_partial_bytes(pl, M, epi);
-            }
-        }
         bytes += need + (with_perm ? (size_t)M * K * 2 : 0);  // + the rows gathered for an act-order call
     } else if ((K % 64) == 0) {
         const int epi = (op == GPTQ4_OP_MLP_GATEUP) ? EPI_SILU_MUL : (op == GPTQ4_OP_QKV_ROTARY ? EPI_ROPE : EPI_PLAIN);
@@ -527,9 +535,9 @@ int gptq4_decode_attention(const void *q, const void *k_cache, const void *v_cac
     if (!q || !k_cache || !v_cache || !positions || !out) return -GPTQ4_E_NULL;
     if (B < 1 || H < 1 || D != 128 || kv_capacity < 1 || (long)B * H > SKINNY_MAX_TILES) return -GPTQ4_E_SHAPE;
     if (misaligned16(q) || misaligned16(k_cache) || misaligned16(v_cache) || misaligned16(out)) return -GPTQ4_E_ALIGN;
-    if (workspace == nullptr || workspace_bytes < GPTQ4_WS_COUNTER_BYTES + attn_decode_partial_bytes(B * H, kv_capacity))
+    if (workspace == nullptr || workspace_bytes < GPTQ4_WS_HEAD_BYTES + attn_decode_partial_bytes(B * H, kv_capacity))
         return -GPTQ4_E_WORKSPACE;
-    float *partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_COUNTER_BYTES);
+    float *partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_HEAD_BYTES);
     return launch_attn_decode(reinterpret_cast<const half_t *>(q), reinterpret_cast<const half_t *>(k_cache),
                               reinterpret_cast<const half_t *>(v_cache), positions, reinterpret_cast<half_t *>(out), out_index, B, H,
                               kv_capacity, scale, reinterpret_cast<int *>(workspace), partials,

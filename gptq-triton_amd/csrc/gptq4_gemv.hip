@@ -18,13 +18,21 @@
 //     the exact fp16 values of the dequantisation kernel;
 //   * at the end of a tile segment the wave publishes its partial sums
 //     [rows][tile columns] in its slot of the workspace (slot = its rank among the waves
-//     that touch the tile) with agent-scope stores, waits for their completion, and adds
-//     its unit count to the tile's counter; the wave that completes the count sums the
-//     slots in rank order (deterministic) and runs the epilogue (bias / SiLU*mul /
-//     rotary + head-major q,k,v store), then clears the counter.
+//     that touch the tile) as 8-byte {fp32 bits, 1} pairs with agent-scope stores, and goes
+//     on: no wait for their completion, no counter.  The wave that owns the tile's last unit
+//     finishes the tile: it polls the slots until every pair carries its 1 (a pair is one
+//     store, so value and mark arrive together), sums them in rank order (deterministic),
+//     runs the epilogue (bias / SiLU*mul / rotary + head-major q,k,v store) and writes the
+//     slots back to zero for the next call.  The region of the workspace that holds the
+//     slots is zero whenever no call is running; nothing else is ever written there.
+//     A finisher only waits for waves of lower rank, which sit in workgroups dispatched no
+//     later than its own and never wait themselves unless they finish a lower tile - so the
+//     waits end even when the grid does not fit the chip at once.  They are bounded all the
+//     same: a wave that gives up sets the error word of the workspace and moves on.
 // The loop is free of branches around loads: loads past the end of the range are
 // redirected to the first bytes of the matrix (one cache line) and never used, so the
 // compiler's wait counters stay exact and DEPTH units are really in flight.
+#include "../../include/gptq4.h"
 #include "gptq4_internal.h"
 #include "gptq4_norm.h"
 
@@ -290,9 +298,10 @@ __global__ __launch_bounds__(64 * NW) void gptq4_gemv_kernel(MatmulArgs p) {
     // touch the tile; the owner of the tile's first unit has rank 0).  Rows 0..3 of the
     // accumulators live in lanes 0..15.
     const size_t tile_elems = (size_t)M * TILE_COLS;
+    constexpr uint64_t MARK = 1ull << 32;
     auto publish = [&](int tile) {
         const int rank = v - wave_of_unit(tile * NB);
-        float *mine = p.partials + ((size_t)tile * p.max_contrib + rank) * tile_elems;
+        uint64_t *mine = p.tagged + ((size_t)tile * p.max_contrib + rank) * tile_elems;
         if (lane < 16) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -301,8 +310,8 @@ __global__ __launch_bounds__(64 * NW) void gptq4_gemv_kernel(MatmulArgs p) {
                     for (int vv = 0; vv < NV; ++vv)
 #pragma unroll
                         for (int t = 0; t < W; ++t)
-                            __hip_atomic_store(&mine[(size_t)e * TILE_COLS + vv * SW + W * lcol + t], acc[vv][t][e],
-                                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            __hip_atomic_store(&mine[(size_t)e * TILE_COLS + vv * SW + W * lcol + t],
+                                               MARK | (uint64_t)__float_as_uint(acc[vv][t][e]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
             }
         }
@@ -328,28 +337,15 @@ __global__ __launch_bounds__(64 * NW) void gptq4_gemv_kernel(MatmulArgs p) {
     WSTAMP(4);
     const bool crossed = n > first_len;
     publish(crossed ? t0 + 1 : t0);
-    // completion, not fences, orders the exchange: the stores above are acknowledged by
-    // the L2 before the counter is touched
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     WSTAMP(5);
 
-    // ---- arrival count per touched tile; the wave completing a tile finishes it
-#pragma unroll 1
-    for (int seg = 0; seg < 2; ++seg) {
-        if (seg == 1 && !crossed) break;
-        const int tile = t0 + seg;
-        const int cnt = (seg == 0) ? first_len : n - first_len;
-        int old = 0;
-        if (lane == 0)
-            old = __hip_atomic_fetch_add(&p.counters[tile * COUNTER_STRIDE], cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        old = __builtin_amdgcn_readfirstlane(old);
-        WSTAMP(6);
-        if (old + cnt != NB) continue;
-        if (lane == 0) __hip_atomic_store(&p.counters[tile * COUNTER_STRIDE], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-
+    // ---- the owner of a tile's last unit finishes it: that can only be tile t0 (a range is at most one tile long)
+    if (bs + n < NB) return;
+    {
+        const int tile = t0;
         const int w_first = wave_of_unit(tile * NB);
-        const int ncontrib = wave_of_unit(tile * NB + NB - 1) - w_first + 1;
-        const float *all = p.partials + (size_t)tile * p.max_contrib * tile_elems;
+        const int ncontrib = v - w_first + 1;
+        uint64_t *const all = p.tagged + (size_t)tile * p.max_contrib * tile_elems;
         const int col0 = col0_of(tile);
         const int total = M << LOG_TC;
         // lane <-> element (row, tile column); with two strips the partner (same row and
@@ -358,19 +354,39 @@ __global__ __launch_bounds__(64 * NW) void gptq4_gemv_kernel(MatmulArgs p) {
         for (int e0 = 0; e0 < total; e0 += 64) {
             const int e = e0 + lane;
             const bool live = e < total;
-            const float *src = all + (live ? e : 0);
+            uint64_t *const src = all + (live ? e : 0);
             float s = 0.f;
             // every load is issued (contributors past the last one re-read the last slot),
             // so one round trip covers 16 slots
 #pragma unroll 1
             for (int c0 = 0; c0 < ncontrib; c0 += 16) {
-                float part[16];
+                uint64_t part[16];
+                uint32_t tries = p.spin_limit;
+                for (;;) {
 #pragma unroll
-                for (int k = 0; k < 16; ++k)
-                    part[k] = __hip_atomic_load(src + (size_t)min(c0 + k, ncontrib - 1) * tile_elems, __ATOMIC_RELAXED,
-                                                __HIP_MEMORY_SCOPE_AGENT);
+                    for (int k = 0; k < 16; ++k)
+                        part[k] = __hip_atomic_load(src + (size_t)min(c0 + k, ncontrib - 1) * tile_elems, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    uint64_t got = MARK;
 #pragma unroll
-                for (int k = 0; k < 16; ++k) s += (c0 + k < ncontrib) ? part[k] : 0.f;
+                    for (int k = 0; k < 16; ++k) got &= part[k];
+                    // (a limit of 0xFFFFFFFF is the test hook: give up even though everything has arrived)
+                    if (p.spin_limit != 0xFFFFFFFFu && __builtin_amdgcn_ballot_w64(live && got == 0) == 0) break;
+                    if (p.spin_limit == 0xFFFFFFFFu || --tries == 0) {
+                        // gave up: the call's result is not valid; the word stays set for the host to find
+                        if (lane == 0) __hip_atomic_store(&p.counters[EXCHANGE_ERROR_WORD], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep(1);
+                }
+#pragma unroll
+                for (int k = 0; k < 16; ++k) s += (c0 + k < ncontrib) ? __uint_as_float((uint32_t)part[k]) : 0.f;
+                // back to zero for the next call
+                if (live) {
+#pragma unroll
+                    for (int k = 0; k < 16; ++k)
+                        if (c0 + k < ncontrib)
+                            __hip_atomic_store(src + (size_t)(c0 + k) * tile_elems, (uint64_t)0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
             }
             const int row = e >> LOG_TC;
             const int c = e & (SW - 1);
@@ -471,7 +487,7 @@ uint32_t magic_of(int d) { return d > 1 ? (uint32_t)(0x100000000ull / (unsigned)
 
 }  // namespace
 
-GemvTuning g_gemv_tuning = {1, 0, 0, 0};
+GemvTuning g_gemv_tuning = {1, 0, 0, 0, 0};
 
 // Launch shape: the grid holds `waves_per_cu` waves per CU on all CUs of the device (or fewer
 // waves when there are fewer units than that), each wave owning q or q+1 units.
@@ -520,12 +536,13 @@ GemvPlan gemv_plan(int epi, int M, int N, int K, bool norm) {
     // (fewer units than waves: every unit has a wave of its own, a tile as many contributors as batches)
     pl.max_contrib = (pl.q > 0) ? (pl.nb + pl.q - 1) / pl.q + 1 : pl.nb;
     if (pl.max_contrib > pl.nb) pl.max_contrib = pl.nb;
+    if (gemv_tagged_bytes(pl, M, epi) > GPTQ4_WS_TAGGED_BYTES) pl.ok = false;
     return pl;
 }
 
-size_t gemv_partial_bytes(const GemvPlan &pl, int M, int epi) {
+size_t gemv_tagged_bytes(const GemvPlan &pl, int M, int epi) {
     const int tile_cols = 32 * (epi == EPI_PLAIN ? 1 : 2);
-    return (size_t)pl.tiles * pl.max_contrib * M * tile_cols * sizeof(float);
+    return (size_t)pl.tiles * pl.max_contrib * M * tile_cols * sizeof(uint64_t);
 }
 
 int launch_gemv(int epi, MatmulArgs &a, const GemvPlan &pl, hipStream_t stream) {
@@ -537,6 +554,7 @@ int launch_gemv(int epi, MatmulArgs &a, const GemvPlan &pl, hipStream_t stream) 
     a.lds_wave_chunks = pl.lds_wave_chunks;
     a.x_chunks_max = (pl.q + 1) << (4 + pl.m_shift);
     a.max_contrib = pl.max_contrib;
+    a.spin_limit = g_gemv_tuning.spin_limit ? g_gemv_tuning.spin_limit : (1u << 22);
     a.batches_per_group = a.groupsize / 128;
     a.groups = a.K / a.groupsize;
     a.group_magic = magic_of(a.batches_per_group);

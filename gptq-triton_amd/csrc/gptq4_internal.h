@@ -15,6 +15,8 @@ struct MatmulArgs {
     QMat w[2];        // w[1] only for EPI_SILU_MUL (w[0] = gate, w[1] = up)
     float *partials;
     int *counters;
+    uint64_t *tagged;     // small-M kernels: marked partial sums, GPTQ4_WS_TAGGED_BYTES of them behind the counters (split-K kernel: null = exchange through counters)
+    uint32_t spin_limit;  // small-M kernels: polls of a slot before a finishing wave gives up
     half_t *y;  // [M, N] (EPI_PLAIN, EPI_SILU_MUL)
     const half_t *bias;
     const int32_t *perm;
@@ -59,6 +61,7 @@ struct SkinnyPlan {
 };
 struct SkinnyTuning {
     int words, depth, splitk, waves;  // 0 = automatic
+    int exchange;                     // 0 = automatic, 1 = always arrival counters and plain partial sums
 };
 extern SkinnyTuning g_skinny_tuning;
 // standard_shape: ignore the tuning overrides of words, depth and waves (the split is still tunable)
@@ -78,11 +81,13 @@ struct GemvPlan {
 struct GemvTuning {
     int mode;                        // 0 never, 1 where it is the faster kernel, 2 wherever it can run
     int depth, waves, waves_per_cu;  // 0 = automatic
+    uint32_t spin_limit;             // 0 = the default bound on a finishing wave's polls
 };
 extern GemvTuning g_gemv_tuning;
 // norm: plan for the variant that normalises its own input (automatic launch shape, room for the rows in LDS)
 GemvPlan gemv_plan(int epi, int M, int N, int K, bool norm = false);
-size_t gemv_partial_bytes(const GemvPlan &plan, int M, int epi);
+// bytes of marked partial sums (8 per value) the plan exchanges; a plan is only ok while they fit GPTQ4_WS_TAGGED_BYTES
+size_t gemv_tagged_bytes(const GemvPlan &plan, int M, int epi);
 int launch_gemv(int epi, MatmulArgs &a, const GemvPlan &plan, hipStream_t stream);
 // Launch shape of the tiled kernel.
 struct GemmPlan {
@@ -146,6 +151,8 @@ DeviceShape device_shape();
 // arrival counters sit one per 128-byte line: atomics on one line are served one after
 // the other by the memory side
 enum { COUNTER_STRIDE = 32 };
+// word of the counter region (between two counter lines' first words) that a kernel sets when a bounded wait ran out
+enum { EXCHANGE_ERROR_WORD = 1 };
 // act-order: activations up to this many bytes are gathered into the workspace ahead of the kernel
 constexpr size_t ACT_ORDER_STAGE_MAX = (size_t)1 << 30;
 enum { GEMV_MAX_M = 4, SKINNY_MAX_M = 16, SKINNY_MAX_SPLITK = 16, SKINNY_MAX_TILES = 4096, GEMM_MAX_SPLITK = 16 };

@@ -324,7 +324,99 @@ __global__ __launch_bounds__(64 * NW) void gptq4_skinny_kernel(MatmulArgs p) {
     }
 
     PHASE_STAMP(2);
-    if (p.splitk > 1) {
+    if (p.splitk > 1 && p.tagged != nullptr) {
+        // Cross-workgroup exchange through marked values: every partial sum travels as one 8-byte
+        // {fp32 bits, 1} store (value and mark arrive together) into a region of the workspace that is zero
+        // whenever no call runs.  The workgroups of splits 0 .. splitk-2 store theirs and leave - no wait for
+        // the stores' completion, no arrival counter; the workgroup of the last split keeps its own sums in
+        // registers, polls the others' slots until every value it needs carries its mark, adds them in split
+        // order and writes the slots back to zero.  It waits only for workgroups with a lower blockIdx.y,
+        // dispatched before it, which never wait themselves; the wait is bounded all the same.
+        constexpr uint64_t MARK = 1ull << 32;
+        const size_t tile_elems = (size_t)M * TILE_COLS;
+        uint64_t *const slots = p.tagged + (size_t)tile * p.splitk * tile_elems;
+        if (split != p.splitk - 1) {
+            uint64_t *const mine = slots + (size_t)split * tile_elems;
+#pragma unroll
+            for (int q = 0; q < Q; ++q) {
+                const int row = ROWS_PER_PASS * q + rbase;
+                if (row < Mf) {
+#pragma unroll
+                    for (int v = 0; v < NV; ++v)
+                        __hip_atomic_store(&mine[(size_t)row * TILE_COLS + v * SW + c], MARK | (uint64_t)__float_as_uint(val[q][v]),
+                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+            PHASE_STAMP(3);
+            return;
+        }
+        // CH splits per round of polls, every element of the thread at once: 16 loads in flight per thread (more
+        // would cost the streaming loop a wave per SIMD in registers), and a round is one round trip however
+        // many elements and splits it covers
+        const int others = p.splitk - 1;
+        constexpr int CH = (Q * NV >= 8) ? 2 : (Q * NV >= 4) ? 4 : 8;
+        float sum[Q][NV];
+#pragma unroll
+        for (int q = 0; q < Q; ++q)
+#pragma unroll
+            for (int v = 0; v < NV; ++v) sum[q][v] = 0.f;
+        uint32_t tries = p.spin_limit;
+#pragma unroll 1
+        for (int c0 = 0; c0 < others; c0 += CH) {
+            uint64_t part[Q][NV][CH];
+            for (;;) {
+                uint64_t got = MARK;
+#pragma unroll
+                for (int q = 0; q < Q; ++q) {
+                    const int row = ROWS_PER_PASS * q + rbase;
+                    const uint64_t *const src = slots + (row < Mf ? (size_t)row * TILE_COLS + c : 0);
+#pragma unroll
+                    for (int v = 0; v < NV; ++v)
+#pragma unroll
+                        for (int k = 0; k < CH; ++k)  // (splits past the last one re-read the last slot)
+                            part[q][v][k] = __hip_atomic_load(src + v * SW + (size_t)min(c0 + k, others - 1) * tile_elems, __ATOMIC_RELAXED,
+                                                              __HIP_MEMORY_SCOPE_AGENT);
+                }
+#pragma unroll
+                for (int q = 0; q < Q; ++q)
+#pragma unroll
+                    for (int v = 0; v < NV; ++v)
+#pragma unroll
+                        for (int k = 0; k < CH; ++k) got &= (ROWS_PER_PASS * q + rbase < Mf) ? part[q][v][k] : MARK;
+                // (a limit of 0xFFFFFFFF is the test hook: give up even though everything has arrived)
+                if (p.spin_limit != 0xFFFFFFFFu && __builtin_amdgcn_ballot_w64(got == 0) == 0) break;
+                if (p.spin_limit == 0xFFFFFFFFu || --tries == 0) {
+                    // gave up: the call's result is not valid; the word stays set for the host to find
+                    if (lane == 0) __hip_atomic_store(&p.counters[EXCHANGE_ERROR_WORD], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    tries = 1;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(4);
+            }
+#pragma unroll
+            for (int q = 0; q < Q; ++q) {
+                const int row = ROWS_PER_PASS * q + rbase;
+                if (row < Mf) {
+                    uint64_t *const src = slots + (size_t)row * TILE_COLS + c;
+#pragma unroll
+                    for (int v = 0; v < NV; ++v)
+#pragma unroll
+                        for (int k = 0; k < CH; ++k)
+                            if (c0 + k < others) {
+                                // a fixed-order sum: splits 0 .. splitk-2, then this workgroup's own
+                                sum[q][v] += __uint_as_float((uint32_t)part[q][v][k]);
+                                // back to zero for the next call
+                                __hip_atomic_store(src + v * SW + (size_t)(c0 + k) * tile_elems, (uint64_t)0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                            }
+                }
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < Q; ++q)
+#pragma unroll
+            for (int v = 0; v < NV; ++v) val[q][v] = sum[q][v] + val[q][v];
+        PHASE_STAMP(5);
+    } else if (p.splitk > 1) {
         // Cross-workgroup exchange without cache maintenance: partial sums are written
         // and read with agent-scope (sc1) relaxed atomics, which are coherent across the
         // XCDs' L2s by themselves.  A release/acquire fence would add an L2 write-back
@@ -482,13 +574,13 @@ int launch_epi(const MatmulArgs &a, const SkinnyPlan &pl, hipStream_t stream) {
         case 424: return launch_variant<EPI, 2, 4, 4>(a, stream);
         case 441: return launch_variant<EPI, 4, 1, 4>(a, stream);
         case 442: return launch_variant<EPI, 4, 2, 4>(a, stream);
-        default: return launch_variant<EPI, 2, 2, 4>(a, stream);
+        default: return (int)hipErrorInvalidValue;  // skinny_plan only makes the pairs above
     }
 }
 
 }  // namespace
 
-SkinnyTuning g_skinny_tuning = {0, 0, 0, 0};
+SkinnyTuning g_skinny_tuning = {0, 0, 0, 0, 0};
 
 // Launch shape for a small-M problem, from sweeps on MI355X at LLaMA-7B / 13B / 30B shapes: split K until
 // there are ~1024 workgroups (4 per CU) but keep >= 2 batches per wave.  8-byte loads (32-column strips,
@@ -520,6 +612,10 @@ SkinnyPlan skinny_plan(int epi, int N, int K, bool standard_shape) {
         pl.depth = (epi == EPI_SILU_MUL) ? 1 : 2;
     }
     if (tuned && g_skinny_tuning.depth > 0) pl.depth = g_skinny_tuning.depth;
+    // the instantiated (width, depth) pairs: 4 bytes x {2, 4}, 8 bytes x {1, 2, 4}, 16 bytes x {1, 2}
+    if (pl.words == 1) pl.depth = (pl.depth <= 2) ? 2 : 4;
+    if (pl.words == 2 && pl.depth == 3) pl.depth = 2;
+    if (pl.words == 4 && pl.depth > 2) pl.depth = 2;
     const int sw = 16 * pl.words;
     pl.tiles = (epi == EPI_ROPE) ? (N / 128) * (64 / sw) : N / sw;
     int s;

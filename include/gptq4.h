@@ -29,10 +29,13 @@
  *    gathers by itself, which is slower).
  *  - `workspace` holds split-K partial sums, arrival counters and, for a call with
  *    `perm`, the gathered activations (M * K * 2 bytes).  Size it with
- *    gptq4_workspace_bytes() (selector | GPTQ4_OP_WITH_PERM for such calls); its first GPTQ4_WS_COUNTER_BYTES bytes must be zero
- *    before the FIRST call that uses it (each call leaves them zero again).  One
- *    workspace may be shared by all calls on one stream; calls that run
- *    concurrently on different streams need a workspace each.
+ *    gptq4_workspace_bytes() (selector | GPTQ4_OP_WITH_PERM for such calls); its first GPTQ4_WS_HEAD_BYTES bytes
+ *    (the arrival counters, then the region where the decode GEMV exchanges marked partial sums) must be zero
+ *    before the FIRST call that uses it (each call leaves them zero again).  Word GPTQ4_WS_ERROR_WORD (32-bit
+ *    words from the start) is the exception: a kernel whose bounded wait for another wave's partial sums ran
+ *    out sets it to 1 and it stays set - the results of that call are not valid and the workspace has to be
+ *    zeroed again before it is reused.  One workspace may be shared by all calls on one stream; calls that
+ *    run concurrently on different streams need a workspace each.
  */
 #ifndef GPTQ4_H
 #define GPTQ4_H
@@ -44,7 +47,7 @@
 extern "C" {
 #endif
 
-#define GPTQ4_ABI_VERSION 1
+#define GPTQ4_ABI_VERSION 2
 
 /* host-side argument errors (returned negated: -GPTQ4_E_SHAPE ...) */
 #define GPTQ4_E_NULL 1       /* a required pointer is NULL                       */
@@ -54,10 +57,14 @@ extern "C" {
 #define GPTQ4_E_ALIGN 5      /* a pointer is not 16-byte aligned                 */
 #define GPTQ4_E_STATIC_LIMIT 6 /* gptq4_matmul_static: the call needs more scratch than the library holds */
 
+/* head of a workspace, kept zero between calls: arrival counters, then marked partial sums (8 bytes each) */
 #define GPTQ4_WS_COUNTER_BYTES 524288
+#define GPTQ4_WS_TAGGED_BYTES (16u << 20)
+#define GPTQ4_WS_HEAD_BYTES (GPTQ4_WS_COUNTER_BYTES + GPTQ4_WS_TAGGED_BYTES)
+#define GPTQ4_WS_ERROR_WORD 1
 #define GPTQ4_KV_AT_POSITION (-1)
-/* scratch memory inside the library for gptq4_matmul_static: the counters plus 8 MiB of partial sums */
-#define GPTQ4_STATIC_SCRATCH_BYTES (GPTQ4_WS_COUNTER_BYTES + (8u << 20))
+/* scratch memory inside the library for gptq4_matmul_static: the head plus 8 MiB of partial sums */
+#define GPTQ4_STATIC_SCRATCH_BYTES (GPTQ4_WS_HEAD_BYTES + (8u << 20))
 
 /* operation selector for gptq4_workspace_bytes */
 #define GPTQ4_OP_MATMUL 0
@@ -280,7 +287,9 @@ void gptq4_set_chain_tuning(int ring_slots, int reserved, unsigned spin_limit, i
 
 /* Host-side launch tuning of the small-M kernels, for measurements: words per lane and
  * load (1, 2 or 4: strips of 16, 32 or 64 columns), batches of loads in flight per
- * wave (1..4) and the split-K factor; 0 = automatic for each.  Process-wide; not
+ * wave (1..4) and the split-K factor; 0 = automatic for each.  words + 10 (10 = automatic width): the workgroups
+ * that share a tile always exchange plain partial sums under an arrival counter; words + 20: marked 8-byte values
+ * wherever those fit GPTQ4_WS_TAGGED_BYTES (by default: up to 4 rows and few splits).  Process-wide; not
  * thread-safe against concurrent launches.  No reference counterpart (the reference
  * tunes through Triton's autotuner, custom_autotune.py:12-172). */
 void gptq4_set_tuning(int words, int depth, int splitk);
@@ -303,6 +312,11 @@ void gptq4_set_midm_tuning(int mode, int mt, int splitk);
  * flight per wave (1..3), waves per workgroup (4, 8, 16), waves per CU (4..32), 0 =
  * automatic. */
 void gptq4_set_gemv_tuning(int mode, int depth, int waves, int waves_per_cu);
+/* How often a finishing wave of the small-M kernels polls for another wave's marked partial sums before it gives up
+ * and sets GPTQ4_WS_ERROR_WORD (0 = the default, about four million polls).  0xFFFFFFFF is the hook for tests of
+ * that error path: every finishing wave polls once and gives up whatever it found, and every kernel still ends
+ * normally.  No reference counterpart. */
+void gptq4_set_exchange_spin_limit(unsigned polls);
 
 #ifdef __cplusplus
 }

@@ -52,7 +52,7 @@ def test_gemv_leaves_the_workspace_head_zero(forced_gemv):
     gptq().matmul4(g, xd, D["qweight"], D["scales"], D["qzeros"])
     ws = _lib.workspace(xd.device, 0)
     torch.cuda.synchronize()
-    assert int(ws[:_lib.WS_COUNTER_BYTES].view(torch.int32).abs().sum()) == 0
+    assert int(ws[:_lib.WS_HEAD_BYTES].view(torch.int32).abs().sum()) == 0
 
 
 @pytest.mark.parametrize("m", [1, 4])

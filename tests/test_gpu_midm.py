@@ -52,7 +52,7 @@ def test_midm_leaves_the_workspace_head_zero(forced_midm):
     gptq().matmul4(g, xd, D["qweight"], D["scales"], D["qzeros"])
     ws = _lib.workspace(xd.device, 0)
     torch.cuda.synchronize()
-    assert int(ws[:_lib.WS_COUNTER_BYTES].view(torch.int32).abs().sum()) == 0
+    assert int(ws[:_lib.WS_HEAD_BYTES].view(torch.int32).abs().sum()) == 0
 
 
 def test_midm_one_hot_rows_reproduce_weight_rows(forced_midm):
@@ -170,7 +170,7 @@ def test_act_order_inputs_reach_the_mid_m_kernel_through_the_staged_copy():
     ref = O.quant_matmul_ref(x, L["qweight"], L["qzeros"], L["scales"], g, g_idx=L["g_idx"])
     assert_close(y.cpu().numpy(), ref, "act-order through the C ABI, M=48")
     need = lib.gptq4_workspace_bytes(_lib.OP_MATMUL | _lib.OP_WITH_PERM, m, k, n)
-    assert need >= _lib.WS_COUNTER_BYTES + m * k * 2
+    assert need >= _lib.WS_HEAD_BYTES + m * k * 2
     # a workspace sized for a call without `perm`: room for any partial sums, none promised for the rows
     y.zero_()
     rc = lib.gptq4_matmul(xd.data_ptr(), Wq.data_ptr(), D["qzeros"].data_ptr(), D["scales"].data_ptr(), perm.data_ptr(), None,

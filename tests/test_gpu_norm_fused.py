@@ -133,7 +133,7 @@ def test_norm_in_the_balanced_gemv_equals_two_launches(balanced_gemv, m):
     from gptq_triton_amd import _lib
     ws = _lib.workspace(hd.device, 0)
     torch.cuda.synchronize()
-    assert int(ws[:_lib.WS_COUNTER_BYTES].view(torch.int32).abs().sum()) == 0
+    assert int(ws[:_lib.WS_HEAD_BYTES].view(torch.int32).abs().sum()) == 0
 
 
 @pytest.mark.parametrize("gemv_mode", [0, 2])

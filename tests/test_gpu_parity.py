@@ -178,7 +178,7 @@ def test_splitk_variants_agree_and_counters_reset(splitk):
     assert_close(y1.cpu().numpy(), ref, f"splitk={splitk}")
     ws = _lib.workspace(xd.device, 0)
     torch.cuda.synchronize()
-    assert int(ws[:_lib.WS_COUNTER_BYTES].view(torch.int32).abs().sum()) == 0
+    assert int(ws[:_lib.WS_HEAD_BYTES].view(torch.int32).abs().sum()) == 0
 
 
 # --------------------------------------------------------------------------- fused MLP

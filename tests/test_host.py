@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol():
     for name in names:
         assert hasattr(lib, name), f"{name} declared in include/gptq4.h but not exported"
     assert set(names) == set(_lib.SIGNATURES), "ctypes binding and header disagree"
-    assert lib.gptq4_abi_version() == 1
+    assert lib.gptq4_abi_version() == 2
 
 
 def test_error_codes_are_returned_before_any_launch():
@@ -65,7 +65,7 @@ def test_error_codes_are_returned_before_any_launch():
 
 def test_workspace_query():
     lib = _lib.load()
-    base = _lib.WS_COUNTER_BYTES
+    base = _lib.WS_HEAD_BYTES
     assert lib.gptq4_workspace_bytes(_lib.OP_MATMUL, 4096, 4096, 12288) == base   # enough tiles: no split-K, only the counters
     one = lib.gptq4_workspace_bytes(_lib.OP_MATMUL, 1, 4096, 4096)
     assert one >= base + 16 * 1 * 4096 * 4                    # 16 split-K slots at least; the decode GEMV may want more
@@ -214,8 +214,8 @@ def test_mid_m_plan_is_declared_and_tunable():
     for args in ((0, 0, 0), (2, 1, 3), (1, 0, 0)):
         lib.gptq4_set_midm_tuning(*args)
     # the workspace query covers whichever kernel the plans pick for a mid-sized call
-    assert lib.gptq4_workspace_bytes(_lib.OP_MATMUL, 64, 4096, 4096) >= _lib.WS_COUNTER_BYTES
-    assert lib.gptq4_workspace_bytes(_lib.OP_QKV_ROTARY, 128, 4096, 12288) >= _lib.WS_COUNTER_BYTES
+    assert lib.gptq4_workspace_bytes(_lib.OP_MATMUL, 64, 4096, 4096) >= _lib.WS_HEAD_BYTES
+    assert lib.gptq4_workspace_bytes(_lib.OP_QKV_ROTARY, 128, 4096, 12288) >= _lib.WS_HEAD_BYTES
 
 
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
