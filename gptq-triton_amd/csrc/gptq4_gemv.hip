@@ -509,11 +509,12 @@ GemvPlan gemv_plan(int epi, int M, int N, int K, bool norm) {
     total_waves = (long)pl.workgroups * pl.waves;
     pl.q = (int)(units / total_waves);
     pl.r = (int)(units % total_waves);
-    // measured on MI355X at LLaMA-7B shapes: ahead of the split-K kernel for the one-row
-    // gate/up pair (344 tiles, the shape that divides worst by 256 CUs: 16.0 against
-    // 17.0 us), level with it for the one-row plain projections and behind it for more
-    // rows and for the rotary epilogue
-    const bool wanted = g_gemv_tuning.mode == 2 || (g_gemv_tuning.mode == 1 && M == 1 && epi == EPI_SILU_MUL);
+    // measured on MI355X at LLaMA-7B / 13B / 30B shapes, one row: ahead of the split-K kernel for the gate/up
+    // pair (15.0 against 17.6 us, 20.3 / 23.8, 32.2 / 32.4) and, from 13B on, for QKV with the rotary epilogue
+    // (7B 12.1 against 11.1 us, 13B 14.5 / 15.8, 30B 20.2 / 23.4: the crossover is put at 8192 units); within
+    // 3 % either way for o_proj, behind for down_proj (7B 12.6 against 10.8 us) and everywhere from 2 rows on
+    const bool wanted = g_gemv_tuning.mode == 2 ||
+                        (g_gemv_tuning.mode == 1 && M == 1 && (epi == EPI_SILU_MUL || (epi == EPI_ROPE && units >= 8192)));
     pl.ok = wanted && M >= 1 && M <= GEMV_MAX_M && pl.tiles <= SKINNY_MAX_TILES && pl.q + 1 <= pl.nb &&
             units < (1L << 24) && (long)K * N < (1L << 32) && (long)M * K < (1L << 30);
     int mshift = 0;

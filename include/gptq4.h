@@ -107,9 +107,10 @@ int gptq4_matmul(const void *x, const int32_t *qweight, const int32_t *qzeros,
                  size_t workspace_bytes, void *stream);
 
 /* gptq4_matmul for callers that cannot allocate device memory (code under HIP graph capture, tight serving
- * loops, harnesses that forbid hipMalloc): no workspace argument - the arrival counters and split-K partial
- * sums live in a fixed array inside the library (GPTQ4_STATIC_SCRATCH_BYTES = 8.5 MiB per GPU, held until the
- * process ends), and the call itself allocates and frees nothing.  No reference counterpart.
+ * loops, harnesses that forbid hipMalloc): no workspace argument - the workspace head (arrival counters, marked
+ * partial sums) and 8 MiB of split-K partial sums live in a fixed array inside the library
+ * (GPTQ4_STATIC_SCRATCH_BYTES = 24.5 MiB per GPU, held until the process ends), and the call itself allocates and
+ * frees nothing.  No reference counterpart.
  * Same kernels and results as gptq4_matmul without `perm` (act-order calls need room for the gathered
  * rows: use gptq4_matmul).  Calls whose workspace requirement - gptq4_workspace_bytes(GPTQ4_OP_MATMUL, M, K, N) -
  * exceeds the array return -GPTQ4_E_STATIC_LIMIT and launch nothing; decode-sized calls fit up to
