@@ -240,6 +240,9 @@ void gptq4_set_gemm_tuning(int mt, int splitk) {
 
 void gptq4_set_midm_tuning(int mode, int mt, int splitk) {
     g_kslice_tuning.mode = (mode >= 0 && mode <= 2) ? mode : 1;
+    // 100 + mt: four waves per workgroup, 200 + mt: eight where they fit (automatic: eight for plain projections)
+    g_kslice_tuning.waves = (mt >= 200) ? 8 : (mt >= 100) ? 4 : 0;
+    mt %= 100;
     // 10 + mt: 128-column strips for plain projections; a plain 1 or 2 also pins the 64-column strips
     g_kslice_tuning.wide = (mt >= 10) ? 1 : ((mt == 1 || mt == 2) ? -1 : 0);
     if (mt >= 10) mt -= 10;

@@ -112,12 +112,14 @@ struct KslicePlan {
     int splitk;  // workgroups sharing one tile along K, on top of the split inside the workgroup
     int tiles;
     bool wide;   // plain epilogue: 128-column strips (two blocks per wave tile) instead of 64
+    int waves;   // waves per workgroup, each with its own slice of K (4 or 8)
     bool ok;     // false: the shape needs another kernel
 };
 struct KsliceTuning {
     int mode;        // 0 never, 1 where it is the faster kernel, 2 wherever it can run
     int mt, splitk;  // 0 = automatic
     int wide;        // plain epilogue: 1 = 128-column strips, -1 = 64-column strips, 0 = automatic
+    int waves;       // waves per workgroup: 4, 8, 0 = automatic
 };
 extern KsliceTuning g_kslice_tuning;
 KslicePlan kslice_plan(int epi, int M, int N, int K, bool has_perm);

@@ -22,17 +22,34 @@
 // chip; the partial sums exchanged are the workgroup's already reduced tile.
 #include "gptq4_internal.h"
 
+// Development aid, compiled out of the product build: per-workgroup stamps of the 100 MHz clock at the
+// phase boundaries of the kernel, written 32 MiB into the workspace (size it so).
+#ifdef GPTQ4_PHASE_TIMERS
+#define KS_STAMP(i)                                                                                             \
+    do {                                                                                                        \
+        if (threadIdx.x == 0)                                                                                   \
+            reinterpret_cast<unsigned long long *>(reinterpret_cast<char *>(p.counters) + (32 << 20))[(blockIdx.y * gridDim.x + blockIdx.x) * 8 + (i)] = \
+                wall_clock64();                                                                                 \
+    } while (0)
+#else
+#define KS_STAMP(i)
+#endif
+
 namespace {
 
 constexpr int BK = 64;
 
 // WIDE (plain epilogue only): two adjacent 64-column blocks per wave tile, like a rotary head.
-template <int EPI, int MT, bool WIDE>
-__global__ __launch_bounds__(256, 2) void gptq4_kslice_kernel(MatmulArgs p) {
+// KS: waves of the workgroup, each with its own slice of K (4 or 8).  A wave spends about half of its life
+// waiting (first loads, the exchanges at the end) and the other half issuing ~20 instructions per MFMA, one wave
+// per SIMD; the matrix cores are busy 15 % of the time (SQ counters at 128 rows, 4096 x 4096).  A second wave
+// per SIMD overlaps the two.  8 waves with 64-row tiles are 128 KiB of LDS: one workgroup per CU.
+template <int EPI, int MT, bool WIDE, int KS>
+__global__ __launch_bounds__(64 * KS, KS == 8 && MT == 2 ? 1 : 2) void gptq4_kslice_kernel(MatmulArgs p) {
+    static_assert(KS == 4 || KS == 8, "four or eight waves");
     static_assert(!WIDE || EPI == EPI_PLAIN, "the other epilogues have two blocks already");
     constexpr bool ADJ = (EPI == EPI_ROPE) || WIDE;     // the second block is columns + 64 of the same matrix
     constexpr int BM = 32 * MT;
-    constexpr int KS = 4;                               // all four waves along K
     constexpr int NB = (EPI == EPI_PLAIN && !WIDE) ? 1 : 2;  // 64-column blocks of the wave tile
     constexpr int BN = ADJ ? 128 : 64;                  // output columns of the workgroup
     constexpr int NSET = NB;                            // value sets the finishing wave combines
@@ -42,15 +59,16 @@ __global__ __launch_bounds__(256, 2) void gptq4_kslice_kernel(MatmulArgs p) {
     // Per-wave activation tiles (two objects, so that the compiler can tell the loads into one
     // from the reads of the other).  Afterwards the same memory is MT * 4 exchange regions of
     // 8 KiB: region (mt, w) = accumulators of row block mt from wave w.
-    __shared__ __attribute__((aligned(16))) half_t As0[4 * A_HALVES];
-    __shared__ __attribute__((aligned(16))) half_t As1[4 * A_HALVES];
-    static_assert(2 * 4 * A_HALVES * sizeof(half_t) >= (size_t)MT * 4 * 32 * 64 * sizeof(float), "exchange regions do not fit");
+    __shared__ __attribute__((aligned(16))) half_t As0[KS * A_HALVES];
+    __shared__ __attribute__((aligned(16))) half_t As1[KS * A_HALVES];
+    static_assert(2 * KS * A_HALVES * sizeof(half_t) >= (size_t)MT * KS * 32 * 64 * sizeof(float), "exchange regions do not fit");
     auto region = [&](int mt, int w) -> float * {
-        const int r = mt * 4 + w;
-        constexpr int HALF = MT * 2;
+        const int r = mt * KS + w;
+        constexpr int HALF = MT * KS / 2;
         return reinterpret_cast<float *>(r < HALF ? As0 : As1) + (r < HALF ? r : r - HALF) * (32 * 64);
     };
 
+    KS_STAMP(0);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -204,10 +222,8 @@ __global__ __launch_bounds__(256, 2) void gptq4_kslice_kernel(MatmulArgs p) {
             // Loads complete in order and this wave issued 4 * NB packed-word loads after the
             // scale/zero words that followed its LDS-direct loads of this tile: at most that
             // many outstanding means the tile has landed.  It is this wave's own tile: no barrier.
-            if (NB == 1)
-                asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
-            else
-                asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
+            // (lgkmcnt: the fragment reads of the tile before are done before its buffer is requested again.)
+            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(4 * NB) : "memory");
             dma_a(nxt, min(kt + 1, nk - 1));
             load_group2(par);
             h8_t araw[MT];
@@ -240,6 +256,7 @@ __global__ __launch_bounds__(256, 2) void gptq4_kslice_kernel(MatmulArgs p) {
                 }
             }
         };
+        KS_STAMP(1);
         int kt = k_begin;
         for (; kt + 1 < nk; kt += 2) {
             k_tile(buf0, buf1, kt, 0);
@@ -250,14 +267,20 @@ __global__ __launch_bounds__(256, 2) void gptq4_kslice_kernel(MatmulArgs p) {
     // every LDS-direct load has landed and every wave is done reading before the tiles are
     // reused for the exchange
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    KS_STAMP(3);
     __syncthreads();
 
-    // ---- the four accumulator sets meet: row block mt goes to wave mt, one column block at a time.
+    // ---- the KS accumulator sets meet, one column block at a time.  Row block mt is finished by PARTS waves
+    // (one with four waves, two with eight): wave mt * PARTS + part takes registers i = part * IW .. + IW - 1.
     // acc[j][mt][t][i]: row = 32*mt + 8*(i/4) + 4*lhi + i%4 of the tile, column = 2*l32 + t of block j.
-    // vals[j]: the sums the epilogue combines - plain: the strip; SiLU*mul: gate and up; rotary:
-    // columns d < 64 and d >= 64 of the head.  Only waves < MT hold any.
-    float vals[NSET][2][16];
-    const bool owner = wave < MT;
+    // vals[j][t][ii], i = part * IW + ii: the sums the epilogue combines - plain: the strip; SiLU*mul: gate and
+    // up; rotary: columns d < 64 and d >= 64 of the head.  Only waves < MT * PARTS hold any.
+    constexpr int PARTS = KS / 4;
+    constexpr int IW = 16 / PARTS;
+    float vals[NSET][2][IW];
+    const bool owner = wave < MT * PARTS;
+    const int own_mt = wave / PARTS, part = wave % PARTS;
+    const int i0 = part * IW;
 #pragma unroll
     for (int j = 0; j < NB; ++j) {
         if (j > 0) __syncthreads();  // the owners are done reading the previous block
@@ -271,28 +294,32 @@ __global__ __launch_bounds__(256, 2) void gptq4_kslice_kernel(MatmulArgs p) {
         }
         __syncthreads();
         if (owner) {
-            const float *src[4];
+            const float *src[KS];
 #pragma unroll
-            for (int w = 0; w < 4; ++w) src[w] = region(wave, w) + lane;
+            for (int w = 0; w < KS; ++w) src[w] = region(own_mt, w) + i0 * 64 + lane;
 #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    float v[4];
+                for (int ii = 0; ii < IW; ++ii) {
+                    float v[KS];
 #pragma unroll
-                    for (int w = 0; w < 4; ++w) v[w] = src[w][(t * 16 + i) * 64];
-                    vals[j][t][i] = ((v[0] + v[1]) + v[2]) + v[3];
+                    for (int w = 0; w < KS; ++w) v[w] = src[w][(t * 16 + ii) * 64];
+                    float sum = v[0];
+#pragma unroll
+                    for (int w = 1; w < KS; ++w) sum += v[w];
+                    vals[j][t][ii] = sum;
                 }
         }
     }
 
+    KS_STAMP(4);
+    constexpr int NREG = NSET * 2 * IW;  // values per lane of an owner wave
     if (p.splitk > 1) {
         // K split across workgroups as well: each publishes its reduced tile (agent-scope
         // atomics, no cache maintenance), the last one to arrive sums them in split order.
         __shared__ int s_is_last;
-        constexpr int NREG = NSET * 32;
         const int tile = logical;
-        const size_t per_split = (size_t)MT * NREG * 64;
+        const size_t per_split = (size_t)MT * PARTS * NREG * 64;
         float *const mine = p.partials + ((size_t)tile * p.splitk + split) * per_split + (size_t)wave * NREG * 64 + lane;
         if (owner) {
 #pragma unroll
@@ -300,56 +327,67 @@ __global__ __launch_bounds__(256, 2) void gptq4_kslice_kernel(MatmulArgs p) {
 #pragma unroll
                 for (int t = 0; t < 2; ++t)
 #pragma unroll
-                    for (int i = 0; i < 16; ++i)
-                        __hip_atomic_store(mine + ((s * 2 + t) * 16 + i) * 64, vals[s][t][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    for (int ii = 0; ii < IW; ++ii)
+                        __hip_atomic_store(mine + ((s * 2 + t) * IW + ii) * 64, vals[s][t][ii], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        KS_STAMP(5);
         __syncthreads();
         if (tid == 0) {
             const int old = __hip_atomic_fetch_add(&p.counters[tile * COUNTER_STRIDE], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             s_is_last = (old == p.splitk - 1);
         }
         __syncthreads();
+        KS_STAMP(6);
         if (!s_is_last) return;
         if (owner) {
+            // E of the lane's values from SPR splits per round, 32 loads in flight per lane: a round is one round trip
+            constexpr int E = NREG < 32 ? NREG : 32;
+            constexpr int SPR = 32 / E;
             const float *const all = p.partials + (size_t)tile * p.splitk * per_split + (size_t)wave * NREG * 64 + lane;
 #pragma unroll
-            for (int s = 0; s < NSET; ++s)
+            for (int e0 = 0; e0 < NREG; e0 += E) {
+                float sum[E];
 #pragma unroll
-                for (int t = 0; t < 2; ++t)
+                for (int e = 0; e < E; ++e) sum[e] = 0.f;
+#pragma unroll 1
+                for (int c0 = 0; c0 < p.splitk; c0 += SPR) {
+                    float got[SPR][E];
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) vals[s][t][i] = 0.f;
-            for (int sp = 0; sp < p.splitk; ++sp) {
+                    for (int k = 0; k < SPR; ++k)
 #pragma unroll
-                for (int s = 0; s < NSET; ++s)
+                        for (int e = 0; e < E; ++e)  // (past the last split: the last one again, not added)
+                            got[k][e] = __hip_atomic_load(all + (size_t)min(c0 + k, p.splitk - 1) * per_split + (e0 + e) * 64, __ATOMIC_RELAXED,
+                                                          __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
-                    for (int t = 0; t < 2; ++t) {
-                        float got[16];
+                    for (int k = 0; k < SPR; ++k)
 #pragma unroll
-                        for (int i = 0; i < 16; ++i)
-                            got[i] = __hip_atomic_load(all + (size_t)sp * per_split + ((s * 2 + t) * 16 + i) * 64, __ATOMIC_RELAXED,
-                                                       __HIP_MEMORY_SCOPE_AGENT);
+                        for (int e = 0; e < E; ++e) sum[e] += (c0 + k < p.splitk) ? got[k][e] : 0.f;
+                }
 #pragma unroll
-                        for (int i = 0; i < 16; ++i) vals[s][t][i] += got[i];
-                    }
+                for (int e = 0; e < E; ++e) {
+                    const int f = e0 + e;  // = (s * 2 + t) * IW + ii
+                    vals[f / (2 * IW)][(f / IW) & 1][f % IW] = sum[e];
+                }
             }
         }
         if (tid == 0) __hip_atomic_store(&p.counters[tile * COUNTER_STRIDE], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     if (!owner) return;
 
-    // ---- epilogue of row block `wave`
-    const int row0 = m0 + wave * 32 + 4 * lhi;
+    // ---- epilogue of registers i0 .. i0 + IW - 1 of row block own_mt
+    const int row0 = m0 + own_mt * 32 + 4 * lhi;
+    auto row_of = [&](int ii) { return row0 + 8 * ((i0 + ii) >> 2) + ((i0 + ii) & 3); };
     if (EPI == EPI_PLAIN) {
 #pragma unroll
         for (int j = 0; j < NSET; ++j) {
             h2_t bias2 = {(half_t)0.f, (half_t)0.f};
             if (p.bias != nullptr) bias2 = as_h2(*reinterpret_cast<const uint32_t *>(p.bias + ncol + 64 * j));
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int row = row0 + 8 * (i >> 2) + (i & 3);
+            for (int ii = 0; ii < IW; ++ii) {
+                const int row = row_of(ii);
                 if (row < M) {
-                    h2_t o = {(half_t)vals[j][0][i], (half_t)vals[j][1][i]};
+                    h2_t o = {(half_t)vals[j][0][ii], (half_t)vals[j][1][ii]};
                     if (p.bias != nullptr) o = o + bias2;
                     *reinterpret_cast<uint32_t *>(p.y + (size_t)row * N + ncol + 64 * j) = as_u32(o);
                 }
@@ -357,11 +395,11 @@ __global__ __launch_bounds__(256, 2) void gptq4_kslice_kernel(MatmulArgs p) {
         }
     } else if (EPI == EPI_SILU_MUL) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int row = row0 + 8 * (i >> 2) + (i & 3);
+        for (int ii = 0; ii < IW; ++ii) {
+            const int row = row_of(ii);
             if (row < M) {
-                const h2_t o = {(half_t)(silu_f32(vals[0][0][i]) * vals[NSET - 1][0][i]),
-                                (half_t)(silu_f32(vals[0][1][i]) * vals[NSET - 1][1][i])};
+                const h2_t o = {(half_t)(silu_f32(vals[0][0][ii]) * vals[NSET - 1][0][ii]),
+                                (half_t)(silu_f32(vals[0][1][ii]) * vals[NSET - 1][1][ii])};
                 *reinterpret_cast<uint32_t *>(p.y + (size_t)row * N + n0 + 2 * l32) = as_u32(o);
             }
         }
@@ -376,33 +414,33 @@ __global__ __launch_bounds__(256, 2) void gptq4_kslice_kernel(MatmulArgs p) {
         const size_t seq_stride = (size_t)r.H * cap * 128;
         const bool at_position = (which != 0) && r.kv_offset < 0;  // cache row = the token's position
         const int row_shift = (which == 0 || r.kv_offset < 0) ? 0 : r.kv_offset;
-        float2 cs[16], sn[16];
-        int pos[16];
+        float2 cs[IW], sn[IW];
+        int pos[IW];
         if (which < 2 || at_position) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) pos[i] = max(r.position_ids[min(row0 + 8 * (i >> 2) + (i & 3), M - 1)], 0);
+            for (int ii = 0; ii < IW; ++ii) pos[ii] = max(r.position_ids[min(row_of(ii), M - 1)], 0);
         }
         if (which < 2) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int tp = min(pos[i], r.max_pos - 1);
-                cs[i] = *reinterpret_cast<const float2 *>(r.cos_table + (size_t)tp * 64 + 2 * l32);
-                sn[i] = *reinterpret_cast<const float2 *>(r.sin_table + (size_t)tp * 64 + 2 * l32);
+            for (int ii = 0; ii < IW; ++ii) {
+                const int tp = min(pos[ii], r.max_pos - 1);
+                cs[ii] = *reinterpret_cast<const float2 *>(r.cos_table + (size_t)tp * 64 + 2 * l32);
+                sn[ii] = *reinterpret_cast<const float2 *>(r.sin_table + (size_t)tp * 64 + 2 * l32);
             }
         }
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int row = row0 + 8 * (i >> 2) + (i & 3);
-            float lo0 = vals[0][0][i], lo1 = vals[0][1][i], hi0 = vals[NSET - 1][0][i], hi1 = vals[NSET - 1][1][i];
+        for (int ii = 0; ii < IW; ++ii) {
+            const int row = row_of(ii);
+            float lo0 = vals[0][0][ii], lo1 = vals[0][1][ii], hi0 = vals[NSET - 1][0][ii], hi1 = vals[NSET - 1][1][ii];
             if (which < 2) {
-                const float a0 = lo0 * cs[i].x - hi0 * sn[i].x, a1 = lo1 * cs[i].y - hi1 * sn[i].y;
-                const float b0 = hi0 * cs[i].x + lo0 * sn[i].x, b1 = hi1 * cs[i].y + lo1 * sn[i].y;
+                const float a0 = lo0 * cs[ii].x - hi0 * sn[ii].x, a1 = lo1 * cs[ii].y - hi1 * sn[ii].y;
+                const float b0 = hi0 * cs[ii].x + lo0 * sn[ii].x, b1 = hi1 * cs[ii].y + lo1 * sn[ii].y;
                 lo0 = a0, lo1 = a1, hi0 = b0, hi1 = b1;
             }
             if (row < M) {
                 int bb, srow;
                 split_row(r, row, bb, srow);
-                const int crow = at_position ? min(pos[i], r.kv_capacity - 1) : srow + row_shift;
+                const int crow = at_position ? min(pos[ii], r.kv_capacity - 1) : srow + row_shift;
                 half_t *const at = dst + (size_t)bb * seq_stride + (size_t)crow * 128;
                 const h2_t olo = {(half_t)lo0, (half_t)lo1}, ohi = {(half_t)hi0, (half_t)hi1};
                 *reinterpret_cast<uint32_t *>(at) = as_u32(olo);
@@ -410,32 +448,44 @@ __global__ __launch_bounds__(256, 2) void gptq4_kslice_kernel(MatmulArgs p) {
             }
         }
     }
+    KS_STAMP(7);
 }
 
-template <int EPI, int MT, bool WIDE>
+template <int EPI, int MT, bool WIDE, int KS>
 int launch_one(const MatmulArgs &a, int tiles, hipStream_t stream) {
-    dim3 grid((unsigned)tiles, (unsigned)a.splitk), block(256);
-    hipLaunchKernelGGL((gptq4_kslice_kernel<EPI, MT, WIDE>), grid, block, 0, stream, a);
+    dim3 grid((unsigned)tiles, (unsigned)a.splitk), block(64 * KS);
+    hipLaunchKernelGGL((gptq4_kslice_kernel<EPI, MT, WIDE, KS>), grid, block, 0, stream, a);
     return (int)hipGetLastError();
+}
+
+template <int EPI, int KS>
+int launch_waves(const MatmulArgs &a, const KslicePlan &pl, hipStream_t stream) {
+    if (EPI == EPI_PLAIN && pl.wide)
+        return pl.mt == 1 ? launch_one<EPI_PLAIN, 1, true, KS>(a, pl.tiles, stream) : launch_one<EPI_PLAIN, 2, true, KS>(a, pl.tiles, stream);
+    return pl.mt == 1 ? launch_one<EPI, 1, false, KS>(a, pl.tiles, stream) : launch_one<EPI, 2, false, KS>(a, pl.tiles, stream);
 }
 
 template <int EPI>
 int launch_epi(const MatmulArgs &a, const KslicePlan &pl, hipStream_t stream) {
-    if (EPI == EPI_PLAIN && pl.wide)
-        return pl.mt == 1 ? launch_one<EPI_PLAIN, 1, true>(a, pl.tiles, stream) : launch_one<EPI_PLAIN, 2, true>(a, pl.tiles, stream);
-    return pl.mt == 1 ? launch_one<EPI, 1, false>(a, pl.tiles, stream) : launch_one<EPI, 2, false>(a, pl.tiles, stream);
+    return pl.waves == 8 ? launch_waves<EPI, 8>(a, pl, stream) : launch_waves<EPI, 4>(a, pl, stream);
 }
 
 }  // namespace
 
-KsliceTuning g_kslice_tuning = {1, 0, 0, 0};
+KsliceTuning g_kslice_tuning = {1, 0, 0, 0, 0};
 
-// Row tile: 32 rows up to M = 32, else 64 (128-row tiles decode each weight once instead of
-// twice at M = 128, but their 128 KiB of LDS leaves one wave per SIMD and they come out no
-// faster).  How far K is split across workgroups on top is scored below.
+// Row tile: 32 rows up to M = 32, else 64.  (128-row tiles decode each weight once instead of twice at M = 128 and
+// halve the instructions per MFMA, but came out no faster: 17.3 against 15.1 us on 4096 x 4096, level on
+// 11008 x 4096.  Four activation tiles per wave instead of two - the tile three K tiles on requested while one is
+// multiplied - gained nothing that eight waves do not gain as well.)  How far K is split across workgroups on top is
+// scored below.
 KslicePlan kslice_plan(int epi, int M, int N, int K, bool has_perm) {
     KslicePlan pl = {};
-    const int ks = 4;
+    // eight waves for plain projections wherever they fit (checked below): ahead of four waves by 4 - 18 % at
+    // LLaMA-7B / 30B shapes from 17 to 256 rows, level at 512; the gate/up pair and the rotary epilogue stay at four
+    // (two column blocks per wave tile need the registers of a whole SIMD; 7B QKV loses 3 % with eight)
+    pl.waves = g_kslice_tuning.waves ? g_kslice_tuning.waves : (epi == EPI_PLAIN ? 8 : 4);
+    int ks = pl.waves;
     // plain projections: 128-column strips (half the activation traffic per weight byte, half the tiles) pay
     // from 256 rows on when K is long (LLaMA-7B down_proj: 39.8 -> 37.3 us at 256 rows, 66.2 -> 61.1 at 512;
     // o_proj with K = 4096 loses below 512 rows)
@@ -445,31 +495,45 @@ KslicePlan kslice_plan(int epi, int M, int N, int K, bool has_perm) {
     pl.mt = g_kslice_tuning.mt ? g_kslice_tuning.mt : (M <= 32 ? 1 : 2);
     const int bm = 32 * pl.mt;
     pl.tiles = ((M + bm - 1) / bm) * (N / bn);
-    int s = 1;
-    if (g_kslice_tuning.splitk > 0) {
-        s = g_kslice_tuning.splitk;
-    } else {
-        // Score 1..8 splits by how evenly tiles * s workgroups fill 256 CUs holding two each (w / 256 up to 256,
-        // else w / (512 * ceil(w / 512)), never below 0.8 from 512 workgroups on: with several rounds the
-        // scheduler evens things out), every extra split at 4 % + 15 / (K tiles) of the time, at least 4 K
-        // tiles per wave.  Fitted to sweeps at LLaMA-7B / 13B / 30B shapes, 32..256 rows: on average 1 % off
-        // the best split (a fixed target of 512 workgroups: 2.3 %, worst case 17 %).
-        const double pen = 0.04 + 15.0 / (double)nk;
-        const long cus = device_shape().cus;  // 256 on MI355X
-        double best = -1.0;
-        for (int c = 1; c <= 8 && c <= nk / (4 * ks); ++c) {
-            const long w = (long)pl.tiles * c;
-            double e = (w <= cus) ? (double)w / (double)cus : (double)w / ((double)(2 * cus) * (double)((w + 2 * cus - 1) / (2 * cus)));
-            if (w >= 2 * cus && e < 0.8) e = 0.8;
-            const double score = e / (1.0 + pen * (c - 1));
-            if (score > best + 1e-9) {
-                best = score;
-                s = c;
+    const long cus = device_shape().cus;  // 256 on MI355X
+    auto choose_split = [&](int ks) {
+        int s = 1;
+        if (g_kslice_tuning.splitk > 0) {
+            s = g_kslice_tuning.splitk;
+        } else {
+            // Score 1..8 splits by how evenly tiles * s workgroups fill 256 CUs holding two each (w / 256 up to 256,
+            // else w / (512 * ceil(w / 512)), never below 0.8 from 512 workgroups on: with several rounds the
+            // scheduler evens things out), every extra split at 4 % + 15 / (K tiles) of the time, at least 4 K
+            // tiles per wave.  Fitted to sweeps at LLaMA-7B / 13B / 30B shapes, 32..256 rows: on average 1 % off
+            // the best split (a fixed target of 512 workgroups: 2.3 %, worst case 17 %).
+            const double pen = 0.04 + 15.0 / (double)nk;
+            double best = -1.0;
+            for (int c = 1; c <= 8 && c <= nk / (4 * ks); ++c) {
+                const long w = (long)pl.tiles * c;
+                double e = (w <= cus) ? (double)w / (double)cus : (double)w / ((double)(2 * cus) * (double)((w + 2 * cus - 1) / (2 * cus)));
+                if (w >= 2 * cus && e < 0.8) e = 0.8;
+                const double score = e / (1.0 + pen * (c - 1));
+                if (score > best + 1e-9) {
+                    best = score;
+                    s = c;
+                }
             }
         }
+        if (s > GEMM_MAX_SPLITK) s = GEMM_MAX_SPLITK;
+        if (s < 1 || pl.tiles > SKINNY_MAX_TILES) s = 1;
+        return s;
+    };
+    int s = choose_split(ks);
+    // eight waves: 128 KiB of LDS with 64-row tiles, so only in launches of at most one workgroup per CU; with 32-row
+    // tiles two workgroups share a CU and four waves a SIMD, which leaves each 128 registers - enough for one
+    // column block per wave tile only; and every wave needs a K tile or two
+    if (pl.waves == 8) {
+        const int nb = (epi == EPI_PLAIN && !pl.wide) ? 1 : 2;
+        if ((pl.mt == 2 && (long)pl.tiles * s > cus) || (pl.mt == 1 && nb == 2) || nk / s < 16) {
+            pl.waves = ks = 4;
+            s = choose_split(ks);
+        }
     }
-    if (s > GEMM_MAX_SPLITK) s = GEMM_MAX_SPLITK;
-    if (s < 1 || pl.tiles > SKINNY_MAX_TILES) s = 1;
     pl.splitk = s;
     // the wave loop needs the activations unpermuted and at least one K tile per wave
     pl.ok = !has_perm && (N % bn) == 0 && nk / s >= ks;
@@ -477,6 +541,7 @@ KslicePlan kslice_plan(int epi, int M, int N, int K, bool has_perm) {
 }
 
 size_t kslice_partial_bytes(int epi, const KslicePlan &pl) {
+    // (the same with four or eight waves: eight split the 32 values per lane and block over two owner waves)
     const int nset = (epi == EPI_PLAIN && !pl.wide) ? 1 : 2;
     return pl.splitk > 1 ? (size_t)pl.tiles * pl.splitk * pl.mt * nset * 32 * 64 * sizeof(float) : 0;
 }

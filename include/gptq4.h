@@ -302,10 +302,11 @@ void gptq4_set_tuning(int words, int depth, int splitk);
 void gptq4_set_gemm_tuning(int mt, int splitk);
 
 /* Same for the mid-M kernel (M > 16 with too few wide tiles for the tiled kernel; K is split
- * across the four waves of a workgroup): mode 0 = never use it, 1 = where it is the faster
+ * across the four or eight waves of a workgroup): mode 0 = never use it, 1 = where it is the faster
  * kernel, 2 = wherever it can run; 32-row blocks per row tile (1, 2; 10 + that, or 10 alone, also
- * selects 128-column strips for plain projections, a plain 1 or 2 the 64-column strips) and the
- * split-K factor across workgroups; 0 = automatic. */
+ * selects 128-column strips for plain projections, a plain 1 or 2 the 64-column strips; 100 + any of
+ * these: four waves per workgroup, 200 +: eight where they fit) and the split-K factor across
+ * workgroups; 0 = automatic. */
 void gptq4_set_midm_tuning(int mode, int mt, int splitk);
 
 /* Same for the balanced decode GEMV (M <= 4): mode 0 = never use it, 1 = where it is the
