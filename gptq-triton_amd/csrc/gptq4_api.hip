@@ -124,7 +124,7 @@ int setup_gemm(MatmulArgs &a, const GemmPlan &pl, void *workspace, size_t worksp
     const int nk = a.K / 64;
     a.slot_q = nk / pl.splitk;
     a.slot_rem = nk % pl.splitk;
-    if (pl.splitk > 1) {
+    if (pl.splitk > 1 || pl.streamed) {
         if (workspace == nullptr || workspace_bytes < GPTQ4_WS_HEAD_BYTES + gemm_partial_bytes(pl))
             return -GPTQ4_E_WORKSPACE;
         a.counters = reinterpret_cast<int *>(workspace);
@@ -168,11 +168,17 @@ int run_tiled(int epi, MatmulArgs &a, void *workspace, size_t workspace_bytes, h
     // kernel can run too); else the tiled kernel gathers by itself
     const size_t rows_bytes = (size_t)a.M * a.K * sizeof(half_t);
     bool stage = a.perm != nullptr && !g_gemm_tuning.own_gather && rows_bytes <= ACT_ORDER_STAGE_MAX;
-    const GemmPlan pl = gemm_plan(epi, a.M, a.N, a.K);
+    GemmPlan pl = gemm_plan(epi, a.M, a.N, a.K, a.perm != nullptr && !stage);
+    // the streamed schedule keeps 128 MiB of partial sums: without the room for them, the unstreamed plan
+    if (pl.streamed && (workspace == nullptr || workspace_bytes < GPTQ4_WS_HEAD_BYTES + gemm_partial_bytes(pl) + (stage ? rows_bytes : 0))) {
+        g_stream_off = true;
+        pl = gemm_plan(epi, a.M, a.N, a.K, a.perm != nullptr && !stage);
+        g_stream_off = false;
+    }
     if (stage) {
         const KslicePlan kp = kslice_plan(epi, a.M, a.N, a.K, false);
         const size_t partial = prefer_kslice(kp, epi, a.M, a.N, a.K) ? (kp.splitk > 1 ? kslice_partial_bytes(epi, kp) : 0)
-                                                                       : (pl.splitk > 1 ? gemm_partial_bytes(pl) : 0);
+                                                                       : gemm_partial_bytes(pl);
         if (workspace == nullptr || workspace_bytes < GPTQ4_WS_HEAD_BYTES + partial + rows_bytes) stage = false;
     }
     const KslicePlan kp = kslice_plan(epi, a.M, a.N, a.K, a.perm != nullptr && !stage);
@@ -197,7 +203,7 @@ int run_tiled(int epi, MatmulArgs &a, void *workspace, size_t workspace_bytes, h
     int rc = setup_gemm(a, pl, workspace, workspace_bytes);
     if (rc) return rc;
     if (stage) {
-        rc = stage_act_order(a, pl.splitk > 1 ? gemm_partial_bytes(pl) : 0, workspace, workspace_bytes, s);
+        rc = stage_act_order(a, gemm_partial_bytes(pl), workspace, workspace_bytes, s);
         if (rc) return rc;
     }
     return launch_gemm(epi, a, pl, s);
@@ -231,6 +237,9 @@ const char *gptq4_strerror(int code) {
 }
 
 void gptq4_set_gemm_tuning(int mt, int splitk) {
+    // 100: never the streamed schedule, 200: the streamed schedule wherever it can run (both with automatic tile and split)
+    g_gemm_tuning.streamed = (mt == 100) ? 1 : (mt == 200) ? 2 : 0;
+    if (mt >= 100) mt = 0;
     // 10 + mt: act-order calls use the tiled kernel's own gather (no staging of the activations)
     g_gemm_tuning.own_gather = (mt >= 10) ? 1 : 0;
     if (mt >= 10) mt -= 10;
@@ -368,8 +377,12 @@ int gptq4_matmul_static(const void *x, const int32_t *qweight, const int32_t *qz
     int g = groupsize;
     int rc = check_dims(K, N, &g);
     if (rc) return rc;
-    // what the same call would ask of a caller's workspace has to fit the static array
-    if (gptq4_workspace_bytes(GPTQ4_OP_MATMUL, M, K, N) > (size_t)GPTQ4_STATIC_SCRATCH_BYTES) return -GPTQ4_E_STATIC_LIMIT;
+    // what the same call would ask of a caller's workspace - planned without the streamed schedule of the tiled
+    // kernel, whose partial sums alone are 128 MiB - has to fit the static array
+    g_stream_off = true;
+    const size_t need = gptq4_workspace_bytes(GPTQ4_OP_MATMUL, M, K, N);
+    g_stream_off = false;
+    if (need > (size_t)GPTQ4_STATIC_SCRATCH_BYTES) return -GPTQ4_E_STATIC_LIMIT;
     void *ws = nullptr;
     rc = static_scratch(&ws);
     if (rc) return rc;

@@ -43,8 +43,17 @@ namespace {
 constexpr int BK = 64;
 constexpr int LDS_ROW = BK + 8;  // halves; 144-byte rows keep 128-bit reads conflict-free
 
-template <int EPI, int MT, bool PERM>
+// STREAM: the workgroups do not own tiles.  The K tiles of all output tiles form one sequence (in the tile order
+// described below), and workgroup g of the resident grid takes the g-th of gridDim.x equal ranges of it: the
+// end of one tile, whole tiles, the beginning of another.  Every CU slot then has the same amount of work whatever
+// the tile count - with tiles dealt whole, 344 tiles on 512 slots leave a third of the slots idle while the CUs
+// that got two set the pace, and 768 tiles are a pair and then a single one per CU.  A tile cut by a range
+// boundary is finished like a split-K tile: its parts are exchanged through the workspace, the last to arrive
+// adds them in K order and runs the epilogue; nobody waits for anybody.  (Measured slower than whole tiles at the
+// shapes of the plan's comment, so only the tuning hook selects it.)
+template <int EPI, int MT, bool PERM, bool STREAM = false>
 __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
+    static_assert(!STREAM || !PERM, "act-order calls reach the streamed schedule with gathered activations");
     constexpr int NW = 4;        // waves
     constexpr int NT = 64 * NW;  // threads
     constexpr int WM = (MT == 4) ? 1 : 2;  // waves along M
@@ -83,7 +92,13 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
 
     const int M = p.M, K = p.K, N = p.N;
     const int tiles_m = (M + BM - 1) / BM;
+    __shared__ int s_is_last;
+    constexpr bool ROPE_TAB = (EPI == EPI_ROPE) && (MT == 4);
+    extern __shared__ __attribute__((aligned(16))) float rope_tab[];  // ROPE_TAB: [2 buffers][cos, sin][32 tokens][64]
 
+    // One (part of a) tile: K tiles [k_begin, nk) of tile `logical`, which `nsplit` workgroups share; this one is
+    // number `idx` of them in K order.  part_slot(c): where sharer c keeps its partial sums.
+    auto run_part = [&](const int logical, const int k_begin, const int nk, const int nsplit, const int idx, auto part_slot) {
     // XCD-contiguous logical tile index: workgroups that run at the same time on one XCD (one
     // L2) have consecutive logical indices.  These walk GROUP_M row tiles, then move to the
     // next column panel, and only after the last panel to the next GROUP_M row tiles: the
@@ -93,10 +108,6 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
     // activation tile by two, and the activation tiles are the larger stream).
     constexpr int GROUP_M = 8;
     const int tiles_n = N / BN;
-    const int total = gridDim.x;
-    const int per = total >> 3, rem = total & 7;
-    const int xcd = blockIdx.x & 7;
-    const int logical = xcd * per + (xcd < rem ? xcd : rem) + (blockIdx.x >> 3);
     const int band = logical / (GROUP_M * tiles_n);  // band of GROUP_M row tiles
     const int in_band = logical - band * (GROUP_M * tiles_n);
     const int band_rows = min(GROUP_M, tiles_m - band * GROUP_M);
@@ -131,8 +142,6 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
     // become free.  Read from memory per lane instead (16 tokens x 2 tables in registers, after the positions
     // they depend on, once per block of 32 rows), the epilogue is four round trips to memory long with the
     // matrix cores idle: the two workgroups of a CU start together and so reach it together.
-    constexpr bool ROPE_TAB = (EPI == EPI_ROPE) && (MT == 4);
-    extern __shared__ __attribute__((aligned(16))) float rope_tab[];  // ROPE_TAB: [2 buffers][cos, sin][32 tokens][64]
     bool need_tab = false;
     int tab_voff[4][2];  // per block and unit of 4 tokens: byte offset of the lane's 16-byte chunk in the tables
     __amdgpu_buffer_rsrc_t cos_rsrc, sin_rsrc;
@@ -166,12 +175,7 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
         }
     };
 
-    // K tiles [k_begin, nk) of this split (host-side quotient / remainder, no division here
-    // except the one that finds the first group)
-    const int split = blockIdx.y;
-    const int k_begin = split * p.slot_q + min(split, p.slot_rem);
-    const int nk = k_begin + p.slot_q + (split < p.slot_rem ? 1 : 0);
-    int group = (p.splitk > 1) ? k_begin / tiles_per_group : 0;
+    int group = (k_begin > 0) ? k_begin / tiles_per_group : 0;
     int left_in_group = tiles_per_group - (k_begin - group * tiles_per_group);  // K tiles left in the group
     if constexpr (PERM) {
         // ---- act-order path: the activations are gathered through registers (x_sorted[k] =
@@ -413,14 +417,13 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     }
 
-    if (p.splitk > 1) {
-        // Split-K for problems with too few tiles to fill the chip: every split publishes its
-        // fp32 accumulators (agent-scope atomics, no cache maintenance - see the small-M
-        // kernel), the last one to arrive sums them in split order and runs the epilogue.
-        __shared__ int s_is_last;
+    if (nsplit > 1) {
+        // Split-K for problems with too few tiles to fill the chip (or a tile cut by the streamed schedule): every
+        // sharer publishes its fp32 accumulators (agent-scope atomics, no cache maintenance - see the small-M
+        // kernel), the last one to arrive sums them in K order and runs the epilogue.
         constexpr int NREG = MT * 32;
         const int tile = logical;
-        float *const mine = p.partials + ((size_t)tile * p.splitk + split) * (NREG * NT) + tid;
+        float *const mine = p.partials + part_slot(idx) * (NREG * NT) + tid;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -433,18 +436,18 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
         __syncthreads();
         if (tid == 0) {
             const int old = __hip_atomic_fetch_add(&p.counters[tile * COUNTER_STRIDE], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            s_is_last = (old == p.splitk - 1);
+            s_is_last = (old == nsplit - 1);
         }
         __syncthreads();
         if (!s_is_last) return;
-        const float *const all = p.partials + (size_t)tile * p.splitk * (NREG * NT) + tid;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
             for (int t = 0; t < 2; ++t)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) acc[mt][t][i] = 0.f;
-        for (int sp = 0; sp < p.splitk; ++sp) {
+        for (int sp = 0; sp < nsplit; ++sp) {
+            const float *const theirs = p.partials + part_slot(sp) * (NREG * NT) + tid;
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -454,8 +457,7 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
                     float got[16];
 #pragma unroll
                     for (int i = 0; i < 16; ++i)
-                        got[i] = __hip_atomic_load(all + ((size_t)sp * NREG + (mt * 2 + t) * 16 + i) * NT,
-                                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        got[i] = __hip_atomic_load(theirs + ((mt * 2 + t) * 16 + i) * NT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
                     for (int i = 0; i < 16; ++i) acc[mt][t][i] += got[i];
                 }
@@ -642,6 +644,47 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
             }
         }
     }
+    };  // run_part
+
+    if constexpr (!STREAM) {
+        // one tile (or one K split of it) per workgroup; K tiles of the split by host-side quotient / remainder
+        const int total = gridDim.x;
+        const int per = total >> 3, rem = total & 7;
+        const int xcd = blockIdx.x & 7;
+        const int logical = xcd * per + (xcd < rem ? xcd : rem) + (blockIdx.x >> 3);
+        const int split = blockIdx.y;
+        const int k_begin = split * p.slot_q + min(split, p.slot_rem);
+        const int nk = k_begin + p.slot_q + (split < p.slot_rem ? 1 : 0);
+        const int nsplit = p.splitk;
+        run_part(logical, k_begin, nk, nsplit, split, [&](int c) { return (size_t)logical * nsplit + c; });
+    } else {
+        // Range of this workgroup in the sequence of all K tiles.  g: its rank with the workgroups of one XCD
+        // (blockIdx.x % 8) adjacent, so that an XCD works on one stretch of the tile order, as it does unstreamed.
+        const int S = gridDim.x;  // a multiple of 8
+        const int nkt = K / BK;
+        const long U = (long)p.tiles * nkt;
+        const int g = (blockIdx.x & 7) * (S >> 3) + (blockIdx.x >> 3);
+        auto start_of = [&](int w) { return (int)((long)w * U / S); };
+        const int u1 = start_of(g + 1);
+        for (int u = start_of(g); u < u1;) {
+            const int tile = u / nkt;
+            const int kb = u - tile * nkt;
+            const int ke = min(nkt, kb + (u1 - u));
+            // the sharers of this tile: workgroups whose ranges meet [tile * nkt, (tile + 1) * nkt)
+            const long x0 = (long)tile * nkt, x1 = x0 + nkt;
+            const int g_first = (int)(((x0 + 1) * S + U - 1) / U) - 1;  // the last workgroup that starts at or before x0
+            const int g_last = (int)((x1 * S + U - 1) / U) - 1;         // the last one that starts before x1
+            // a sharer keeps the part with which its range begins in slot 0 and the one with which it ends in
+            // slot 1: only the first sharer of a tile can hold the tile at the end of its range
+            const bool first_ends_here = start_of(g_first) < (int)x0;
+            run_part(tile, kb, ke, g_last - g_first + 1, g - g_first,
+                     [&](int c) { return (size_t)(g_first + c) * 2 + ((c == 0 && first_ends_here) ? 1 : 0); });
+            u += ke - kb;
+            // the epilogue's exchange regions (and table buffers) are the next part's activation tiles
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+            __syncthreads();
+        }
+    }
 }
 
 template <int EPI, int MT>
@@ -668,14 +711,35 @@ int launch_one(const MatmulArgs &a, int tiles, hipStream_t stream) {
     return (int)hipGetLastError();
 }
 
+// The streamed schedule: wide tiles only, a grid of exactly the workgroups that are resident at one time.
+template <int EPI>
+int launch_streamed(const MatmulArgs &a, int workgroups, hipStream_t stream) {
+    dim3 grid((unsigned)workgroups), block(256);
+    const size_t lds = (EPI == EPI_ROPE) ? 2 * 2 * 32 * 64 * sizeof(float) : 0;
+    if (a.perm != nullptr) return (int)hipErrorInvalidValue;
+    if (lds) {
+        static bool allowed = false;
+        if (!allowed) {
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gptq4_gemm_kernel<EPI, 4, false, true>),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return (int)e;
+            allowed = true;
+        }
+    }
+    hipLaunchKernelGGL((gptq4_gemm_kernel<EPI, 4, false, true>), grid, block, lds, stream, a);
+    return (int)hipGetLastError();
+}
+
 template <int EPI>
 int launch_epi(const MatmulArgs &a, const GemmPlan &pl, hipStream_t stream) {
+    if (pl.streamed) return launch_streamed<EPI>(a, pl.streamed, stream);
     return pl.mt == 4 ? launch_one<EPI, 4>(a, pl.tiles, stream) : launch_one<EPI, 2>(a, pl.tiles, stream);
 }
 
 }  // namespace
 
-GemmTuning g_gemm_tuning = {0, 0, 0};
+GemmTuning g_gemm_tuning = {0, 0, 0, 0};
+thread_local bool g_stream_off = false;
 
 // Tile shape and split-K factor of the tiled kernel.  The wide tile (128 x 256, half as
 // wide for SiLU*mul) is the faster one as soon as there are enough of them to give three
@@ -692,9 +756,10 @@ static double fill_efficiency(long w) {
     return (double)w / ((double)(2 * cus) * (double)((w + 2 * cus - 1) / (2 * cus)));
 }
 
-GemmPlan gemm_plan(int epi, int M, int N, int K) {
+GemmPlan gemm_plan(int epi, int M, int N, int K, bool has_perm) {
     GemmPlan pl;
     pl.score = 1.0;
+    pl.streamed = 0;
     const int bn2 = (epi == EPI_SILU_MUL) ? 64 : 128;  // tile width at MT = 2; twice that at MT = 4
     const int nk = K / 64;
     const long wide = (long)((M + 127) / 128) * (N / (2 * bn2));
@@ -741,10 +806,33 @@ GemmPlan gemm_plan(int epi, int M, int N, int K) {
     if (s > nk) s = nk;
     if (s < 1 || pl.tiles > SKINNY_MAX_TILES) s = 1;
     pl.splitk = s;
+    // The streamed schedule (wide tiles; the K tiles of all of them dealt evenly to the 2 x CUs workgroups that are
+    // resident at one time) is never chosen automatically: it evens out the work - 344 tiles on 512 slots, or 768 (a
+    // pair and then a single one per CU) - but every workgroup then exchanges a 128 KiB tile of fp32 partial sums,
+    // 128 MB per launch, at the moment all of them finish, and that costs more than the idle slots did.  Measured at
+    // LLaMA-7B / 13B / 30B shapes, 512 .. 4096 rows: 0 - 25 % slower (7B gate/up at 512 rows 122 -> 133 us, QKV at
+    // 2048 rows 216 -> 240), ahead only where K is long and the tile count large (30B down_proj at 4096 rows
+    // 970 -> 942 us).  gptq4_set_gemm_tuning(200, 0) runs it wherever it can run.
+    const long slots = 2 * cus;
+    const bool can_stream = !has_perm && !g_stream_off && g_gemm_tuning.streamed == 2 && g_gemm_tuning.mt == 0 && g_gemm_tuning.splitk == 0 &&
+                            wide >= 1 && wide <= SKINNY_MAX_TILES;
+    if (can_stream) {
+        // every workgroup of the grid needs at least one K tile (the sharers of a tile are counted from the
+        // ranges), and the grid is a multiple of 8 (the XCDs)
+        const long grid = (wide * nk < slots ? wide * nk : slots) & ~7L;
+        if (grid >= 8) {
+            pl.mt = 4;
+            pl.tiles = (int)wide;
+            pl.splitk = 1;
+            pl.streamed = (int)grid;
+        }
+    }
     return pl;
 }
 
 size_t gemm_partial_bytes(const GemmPlan &pl) {
+    // streamed: two slots of a whole wide tile per workgroup (the part that begins its range, the part that ends it)
+    if (pl.streamed) return (size_t)pl.streamed * 2 * (4 * 32 * 256) * sizeof(float);
     return pl.splitk > 1 ? (size_t)pl.tiles * pl.splitk * (pl.mt * 32 * 256) * sizeof(float) : 0;
 }
 

@@ -95,13 +95,18 @@ struct GemmPlan {
     int splitk;  // workgroups sharing one tile along K
     int tiles;
     double score;  // expected efficiency of the choice: fill of the chip / cost of the splits (1 where the tile count is large)
+    int streamed;  // 0, or the grid of the streamed schedule (wide tiles, K tiles of all tiles dealt evenly to that many workgroups)
 };
 struct GemmTuning {
     int mt, splitk;  // 0 = automatic
     int own_gather;  // 1: act-order calls run the tiled kernel's own gather instead of staging the activations
+    int streamed;    // 0 = automatic, 1 = never, 2 = wherever it can run
 };
 extern GemmTuning g_gemm_tuning;
-GemmPlan gemm_plan(int epi, int M, int N, int K);
+// set around a call that must not plan the streamed schedule (its partial sums would not fit the caller's scratch memory)
+extern thread_local bool g_stream_off;
+// has_perm: the kernel will gather act-order activations itself (no streamed schedule then)
+GemmPlan gemm_plan(int epi, int M, int N, int K, bool has_perm = false);
 size_t gemm_partial_bytes(const GemmPlan &plan);
 // Tiled matrix-core GEMM for any M.  Returns hipError_t.
 int launch_gemm(int epi, const MatmulArgs &a, const GemmPlan &plan, hipStream_t stream);

@@ -298,7 +298,9 @@ void gptq4_set_tuning(int words, int depth, int splitk);
 /* Same for the tiled (M > 16) kernel: workgroup tile (mt = 2: 128 x 128, mt = 4: 128 x 256
  * outputs; half as wide for the fused gate/up) and the split-K factor; 0 = automatic.
  * mt = 10, 12 or 14: the same tile choice, and act-order calls use the tiled kernel's own
- * gather of the activations instead of the copy staged in the workspace. */
+ * gather of the activations instead of the copy staged in the workspace.  mt = 200: the streamed
+ * schedule (K tiles of all wide tiles dealt evenly to the resident workgroups; never chosen
+ * automatically, it measured slower) wherever it can run, mt = 100: never; tile and split automatic with both. */
 void gptq4_set_gemm_tuning(int mt, int splitk);
 
 /* Same for the mid-M kernel (M > 16 with too few wide tiles for the tiled kernel; K is split

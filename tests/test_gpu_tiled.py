@@ -12,8 +12,10 @@ from test_gpu_parity import assert_close, gptq
 
 pytestmark = pytest.mark.gpu
 
-# (32-row blocks per wave: 2 = 128 x 128 tile, 4 = 128 x 256 tile; split-K); 0 = automatic
-CONFIGS = [(2, 1), (4, 1), (2, 3), (4, 2), (0, 0)]
+# (32-row blocks per wave: 2 = 128 x 128 tile, 4 = 128 x 256 tile; split-K); 0 = automatic; 200 = the streamed
+# schedule (K tiles of all wide tiles dealt evenly to 512 workgroups: at these sizes one K tile each and up to
+# 64 sharers per tile), 100 = never streamed
+CONFIGS = [(2, 1), (4, 1), (2, 3), (4, 2), (0, 0), (200, 0), (100, 0)]
 
 
 @pytest.fixture(params=CONFIGS, ids=lambda c: "mt%d_s%d" % c)
@@ -107,6 +109,56 @@ def test_tiled_rotary_by_position_with_positions_outside_the_table(forced_tiled)
         untouched = torch.ones(cap, dtype=torch.bool)
         untouched[cache_row[bi]] = False
         assert bool((kc[bi][:, untouched] == 7.0).all()) and bool((vc[bi][:, untouched] == 7.0).all())
+
+
+@pytest.mark.parametrize("m", [1100, 2048])
+def test_streamed_schedule_at_prefill_size(m):
+    """The streamed schedule on a tile count that does not divide by the resident workgroups (1100 rows x 8192
+    columns = 9 x 32 wide tiles, the last row tile ragged; 2048 x 8192 = 512 tiles, one each): every workgroup gets
+    the same number of K tiles, tiles cut by a range boundary are finished by whoever arrives last.  Against the
+    oracle on sampled rows and the tile-boundary rows, and against the unstreamed schedule within rounding (the
+    partial sums meet in another order); two calls give the same bits."""
+    from gptq_triton_amd import _lib
+    lib = _lib.load()
+    G = gptq()
+    k, n, g, heads = 2048, 8192, 128, 16
+    L = O.make_layer(k, n, g, seed=700, bias=True)
+    up = O.make_layer(k, n, g, seed=701)
+    qkv = O.make_layer(k, 3 * k, g, seed=702)
+    x = O.make_x(m, k, seed=703)
+    xd = torch.from_numpy(x).cuda()
+    D, Du, Dq = to_dev(L), to_dev(up), to_dev(qkv)
+    cos, sin = G.RotaryTable(128, 4096).get(torch.device("cuda"), 4096)
+    pos = np.arange(m, dtype=np.int32)[None, :]
+    pd = torch.from_numpy(pos).cuda()
+    out = {}
+    lib.gptq4_set_midm_tuning(0, 0, 0)
+    try:
+        for mode in (200, 100):
+            lib.gptq4_set_gemm_tuning(mode, 0)
+            y = G.matmul4(g, xd, D["qweight"], D["scales"], D["qzeros"], D["bias"])
+            y2 = G.matmul4(g, xd, D["qweight"], D["scales"], D["qzeros"], D["bias"])
+            assert torch.equal(y, y2)
+            h = G.llama_mlp_4(g, xd, D["qweight"], D["scales"], D["qzeros"], Du["qweight"], Du["scales"], Du["qzeros"])
+            q, kk, vv = G.qkv_rotary(g, xd.view(1, m, k), Dq["qweight"], Dq["scales"], Dq["qzeros"], pd, cos, sin, heads)
+            out[mode] = (y, h, q, kk, vv)
+    finally:
+        lib.gptq4_set_gemm_tuning(0, 0)
+        lib.gptq4_set_midm_tuning(1, 0, 0)
+    for a, b, name in zip(out[200], out[100], ("matmul", "gate/up", "q", "k", "v")):
+        a, b = a.float(), b.float()
+        assert bool(((a - b).abs() <= 2e-3 + 2e-3 * b.abs()).all()), f"{name}: streamed and unstreamed schedules differ beyond rounding"
+    rows = sorted(set([0, 1, 127, 128, 129, 1023, 1024, m - 129, m - 1] + list(np.random.default_rng(5).integers(0, m, 24))))
+    xs = x[rows]
+    y, h, q, kk, vv = out[200]
+    assert_close_bias = O.within_tolerance(y[rows].cpu().numpy(), O.quant_matmul_ref(xs, L["qweight"], L["qzeros"], L["scales"], g, bias=L["bias"]))
+    assert assert_close_bias[0], assert_close_bias[1]
+    href = O.mlp_gateup_ref(xs, (L["qweight"], L["qzeros"], L["scales"]), (up["qweight"], up["qzeros"], up["scales"]), g)
+    assert_close(h[rows].cpu().numpy(), href, f"streamed gate/up M={m}")
+    qr, kr, vr = O.qkv_rotary_ref(xs.reshape(1, len(rows), k), qkv["qweight"], qkv["qzeros"], qkv["scales"], g, pos[:, rows], heads, 128,
+                                  max_pos=4096)
+    for got, want, name in ((q, qr, "q"), (kk, kr, "k"), (vv, vr, "v")):
+        assert_close(got[:, :, rows].cpu().numpy(), want, f"streamed {name} M={m}")
 
 
 def test_prefill_sized_call_takes_the_wide_tiles_by_itself():
