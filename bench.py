@@ -17,10 +17,23 @@ Also reported on the same line:
                 the 8 TB/s HBM peak
   cpu_baseline  the PyTorch CPU dequantise-then-fp32-matmul path (oracle/torch_cpu.py)
                 on the host cores for 1 of the 32 layers, extrapolated to a token
-  extra         per-operator decode timings ("hot" = one layer's weights over and over, served by
+                (+ step_frac: the weights of the whole 128-launch step over the step time;
+                traffic: HBM bytes per launch from rocprofv3 counters, a constant taken from
+                profiles/decode_gemv_llama7b_m1.md, see traffic_source)
+  extra         baseline_configs: one row per configuration of BASELINE.json that fits this
+                path - C1 QuantLinear 4096 x 4096 (one group) at M = 1 and 128, C2 the fused
+                MLP (gate/up + SiLU*mul, then down; groupsize 128) at M = 1, 16 and 512, C3
+                fused QKV + rotary (one group) at M = 1 (position 2047) and M = 2048 - each
+                with its time, algorithmic bytes and flops, and the fraction of the HBM or
+                fp16 MFMA peak that bounds it;
+                decoders: the whole-decoder workloads below (7B, 13B act-order, 30B at batch
+                1 and 8), unless --no-decoders;
+                per-operator decode timings ("hot" = one layer's weights over and over, served by
                 the Infinity Cache; everything else streams from HBM), batched and prefill
                 TFLOP/s (M = 16 ... 8192) and the vendor library's dense fp16 GEMM on the
                 M = 2048 shapes
+  --chain-probe / --chain-timeline: the chained decode launch (gptq4_decode_chain) against the
+                separate launches it would replace
 
 Other workloads (--workload llama7b | llama13b | llama30b): a full random-init decoder of
 that shape (embedding, RMSNorm, fused QKV + rotary into a preallocated KV cache, torch
@@ -461,7 +474,7 @@ def main():
                 "frac": round(gu_gbs / HBM_PEAK_GBS, 4),
                 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
                 # `bench.py --traffic-probe`, scaled by a 256 MiB copy (x2.000 / x1.000)
-                "traffic": 50_601_000 + 1_286_000,
+                "traffic": 51_322_000 + 3_561_000,
                 "traffic_source": "constant: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this kernel, profiles/decode_gemv_llama7b_m1.md",
                 "step_frac": round(LAYERS * layer_bytes / ms_per_step / 1e6 / HBM_PEAK_GBS, 4),
                 "step_GBps": round(LAYERS * layer_bytes / ms_per_step / 1e6, 1),
