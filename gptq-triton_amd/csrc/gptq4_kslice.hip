@@ -460,9 +460,18 @@ int launch_one(const MatmulArgs &a, int tiles, hipStream_t stream) {
 
 template <int EPI, int KS>
 int launch_waves(const MatmulArgs &a, const KslicePlan &pl, hipStream_t stream) {
-    if (EPI == EPI_PLAIN && pl.wide)
-        return pl.mt == 1 ? launch_one<EPI_PLAIN, 1, true, KS>(a, pl.tiles, stream) : launch_one<EPI_PLAIN, 2, true, KS>(a, pl.tiles, stream);
-    return pl.mt == 1 ? launch_one<EPI, 1, false, KS>(a, pl.tiles, stream) : launch_one<EPI, 2, false, KS>(a, pl.tiles, stream);
+    if constexpr (KS == 8) {
+        // 32-row tiles with two column blocks per wave tile are never planned with eight waves (kslice_plan)
+        if (EPI == EPI_PLAIN && !pl.wide)
+            return pl.mt == 1 ? launch_one<EPI_PLAIN, 1, false, 8>(a, pl.tiles, stream) : launch_one<EPI_PLAIN, 2, false, 8>(a, pl.tiles, stream);
+        if (pl.mt == 1) return (int)hipErrorInvalidValue;
+        if (EPI == EPI_PLAIN) return launch_one<EPI_PLAIN, 2, true, 8>(a, pl.tiles, stream);
+        return launch_one<EPI, 2, false, 8>(a, pl.tiles, stream);
+    } else {
+        if (EPI == EPI_PLAIN && pl.wide)
+            return pl.mt == 1 ? launch_one<EPI_PLAIN, 1, true, KS>(a, pl.tiles, stream) : launch_one<EPI_PLAIN, 2, true, KS>(a, pl.tiles, stream);
+        return pl.mt == 1 ? launch_one<EPI, 1, false, KS>(a, pl.tiles, stream) : launch_one<EPI, 2, false, KS>(a, pl.tiles, stream);
+    }
 }
 
 template <int EPI>
