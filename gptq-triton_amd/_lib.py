@@ -116,8 +116,9 @@ def current_stream(device: torch.device):
     return torch.cuda.current_stream(device).cuda_stream
 
 
-# One workspace per (device, stream): split-K partials + arrival counters (+ the gathered rows of
-# an act-order call).  The counter region must start zeroed; the kernels restore it to zero.
+# One workspace per (device, stream): arrival counters and the marked partial sums of the small-M kernels (the
+# head, WS_HEAD_BYTES), then plain split-K partial sums (+ the gathered rows of an act-order call).  The head
+# must start zeroed; the kernels restore it to zero.
 # A workspace that has to grow is replaced by one at least twice as large; the old one is kept
 # alive, because captured graphs may still launch kernels that point into it.
 _workspaces: dict = {}
@@ -135,6 +136,31 @@ def workspace(device: torch.device, need: int):
         ws = torch.zeros(max(need, _WS_BYTES, 2 * ws.numel() if ws is not None else 0), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
+
+
+def exchange_errors() -> list:
+    """(device, stream) keys of the workspaces whose error word is set: a kernel's bounded wait for another
+    workgroup's partial sums ran out there, and the results of that call are not valid.  Synchronises."""
+    bad = []
+    for key, ws in list(_workspaces.items()) + [(None, w) for w in _outgrown]:
+        if int(ws[4 * WS_ERROR_WORD:4 * WS_ERROR_WORD + 4].view(torch.int32).item()) != 0:
+            bad.append(key)
+    return bad
+
+
+def check_exchange_errors() -> None:
+    bad = exchange_errors()
+    if bad:
+        raise RuntimeError(f"a small-M kernel gave up waiting for partial sums on workspace(s) {bad}: results computed on them "
+                           "since the last check are not valid; call reset_workspaces() before reusing them")
+
+
+def reset_workspaces() -> None:
+    """Zero every workspace (after an exchange error, which leaves marked values and the error word behind)."""
+    torch.cuda.synchronize()
+    for ws in list(_workspaces.values()) + _outgrown:
+        ws.zero_()
+    torch.cuda.synchronize()
 
 
 def require_cuda(t: torch.Tensor, name: str) -> None:

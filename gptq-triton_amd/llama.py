@@ -17,6 +17,7 @@ from typing import List, Optional, Tuple
 import torch
 import torch.nn as nn
 
+from . import _lib
 from .decoder_ops import add_rms_norm, decode_attention, rms_norm
 from .fused_attention import LlamaConfigLite
 
@@ -269,6 +270,8 @@ class GreedyDecoder:
             else:
                 self._step()
             out[:, i:i + 1].copy_(self.tokens)
+        # one 4-byte read per workspace: a bounded wait of the small-M kernels that ran out would have made tokens wrong silently
+        _lib.check_exchange_errors()
         return out
 
     def _capture(self):

@@ -135,3 +135,28 @@ def test_a_wait_that_runs_out_sets_the_error_word_and_the_kernel_still_ends(kern
         lib.gptq4_set_exchange_spin_limit(0)
         lib.gptq4_set_tuning(0, 0, 0)
         lib.gptq4_set_gemv_tuning(1, 0, 0, 0)
+
+
+def test_the_python_layer_reports_and_clears_an_exchange_error():
+    """The module-level workspaces: after a forced give-up `check_exchange_errors` raises and names the workspace,
+    `reset_workspaces` zeroes it, and the next call is right again."""
+    from gptq_triton_amd import _lib
+    lib = _lib.load()
+    G = gptq()
+    k, n, g, m = 4096, 4096, 128, 1
+    L = O.make_layer(k, n, g, seed=15)
+    D = to_dev(L)
+    x = O.make_x(m, k, seed=16)
+    xd = torch.from_numpy(x).cuda()
+    _lib.check_exchange_errors()
+    try:
+        lib.gptq4_set_exchange_spin_limit(0xFFFFFFFF)
+        G.matmul4(g, xd, D["qweight"], D["scales"], D["qzeros"])
+        with pytest.raises(RuntimeError, match="gave up waiting"):
+            _lib.check_exchange_errors()
+    finally:
+        lib.gptq4_set_exchange_spin_limit(0)
+        _lib.reset_workspaces()
+    assert _lib.exchange_errors() == []
+    y = G.matmul4(g, xd, D["qweight"], D["scales"], D["qzeros"])
+    assert_close(y.cpu().numpy(), O.quant_matmul_ref(x, L["qweight"], L["qzeros"], L["scales"], g), "after the reset")
