@@ -81,6 +81,7 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
         return reinterpret_cast<float *>(w < HALF ? As0 : As1) + (w < HALF ? w : w - HALF) * (32 * 64);
     };
 
+    GPTQ4_FETCH_MATMUL_ARGS(p);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);

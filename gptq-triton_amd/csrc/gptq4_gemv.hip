@@ -88,6 +88,7 @@ __global__ __launch_bounds__(64 * NW) void gptq4_gemv_kernel(MatmulArgs p) {
 
     extern __shared__ uint4 smem[];
 
+    GPTQ4_FETCH_MATMUL_ARGS(p);
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int lrow = lane >> 4;

@@ -69,6 +69,7 @@ __global__ __launch_bounds__(64 * KS, KS == 8 && MT == 2 ? 1 : 2) void gptq4_ksl
     };
 
     KS_STAMP(0);
+    GPTQ4_FETCH_MATMUL_ARGS(p);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);

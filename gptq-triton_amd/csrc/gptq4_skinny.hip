@@ -92,6 +92,7 @@ __global__ __launch_bounds__(64 * NW) void gptq4_skinny_kernel(MatmulArgs p) {
     __shared__ float norm_part[NORM ? NORM_MAX_M * 4 : 1];
     extern __shared__ uint4 xs[];  // NORM: [M][K / 8] normalised activations
 
+    GPTQ4_FETCH_MATMUL_ARGS(p);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     // the wave index is uniform: keep it (and everything derived from it - batch range,
