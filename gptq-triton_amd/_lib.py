@@ -60,6 +60,7 @@ SIGNATURES = {
     "gptq4_set_midm_tuning": (None, [c_int, c_int, c_int]),
     "gptq4_set_gemv_tuning": (None, [c_int, c_int, c_int, c_int]),
     "gptq4_set_exchange_spin_limit": (None, [ctypes.c_uint]),
+    "gptq4_column_parts": (c_int, [c_int, c_int, c_int, c_int, POINTER(c_int), POINTER(c_int)]),
 }
 
 

@@ -163,50 +163,135 @@ bool prefer_kslice(const KslicePlan &kp, int epi, int M, int N, int K) {
     return wide < 3 * cus / 4 || gemm_plan(epi, M, N, K).score < 0.65;
 }
 
+// Which kernel computes columns [.., .. + n) of an M > 16 call, with what plan, and the partial sums it exchanges.
+struct TiledChoice {
+    bool kslice;
+    KslicePlan kp;
+    GemmPlan gp;
+    size_t partial;
+};
+
+TiledChoice choose_tiled(int epi, int M, int n, int K, bool kernel_gathers) {
+    TiledChoice c = {};
+    c.kp = kslice_plan(epi, M, n, K, kernel_gathers);
+    c.kslice = prefer_kslice(c.kp, epi, M, n, K);
+    c.gp = gemm_plan(epi, M, n, K, kernel_gathers);
+    c.partial = c.kslice ? (c.kp.splitk > 1 ? kslice_partial_bytes(epi, c.kp) : 0) : gemm_partial_bytes(c.gp);
+    return c;
+}
+
+// An M > 16 call as one launch or as two launches over adjacent column ranges.  Whole wide tiles are dealt one per
+// CU and round; a count just above a multiple of the CU count leaves most CUs idle for a whole round (344 tiles of
+// the LLaMA-7B gate/up pair at 512 rows: 88 CUs work through two tiles, 168 through one; 516 at 768 rows: four CUs
+// take a third).  Then the columns of the full rounds go to one launch of wide tiles and the remaining columns to a
+// second launch that is planned by itself - narrower tiles, a K split or the mid-M kernel spread the remainder over
+// the chip.  Nothing is exchanged between the two: they write different columns.
+struct ColumnParts {
+    int count;
+    int begin[2], cols[2];
+    bool first_is_wide;  // part 0 runs wide unsplit tiles whatever its own plan would say
+};
+
+ColumnParts tiled_parts(int epi, int M, int N, int K, bool kernel_gathers) {
+    ColumnParts parts = {1, {0, 0}, {N, 0}, false};
+    if (g_gemm_tuning.parts == 1 || g_gemm_tuning.mt != 0 || g_gemm_tuning.splitk != 0 || g_gemm_tuning.streamed == 2 || g_kslice_tuning.mode == 2)
+        return parts;
+    const TiledChoice whole = choose_tiled(epi, M, N, K, kernel_gathers);
+    if (whole.kslice || whole.gp.mt != 4 || whole.gp.splitk != 1 || whole.gp.streamed) return parts;
+    const long cus = device_shape().cus;
+    const int bnw = (epi == EPI_SILU_MUL) ? 128 : 256;  // output columns of a wide tile
+    const long tiles_m = (M + 127) / 128, tiles_n = N / bnw, tiles = tiles_m * tiles_n;
+    const long rest = tiles % cus;
+    // From one full round on, and only for a small remainder (up to an eighth of a round).  A second launch costs
+    // 30 - 50 us at K = 4096 however little it computes, a round of wide tiles 55 - 75 us: LLaMA-7B gate/up at 384
+    // rows (258 tiles) 108 -> 89 us, at 768 rows (516) 167 -> 143, at 1536 rows (1032) 283 -> 269; with 88 tiles left
+    // over (512 rows) the two launches take what the one took, with 128 (QKV at 1024 rows) 7 % more.
+    if (tiles <= cus || tiles > 8 * cus || rest == 0 || 8 * rest > cus || K < 2048) return parts;
+    const long cols_a = (tiles - rest) / tiles_m;  // column tiles of the full rounds
+    if (cols_a < 1 || cols_a >= tiles_n) return parts;
+    parts.count = 2;
+    parts.first_is_wide = true;
+    parts.begin[0] = 0;
+    parts.cols[0] = (int)(cols_a * bnw);
+    parts.begin[1] = parts.cols[0];
+    parts.cols[1] = N - parts.cols[0];
+    return parts;
+}
+
+TiledChoice choose_part(int epi, int M, int K, const ColumnParts &parts, int i, bool kernel_gathers) {
+    if (i == 0 && parts.first_is_wide) {
+        TiledChoice c = {};
+        c.kslice = false;
+        c.gp.mt = 4;
+        c.gp.splitk = 1;
+        c.gp.score = 1.0;
+        c.gp.streamed = 0;
+        c.gp.tiles = ((M + 127) / 128) * (parts.cols[0] / ((epi == EPI_SILU_MUL) ? 128 : 256));
+        c.partial = 0;
+        return c;
+    }
+    return choose_tiled(epi, M, parts.cols[i], K, kernel_gathers);
+}
+
 int run_tiled(int epi, MatmulArgs &a, void *workspace, size_t workspace_bytes, hipStream_t s) {
     // act-order: staged activations wherever they fit the staging limit and the workspace (then the mid-M
     // kernel can run too); else the tiled kernel gathers by itself
     const size_t rows_bytes = (size_t)a.M * a.K * sizeof(half_t);
     bool stage = a.perm != nullptr && !g_gemm_tuning.own_gather && rows_bytes <= ACT_ORDER_STAGE_MAX;
-    GemmPlan pl = gemm_plan(epi, a.M, a.N, a.K, a.perm != nullptr && !stage);
+    ColumnParts parts;
+    TiledChoice choice[2];
+    size_t partial = 0;
+    auto plan_all = [&]() {
+        const bool kernel_gathers = a.perm != nullptr && !stage;
+        parts = tiled_parts(epi, a.M, a.N, a.K, kernel_gathers);
+        partial = 0;
+        for (int i = 0; i < parts.count; ++i) {
+            choice[i] = choose_part(epi, a.M, a.K, parts, i, kernel_gathers);
+            if (choice[i].partial > partial) partial = choice[i].partial;
+        }
+    };
+    plan_all();
     // the streamed schedule keeps 128 MiB of partial sums: without the room for them, the unstreamed plan
-    if (pl.streamed && (workspace == nullptr || workspace_bytes < GPTQ4_WS_HEAD_BYTES + gemm_partial_bytes(pl) + (stage ? rows_bytes : 0))) {
+    if (parts.count == 1 && !choice[0].kslice && choice[0].gp.streamed &&
+        (workspace == nullptr || workspace_bytes < GPTQ4_WS_HEAD_BYTES + partial + (stage ? rows_bytes : 0))) {
         g_stream_off = true;
-        pl = gemm_plan(epi, a.M, a.N, a.K, a.perm != nullptr && !stage);
+        plan_all();
         g_stream_off = false;
     }
-    if (stage) {
-        const KslicePlan kp = kslice_plan(epi, a.M, a.N, a.K, false);
-        const size_t partial = prefer_kslice(kp, epi, a.M, a.N, a.K) ? (kp.splitk > 1 ? kslice_partial_bytes(epi, kp) : 0)
-                                                                       : gemm_partial_bytes(pl);
-        if (workspace == nullptr || workspace_bytes < GPTQ4_WS_HEAD_BYTES + partial + rows_bytes) stage = false;
+    if (stage && (workspace == nullptr || workspace_bytes < GPTQ4_WS_HEAD_BYTES + partial + rows_bytes)) {
+        stage = false;
+        plan_all();
     }
-    const KslicePlan kp = kslice_plan(epi, a.M, a.N, a.K, a.perm != nullptr && !stage);
-    if (prefer_kslice(kp, epi, a.M, a.N, a.K)) {
-        a.tiles = kp.tiles;
-        a.splitk = kp.splitk;
-        const int nk = a.K / 64;
-        a.slot_q = nk / kp.splitk;
-        a.slot_rem = nk % kp.splitk;
-        const size_t partial = kp.splitk > 1 ? kslice_partial_bytes(epi, kp) : 0;
-        if (kp.splitk > 1) {
-            if (workspace == nullptr || workspace_bytes < GPTQ4_WS_HEAD_BYTES + partial) return -GPTQ4_E_WORKSPACE;
-            a.counters = reinterpret_cast<int *>(workspace);
-            a.partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_HEAD_BYTES);
-        }
-        if (stage) {
-            const int rc = stage_act_order(a, partial, workspace, workspace_bytes, s);
-            if (rc) return rc;
-        }
-        return launch_kslice(epi, a, kp, s);
-    }
-    int rc = setup_gemm(a, pl, workspace, workspace_bytes);
-    if (rc) return rc;
+    if (partial > 0 && (workspace == nullptr || workspace_bytes < GPTQ4_WS_HEAD_BYTES + partial)) return -GPTQ4_E_WORKSPACE;
     if (stage) {
-        rc = stage_act_order(a, gemm_partial_bytes(pl), workspace, workspace_bytes, s);
+        // once, behind the largest partial-sum region any part uses
+        const int rc = stage_act_order(a, partial, workspace, workspace_bytes, s);
         if (rc) return rc;
     }
-    return launch_gemm(epi, a, pl, s);
+    for (int i = 0; i < parts.count; ++i) {
+        a.n_begin = parts.begin[i];
+        a.n_count = parts.cols[i];
+        const TiledChoice &c = choice[i];
+        int rc;
+        if (c.kslice) {
+            a.tiles = c.kp.tiles;
+            a.splitk = c.kp.splitk;
+            const int nk = a.K / 64;
+            a.slot_q = nk / c.kp.splitk;
+            a.slot_rem = nk % c.kp.splitk;
+            if (c.kp.splitk > 1) {
+                a.counters = reinterpret_cast<int *>(workspace);
+                a.partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_HEAD_BYTES);
+            }
+            rc = launch_kslice(epi, a, c.kp, s);
+        } else {
+            rc = setup_gemm(a, c.gp, workspace, workspace_bytes);
+            if (rc) return rc;
+            rc = launch_gemm(epi, a, c.gp, s);
+        }
+        if (rc) return rc;
+    }
+    return 0;
 }
 
 }  // namespace
@@ -237,8 +322,10 @@ const char *gptq4_strerror(int code) {
 }
 
 void gptq4_set_gemm_tuning(int mt, int splitk) {
-    // 100: never the streamed schedule, 200: the streamed schedule wherever it can run (both with automatic tile and split)
+    // 100: never the streamed schedule, 200: the streamed schedule wherever it can run (both with automatic tile and split);
+    // 300: never two launches over column ranges (automatic otherwise)
     g_gemm_tuning.streamed = (mt == 100) ? 1 : (mt == 200) ? 2 : 0;
+    g_gemm_tuning.parts = (mt == 300) ? 1 : 0;
     if (mt >= 100) mt = 0;
     // 10 + mt: act-order calls use the tiled kernel's own gather (no staging of the activations)
     g_gemm_tuning.own_gather = (mt >= 10) ? 1 : 0;
@@ -291,15 +378,39 @@ size_t gptq4_workspace_bytes(int op, int M, int K, int N) {
         bytes += need + (with_perm ? (size_t)M * K * 2 : 0);  // + the rows gathered for an act-order call
     } else if ((K % 64) == 0) {
         const int epi = (op == GPTQ4_OP_MLP_GATEUP) ? EPI_SILU_MUL : (op == GPTQ4_OP_QKV_ROTARY ? EPI_ROPE : EPI_PLAIN);
-        // whichever kernel the current (automatic or forced) plans pick, with or without act-order
+        // whichever kernel the current (automatic or forced) plans pick, with or without act-order, for the whole
+        // matrix and for each of the column ranges a call may be cut into
         size_t need = gemm_partial_bytes(gemm_plan(epi, M, N, K));
         const KslicePlan kp = kslice_plan(epi, M, N, K, false);
         if (kp.ok && kslice_partial_bytes(epi, kp) > need) need = kslice_partial_bytes(epi, kp);
+        const ColumnParts parts = tiled_parts(epi, M, N, K, false);
+        for (int i = 0; i < parts.count; ++i) {
+            const TiledChoice c = choose_part(epi, M, K, parts, i, false);
+            if (c.partial > need) need = c.partial;
+            const KslicePlan pk = kslice_plan(epi, M, parts.cols[i], K, false);
+            if (pk.ok && kslice_partial_bytes(epi, pk) > need) need = kslice_partial_bytes(epi, pk);
+        }
         bytes += need;
         // + the rows gathered for an act-order call
         if (with_perm && (size_t)M * K * 2 <= ACT_ORDER_STAGE_MAX) bytes += (size_t)M * K * 2;
     }
     return bytes;
+}
+
+int gptq4_column_parts(int op, int M, int K, int N, int *begin, int *cols) {
+    op &= ~GPTQ4_OP_WITH_PERM;
+    if (M <= SKINNY_MAX_M || N <= 0 || K <= 0 || (K % 64) != 0 || (N % 256) != 0 || op < GPTQ4_OP_MATMUL || op > GPTQ4_OP_QKV_ROTARY) {
+        if (begin) begin[0] = 0;
+        if (cols) cols[0] = N > 0 ? N : 0;
+        return 1;
+    }
+    const int epi = (op == GPTQ4_OP_MLP_GATEUP) ? EPI_SILU_MUL : (op == GPTQ4_OP_QKV_ROTARY ? EPI_ROPE : EPI_PLAIN);
+    const ColumnParts parts = tiled_parts(epi, M, N, K, false);
+    for (int i = 0; i < parts.count; ++i) {
+        if (begin) begin[i] = parts.begin[i];
+        if (cols) cols[i] = parts.cols[i];
+    }
+    return parts.count;
 }
 
 int gptq4_dequant(const int32_t *qweight, const int32_t *qzeros, const void *scales, const int32_t *g_idx,
@@ -341,6 +452,8 @@ int gptq4_matmul(const void *x, const int32_t *qweight, const int32_t *qzeros, c
     a.M = M;
     a.K = K;
     a.N = N;
+    a.n_begin = 0;
+    a.n_count = N;
     a.groupsize = groupsize;
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     if (M <= SKINNY_MAX_M) {
@@ -413,6 +526,8 @@ static int mlp_gateup_impl(const void *x, const void *delta, const void *norm_we
     a.M = M;
     a.K = K;
     a.N = I;
+    a.n_begin = 0;
+    a.n_count = I;
     a.groupsize = groupsize;
     if (norm) {
         rc = setup_norm(a, delta, norm_weight, sum_out, eps);
@@ -473,6 +588,8 @@ static int qkv_rotary_impl(const void *x, const void *delta, const void *norm_we
     a.M = B * S;
     a.K = K;
     a.N = N;
+    a.n_begin = 0;
+    a.n_count = N;
     a.groupsize = groupsize;
     a.rope.position_ids = position_ids;
     a.rope.cos_table = cos_table;

@@ -108,14 +108,14 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
     // the L2 (row tiles fastest over all of M left a weight panel shared by many but an
     // activation tile by two, and the activation tiles are the larger stream).
     constexpr int GROUP_M = 8;
-    const int tiles_n = N / BN;
+    const int tiles_n = p.n_count / BN;  // the launch covers columns [n_begin, n_begin + n_count) of the N
     const int band = logical / (GROUP_M * tiles_n);  // band of GROUP_M row tiles
     const int in_band = logical - band * (GROUP_M * tiles_n);
     const int band_rows = min(GROUP_M, tiles_m - band * GROUP_M);
     const int tile_n = in_band / band_rows;
     const int tile_m = band * GROUP_M + (in_band - tile_n * band_rows);
     const int m0 = tile_m * BM;
-    const int n0 = tile_n * BN;
+    const int n0 = p.n_begin + tile_n * BN;
 
     const int mat = (EPI == EPI_SILU_MUL) ? wn_odd : 0;
     const int nw0 = n0 + ((EPI == EPI_SILU_MUL) ? wn_pair : wn) * 64;  // first column of the wave
@@ -739,7 +739,7 @@ int launch_epi(const MatmulArgs &a, const GemmPlan &pl, hipStream_t stream) {
 
 }  // namespace
 
-GemmTuning g_gemm_tuning = {0, 0, 0, 0};
+GemmTuning g_gemm_tuning = {0, 0, 0, 0, 0};
 thread_local bool g_stream_off = false;
 
 // Tile shape and split-K factor of the tiled kernel.  The wide tile (128 x 256, half as

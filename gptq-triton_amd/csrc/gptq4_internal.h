@@ -31,6 +31,9 @@ struct MatmulArgs {
     const half_t *bias;
     const int32_t *perm;
     int M, K, N;
+    // M > 16 kernels: the launch computes output columns [n_begin, n_begin + n_count) only (N stays the row length of
+    // the weights and of the result); the whole matrix: 0, N
+    int n_begin, n_count;
     int groupsize;  // normalised: K when the caller passed -1
     int splitk;
     int tiles;
@@ -111,6 +114,7 @@ struct GemmTuning {
     int mt, splitk;  // 0 = automatic
     int own_gather;  // 1: act-order calls run the tiled kernel's own gather instead of staging the activations
     int streamed;    // 0 = automatic, 1 = never, 2 = wherever it can run
+    int parts;       // 0 = automatic, 1 = never cut a call into two launches over column ranges
 };
 extern GemmTuning g_gemm_tuning;
 // set around a call that must not plan the streamed schedule (its partial sums would not fit the caller's scratch memory)

@@ -88,7 +88,7 @@ __global__ __launch_bounds__(64 * KS, KS == 8 && MT == 2 ? 1 : 2) void gptq4_ksl
     const int tile_n = logical / tiles_m;
     const int tile_m = logical - tile_n * tiles_m;
     const int m0 = tile_m * BM;
-    const int n0 = tile_n * BN;
+    const int n0 = p.n_begin + tile_n * BN;  // the launch covers columns [n_begin, n_begin + n_count) of the N
 
     // block j of the wave tile: matrix j at the strip's columns (SiLU*mul), or columns
     // 64*j .. 64*j + 63 of the head (rotary); the lane's 2 columns of it

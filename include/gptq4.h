@@ -300,7 +300,9 @@ void gptq4_set_tuning(int words, int depth, int splitk);
  * mt = 10, 12 or 14: the same tile choice, and act-order calls use the tiled kernel's own
  * gather of the activations instead of the copy staged in the workspace.  mt = 200: the streamed
  * schedule (K tiles of all wide tiles dealt evenly to the resident workgroups; never chosen
- * automatically, it measured slower) wherever it can run, mt = 100: never; tile and split automatic with both. */
+ * automatically, it measured slower) wherever it can run, mt = 100: never; mt = 300: never cut a call into two
+ * launches over adjacent column ranges (done automatically where the wide-tile count is just above a multiple of
+ * the CU count); tile and split automatic with all three. */
 void gptq4_set_gemm_tuning(int mt, int splitk);
 
 /* Same for the mid-M kernel (M > 16 with too few wide tiles for the tiled kernel; K is split
@@ -316,6 +318,13 @@ void gptq4_set_midm_tuning(int mode, int mt, int splitk);
  * flight per wave (1..3), waves per workgroup (4, 8, 16), waves per CU (4..32), 0 =
  * automatic. */
 void gptq4_set_gemv_tuning(int mode, int depth, int waves, int waves_per_cu);
+/* How a call with more than 16 rows is launched: as one launch over all N output columns (returns 1) or as two
+ * launches over adjacent column ranges (returns 2; begin[i], cols[i] describe them) - the second where the count of
+ * wide tiles is just above a multiple of the CU count, so that a few left-over tiles do not cost a round of their
+ * own.  `op` is a GPTQ4_OP_* selector (N of one matrix for the gate/up pair); begin and cols have room for two
+ * values (or are NULL).  For diagnostics and tests; no reference counterpart. */
+int gptq4_column_parts(int op, int M, int K, int N, int *begin, int *cols);
+
 /* How often a finishing wave of the small-M kernels polls for another wave's marked partial sums before it gives up
  * and sets GPTQ4_WS_ERROR_WORD (0 = the default, about four million polls).  0xFFFFFFFF is the hook for tests of
  * that error path: every finishing wave polls once and gives up whatever it found, and every kernel still ends
