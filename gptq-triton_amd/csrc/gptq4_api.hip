@@ -118,13 +118,17 @@ int run_small(int epi, MatmulArgs &a, int nmat, void *workspace, size_t workspac
 }
 
 // Fill the split-K fields of `a` for the tiled kernel.
-int setup_gemm(MatmulArgs &a, const GemmPlan &pl, void *workspace, size_t workspace_bytes) {
+int setup_gemm(int epi, MatmulArgs &a, const GemmPlan &pl, void *workspace, size_t workspace_bytes) {
     a.tiles = pl.tiles;
     a.splitk = pl.splitk;
     const int nk = a.K / 64;
     a.slot_q = nk / pl.splitk;
     a.slot_rem = nk % pl.splitk;
-    if (pl.splitk > 1 || pl.streamed) {
+    a.tail_first = pl.tail_first;
+    a.tail_split = pl.tail_split;
+    // the tiles cut along K are the last column panels: the whole tiles cover the columns before them
+    if (pl.tail_split > 1) a.n_count = (pl.tail_first / ((a.M + 127) / 128)) * ((epi == EPI_SILU_MUL) ? 128 : 256);
+    if (pl.splitk > 1 || pl.streamed || pl.tail_split > 1) {
         if (workspace == nullptr || workspace_bytes < GPTQ4_WS_HEAD_BYTES + gemm_partial_bytes(pl))
             return -GPTQ4_E_WORKSPACE;
         a.counters = reinterpret_cast<int *>(workspace);
@@ -197,7 +201,7 @@ ColumnParts tiled_parts(int epi, int M, int N, int K, bool kernel_gathers) {
     if (g_gemm_tuning.parts == 1 || g_gemm_tuning.mt != 0 || g_gemm_tuning.splitk != 0 || g_gemm_tuning.streamed == 2 || g_kslice_tuning.mode == 2)
         return parts;
     const TiledChoice whole = choose_tiled(epi, M, N, K, kernel_gathers);
-    if (whole.kslice || whole.gp.mt != 4 || whole.gp.splitk != 1 || whole.gp.streamed) return parts;
+    if (whole.kslice || whole.gp.mt != 4 || whole.gp.splitk != 1 || whole.gp.streamed || whole.gp.tail_split > 1) return parts;
     const long cus = device_shape().cus;
     const int bnw = (epi == EPI_SILU_MUL) ? 128 : 256;  // output columns of a wide tile
     const long tiles_m = (M + 127) / 128, tiles_n = N / bnw, tiles = tiles_m * tiles_n;
@@ -226,6 +230,8 @@ TiledChoice choose_part(int epi, int M, int K, const ColumnParts &parts, int i, 
         c.gp.splitk = 1;
         c.gp.score = 1.0;
         c.gp.streamed = 0;
+        c.gp.tail_first = 0;
+        c.gp.tail_split = 1;
         c.gp.tiles = ((M + 127) / 128) * (parts.cols[0] / ((epi == EPI_SILU_MUL) ? 128 : 256));
         c.partial = 0;
         return c;
@@ -285,7 +291,7 @@ int run_tiled(int epi, MatmulArgs &a, void *workspace, size_t workspace_bytes, h
             }
             rc = launch_kslice(epi, a, c.kp, s);
         } else {
-            rc = setup_gemm(a, c.gp, workspace, workspace_bytes);
+            rc = setup_gemm(epi, a, c.gp, workspace, workspace_bytes);
             if (rc) return rc;
             rc = launch_gemm(epi, a, c.gp, s);
         }
@@ -325,7 +331,9 @@ void gptq4_set_gemm_tuning(int mt, int splitk) {
     // 100: never the streamed schedule, 200: the streamed schedule wherever it can run (both with automatic tile and split);
     // 300: never two launches over column ranges (automatic otherwise)
     g_gemm_tuning.streamed = (mt == 100) ? 1 : (mt == 200) ? 2 : 0;
-    g_gemm_tuning.parts = (mt == 300) ? 1 : 0;
+    g_gemm_tuning.parts = (mt == 300 || mt == 500) ? 1 : 0;
+    // 400: never cut the tiles past a whole number of rounds along K; 500: neither that nor the two launches
+    g_gemm_tuning.tail = (mt == 400 || mt == 500) ? 1 : 0;
     if (mt >= 100) mt = 0;
     // 10 + mt: act-order calls use the tiled kernel's own gather (no staging of the activations)
     g_gemm_tuning.own_gather = (mt >= 10) ? 1 : 0;

@@ -108,12 +108,20 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
     // the L2 (row tiles fastest over all of M left a weight panel shared by many but an
     // activation tile by two, and the activation tiles are the larger stream).
     constexpr int GROUP_M = 8;
-    const int tiles_n = p.n_count / BN;  // the launch covers columns [n_begin, n_begin + n_count) of the N
-    const int band = logical / (GROUP_M * tiles_n);  // band of GROUP_M row tiles
-    const int in_band = logical - band * (GROUP_M * tiles_n);
-    const int band_rows = min(GROUP_M, tiles_m - band * GROUP_M);
-    const int tile_n = in_band / band_rows;
-    const int tile_m = band * GROUP_M + (in_band - tile_n * band_rows);
+    const int tiles_n = p.n_count / BN;  // the tiles in this order cover columns [n_begin, n_begin + n_count) of the N
+    int tile_m, tile_n;
+    if (logical < tiles_m * tiles_n) {
+        const int band = logical / (GROUP_M * tiles_n);  // band of GROUP_M row tiles
+        const int in_band = logical - band * (GROUP_M * tiles_n);
+        const int band_rows = min(GROUP_M, tiles_m - band * GROUP_M);
+        tile_n = in_band / band_rows;
+        tile_m = band * GROUP_M + (in_band - tile_n * band_rows);
+    } else {
+        // tiles cut along K: whole column panels behind those columns, row tiles fastest
+        const int t = logical - tiles_m * tiles_n;
+        tile_n = tiles_n + t / tiles_m;
+        tile_m = t - (t / tiles_m) * tiles_m;
+    }
     const int m0 = tile_m * BM;
     const int n0 = p.n_begin + tile_n * BN;
 
@@ -648,6 +656,28 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
     };  // run_part
 
     if constexpr (!STREAM) {
+        if (p.tail_split > 1) {
+            // Tiles [0, tail_first) whole, one workgroup each; every tile from tail_first on - the last column
+            // panels, all their row tiles, so that a row is summed in the same order wherever it sits in the
+            // batch - cut into tail_split parts along K with a workgroup each.  The parts come last in the grid:
+            // they are dispatched onto CUs that are working on a whole tile already and run beside it, so the few
+            // tiles past a whole number of rounds cost a fraction of a round instead of one.
+            const int full = p.tail_first;
+            if ((int)blockIdx.x < full) {
+                const int per = full >> 3, rem = full & 7;
+                const int xcd = blockIdx.x & 7;
+                const int logical = xcd * per + (xcd < rem ? xcd : rem) + (blockIdx.x >> 3);
+                run_part(logical, 0, K / BK, 1, 0, [&](int c) { return (size_t)c; });
+            } else {
+                const int s = p.tail_split;
+                const int w = blockIdx.x - full;
+                const int t = w / s, idx = w - t * s;
+                const int nkt = K / BK, q = nkt / s, r = nkt % s;
+                const int kb = idx * q + min(idx, r);
+                run_part(full + t, kb, kb + q + (idx < r ? 1 : 0), s, idx, [&](int c) { return (size_t)t * s + c; });
+            }
+            return;
+        }
         // one tile (or one K split of it) per workgroup; K tiles of the split by host-side quotient / remainder
         const int total = gridDim.x;
         const int per = total >> 3, rem = total & 7;
@@ -734,12 +764,13 @@ int launch_streamed(const MatmulArgs &a, int workgroups, hipStream_t stream) {
 template <int EPI>
 int launch_epi(const MatmulArgs &a, const GemmPlan &pl, hipStream_t stream) {
     if (pl.streamed) return launch_streamed<EPI>(a, pl.streamed, stream);
+    if (pl.tail_split > 1) return launch_one<EPI, 4>(a, pl.tail_first + (pl.tiles - pl.tail_first) * pl.tail_split, stream);
     return pl.mt == 4 ? launch_one<EPI, 4>(a, pl.tiles, stream) : launch_one<EPI, 2>(a, pl.tiles, stream);
 }
 
 }  // namespace
 
-GemmTuning g_gemm_tuning = {0, 0, 0, 0, 0};
+GemmTuning g_gemm_tuning = {0, 0, 0, 0, 0, 0};
 thread_local bool g_stream_off = false;
 
 // Tile shape and split-K factor of the tiled kernel.  The wide tile (128 x 256, half as
@@ -761,6 +792,8 @@ GemmPlan gemm_plan(int epi, int M, int N, int K, bool has_perm) {
     GemmPlan pl;
     pl.score = 1.0;
     pl.streamed = 0;
+    pl.tail_first = 0;
+    pl.tail_split = 1;
     const int bn2 = (epi == EPI_SILU_MUL) ? 64 : 128;  // tile width at MT = 2; twice that at MT = 4
     const int nk = K / 64;
     const long wide = (long)((M + 127) / 128) * (N / (2 * bn2));
@@ -807,6 +840,28 @@ GemmPlan gemm_plan(int epi, int M, int N, int K, bool has_perm) {
     if (s > nk) s = nk;
     if (s < 1 || pl.tiles > SKINNY_MAX_TILES) s = 1;
     pl.splitk = s;
+    // Wide unsplit tiles past a whole number of rounds (one tile per CU and round): up to half a round of them is cut
+    // along K, each into as many parts as spread the left-over tiles over the chip, and the parts run beside the whole
+    // tiles of the last round instead of after them.
+    if (pl.mt == 4 && s == 1 && g_gemm_tuning.tail != 1 && g_gemm_tuning.mt == 0 && g_gemm_tuning.splitk == 0 && wide > cus &&
+        wide <= SKINNY_MAX_TILES) {
+        const long rest = wide % cus;
+        // (after an even number of rounds every CU holds its two workgroups and the parts have to wait for a free
+        // place: a small remainder is then better off as a launch of its own, see tiled_parts)
+        const bool own_launch = ((wide - rest) / cus) % 2 == 0 && 8 * rest <= cus && K >= 2048 && g_gemm_tuning.parts != 1;
+        // whole column panels are cut: at least `rest` tiles
+        const long tiles_m = (M + 127) / 128, tiles_n = wide / tiles_m;
+        const long panels = (rest + tiles_m - 1) / tiles_m, cut = panels * tiles_m;
+        if (rest > 0 && 2 * cut <= cus && panels < tiles_n && !own_launch) {
+            long parts = cus / cut;
+            if (parts > nk / 8) parts = nk / 8;  // at least 8 K tiles (512 k) per part
+            if (parts > GEMM_MAX_SPLITK) parts = GEMM_MAX_SPLITK;
+            if (parts >= 2) {
+                pl.tail_first = (int)(wide - cut);
+                pl.tail_split = (int)parts;
+            }
+        }
+    }
     // The streamed schedule (wide tiles; the K tiles of all of them dealt evenly to the 2 x CUs workgroups that are
     // resident at one time) is never chosen automatically: it evens out the work - 344 tiles on 512 slots, or 768 (a
     // pair and then a single one per CU) - but every workgroup then exchanges a 128 KiB tile of fp32 partial sums,
@@ -826,6 +881,7 @@ GemmPlan gemm_plan(int epi, int M, int N, int K, bool has_perm) {
             pl.tiles = (int)wide;
             pl.splitk = 1;
             pl.streamed = (int)grid;
+            pl.tail_split = 1;
         }
     }
     return pl;
@@ -834,6 +890,7 @@ GemmPlan gemm_plan(int epi, int M, int N, int K, bool has_perm) {
 size_t gemm_partial_bytes(const GemmPlan &pl) {
     // streamed: two slots of a whole wide tile per workgroup (the part that begins its range, the part that ends it)
     if (pl.streamed) return (size_t)pl.streamed * 2 * (4 * 32 * 256) * sizeof(float);
+    if (pl.tail_split > 1) return (size_t)(pl.tiles - pl.tail_first) * pl.tail_split * (4 * 32 * 256) * sizeof(float);
     return pl.splitk > 1 ? (size_t)pl.tiles * pl.splitk * (pl.mt * 32 * 256) * sizeof(float) : 0;
 }
 

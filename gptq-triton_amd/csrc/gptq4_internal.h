@@ -34,6 +34,7 @@ struct MatmulArgs {
     // M > 16 kernels: the launch computes output columns [n_begin, n_begin + n_count) only (N stays the row length of
     // the weights and of the result); the whole matrix: 0, N
     int n_begin, n_count;
+    int tail_first, tail_split;  // tiled kernel, wide unsplit tiles: see GemmPlan
     int groupsize;  // normalised: K when the caller passed -1
     int splitk;
     int tiles;
@@ -109,12 +110,16 @@ struct GemmPlan {
     int tiles;
     double score;  // expected efficiency of the choice: fill of the chip / cost of the splits (1 where the tile count is large)
     int streamed;  // 0, or the grid of the streamed schedule (wide tiles, K tiles of all tiles dealt evenly to that many workgroups)
+    // wide tiles, unsplit: tiles [0, tail_first) whole, the tiles from tail_first on cut into tail_split parts along K
+    // (1 = no tile is cut)
+    int tail_first, tail_split;
 };
 struct GemmTuning {
     int mt, splitk;  // 0 = automatic
     int own_gather;  // 1: act-order calls run the tiled kernel's own gather instead of staging the activations
     int streamed;    // 0 = automatic, 1 = never, 2 = wherever it can run
     int parts;       // 0 = automatic, 1 = never cut a call into two launches over column ranges
+    int tail;        // 0 = automatic, 1 = never cut the tiles past a whole number of rounds along K
 };
 extern GemmTuning g_gemm_tuning;
 // set around a call that must not plan the streamed schedule (its partial sums would not fit the caller's scratch memory)

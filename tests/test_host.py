@@ -220,9 +220,9 @@ def test_mid_m_plan_is_declared_and_tunable():
 
 def test_column_parts_plan_without_a_gpu():
     """The plan that cuts a call into two launches over column ranges is host arithmetic (256 CUs assumed where no
-    device can be asked): LLaMA-7B gate/up has 86 column tiles, so 3, 6 or 12 row tiles are 2, 4 or 8 tiles more than
-    a whole number of rounds; 4 row tiles (88 over) and decode-sized calls are never cut; the tuning hook switches
-    it off."""
+    device can be asked): LLaMA-7B gate/up has 86 column tiles, so 6 or 12 row tiles are 4 or 8 tiles more than an
+    even number of rounds; 3 row tiles (2 over one round) and 4 (88 over) are cut along K inside one launch instead,
+    decode-sized calls are never cut; the tuning hook switches it off."""
     import ctypes
     lib = _lib.load()
 
@@ -231,7 +231,7 @@ def test_column_parts_plan_without_a_gpu():
         count = lib.gptq4_column_parts(op, m, k, n, begin, cols)
         return [(begin[i], cols[i]) for i in range(count)]
 
-    assert parts(_lib.OP_MLP_GATEUP, 384, 4096, 11008) == [(0, 85 * 128), (85 * 128, 128)]
+    assert parts(_lib.OP_MLP_GATEUP, 384, 4096, 11008) == [(0, 11008)]                            # 258 tiles: cut along K instead
     assert parts(_lib.OP_MLP_GATEUP, 768, 4096, 11008) == [(0, 85 * 128), (85 * 128, 128)]       # 516 tiles: 512 + 4
     assert parts(_lib.OP_MLP_GATEUP, 1536, 4096, 11008) == [(0, 85 * 128), (85 * 128, 128)]      # 1032: 1024 + 8
     assert parts(_lib.OP_MLP_GATEUP, 512, 4096, 11008) == [(0, 11008)]
@@ -239,7 +239,7 @@ def test_column_parts_plan_without_a_gpu():
     assert parts(_lib.OP_MATMUL, 2048, 4096, 4096) == [(0, 4096)]
     lib.gptq4_set_gemm_tuning(300, 0)
     try:
-        assert parts(_lib.OP_MLP_GATEUP, 384, 4096, 11008) == [(0, 11008)]
+        assert parts(_lib.OP_MLP_GATEUP, 768, 4096, 11008) == [(0, 11008)]
     finally:
         lib.gptq4_set_gemm_tuning(0, 0)
     assert parts(_lib.OP_QKV_ROTARY, 1408, 4096, 12288) == [(0, 46 * 256), (46 * 256, 2 * 256)]  # 11 x 48 = 528: 512 + 16
