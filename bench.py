@@ -150,7 +150,7 @@ def decoder_figures(workload, bsz, prompt, new):
     dec.prefill(ids)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    dec.prefill(ids)
+    first = dec.prefill(ids)
     torch.cuda.synchronize()
     prefill_s = time.perf_counter() - t0
     per_token_kn = layers * (hidden * 3 * hidden + hidden * hidden + 2 * hidden * inter + inter * hidden)
@@ -160,10 +160,10 @@ def decoder_figures(workload, bsz, prompt, new):
     eager_steps = min(8, new - 1)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    dec.decode(eager_steps)
+    generated = [first, dec.decode(eager_steps)]
     torch.cuda.synchronize()
     eager_s = (time.perf_counter() - t0) / max(eager_steps, 1)
-    dec.decode(2, use_graph=True)  # captures the step
+    generated.append(dec.decode(2, use_graph=True))  # captures the step
     steps = new - 1 - eager_steps - 2
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -173,6 +173,17 @@ def decoder_figures(workload, bsz, prompt, new):
     kv_bytes = 2 * layers * bsz * heads * (prompt + new) * 128 * 2
     step_bytes = qbytes + model.lm_head.weight.numel() * 2 + kv_bytes
     gbs = step_bytes / step_s / 1e9
+    # Check beyond "tokens came out": the prompt + the first j generated tokens through the prefill path (tiled GEMM, torch's
+    # attention over the whole sequence) must choose generated token j, which the decode path (GEMV kernels, one-token
+    # attention over the cache, graph replay) chose.  Random-init logits have near-ties, so the count is reported, not asserted.
+    generated = torch.cat(generated + [toks], dim=1)
+    probes = sorted({1, eager_steps + 3, generated.shape[1] // 2, generated.shape[1] - 1})
+    agree = 0
+    for j in probes:
+        nxt = dec.prefill(torch.cat([ids, generated[:, :j]], dim=1))
+        agree += int((nxt[:, 0] == generated[:, j]).sum())
+    agreement = f"{agree}/{len(probes) * bsz}"
+    log(f"prefill path re-run on prompt + generated tokens agrees with the decode path on {agreement} next tokens (probes {probes})")
     log(f"decode: {step_s * 1e3:.3f} ms/step graph-replayed ({bsz / step_s:.1f} tok/s), {eager_s * 1e3:.3f} ms/step eager; "
         f"{step_bytes / 1e9:.2f} GB per step -> {gbs:.0f} GB/s")
     result = {
@@ -191,7 +202,8 @@ def decoder_figures(workload, bsz, prompt, new):
         "cpu_baseline": None,
         "extra": {"prefill_ms": round(prefill_s * 1e3, 2), "prefill_linear_TFLOPs": round(prefill_tf, 1),
                   "prefill_frac_of_fp16_mfma_peak": round(prefill_tf / MFMA_FP16_PEAK_TFLOPS, 4),
-                  "eager_decode_ms_per_step": round(eager_s * 1e3, 3), "last_tokens": toks[0, -4:].tolist()},
+                  "eager_decode_ms_per_step": round(eager_s * 1e3, 3), "last_tokens": toks[0, -4:].tolist(),
+                  "prefill_path_agrees_with_decode_path_on_next_tokens": agreement},
     }
     del dec, model, toks, ids
     gc.collect()
