@@ -580,29 +580,42 @@ def main():
         del c3, xp
         extra["baseline_configs"] = rows
 
-        # Yardstick: the vendor library's DENSE fp16 GEMM (torch.matmul) on the same M = 2048
-        # shapes, weights already dequantised.  It does no 4-bit decode and reads 4x the
-        # weight bytes; it shows what fraction of the nominal MFMA peak a tuned kernel
-        # sustains on this chip at these shapes.
-        def dense(name, k, n, m=2048, reps=20):
+        # Yardstick: the vendor library's DENSE fp16 GEMM (torch) on the same shapes at 128, 512 and 2048 rows,
+        # weights already dequantised, in the faster of its two weight layouts ([K, N] and [N, K]), 20 calls
+        # replayed from one graph.  It does no 4-bit decode, no fused epilogue and reads 4x the weight bytes; it
+        # shows what a tuned kernel sustains on this chip at these shapes.
+        def dense(shape, k, n, m, reps=20):
             a = torch.randn((m, k), device=dev, generator=gen).half()
-            ws = [(torch.randn((k, n), device=dev, generator=gen) * 0.02).half() for _ in range(2)]
-            for w in ws:
-                torch.matmul(a, w)
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            for i in range(reps):
-                torch.matmul(a, ws[i & 1])
-            e1.record()
-            torch.cuda.synchronize()
-            us = e0.elapsed_time(e1) * 1e3 / reps
-            extra[name] = {"us": round(us, 2), "TFLOPs": round(2.0 * m * k * n / us / 1e6, 2)}
-            log(f"  {name:34s} {us:9.2f} us  {'':8s}       {2.0 * m * k * n / us / 1e6:8.1f} TFLOP/s")
-        dense("dense fp16 library M=2048 qkv shape", HIDDEN, 3 * HIDDEN)
-        dense("dense fp16 library M=2048 gate+up shape", HIDDEN, 2 * INTER)
-        dense("dense fp16 library M=2048 down shape", INTER, HIDDEN)
-        dense("dense fp16 library M=2048 o_proj shape", HIDDEN, HIDDEN)
+            w = (torch.randn((k, n), device=dev, generator=gen) * 0.02).half()
+            wt = w.t().contiguous()
+            best = None
+            for fn in (lambda: torch.matmul(a, w), lambda: torch.nn.functional.linear(a, wt)):
+                for _ in range(3):
+                    fn()
+                torch.cuda.synchronize()
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    for _ in range(reps):
+                        fn()
+                g.replay()
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(3):
+                    g.replay()
+                e1.record()
+                torch.cuda.synchronize()
+                us = e0.elapsed_time(e1) * 1e3 / (3 * reps)
+                best = us if best is None else min(best, us)
+                del g
+            name = f"dense fp16 library M={m} {shape} shape"
+            extra[name] = {"us": round(best, 2), "TFLOPs": round(2.0 * m * k * n / best / 1e6, 2)}
+            log(f"  {name:34s} {best:9.2f} us  {'':8s}       {2.0 * m * k * n / best / 1e6:8.1f} TFLOP/s")
+        for m in (128, 512, 2048):
+            dense("qkv", HIDDEN, 3 * HIDDEN, m)
+            dense("gate+up", HIDDEN, 2 * INTER, m)
+            dense("down", INTER, HIDDEN, m)
+            dense("o_proj", HIDDEN, HIDDEN, m)
         best_prefill = max(v["TFLOPs"] for k, v in extra.items() if k.startswith("M=2048"))
         extra["prefill_best_TFLOPs"] = best_prefill
         extra["prefill_frac_of_fp16_mfma_peak"] = round(best_prefill / MFMA_FP16_PEAK_TFLOPS, 4)

@@ -153,7 +153,7 @@ int setup_norm(MatmulArgs &a, const void *delta, const void *norm_weight, void *
 
 // M > 16: the mid-M kernel where it is the faster one, else the tiled kernel.  Measured at LLaMA-7B /
 // 13B / 30B shapes, 256..768 rows: the tiled kernel takes over once it has enough wide tiles (72 for a plain
-// projection, 160 for the gate/up pair, 192 with the rotary epilogue) - with the rotary epilogue not while
+// projection, 160 for the gate/up pair, more than 192 with the rotary epilogue: LLaMA-7B QKV at 512 rows, 192 tiles, 75 -> 68 us) - with the rotary epilogue not while
 // their number fills the chip badly (just over one per CU with a short K, where splitting does not pay either).
 bool prefer_kslice(const KslicePlan &kp, int epi, int M, int N, int K) {
     if (!kp.ok || g_kslice_tuning.mode == 0) return false;
@@ -164,7 +164,7 @@ bool prefer_kslice(const KslicePlan &kp, int epi, int M, int N, int K) {
     const long cus = device_shape().cus;  // the crossovers were measured on 256 CUs: 72, 160 and 192 wide tiles
     if (epi == EPI_PLAIN) return wide < 9 * cus / 32;
     if (epi == EPI_SILU_MUL) return wide < 5 * cus / 8;
-    return wide < 3 * cus / 4 || gemm_plan(epi, M, N, K).score < 0.65;
+    return wide <= 3 * cus / 4 || gemm_plan(epi, M, N, K).score < 0.65;
 }
 
 // Which kernel computes columns [.., .. + n) of an M > 16 call, with what plan, and the partial sums it exchanges.
@@ -180,7 +180,7 @@ TiledChoice choose_tiled(int epi, int M, int n, int K, bool kernel_gathers) {
     c.kp = kslice_plan(epi, M, n, K, kernel_gathers);
     c.kslice = prefer_kslice(c.kp, epi, M, n, K);
     c.gp = gemm_plan(epi, M, n, K, kernel_gathers);
-    c.partial = c.kslice ? (c.kp.splitk > 1 ? kslice_partial_bytes(epi, c.kp) : 0) : gemm_partial_bytes(c.gp);
+    c.partial = c.kslice ? kslice_partial_bytes(epi, c.kp) : gemm_partial_bytes(c.gp);
     return c;
 }
 
@@ -285,7 +285,9 @@ int run_tiled(int epi, MatmulArgs &a, void *workspace, size_t workspace_bytes, h
             const int nk = a.K / 64;
             a.slot_q = nk / c.kp.splitk;
             a.slot_rem = nk % c.kp.splitk;
-            if (c.kp.splitk > 1) {
+            a.tail_first = c.kp.tail_first;
+            a.tail_split = c.kp.tail_split;
+            if (c.kp.splitk > 1 || c.kp.tail_split > 1) {
                 a.counters = reinterpret_cast<int *>(workspace);
                 a.partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_HEAD_BYTES);
             }

@@ -138,6 +138,9 @@ struct KslicePlan {
     bool wide;   // plain epilogue: 128-column strips (two blocks per wave tile) instead of 64
     int waves;   // waves per workgroup, each with its own slice of K (4 or 8)
     bool ok;     // false: the shape needs another kernel
+    // tail_split > 1 (only with splitk == 1): tiles [0, tail_first) whole, every later one - the last column strips
+    // of the launch, all their row tiles - shared by tail_split workgroups along K
+    int tail_first, tail_split;
 };
 struct KsliceTuning {
     int mode;        // 0 never, 1 where it is the faster kernel, 2 wherever it can run

@@ -80,11 +80,35 @@ __global__ __launch_bounds__(64 * KS, KS == 8 && MT == 2 ? 1 : 2) void gptq4_ksl
     const int M = p.M, K = p.K, N = p.N;
     const int tiles_m = (M + BM - 1) / BM;
 
-    // XCD-contiguous logical tile index, row tiles fastest
-    const int total = gridDim.x;
-    const int per = total >> 3, rem = total & 7;
-    const int xcd = blockIdx.x & 7;
-    const int logical = xcd * per + (xcd < rem ? xcd : rem) + (blockIdx.x >> 3);
+    // XCD-contiguous logical tile index, row tiles fastest; the workgroup's K tiles [wg_begin, wg_begin + wg_len), its
+    // rank `split` among the `nsplit` workgroups that share the tile, and the tile's index `xtile` among those that
+    // exchange partial sums
+    int logical, split, nsplit, wg_begin, wg_len, xtile;
+    {
+        const bool tail = p.tail_split > 1;  // one-dimensional grid: whole tiles first, then the parts of the shared ones
+        const int total = tail ? p.tail_first : (int)gridDim.x;
+        const int per = total >> 3, rem = total & 7;
+        const int xcd = blockIdx.x & 7;
+        logical = xcd * per + (xcd < rem ? xcd : rem) + (blockIdx.x >> 3);
+        if (!tail) {
+            split = blockIdx.y;
+            nsplit = p.splitk;
+            wg_begin = split * p.slot_q + min(split, p.slot_rem);
+            wg_len = p.slot_q + (split < p.slot_rem ? 1 : 0);
+            xtile = logical;
+        } else if ((int)blockIdx.x < total) {
+            split = 0, nsplit = 1, wg_begin = 0, wg_len = p.K / BK, xtile = 0;
+        } else {
+            const int s = p.tail_split, w = (int)blockIdx.x - total;
+            xtile = w / s;
+            split = w - xtile * s;
+            logical = total + xtile;
+            nsplit = s;
+            const int nkt = p.K / BK, q = nkt / s, r = nkt - q * s;
+            wg_begin = split * q + min(split, r);
+            wg_len = q + (split < r ? 1 : 0);
+        }
+    }
     const int tile_n = logical / tiles_m;
     const int tile_m = logical - tile_n * tiles_m;
     const int m0 = tile_m * BM;
@@ -121,9 +145,6 @@ __global__ __launch_bounds__(64 * KS, KS == 8 && MT == 2 ? 1 : 2) void gptq4_ksl
                 for (int i = 0; i < 16; ++i) acc[j][mt][t][i] = 0.f;
 
     // K tiles of the workgroup (split across workgroups), then of this wave
-    const int split = blockIdx.y;
-    const int wg_begin = split * p.slot_q + min(split, p.slot_rem);
-    const int wg_len = p.slot_q + (split < p.slot_rem ? 1 : 0);
     const int wq = wg_len / KS, wr = wg_len % KS;
     const int k_begin = wg_begin + ksl * wq + min(ksl, wr);
     const int nk = k_begin + wq + (ksl < wr ? 1 : 0);
@@ -315,13 +336,13 @@ __global__ __launch_bounds__(64 * KS, KS == 8 && MT == 2 ? 1 : 2) void gptq4_ksl
 
     KS_STAMP(4);
     constexpr int NREG = NSET * 2 * IW;  // values per lane of an owner wave
-    if (p.splitk > 1) {
+    if (nsplit > 1) {
         // K split across workgroups as well: each publishes its reduced tile (agent-scope
         // atomics, no cache maintenance), the last one to arrive sums them in split order.
         __shared__ int s_is_last;
-        const int tile = logical;
+        const int tile = xtile;
         const size_t per_split = (size_t)MT * PARTS * NREG * 64;
-        float *const mine = p.partials + ((size_t)tile * p.splitk + split) * per_split + (size_t)wave * NREG * 64 + lane;
+        float *const mine = p.partials + ((size_t)tile * nsplit + split) * per_split + (size_t)wave * NREG * 64 + lane;
         if (owner) {
 #pragma unroll
             for (int s = 0; s < NSET; ++s)
@@ -336,7 +357,7 @@ __global__ __launch_bounds__(64 * KS, KS == 8 && MT == 2 ? 1 : 2) void gptq4_ksl
         __syncthreads();
         if (tid == 0) {
             const int old = __hip_atomic_fetch_add(&p.counters[tile * COUNTER_STRIDE], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            s_is_last = (old == p.splitk - 1);
+            s_is_last = (old == nsplit - 1);
         }
         __syncthreads();
         KS_STAMP(6);
@@ -345,25 +366,25 @@ __global__ __launch_bounds__(64 * KS, KS == 8 && MT == 2 ? 1 : 2) void gptq4_ksl
             // E of the lane's values from SPR splits per round, 32 loads in flight per lane: a round is one round trip
             constexpr int E = NREG < 32 ? NREG : 32;
             constexpr int SPR = 32 / E;
-            const float *const all = p.partials + (size_t)tile * p.splitk * per_split + (size_t)wave * NREG * 64 + lane;
+            const float *const all = p.partials + (size_t)tile * nsplit * per_split + (size_t)wave * NREG * 64 + lane;
 #pragma unroll
             for (int e0 = 0; e0 < NREG; e0 += E) {
                 float sum[E];
 #pragma unroll
                 for (int e = 0; e < E; ++e) sum[e] = 0.f;
 #pragma unroll 1
-                for (int c0 = 0; c0 < p.splitk; c0 += SPR) {
+                for (int c0 = 0; c0 < nsplit; c0 += SPR) {
                     float got[SPR][E];
 #pragma unroll
                     for (int k = 0; k < SPR; ++k)
 #pragma unroll
                         for (int e = 0; e < E; ++e)  // (past the last split: the last one again, not added)
-                            got[k][e] = __hip_atomic_load(all + (size_t)min(c0 + k, p.splitk - 1) * per_split + (e0 + e) * 64, __ATOMIC_RELAXED,
+                            got[k][e] = __hip_atomic_load(all + (size_t)min(c0 + k, nsplit - 1) * per_split + (e0 + e) * 64, __ATOMIC_RELAXED,
                                                           __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
                     for (int k = 0; k < SPR; ++k)
 #pragma unroll
-                        for (int e = 0; e < E; ++e) sum[e] += (c0 + k < p.splitk) ? got[k][e] : 0.f;
+                        for (int e = 0; e < E; ++e) sum[e] += (c0 + k < nsplit) ? got[k][e] : 0.f;
                 }
 #pragma unroll
                 for (int e = 0; e < E; ++e) {
@@ -455,6 +476,7 @@ __global__ __launch_bounds__(64 * KS, KS == 8 && MT == 2 ? 1 : 2) void gptq4_ksl
 template <int EPI, int MT, bool WIDE, int KS>
 int launch_one(const MatmulArgs &a, int tiles, hipStream_t stream) {
     dim3 grid((unsigned)tiles, (unsigned)a.splitk), block(64 * KS);
+    if (a.tail_split > 1) grid = dim3((unsigned)(a.tail_first + (tiles - a.tail_first) * a.tail_split), 1u);
     hipLaunchKernelGGL((gptq4_kslice_kernel<EPI, MT, WIDE, KS>), grid, block, 0, stream, a);
     return (int)hipGetLastError();
 }
@@ -545,6 +567,27 @@ KslicePlan kslice_plan(int epi, int M, int N, int K, bool has_perm) {
         }
     }
     pl.splitk = s;
+    // Unsplit tiles past a whole number of rounds (one per CU and round; two workgroups of four waves are resident
+    // per CU, and two that share a CU take 1.6 times what one takes alone): up to half a round of them - whole column
+    // strips, every row tile, so that a row's summation order does not depend on its place in the batch - are cut along
+    // K into as many parts as spread them over the chip, and the parts run beside the whole tiles.  LLaMA-7B gate/up
+    // at 128 rows: 344 tiles, 88 of them in two parts each.
+    pl.tail_first = 0;
+    pl.tail_split = 1;
+    if (s == 1 && pl.waves == 4 && g_kslice_tuning.splitk == 0 && g_gemm_tuning.tail != 1 && pl.tiles > cus && pl.tiles <= SKINNY_MAX_TILES) {
+        const long tiles_m = (M + bm - 1) / bm, strips = N / bn;
+        const long rest = pl.tiles % cus;
+        const long cut_strips = (rest + tiles_m - 1) / tiles_m, cut = cut_strips * tiles_m;
+        if (rest > 0 && 2 * cut <= cus && cut_strips < strips) {
+            long parts = cus / cut;
+            if (parts > nk / (4 * ks)) parts = nk / (4 * ks);  // at least 4 K tiles per wave
+            if (parts > GEMM_MAX_SPLITK) parts = GEMM_MAX_SPLITK;
+            if (parts >= 2) {
+                pl.tail_first = (int)(pl.tiles - cut);
+                pl.tail_split = (int)parts;
+            }
+        }
+    }
     // the wave loop needs the activations unpermuted and at least one K tile per wave
     pl.ok = !has_perm && (N % bn) == 0 && nk / s >= ks;
     return pl;
@@ -553,6 +596,7 @@ KslicePlan kslice_plan(int epi, int M, int N, int K, bool has_perm) {
 size_t kslice_partial_bytes(int epi, const KslicePlan &pl) {
     // (the same with four or eight waves: eight split the 32 values per lane and block over two owner waves)
     const int nset = (epi == EPI_PLAIN && !pl.wide) ? 1 : 2;
+    if (pl.tail_split > 1) return (size_t)(pl.tiles - pl.tail_first) * pl.tail_split * pl.mt * nset * 32 * 64 * sizeof(float);
     return pl.splitk > 1 ? (size_t)pl.tiles * pl.splitk * pl.mt * nset * 32 * 64 * sizeof(float) : 0;
 }
 

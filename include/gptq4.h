@@ -302,7 +302,7 @@ void gptq4_set_tuning(int words, int depth, int splitk);
  * schedule (K tiles of all wide tiles dealt evenly to the resident workgroups; never chosen
  * automatically, it measured slower) wherever it can run, mt = 100: never; mt = 300: never cut a call into two
  * launches over adjacent column ranges, mt = 400: never cut the column panels past the last whole round of wide tiles
- * along K inside the launch, mt = 500: neither (both are done automatically where the wide-tile count is just above
+ * along K inside the launch (the mid-M kernel's launches included), mt = 500: neither (both are done automatically where the wide-tile count is just above
  * a multiple of the CU count); tile and split automatic with all five. */
 void gptq4_set_gemm_tuning(int mt, int splitk);
 

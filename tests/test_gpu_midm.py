@@ -181,3 +181,64 @@ def test_act_order_inputs_reach_the_mid_m_kernel_through_the_staged_copy():
                           _lib.current_stream(xd.device))
     assert rc == 0
     assert_close(y.cpu().numpy(), ref, "act-order through the C ABI, M=48, no room for the gathered rows")
+
+
+def test_tile_counts_just_above_a_whole_number_of_rounds_share_their_last_strips():
+    """More tiles than CUs, fewer than one and a half times as many: the last column strips (every row tile of them) are
+    shared by two workgroups along K inside the launch.  Against the oracle, against the same plan without the sharing
+    (`gptq4_set_gemm_tuning(400, 0)`; another summation order in the shared strips, the same bits elsewhere), and a row
+    keeps its bits wherever it sits in the batch."""
+    from gptq_triton_amd import _lib
+    lib = _lib.load()
+    G = gptq()
+    g = 128
+    # gate/up: 88 strips x 4 row tiles = 352 tiles
+    k, n, m = 2048, 5632, 200
+    gate, up = O.make_layer(k, n, g, seed=400), O.make_layer(k, n, g, seed=401)
+    Dg, Du = to_dev(gate), to_dev(up)
+    x = O.make_x(m, k, seed=402)
+    xd = torch.from_numpy(x).cuda()
+    run = lambda xx: G.llama_mlp_4(g, xx, Dg["qweight"], Dg["scales"], Dg["qzeros"], Du["qweight"], Du["scales"], Du["qzeros"])
+    h = run(xd)
+    assert torch.equal(h, run(xd))
+    perm = torch.randperm(m, generator=torch.Generator().manual_seed(3)).cuda()
+    assert torch.equal(run(xd[perm]), h[perm])
+    ref = O.mlp_gateup_ref(x, (gate["qweight"], gate["qzeros"], gate["scales"]), (up["qweight"], up["qzeros"], up["scales"]), g)
+    assert_close(h.cpu().numpy(), ref, "gate/up, shared last strips")
+    try:
+        lib.gptq4_set_gemm_tuning(400, 0)
+        h0 = run(xd)
+    finally:
+        lib.gptq4_set_gemm_tuning(0, 0)
+    assert_close(h0.cpu().numpy(), ref, "gate/up, no sharing")
+    whole = (352 - 96) // 4 * 64          # columns of the strips that stay whole: 256 CUs -> 96 tiles = 24 strips shared
+    assert torch.equal(h[:, :whole], h0[:, :whole]) and not torch.equal(h[:, whole:], h0[:, whole:])
+
+    # QKV + rotary: 48 heads' strips x 7 row tiles = 336 tiles
+    hidden, heads, m = 2048, 16, 400
+    L = O.make_layer(hidden, 3 * hidden, g, seed=410)
+    D = to_dev(L)
+    x = O.make_x(m, hidden, seed=411).reshape(1, m, hidden)
+    pos = np.arange(m)[None, :].astype(np.int32)
+    cos, sin = G.RotaryTable(128, 512).get(torch.device("cuda"), 512)
+    q, kk, v = G.qkv_rotary(g, torch.from_numpy(x).cuda(), D["qweight"], D["scales"], D["qzeros"], torch.from_numpy(pos).cuda(), cos, sin, heads)
+    qr, kr, vr = O.qkv_rotary_ref(x, L["qweight"], L["qzeros"], L["scales"], g, pos, heads, 128, max_pos=512)
+    for got, want, name in ((q, qr, "q"), (kk, kr, "k"), (v, vr, "v")):
+        assert_close(got.cpu().numpy(), want, f"{name}, shared last strips")
+
+    # a plain projection with four waves per workgroup: 96 strips x 3 row tiles = 288 tiles
+    k, n, m = 2048, 6144, 150
+    L = O.make_layer(k, n, g, seed=420, bias=True)
+    D = to_dev(L)
+    x = O.make_x(m, k, seed=421)
+    try:
+        lib.gptq4_set_midm_tuning(2, 100, 0)
+        y = G.matmul4(g, torch.from_numpy(x).cuda(), D["qweight"], D["scales"], D["qzeros"], D["bias"])
+    finally:
+        lib.gptq4_set_midm_tuning(1, 0, 0)
+    ok, max_abs, _ = O.within_tolerance(y.cpu().numpy(), O.quant_matmul_ref(x, L["qweight"], L["qzeros"], L["scales"], g, bias=L["bias"]))
+    assert ok, max_abs
+    from gptq_triton_amd import _lib as L_
+    ws = L_.workspace(torch.device("cuda", torch.cuda.current_device()), 0)
+    torch.cuda.synchronize()
+    assert int(ws[:L_.WS_HEAD_BYTES].view(torch.int32).abs().sum()) == 0
