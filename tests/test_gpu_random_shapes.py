@@ -135,3 +135,24 @@ def test_the_checker_agrees_with_the_oracle(idx):
     mine = (torch.from_numpy(x).cuda().double() @ dequant64(G, D, k, g)).cpu().numpy()
     # (the oracle hands its float64 sums back rounded to float32)
     assert (np.abs(mine - ref) <= 2.0 ** -23 * np.abs(ref) + 1e-9).all()
+
+
+@pytest.mark.parametrize("m,k,n,g", [s for s in draw_shapes(4, 90, 256, 8192) if s[3] != -1][:60])
+def test_act_order_projection(m, k, n, g):
+    """Rows of the weight in a random group order (g_idx): the sorted copy and the permutation made at load time, the
+    activations gathered by the call; plain projection and the gate/up pair on the same draw."""
+    G = gptq()
+    rng = np.random.default_rng(m + k)
+    g_idx = torch.from_numpy(rng.permutation(np.repeat(np.arange(k // g), g)).astype(np.int32)).cuda()
+    Dg, Du = to_dev(layer(k, n, g, seed=m + n + 5)), to_dev(layer(k, n, g, seed=m + n + 6))
+    x = torch.from_numpy(O.make_x(m, k, seed=m + 2)).cuda()
+    wg = G.dequantize(Dg["qweight"], Dg["qzeros"], Dg["scales"], g, g_idx).double()
+    wu = G.dequantize(Du["qweight"], Du["qzeros"], Du["scales"], g, g_idx).double()
+    gq, perm = G.prepare_act_order(Dg["qweight"], g_idx, g)
+    uq, _ = G.prepare_act_order(Du["qweight"], g_idx, g)
+    y = G.matmul4(g, x, gq, Dg["scales"], Dg["qzeros"], None, perm)
+    close(y, x.double() @ wg, sum_noise(x, wg), f"act-order matmul M={m} K={k} N={n} g={g}")
+    h = G.llama_mlp_4(g, x, gq, Dg["scales"], Dg["qzeros"], uq, Du["scales"], Du["qzeros"], perm=perm)
+    a, b = x.double() @ wg, x.double() @ wu
+    silu = a / (1.0 + torch.exp(-a))
+    close(h, silu * b, 1.1 * b.abs() * sum_noise(x, wg) + silu.abs() * sum_noise(x, wu), f"act-order gate/up M={m} K={k} N={n} g={g}")
