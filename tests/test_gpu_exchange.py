@@ -160,3 +160,33 @@ def test_the_python_layer_reports_and_clears_an_exchange_error():
     assert _lib.exchange_errors() == []
     y = G.matmul4(g, xd, D["qweight"], D["scales"], D["qzeros"])
     assert_close(y.cpu().numpy(), O.quant_matmul_ref(x, L["qweight"], L["qzeros"], L["scales"], g), "after the reset")
+
+
+def test_two_streams_with_a_workspace_each_do_not_disturb_each_other():
+    """Calls that overlap in time on two streams (default priority), each stream with the workspace the Python layer
+    keeps for it: the same bits as the same calls made alone, for the marked exchange, the counter exchange and the
+    mid-M kernel's split across workgroups."""
+    from gptq_triton_amd import _lib
+    G = gptq()
+    k, n, g = 4096, 4096, 128
+    La, Lb = O.make_layer(k, n, g, seed=70), O.make_layer(11008, n, g, seed=71)
+    Da, Db = to_dev(La), to_dev(Lb)
+    xs = {m: torch.from_numpy(O.make_x(m, k, seed=72 + m)).cuda() for m in (1, 8, 48)}
+    xb = {m: torch.from_numpy(O.make_x(m, 11008, seed=80 + m)).cuda() for m in (1, 8, 48)}
+    alone_a = {m: G.matmul4(g, xs[m], Da["qweight"], Da["scales"], Da["qzeros"]) for m in xs}
+    alone_b = {m: G.matmul4(g, xb[m], Db["qweight"], Db["scales"], Db["qzeros"]) for m in xb}
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    got_a, got_b = [], []
+    for rep in range(40):
+        for m in (1, 8, 48):
+            with torch.cuda.stream(s1):
+                got_a.append((m, G.matmul4(g, xs[m], Da["qweight"], Da["scales"], Da["qzeros"])))
+            with torch.cuda.stream(s2):
+                got_b.append((m, G.matmul4(g, xb[m], Db["qweight"], Db["scales"], Db["qzeros"])))
+    torch.cuda.synchronize()
+    assert all(torch.equal(y, alone_a[m]) for m, y in got_a)
+    assert all(torch.equal(y, alone_b[m]) for m, y in got_b)
+    _lib.check_exchange_errors()
+    keys = {key[1] for key in _lib._workspaces}
+    assert s1.cuda_stream in keys and s2.cuda_stream in keys
