@@ -62,8 +62,8 @@ __global__ __launch_bounds__(256) void gptq4_rmsnorm_kernel(const half_t *x, con
     for (int c = tid + 256 * KEEP; c < chunks; c += 256) put(c, ADD ? sr[c] : xr[c]);
 }
 
-// Single-query attention, split over the cache length.  Workgroup (split, b*H + h) takes
-// rows [split*chunk, ...) of the valid prefix 0..positions[b]; 16 lanes share a row (8
+// Single-query attention, split over the valid prefix 0..positions[b] of the cache.  Workgroup (split, b*H + h) takes
+// an equal share of its rows (at most `chunk`, the share at full capacity); 16 lanes share a row (8
 // head dimensions each, one 16-byte load of K and of V per lane), 16 rows per pass,
 // running (max, sum, weighted V) per thread in fp32; the 16 row slots are merged through
 // LDS and the partial [max, sum, acc[128]] goes to the workspace.  The splits of one (b, h)
@@ -86,7 +86,10 @@ __global__ __launch_bounds__(256) void gptq4_attn_decode_kernel(const half_t *__
     const int bh = blockIdx.y, split = blockIdx.x, nsplit = gridDim.x;
     const int b = bh / H;
     const int len = min(max(positions[b], 0), capacity - 1) + 1;
-    const int r0 = split * chunk, r1 = min(r0 + chunk, len);
+    // the valid prefix, not the capacity, is dealt to the splits (in multiples of the 16 rows of a pass): a short
+    // context in a long cache still spreads over all of them
+    const int mine = min(chunk, (((len + nsplit - 1) / nsplit) + 15) & ~15);
+    const int r0 = split * mine, r1 = min(r0 + mine, len);
 
     float qf[8];
     {
