@@ -93,7 +93,7 @@ int run_small(int epi, MatmulArgs &a, int nmat, void *workspace, size_t workspac
                 return launch_gemv(epi, a, gp, s);
             }
         }
-        const SkinnyPlan pl = skinny_plan(epi, a.N, a.K, true);
+        const SkinnyPlan pl = skinny_plan(epi, a.M, a.N, a.K, true);
         int rc = setup_skinny(a, pl, nmat, workspace, workspace_bytes);
         if (rc) return rc;
         return launch_skinny(epi, a, pl, s);
@@ -107,7 +107,7 @@ int run_small(int epi, MatmulArgs &a, int nmat, void *workspace, size_t workspac
             return launch_gemv(epi, a, pl, s);
         }
     }
-    const SkinnyPlan pl = skinny_plan(epi, a.N, a.K);
+    const SkinnyPlan pl = skinny_plan(epi, a.M, a.N, a.K);
     int rc = setup_skinny(a, pl, nmat, workspace, workspace_bytes);
     if (rc) return rc;
     if (a.perm != nullptr) {

@@ -79,7 +79,7 @@ struct SkinnyTuning {
 };
 extern SkinnyTuning g_skinny_tuning;
 // standard_shape: ignore the tuning overrides of words, depth and waves (the split is still tunable)
-SkinnyPlan skinny_plan(int epi, int N, int K, bool standard_shape = false);
+SkinnyPlan skinny_plan(int epi, int M, int N, int K, bool standard_shape = false);
 // Small-M (M <= 16) split-K matrix-core GEMV.  Returns hipError_t.
 int launch_skinny(int epi, const MatmulArgs &a, const SkinnyPlan &plan, hipStream_t stream);
 // Balanced decode GEMV (M <= GEMV_MAX_M): (tile, batch) units dealt evenly to waves.

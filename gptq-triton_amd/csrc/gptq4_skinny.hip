@@ -597,20 +597,24 @@ static int split_for(int tiles, int k_batches, int waves) {
     return s < 1 ? 1 : s;
 }
 
-SkinnyPlan skinny_plan(int epi, int N, int K, bool standard_shape) {
+SkinnyPlan skinny_plan(int epi, int M, int N, int K, bool standard_shape) {
     SkinnyPlan pl;
     const bool tuned = !standard_shape;
     const int k_batches = K / 128;
     pl.waves = (tuned && g_skinny_tuning.waves > 0) ? g_skinny_tuning.waves : 4;
     pl.words = 2;
-    pl.depth = (epi == EPI_SILU_MUL) ? 1 : 2;
+    // Batches of loads in flight per wave: two, but one for the gate/up pair (two matrices' worth of registers) and for
+    // plain projections of up to 4 rows - measured at LLaMA-7B / 13B / 30B shapes with the weights coming from HBM:
+    // 7B o_proj 6.2 -> 5.9 us and down_proj 9.6 -> 8.6 at one row, 13B down_proj 12.5 -> 11.4, 30B o_proj 9.5 -> 8.6,
+    // level elsewhere; from 8 rows on and with the rotary epilogue two are level or ahead.
+    pl.depth = (epi == EPI_SILU_MUL || (epi == EPI_PLAIN && M <= 4)) ? 1 : 2;
     if (tuned && epi != EPI_ROPE && (long)(N / 64) * split_for(N / 64, k_batches, pl.waves) >= 900) {
         pl.words = 4;
         pl.depth = 1;
     }
     if (tuned && g_skinny_tuning.words > 0) {
         pl.words = g_skinny_tuning.words;
-        pl.depth = (epi == EPI_SILU_MUL) ? 1 : 2;
+        pl.depth = (epi == EPI_SILU_MUL || (epi == EPI_PLAIN && M <= 4)) ? 1 : 2;
     }
     if (tuned && g_skinny_tuning.depth > 0) pl.depth = g_skinny_tuning.depth;
     // the instantiated (width, depth) pairs: 4 bytes x {2, 4}, 8 bytes x {1, 2, 4}, 16 bytes x {1, 2}
