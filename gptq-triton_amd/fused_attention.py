@@ -143,6 +143,20 @@ def _fuse_qkv(q_proj: QuantLinear, k_proj: QuantLinear, v_proj: QuantLinear) -> 
     return layer
 
 
+def _rope_base(config) -> float:
+    """Base of the rotary embedding: `rope_theta` of the config, which newer transformers keep inside
+    `rope_parameters`; only the default (unscaled) embedding is supported, as in the reference."""
+    params = getattr(config, 'rope_parameters', None) or getattr(config, 'rope_scaling', None)
+    if isinstance(params, dict):
+        kind = params.get('rope_type', params.get('type', 'default'))
+        if kind not in (None, 'default'):
+            raise NotImplementedError(f"rotary embedding of type {kind!r} is not supported (only the default one)")
+        if params.get('rope_theta') is not None:
+            return float(params['rope_theta'])
+    theta = getattr(config, 'rope_theta', None)
+    return float(theta) if theta is not None else 10000.0
+
+
 def _is_llama_attention(m: nn.Module) -> bool:
     if isinstance(m, QuantLlamaAttention):
         return False
@@ -155,8 +169,12 @@ def make_quant_attn(model: nn.Module):
     for name, m in list(model.named_modules()):
         if not _is_llama_attention(m):
             continue
+        if not (m.q_proj.outfeatures == m.k_proj.outfeatures == m.v_proj.outfeatures):
+            raise NotImplementedError("grouped-query attention (fewer key/value heads than query heads) is not supported: "
+                                      "the fused kernel takes q, k and v of one width, as the reference's does")
         qkv = _fuse_qkv(m.q_proj, m.k_proj, m.v_proj)
         attn = QuantLlamaAttention(m.config, qkv, m.o_proj, getattr(m, 'rotary_emb', None))
+        attn.layer_idx = getattr(m, 'layer_idx', None)  # the slot of a transformers Cache this block updates
         parent_name, _, child = name.rpartition('.')
         parent = model.get_submodule(parent_name) if parent_name else model
         if not name:
@@ -184,8 +202,8 @@ class QuantLlamaAttention(nn.Module):
         # kept for interface compatibility; the kernel reads its own table, which follows
         # the same closed form (base from config.rope_theta, default 10000)
         self.rotary_emb = rotary_emb
-        self.rope = RotaryTable(self.head_dim, self.max_position_embeddings,
-                                float(getattr(config, 'rope_theta', 10000.0)))
+        self.rope = RotaryTable(self.head_dim, self.max_position_embeddings, _rope_base(config))
+        self.layer_idx = None
         self._context_order = None
         self._input_order = None
 
@@ -247,8 +265,21 @@ class QuantLlamaAttention(nn.Module):
         past_key_value: Optional[Tuple[torch.Tensor]] = None,
         output_attentions: bool = False,
         use_cache: bool = False,
+        past_key_values=None,
+        position_embeddings=None,
+        **kwargs,
     ) -> Tuple[torch.Tensor, Optional[torch.Tensor], Optional[Tuple[torch.Tensor]]]:
-        """Input shape: Batch x Time x Channel"""
+        """Input shape: Batch x Time x Channel.
+
+        Two calling conventions.  The reference's (fused_attention.py:80-153, transformers of 2023): `past_key_value` is a
+        (key, value) pair or None, the result is (output, weights or None, (key, value) or None).  Called the way the
+        decoder layer of current transformers calls its attention block - `past_key_values` (a Cache object or None)
+        and / or `position_embeddings` given - it updates the Cache in slot `layer_idx` and returns (output, weights or
+        None); the cos / sin handed in are not used: the kernel turns q and k itself, from `position_ids`."""
+        if past_key_values is not None or position_embeddings is not None:
+            return self._forward_with_cache(hidden_states, attention_mask, position_ids, past_key_values,
+                                            output_attentions or bool(kwargs.get('output_attentions', False)),
+                                            kwargs.get('cache_position'))
         bsz, q_len, _ = hidden_states.size()
         past_len = 0 if past_key_value is None else past_key_value[0].shape[-2]
         kv_seq_len = past_len + q_len
@@ -296,3 +327,48 @@ class QuantLlamaAttention(nn.Module):
         attn_output = attn_output.transpose(1, 2).reshape(bsz, q_len, self.hidden_size)
         attn_output = self.o_proj(attn_output)
         return attn_output, attn_weights, past_key_value
+
+
+def _forward_with_cache(self, hidden_states, attention_mask, position_ids, cache, output_attentions, cache_position):
+    """The call of a current transformers decoder layer (see QuantLlamaAttention.forward)."""
+    bsz, q_len, _ = hidden_states.size()
+    if position_ids is None:
+        if cache_position is not None:
+            position_ids = cache_position.unsqueeze(0)
+        else:
+            past = 0 if cache is None else int(cache.get_seq_length(self.layer_idx))
+            position_ids = torch.arange(past, past + q_len, device=hidden_states.device).unsqueeze(0)
+    if position_ids.shape[0] != bsz:
+        position_ids = position_ids.expand(bsz, -1)
+    query_states, key_states, value_states = self.project_qkv(hidden_states, position_ids.contiguous())
+    if cache is not None:
+        if self.layer_idx is None:
+            raise ValueError("this attention block does not know its layer index and cannot update a Cache")
+        key_states, value_states = cache.update(key_states, value_states, self.layer_idx)
+    kv_len = key_states.shape[-2]
+    attn_weights = None
+    if output_attentions:
+        attn_weights = torch.matmul(query_states, key_states.transpose(2, 3)) / math.sqrt(self.head_dim)
+        if attention_mask is not None:
+            if attention_mask.dtype == torch.bool:
+                attn_weights = attn_weights.masked_fill(~attention_mask[..., :kv_len], torch.finfo(attn_weights.dtype).min)
+            else:
+                attn_weights = torch.clamp_min(attn_weights + attention_mask[..., :kv_len], torch.finfo(attn_weights.dtype).min)
+        elif q_len > 1:
+            causal = torch.ones(q_len, kv_len, dtype=torch.bool, device=attn_weights.device).tril(kv_len - q_len)
+            attn_weights = attn_weights.masked_fill(~causal, torch.finfo(attn_weights.dtype).min)
+        attn_weights = nn.functional.softmax(attn_weights, dim=-1, dtype=torch.float32).to(query_states.dtype)
+        attn_output = torch.matmul(attn_weights, value_states)
+    else:
+        # as transformers' own scaled-dot-product path: a given mask is used as it is, none means causal for a prompt
+        # and full attention for a single token
+        mask = None if attention_mask is None else attention_mask[..., :kv_len]
+        attn_output = nn.functional.scaled_dot_product_attention(query_states, key_states, value_states, attn_mask=mask,
+                                                                 is_causal=(mask is None and q_len > 1 and kv_len == q_len))
+        if mask is None and q_len > 1 and kv_len != q_len:
+            raise ValueError("a prompt chunk behind cached tokens needs an attention mask")
+    attn_output = attn_output.transpose(1, 2).reshape(bsz, q_len, self.hidden_size)
+    return self.o_proj(attn_output), attn_weights
+
+
+QuantLlamaAttention._forward_with_cache = _forward_with_cache

@@ -22,8 +22,13 @@ from .quant_linear import QuantLinear, make_quant
 
 
 def load_quant(checkpoint: str, warmup_autotune: bool = True, device: Optional[str] = 'cuda',
-               fuse_mlp: Optional[bool] = None):
+               fuse_mlp: Optional[bool] = None, use_transformers: bool = False):
     """Load a quantised model from a checkpoint directory.
+
+    use_transformers: build the skeleton as the reference does (src/gptq_triton/__init__.py:32-52): a
+    `transformers.LlamaForCausalLM` from the checkpoint's config.json, whose linears, attention blocks and MLPs are
+    then replaced - the result is a transformers model (`generate`, Cache objects, pipelines).  Default: this
+    package's own minimal decoder, which needs no transformers at run time.
 
     warmup_autotune is accepted for compatibility: launch shapes are static, there is
     nothing to tune (the reference spends 18-49 s here).  It still requires a device, as
@@ -38,10 +43,22 @@ def load_quant(checkpoint: str, warmup_autotune: bool = True, device: Optional[s
     torch.set_default_dtype(torch.half)
     try:
         with torch.device('meta'):
-            model = LlamaForCausalLM(config)
+            if use_transformers:
+                import transformers
+                hf_config = transformers.LlamaConfig.from_pretrained(str(ckpt))
+                model = transformers.LlamaForCausalLM(hf_config)
+            else:
+                model = LlamaForCausalLM(config)
     finally:
         torch.set_default_dtype(default_dtype)
     model = model.to_empty(device='cpu')
+    if use_transformers:
+        # buffers that are computed, not stored (the rotary frequencies), are lost on the meta device: rebuild their modules
+        for name, m in list(model.named_modules()):
+            if name and any(b == 'inv_freq' for b, _ in m.named_buffers(recurse=False)):
+                parent_name, _, child = name.rpartition('.')
+                parent = model.get_submodule(parent_name) if parent_name else model
+                setattr(parent, child, type(m)(config=hf_config))
 
     if (ckpt / 'model.safetensors').exists():
         from safetensors.torch import load_file
