@@ -143,6 +143,8 @@ def decoder_figures(workload, bsz, prompt, new):
     model.lm_head.weight.copy_(torch.randn(model.lm_head.weight.shape, device=dev, generator=gen) * 0.02)
     G.make_quant_attn(model)
     G.make_fused_mlp(model)
+    if act_order:
+        G.quant_linear.compact_act_order(model)  # one copy of every packed weight, in the layout the kernels read
 
     ids = torch.randint(0, cfg.vocab_size, (bsz, prompt), device=dev, generator=gen)
     dec = GreedyDecoder(model, bsz, prompt + new)

@@ -114,8 +114,65 @@ class QuantLlamaMLP(nn.Module):
         self._sorted = None
         self._chained = None
         self._input_order = None
+        # compact(): the six gate / up buffers hold the layout forward() multiplies with; these say how it was made
+        self._is_compact = False
+        self.register_buffer('_compact_rows', None, persistent=False)   # row permutation (act-order input), or None
+        self.register_buffer('_compact_cols', None, persistent=False)   # column order (act-order down_proj), or None
+
+    _SIX = ('gate_proj_qweight', 'gate_proj_scales', 'gate_proj_qzeros', 'up_proj_qweight', 'up_proj_scales', 'up_proj_qzeros')
+
+    def compact(self) -> None:
+        """Act-order, on the GPU: keep ONE copy of the gate and up tensors, in the layout forward() reads (rows sorted
+        by group, columns in the order of an act-order down_proj's rows), in the module's own buffers - otherwise that
+        layout lives beside the checkpoint tensors.  state_dict() still gives the checkpoint layout (rows and columns
+        put back on the way out) and load_state_dict() brings the module back to it."""
+        if self._is_compact or not self.gate_proj_qweight.is_cuda:
+            return
+        self.down_proj.compact()
+        w, perm, _ = self._chained_weights()
+        _, down_perm = self.down_proj.kernel_weights()
+        if perm is None and down_perm is None:
+            return
+        for name, t in zip(self._SIX, w):
+            setattr(self, name, t)
+        self._compact_rows = perm
+        self._compact_cols = None if down_perm is None else down_perm.long()
+        self._is_compact = True
+        self._sorted = self._chained = None
+
+    def checkpoint_tensors(self) -> dict:
+        """The six gate / up tensors in the checkpoint's layout, by buffer name."""
+        out = {name: getattr(self, name) for name in self._SIX}
+        if not self._is_compact:
+            return out
+        from .quant_linear import inverse_permutation, sort_rows
+        if self._compact_cols is not None:
+            inv = inverse_permutation(self._compact_cols)
+            for name in self._SIX:
+                out[name] = _move_zero_columns(out[name], inv) if name.endswith('qzeros') else out[name].index_select(1, inv).contiguous()
+        if self._compact_rows is not None:
+            back = inverse_permutation(self._compact_rows)
+            for name in ('gate_proj_qweight', 'up_proj_qweight'):
+                out[name] = sort_rows(out[name], back)
+        return out
+
+    def _save_to_state_dict(self, destination, prefix, keep_vars):
+        super()._save_to_state_dict(destination, prefix, keep_vars)
+        if self._is_compact:
+            for name, t in self.checkpoint_tensors().items():
+                destination[prefix + name] = t
+
+    def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
+        if self._is_compact:
+            for name, t in self.checkpoint_tensors().items():
+                setattr(self, name, t)
+            self._is_compact = False
+            self._compact_rows = self._compact_cols = None
+        super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
 
     def _kernel_weights(self):
+        if self._is_compact:
+            raise RuntimeError("a compacted module multiplies through _chained_weights()")
         if self.g_idx is None:
             return self.gate_proj_qweight, self.up_proj_qweight, None
         key = tensor_key(self.gate_proj_qweight, self.up_proj_qweight, self.g_idx)
@@ -127,6 +184,12 @@ class QuantLlamaMLP(nn.Module):
         return self._sorted[1], self._sorted[2], self._sorted[3]
 
     def gate_up(self, x: torch.Tensor) -> torch.Tensor:
+        if self._is_compact:
+            mid = llama_mlp_4(self.groupsize, x, *(getattr(self, n) for n in self._SIX), self._compact_rows)
+            if self._compact_cols is None:
+                return mid
+            from .quant_linear import inverse_permutation
+            return mid.index_select(-1, inverse_permutation(self._compact_cols))
         gq, uq, perm = self._kernel_weights()
         return llama_mlp_4(self.groupsize, x, gq, self.gate_proj_scales, self.gate_proj_qzeros,
                            uq, self.up_proj_scales, self.up_proj_qzeros, perm)
@@ -139,6 +202,8 @@ class QuantLlamaMLP(nn.Module):
         column only moves, its values do not change).  The intermediate then comes out of the gate/up
         launch already in the order down_proj's kernel reads, and down_proj runs without a gather."""
         down_q, down_perm = self.down_proj.kernel_weights()
+        if self._is_compact:
+            return tuple(getattr(self, n) for n in self._SIX), self._compact_rows, down_q
         if down_perm is None:
             gq, uq, perm = self._kernel_weights()
             return (gq, self.gate_proj_scales, self.gate_proj_qzeros, uq, self.up_proj_scales, self.up_proj_qzeros), perm, down_q

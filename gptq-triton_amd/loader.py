@@ -22,13 +22,17 @@ from .quant_linear import QuantLinear, make_quant
 
 
 def load_quant(checkpoint: str, warmup_autotune: bool = True, device: Optional[str] = 'cuda',
-               fuse_mlp: Optional[bool] = None, use_transformers: bool = False):
+               fuse_mlp: Optional[bool] = None, use_transformers: bool = False, compact: bool = True):
     """Load a quantised model from a checkpoint directory.
 
     use_transformers: build the skeleton as the reference does (src/gptq_triton/__init__.py:32-52): a
     `transformers.LlamaForCausalLM` from the checkpoint's config.json, whose linears, attention blocks and MLPs are
     then replaced - the result is a transformers model (`generate`, Cache objects, pipelines).  Default: this
     package's own minimal decoder, which needs no transformers at run time.
+
+    compact: act-order checkpoints on a GPU keep ONE copy of every packed weight, in the layout the kernels read
+    (QuantLinear.compact, QuantLlamaMLP.compact); state_dict() / save_quant() still produce the checkpoint layout.
+    With False the kernel layout is built at first use beside the checkpoint tensors (twice the weight memory).
 
     warmup_autotune is accepted for compatibility: launch shapes are static, there is
     nothing to tune (the reference spends 18-49 s here).  It still requires a device, as
@@ -94,6 +98,8 @@ def load_quant(checkpoint: str, warmup_autotune: bool = True, device: Optional[s
 
     if device is not None:
         model = model.to(device)
+        if compact and act_order and torch.device(device).type == 'cuda':
+            quant_linear.compact_act_order(model)
     if warmup_autotune:
         if device is None:
             raise ValueError("You must specify a device when warmup_autotune is True.")

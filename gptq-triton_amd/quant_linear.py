@@ -101,6 +101,16 @@ def inverse_permutation(perm: torch.Tensor) -> torch.Tensor:
     return inv
 
 
+def sort_rows(qweight: torch.Tensor, perm: torch.Tensor) -> torch.Tensor:
+    """Packed weight whose nibble row j is row perm[j] of `qweight` (perm int32 [K])."""
+    _lib.require_cuda(qweight, "qweight")
+    out = torch.empty_like(qweight)
+    rc = _lib.load().gptq4_actorder_sort_rows(qweight.data_ptr(), perm.data_ptr(), out.data_ptr(), qweight.shape[0] * 8,
+                                              qweight.shape[1], _lib.current_stream(qweight.device))
+    _lib.check(rc, "gptq4_actorder_sort_rows")
+    return out
+
+
 def prepare_act_order(qweight: torch.Tensor, g_idx: torch.Tensor, groupsize: int):
     """Load-time re-layout for act-order checkpoints.
 
@@ -117,12 +127,7 @@ def prepare_act_order(qweight: torch.Tensor, g_idx: torch.Tensor, groupsize: int
     if g.numel() != k or bool((counts != gs).any()):
         raise NotImplementedError("act-order g_idx must assign exactly `groupsize` rows to every group")
     perm = torch.argsort(g, stable=True).to(torch.int32).contiguous()
-    out = torch.empty_like(qweight)
-    lib = _lib.load()
-    rc = lib.gptq4_actorder_sort_rows(qweight.data_ptr(), perm.data_ptr(), out.data_ptr(), k, n,
-                                      _lib.current_stream(qweight.device))
-    _lib.check(rc, "gptq4_actorder_sort_rows")
-    return out, perm
+    return sort_rows(qweight, perm), perm
 
 
 class QuantLinear(nn.Module):
@@ -154,6 +159,38 @@ class QuantLinear(nn.Module):
         else:
             self.g_idx = None
         self._sorted = None  # (key, qweight_sorted, perm), built at first use
+        # compact(): `qweight` holds the row-sorted layout and this the permutation that made it
+        self.register_buffer('_compact_perm', None, persistent=False)
+
+    def compact(self) -> None:
+        """Act-order, on the GPU: keep ONE copy of the packed weight, the row-sorted one the kernels read, in the
+        `qweight` buffer (otherwise the sorted copy lives beside the checkpoint tensor).  state_dict() and
+        dequantize() still give the checkpoint layout (rows put back on the way out); load_state_dict() brings the
+        module back to the checkpoint layout.  Code that reads or writes `.qweight` directly should use
+        checkpoint_qweight() / load_state_dict() on a compacted module."""
+        if self.g_idx is None or self._compact_perm is not None or not self.qweight.is_cuda:
+            return
+        qs, perm = self._act_order()
+        self.qweight = qs
+        self._compact_perm = perm
+        self._sorted = None
+
+    def checkpoint_qweight(self) -> torch.Tensor:
+        """The packed weight in the checkpoint's row order."""
+        if self._compact_perm is None:
+            return self.qweight
+        return sort_rows(self.qweight, inverse_permutation(self._compact_perm))
+
+    def _save_to_state_dict(self, destination, prefix, keep_vars):
+        super()._save_to_state_dict(destination, prefix, keep_vars)
+        if self._compact_perm is not None:
+            destination[prefix + 'qweight'] = self.checkpoint_qweight()
+
+    def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
+        if self._compact_perm is not None:
+            self.qweight = self.checkpoint_qweight()
+            self._compact_perm = None
+        super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
 
     def _act_order(self):
         key = tensor_key(self.qweight, self.g_idx)
@@ -166,6 +203,8 @@ class QuantLinear(nn.Module):
         """(qweight, perm) as the kernels consume them."""
         if self.g_idx is None:
             return self.qweight, None
+        if self._compact_perm is not None:
+            return self.qweight, self._compact_perm
         return self._act_order()
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
@@ -173,7 +212,7 @@ class QuantLinear(nn.Module):
         return matmul4(self.groupsize, x, qweight, self.scales, self.qzeros, self.bias, perm)
 
     def dequantize(self) -> torch.Tensor:
-        return dequantize(self.qweight, self.qzeros, self.scales, self.groupsize, self.g_idx)
+        return dequantize(self.checkpoint_qweight(), self.qzeros, self.scales, self.groupsize, self.g_idx)
 
 
 def make_quant(model: nn.Module, bits: int, groupsize: int, act_order: bool = False):
@@ -193,3 +232,12 @@ def autotune_warmup(model):
     kernels pick their launch shape statically, so there is nothing to tune: yields no
     warm-up work and keeps the call site valid."""
     return iter(())
+
+
+def compact_act_order(model: nn.Module) -> None:
+    """compact() every act-order module of a model that is on the GPU: one copy of each packed weight instead of the
+    checkpoint tensor plus the layout the kernels read (see QuantLinear.compact)."""
+    from .fused_mlp import QuantLlamaMLP
+    for m in model.modules():
+        if isinstance(m, (QuantLinear, QuantLlamaMLP)):
+            m.compact()

@@ -256,3 +256,51 @@ def test_decode_past_max_position_embeddings_keeps_rotating(tmp_path, use_graph)
     for (kc, vc), (k_full, v_full) in zip(dec.caches, past):
         assert (kc[:, :, :20].float() - k_full.float()).abs().max().item() < 0.03 * k_full.float().abs().max().item()
         assert (vc[:, :, :20].float() - v_full.float()).abs().max().item() < 0.03 * v_full.float().abs().max().item()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fuse_mlp", [True, False])
+def test_compacted_act_order_model_keeps_one_copy_and_the_checkpoint_layout_outside(tmp_path, fuse_mlp):
+    """load_quant(compact=True), the default: an act-order model on the GPU holds each packed weight once, in the
+    layout the kernels read.  Same logits bit for bit as the uncompacted model, state_dict() / save_quant() give the
+    checkpoint's tensors, and load_state_dict() of other weights is followed."""
+    from safetensors.torch import load_file
+    cfg = make_checkpoint(tmp_path / "a", 128, act_order=True, seed=21)
+    make_checkpoint(tmp_path / "b", 128, act_order=True, seed=22)
+    state_a = load_file(str(tmp_path / "a" / "model.safetensors"))
+    plain = G.load_quant(str(tmp_path / "a"), device="cuda", fuse_mlp=fuse_mlp, compact=False)
+    compact = G.load_quant(str(tmp_path / "a"), device="cuda", fuse_mlp=fuse_mlp)
+    ids = torch.randint(0, cfg.vocab_size, (2, 24), generator=torch.Generator().manual_seed(4)).cuda()
+    want, _ = plain(ids)
+    got, _ = compact(ids)
+    assert torch.equal(got, want)
+
+    # one copy: no derived copies beside the buffers, and the buffers are not the checkpoint layout
+    attn, mlp = compact.model.layers[0].self_attn, compact.model.layers[0].mlp
+    assert attn.o_proj._sorted is None and attn.o_proj._compact_perm is not None
+    assert not torch.equal(attn.o_proj.qweight.cpu(), state_a["model.layers.0.self_attn.o_proj.qweight"])
+    assert torch.equal(attn.o_proj.checkpoint_qweight().cpu(), state_a["model.layers.0.self_attn.o_proj.qweight"])
+    if fuse_mlp:
+        assert mlp._is_compact and mlp._sorted is None and mlp._chained is None
+        x = torch.randn(3, cfg.hidden_size, device="cuda").half()
+        assert torch.equal(mlp.gate_up(x), plain.model.layers[0].mlp.gate_up(x))
+
+    # the checkpoint layout on the way out: the same tensors as the uncompacted model's state_dict
+    sd_plain, sd_compact = plain.state_dict(), compact.state_dict()
+    assert sd_plain.keys() == sd_compact.keys()
+    for key in sd_plain:
+        assert torch.equal(sd_plain[key], sd_compact[key]), key
+    # dequantised weights too
+    assert torch.equal(attn.o_proj.dequantize(), plain.model.layers[0].self_attn.o_proj.dequantize())
+
+    # other weights loaded into the compacted model: back to the checkpoint layout, then the new model's logits
+    other = G.load_quant(str(tmp_path / "b"), device="cuda", fuse_mlp=fuse_mlp, compact=False)
+    compact.load_state_dict(other.state_dict())
+    assert compact.model.layers[0].self_attn.o_proj._compact_perm is None
+    want_b, _ = other(ids)
+    got_b, _ = compact(ids)
+    assert torch.equal(got_b, want_b) and not torch.equal(got_b, want)
+    # and compacting again by hand
+    G.quant_linear.compact_act_order(compact)
+    again, _ = compact(ids)
+    assert torch.equal(again, want_b)
