@@ -34,3 +34,20 @@ def to_dev(layer, device="cuda"):
 
 def bits(a):
     return np.asarray(a, dtype=np.float16).view(np.uint16)
+
+
+@pytest.fixture(autouse=True)
+def _automatic_launch_plans_after_every_test():
+    """The library's tuning hooks are process-wide: whatever a test forced - also one that failed before its own
+    clean-up ran - is back to automatic before the next test starts.  (Only if the library is loaded already.)"""
+    yield
+    mod = sys.modules.get("gptq_triton_amd._lib")
+    lib = getattr(mod, "_lib", None) if mod is not None else None
+    if lib is None:
+        return
+    lib.gptq4_set_tuning(0, 0, 0)
+    lib.gptq4_set_gemv_tuning(1, 0, 0, 0)
+    lib.gptq4_set_midm_tuning(1, 0, 0)
+    lib.gptq4_set_gemm_tuning(0, 0)
+    lib.gptq4_set_exchange_spin_limit(0)
+    lib.gptq4_set_chain_tuning(0, 0, 0, -1)
