@@ -156,3 +156,34 @@ def test_act_order_projection(m, k, n, g):
     a, b = x.double() @ wg, x.double() @ wu
     silu = a / (1.0 + torch.exp(-a))
     close(h, silu * b, 1.1 * b.abs() * sum_noise(x, wg) + silu.abs() * sum_noise(x, wu), f"act-order gate/up M={m} K={k} N={n} g={g}")
+
+
+@pytest.mark.parametrize("m,k,n", [(3400, 2048, 2560), (700, 4096, 6144), (1300, 2048, 5632)])
+def test_act_order_gathered_by_the_tiled_kernel_itself_with_shared_panels(m, k, n):
+    """The tiled kernel's own act-order gather (what calls too large to stage use; forced here) on tile counts just above
+    a whole number of rounds, where the last column panels are cut along K inside the launch: plain projection and the
+    gate/up pair."""
+    from gptq_triton_amd import _lib
+    lib = _lib.load()
+    G = gptq()
+    g = 128
+    rng = np.random.default_rng(m)
+    g_idx = torch.from_numpy(rng.permutation(np.repeat(np.arange(k // g), g)).astype(np.int32)).cuda()
+    Dg, Du = to_dev(layer(k, n, g, seed=m + 7)), to_dev(layer(k, n, g, seed=m + 8))
+    x = torch.from_numpy(O.make_x(m, k, seed=m + 3)).cuda()
+    wg = G.dequantize(Dg["qweight"], Dg["qzeros"], Dg["scales"], g, g_idx).double()
+    wu = G.dequantize(Du["qweight"], Du["qzeros"], Du["scales"], g, g_idx).double()
+    gq, perm = G.prepare_act_order(Dg["qweight"], g_idx, g)
+    uq, _ = G.prepare_act_order(Du["qweight"], g_idx, g)
+    try:
+        lib.gptq4_set_midm_tuning(0, 0, 0)
+        lib.gptq4_set_gemm_tuning(10, 0)
+        y = G.matmul4(g, x, gq, Dg["scales"], Dg["qzeros"], None, perm)
+        h = G.llama_mlp_4(g, x, gq, Dg["scales"], Dg["qzeros"], uq, Du["scales"], Du["qzeros"], perm=perm)
+    finally:
+        lib.gptq4_set_gemm_tuning(0, 0)
+        lib.gptq4_set_midm_tuning(1, 0, 0)
+    close(y, x.double() @ wg, sum_noise(x, wg), f"own gather, matmul M={m} K={k} N={n}")
+    a, b = x.double() @ wg, x.double() @ wu
+    silu = a / (1.0 + torch.exp(-a))
+    close(h, silu * b, 1.1 * b.abs() * sum_noise(x, wg) + silu.abs() * sum_noise(x, wu), f"own gather, gate/up M={m} K={k} N={n}")
