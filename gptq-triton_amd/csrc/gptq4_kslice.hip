@@ -506,7 +506,7 @@ int launch_epi(const MatmulArgs &a, const KslicePlan &pl, hipStream_t stream) {
 
 KsliceTuning g_kslice_tuning = {1, 0, 0, 0, 0};
 
-// Row tile: 32 rows up to M = 32, else 64.  (128-row tiles decode each weight once instead of twice at M = 128 and
+// Row tile: 32 rows up to M = 32, else 64 - or 32 for plain projections where that scores higher, see below.  (128-row tiles decode each weight once instead of twice at M = 128 and
 // halve the instructions per MFMA, but came out no faster: 17.3 against 15.1 us on 4096 x 4096, level on
 // 11008 x 4096.  Four activation tiles per wave instead of two - the tile three K tiles on requested while one is
 // multiplied - gained nothing that eight waves do not gain as well.)  How far K is split across workgroups on top is
@@ -525,11 +525,13 @@ KslicePlan kslice_plan(int epi, int M, int N, int K, bool has_perm) {
     const int bn = (epi == EPI_ROPE || pl.wide) ? 128 : 64;
     const int nk = K / 64;
     pl.mt = g_kslice_tuning.mt ? g_kslice_tuning.mt : (M <= 32 ? 1 : 2);
-    const int bm = 32 * pl.mt;
+    int bm = 32 * pl.mt;
     pl.tiles = ((M + bm - 1) / bm) * (N / bn);
     const long cus = device_shape().cus;  // 256 on MI355X
+    double split_score = 0.0;  // of the split choose_split returned last (automatic choice only)
     auto choose_split = [&](int ks) {
         int s = 1;
+        split_score = 0.0;
         if (g_kslice_tuning.splitk > 0) {
             s = g_kslice_tuning.splitk;
         } else {
@@ -550,12 +552,32 @@ KslicePlan kslice_plan(int epi, int M, int N, int K, bool has_perm) {
                     s = c;
                 }
             }
+            split_score = best;
         }
         if (s > GEMM_MAX_SPLITK) s = GEMM_MAX_SPLITK;
         if (s < 1 || pl.tiles > SKINNY_MAX_TILES) s = 1;
         return s;
     };
     int s = choose_split(ks);
+    // Plain projections on 64-column strips, 33 rows and more: 32-row tiles as well, where twice as many tiles fill
+    // the chip without a split across workgroups (or with a smaller one) - each weight is then decoded once per 32
+    // rows instead of once per 64, priced at 0.85 of the rate, but the exchange through memory goes.  Same score as
+    // for the splits.  4096 x 4096 at 128 rows: 256 tiles of 32 rows, 12.8 -> 11.5 us; 5120 x 5120 at 96 rows 16.2 ->
+    // 12.9, 13824 x 5120 at 96 rows 32.3 -> 28.8; 64-row tiles stay where they score higher (11008 x 4096 at 128
+    // rows, 5120 x 5120 at 128 rows: 320 tiles of 32 rows would not fit one round).
+    if (epi == EPI_PLAIN && !pl.wide && M > 32 && g_kslice_tuning.mt == 0 && g_kslice_tuning.splitk == 0) {
+        const double score2 = split_score;
+        const int tiles2 = pl.tiles;
+        pl.tiles = ((M + 31) / 32) * (N / bn);
+        const int s1 = choose_split(ks);
+        if (score2 > 0.0 && 0.85 * split_score > score2 + 1e-9 && pl.tiles <= SKINNY_MAX_TILES) {
+            pl.mt = 1;
+            bm = 32;
+            s = s1;
+        } else {
+            pl.tiles = tiles2;
+        }
+    }
     // eight waves: 128 KiB of LDS with 64-row tiles, so only in launches of at most one workgroup per CU; with 32-row
     // tiles two workgroups share a CU and four waves a SIMD, which leaves each 128 registers - enough for one
     // column block per wave tile only; and every wave needs a K tile or two
