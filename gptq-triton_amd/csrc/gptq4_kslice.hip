@@ -45,7 +45,8 @@ constexpr int BK = 64;
 // per SIMD; the matrix cores are busy 15 % of the time (SQ counters at 128 rows, 4096 x 4096).  A second wave
 // per SIMD overlaps the two.  8 waves with 64-row tiles are 128 KiB of LDS: one workgroup per CU.
 template <int EPI, int MT, bool WIDE, int KS>
-__global__ __launch_bounds__(64 * KS, KS == 8 && MT == 2 ? 1 : 2) void gptq4_kslice_kernel(MatmulArgs p) {
+// (eight waves: one workgroup per CU - all its registers - wherever the wave tile has two column blocks or two row blocks)
+__global__ __launch_bounds__(64 * KS, KS == 8 && (MT == 2 || EPI != EPI_PLAIN || WIDE) ? 1 : 2) void gptq4_kslice_kernel(MatmulArgs p) {
     static_assert(KS == 4 || KS == 8, "four or eight waves");
     static_assert(!WIDE || EPI == EPI_PLAIN, "the other epilogues have two blocks already");
     constexpr bool ADJ = (EPI == EPI_ROPE) || WIDE;     // the second block is columns + 64 of the same matrix
@@ -487,9 +488,9 @@ int launch_waves(const MatmulArgs &a, const KslicePlan &pl, hipStream_t stream) 
         // 32-row tiles with two column blocks per wave tile are never planned with eight waves (kslice_plan)
         if (EPI == EPI_PLAIN && !pl.wide)
             return pl.mt == 1 ? launch_one<EPI_PLAIN, 1, false, 8>(a, pl.tiles, stream) : launch_one<EPI_PLAIN, 2, false, 8>(a, pl.tiles, stream);
-        if (pl.mt == 1) return (int)hipErrorInvalidValue;
-        if (EPI == EPI_PLAIN) return launch_one<EPI_PLAIN, 2, true, 8>(a, pl.tiles, stream);
-        return launch_one<EPI, 2, false, 8>(a, pl.tiles, stream);
+        // (128-column strips of a plain projection on 32-row tiles are never planned with eight waves)
+        if (EPI == EPI_PLAIN) return pl.mt == 1 ? (int)hipErrorInvalidValue : launch_one<EPI_PLAIN, 2, true, 8>(a, pl.tiles, stream);
+        return pl.mt == 1 ? launch_one<EPI, 1, false, 8>(a, pl.tiles, stream) : launch_one<EPI, 2, false, 8>(a, pl.tiles, stream);
     } else {
         if (EPI == EPI_PLAIN && pl.wide)
             return pl.mt == 1 ? launch_one<EPI_PLAIN, 1, true, KS>(a, pl.tiles, stream) : launch_one<EPI_PLAIN, 2, true, KS>(a, pl.tiles, stream);
@@ -514,9 +515,10 @@ KsliceTuning g_kslice_tuning = {1, 0, 0, 0, 0};
 KslicePlan kslice_plan(int epi, int M, int N, int K, bool has_perm) {
     KslicePlan pl = {};
     // eight waves for plain projections wherever they fit (checked below): ahead of four waves by 4 - 18 % at
-    // LLaMA-7B / 30B shapes from 17 to 256 rows, level at 512; the gate/up pair and the rotary epilogue stay at four
-    // (two column blocks per wave tile need the registers of a whole SIMD; 7B QKV loses 3 % with eight)
-    pl.waves = g_kslice_tuning.waves ? g_kslice_tuning.waves : (epi == EPI_PLAIN ? 8 : 4);
+    // LLaMA-7B / 30B shapes from 17 to 256 rows, level at 512; the gate/up pair and the rotary epilogue take eight up to
+    // 32 rows (one workgroup per CU then: two column blocks per wave tile need the registers of a whole SIMD; 7B QKV
+    // 16.9 -> 15.6 us, gate/up 19.6 -> 18.6, 13B QKV 19.3 -> 18.0) and stay at four beyond (level or 3 % behind)
+    pl.waves = g_kslice_tuning.waves ? g_kslice_tuning.waves : ((epi == EPI_PLAIN || M <= 32) ? 8 : 4);
     int ks = pl.waves;
     // plain projections: 128-column strips (half the activation traffic per weight byte, half the tiles) pay
     // from 256 rows on when K is long (LLaMA-7B down_proj: 39.8 -> 37.3 us at 256 rows, 66.2 -> 61.1 at 512;
@@ -580,10 +582,11 @@ KslicePlan kslice_plan(int epi, int M, int N, int K, bool has_perm) {
     }
     // eight waves: 128 KiB of LDS with 64-row tiles, so only in launches of at most one workgroup per CU; with 32-row
     // tiles two workgroups share a CU and four waves a SIMD, which leaves each 128 registers - enough for one
-    // column block per wave tile only; and every wave needs a K tile or two
+    // column block per wave tile only, so two blocks also need the CU to themselves; and every wave needs a K tile
+    // or two
     if (pl.waves == 8) {
         const int nb = (epi == EPI_PLAIN && !pl.wide) ? 1 : 2;
-        if ((pl.mt == 2 && (long)pl.tiles * s > cus) || (pl.mt == 1 && nb == 2) || nk / s < 16) {
+        if (((pl.mt == 2 || nb == 2) && (long)pl.tiles * s > cus) || (pl.mt == 1 && nb == 2 && epi == EPI_PLAIN) || nk / s < 16) {
             pl.waves = ks = 4;
             s = choose_split(ks);
         }
