@@ -639,6 +639,8 @@ def main():
             decs[f"{name}_b{bsz}"] = {"tok_s": r["value"], "ms_per_step": r["ms_per_step"], "prefill_ms": r["extra"]["prefill_ms"],
                                       "prefill_linear_TFLOPs": r["extra"]["prefill_linear_TFLOPs"],
                                       "step_GBps": r["roofline"]["achieved"], "step_frac_hbm": r["roofline"]["frac"],
+                                      "prefill_path_agrees_with_decode_path_on_next_tokens":
+                                          r["extra"]["prefill_path_agrees_with_decode_path_on_next_tokens"],
                                       "workload": r["config"]["workload"]}
         extra["decoders"] = decs
 
