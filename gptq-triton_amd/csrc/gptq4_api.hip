@@ -346,6 +346,9 @@ void gptq4_set_gemm_tuning(int mt, int splitk) {
 
 void gptq4_set_midm_tuning(int mode, int mt, int splitk) {
     g_kslice_tuning.mode = (mode >= 0 && mode <= 2) ? mode : 1;
+    // 1000 + mt: the rotary epilogue on tiles of 32 + 32 paired columns wherever the mid-M kernel runs, 2000 + mt: never
+    g_kslice_tuning.paired = (mt >= 2000) ? 2 : (mt >= 1000) ? 1 : 0;
+    mt %= 1000;
     // 100 + mt: four waves per workgroup, 200 + mt: eight where they fit (automatic: eight for plain projections)
     g_kslice_tuning.waves = (mt >= 200) ? 8 : (mt >= 100) ? 4 : 0;
     mt %= 100;

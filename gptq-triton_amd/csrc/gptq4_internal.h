@@ -137,6 +137,7 @@ struct KslicePlan {
     int tiles;
     bool wide;   // plain epilogue: 128-column strips (two blocks per wave tile) instead of 64
     int waves;   // waves per workgroup, each with its own slice of K (4 or 8)
+    bool paired; // rotary epilogue: tiles of 32 columns of a head plus their 32 rotation partners instead of whole heads
     bool ok;     // false: the shape needs another kernel
     // tail_split > 1 (only with splitk == 1): tiles [0, tail_first) whole, every later one - the last column strips
     // of the launch, all their row tiles - shared by tail_split workgroups along K
@@ -147,6 +148,7 @@ struct KsliceTuning {
     int mt, splitk;  // 0 = automatic
     int wide;        // plain epilogue: 1 = 128-column strips, -1 = 64-column strips, 0 = automatic
     int waves;       // waves per workgroup: 4, 8, 0 = automatic
+    int paired;      // rotary epilogue, tiles of 32 + 32 paired columns: 0 = automatic, 1 = always, 2 = never
 };
 extern KsliceTuning g_kslice_tuning;
 KslicePlan kslice_plan(int epi, int M, int N, int K, bool has_perm);

@@ -14,7 +14,8 @@
 //   plain   : NB = 1, one 64-column strip; or (WIDE, long K and many rows) NB = 2, two adjacent strips.
 //   SiLU*mul: NB = 2, the same 64 columns of the gate and of the up matrix.
 //   rotary  : NB = 2, columns [0, 64) and [64, 128) of one head, so the wave that finishes
-//             a row block holds d and d + 64 itself.
+//             a row block holds d and d + 64 itself; or (PAIRED, few rows) NB = 1: 32 columns of a head and their
+//             32 rotation partners, the two columns of a lane being d and d + 64.
 // With NB = 2 every activation fragment read from LDS feeds twice as many MFMAs.
 //
 // Weights are decoded exactly once per row tile.  K can still be split across workgroups
@@ -44,14 +45,19 @@ constexpr int BK = 64;
 // waiting (first loads, the exchanges at the end) and the other half issuing ~20 instructions per MFMA, one wave
 // per SIMD; the matrix cores are busy 15 % of the time (SQ counters at 128 rows, 4096 x 4096).  A second wave
 // per SIMD overlaps the two.  8 waves with 64-row tiles are 128 KiB of LDS: one workgroup per CU.
-template <int EPI, int MT, bool WIDE, int KS>
+// PAIRED (rotary epilogue only): the workgroup owns 32 columns of a head and their 32 rotation partners (d, d + 64)
+// instead of the whole head.  The two columns of a lane are then d and d + 64 - two 4-byte loads per row instead of one
+// 8-byte load of adjacent columns - so the wave tile has ONE column block, like a plain strip, twice as many workgroups
+// share the projection without splitting K, and the lane that finishes a value holds its rotation partner itself.
+template <int EPI, int MT, bool WIDE, int KS, bool PAIRED = false>
 // (eight waves: one workgroup per CU - all its registers - wherever the wave tile has two column blocks or two row blocks)
-__global__ __launch_bounds__(64 * KS, KS == 8 && (MT == 2 || EPI != EPI_PLAIN || WIDE) ? 1 : 2) void gptq4_kslice_kernel(MatmulArgs p) {
+__global__ __launch_bounds__(64 * KS, KS == 8 && (MT == 2 || (EPI != EPI_PLAIN && !PAIRED) || WIDE) ? 1 : 2) void gptq4_kslice_kernel(MatmulArgs p) {
     static_assert(KS == 4 || KS == 8, "four or eight waves");
     static_assert(!WIDE || EPI == EPI_PLAIN, "the other epilogues have two blocks already");
-    constexpr bool ADJ = (EPI == EPI_ROPE) || WIDE;     // the second block is columns + 64 of the same matrix
+    static_assert(!PAIRED || EPI == EPI_ROPE, "paired columns are a rotary head's");
+    constexpr bool ADJ = (EPI == EPI_ROPE && !PAIRED) || WIDE;  // the second block is columns + 64 of the same matrix
     constexpr int BM = 32 * MT;
-    constexpr int NB = (EPI == EPI_PLAIN && !WIDE) ? 1 : 2;  // 64-column blocks of the wave tile
+    constexpr int NB = ((EPI == EPI_PLAIN && !WIDE) || PAIRED) ? 1 : 2;  // 64-column blocks of the wave tile
     constexpr int BN = ADJ ? 128 : 64;                  // output columns of the workgroup
     constexpr int NSET = NB;                            // value sets the finishing wave combines
     constexpr int A_HALVES = BM * BK;                   // one wave's K tile of activations
@@ -113,11 +119,13 @@ __global__ __launch_bounds__(64 * KS, KS == 8 && (MT == 2 || EPI != EPI_PLAIN ||
     const int tile_n = logical / tiles_m;
     const int tile_m = logical - tile_n * tiles_m;
     const int m0 = tile_m * BM;
-    const int n0 = p.n_begin + tile_n * BN;  // the launch covers columns [n_begin, n_begin + n_count) of the N
+    // the launch covers columns [n_begin, n_begin + n_count) of the N; PAIRED: tile_n counts quarter heads,
+    // n0 = the first of the tile's 32 low columns
+    const int n0 = PAIRED ? p.n_begin + (tile_n >> 1) * 128 + (tile_n & 1) * 32 : p.n_begin + tile_n * BN;
 
     // block j of the wave tile: matrix j at the strip's columns (SiLU*mul), or columns
-    // 64*j .. 64*j + 63 of the head (rotary); the lane's 2 columns of it
-    const int ncol = n0 + 2 * l32;
+    // 64*j .. 64*j + 63 of the head (rotary); the lane's 2 columns of it (PAIRED: ncol and ncol + 64)
+    const int ncol = PAIRED ? n0 + l32 : n0 + 2 * l32;
     // (for rotary the second block is a constant offset from the first: no second set of pointers)
     constexpr int NPTR = (EPI == EPI_SILU_MUL) ? 2 : 1;
     const uint32_t *bptr_[NPTR];
@@ -192,20 +200,34 @@ __global__ __launch_bounds__(64 * KS, KS == 8 && (MT == 2 || EPI != EPI_PLAIN ||
         uint2 b2[NB][2][4];
         auto load_b2 = [&](int par, int kt, int ks) {
             const size_t off = ((size_t)min(kt, nk - 1) * (BK / 8) + 2 * ks) * N;
+            if constexpr (PAIRED) {
+                b2[0][par][ks].x = bptr_[0][off];
+                b2[0][par][ks].y = bptr_[0][off + 64];
+            } else {
 #pragma unroll
-            for (int j = 0; j < NB; ++j) b2[j][par][ks] = *reinterpret_cast<const uint2 *>(bptr(j) + off);
+                for (int j = 0; j < NB; ++j) b2[j][par][ks] = *reinterpret_cast<const uint2 *>(bptr(j) + off);
+            }
         };
         // Scale and zero words two tiles ahead as well; the group of the look-ahead tile is
         // tracked by counting.
         int group2 = k_begin / tiles_per_group;
         int left2 = tiles_per_group - (k_begin - group2 * tiles_per_group);
         uint32_t g_s[NB][2], g_z[NB][2];
+        uint32_t g_s_hi[2], g_z_hi[2];  // PAIRED: scale and zero word of the lane's second column
         auto load_group2 = [&](int par) {
             const int g = min(group2, last_group);
+            if constexpr (PAIRED) {
+                const uint16_t *const sp = reinterpret_cast<const uint16_t *>(sc_[0] + (size_t)g * N);
+                g_s[0][par] = sp[0];
+                g_s_hi[par] = sp[64];
+                g_z[0][par] = qz_[0][(size_t)g * (N >> 3)];
+                g_z_hi[par] = qz_[0][(size_t)g * (N >> 3) + 8];
+            } else {
 #pragma unroll
-            for (int j = 0; j < NB; ++j) {
-                g_s[j][par] = *reinterpret_cast<const uint32_t *>(sc(j) + (size_t)g * N);
-                g_z[j][par] = qz(j)[(size_t)g * (N >> 3)];
+                for (int j = 0; j < NB; ++j) {
+                    g_s[j][par] = *reinterpret_cast<const uint32_t *>(sc(j) + (size_t)g * N);
+                    g_z[j][par] = qz(j)[(size_t)g * (N >> 3)];
+                }
             }
             if (left2 == 1) {
                 ++group2;
@@ -216,6 +238,12 @@ __global__ __launch_bounds__(64 * KS, KS == 8 && (MT == 2 || EPI != EPI_PLAIN ||
         };
         ColDecodeNat cn[NB][2];
         auto make_cn = [&](int par) {
+            if constexpr (PAIRED) {
+                const int sh = (l32 & 7) * 4;
+                cn[0][0] = make_col_decode_nat((g_z[0][par] >> sh) & 0xFu, g_s[0][par]);
+                cn[0][1] = make_col_decode_nat((g_z_hi[par] >> sh) & 0xFu, g_s_hi[par]);
+                return;
+            }
 #pragma unroll
             for (int j = 0; j < NB; ++j) {
                 const uint32_t z2 = g_z[j][par] >> (((2 * l32) & 7) * 4);
@@ -246,7 +274,7 @@ __global__ __launch_bounds__(64 * KS, KS == 8 && (MT == 2 || EPI != EPI_PLAIN ||
             // scale/zero words that followed its LDS-direct loads of this tile: at most that
             // many outstanding means the tile has landed.  It is this wave's own tile: no barrier.
             // (lgkmcnt: the fragment reads of the tile before are done before its buffer is requested again.)
-            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(4 * NB) : "memory");
+            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(4 * NB * (PAIRED ? 2 : 1)) : "memory");
             dma_a(nxt, min(kt + 1, nk - 1));
             load_group2(par);
             h8_t araw[MT];
@@ -437,12 +465,45 @@ __global__ __launch_bounds__(64 * KS, KS == 8 && (MT == 2 || EPI != EPI_PLAIN ||
         const size_t seq_stride = (size_t)r.H * cap * 128;
         const bool at_position = (which != 0) && r.kv_offset < 0;  // cache row = the token's position
         const int row_shift = (which == 0 || r.kv_offset < 0) ? 0 : r.kv_offset;
-        float2 cs[IW], sn[IW];
         int pos[IW];
         if (which < 2 || at_position) {
 #pragma unroll
             for (int ii = 0; ii < IW; ++ii) pos[ii] = max(r.position_ids[min(row_of(ii), M - 1)], 0);
         }
+        if constexpr (PAIRED) {
+            // the lane's two values are columns d and d + 64 of the head: the same products and sums as below
+            const int d = (n0 & 127) + l32;
+            float c1[IW], s1[IW];
+            if (which < 2) {
+#pragma unroll
+                for (int ii = 0; ii < IW; ++ii) {
+                    const int tp = min(pos[ii], r.max_pos - 1);
+                    c1[ii] = r.cos_table[(size_t)tp * 64 + d];
+                    s1[ii] = r.sin_table[(size_t)tp * 64 + d];
+                }
+            }
+#pragma unroll
+            for (int ii = 0; ii < IW; ++ii) {
+                const int row = row_of(ii);
+                float lo = vals[0][0][ii], hi = vals[0][1][ii];
+                if (which < 2) {
+                    const float a = lo * c1[ii] - hi * s1[ii];
+                    const float b = hi * c1[ii] + lo * s1[ii];
+                    lo = a, hi = b;
+                }
+                if (row < M) {
+                    int bb, srow;
+                    split_row(r, row, bb, srow);
+                    const int crow = at_position ? min(pos[ii], r.kv_capacity - 1) : srow + row_shift;
+                    half_t *const at = dst - 2 * l32 + d + (size_t)bb * seq_stride + (size_t)crow * 128;
+                    at[0] = (half_t)lo;
+                    at[64] = (half_t)hi;
+                }
+            }
+            KS_STAMP(7);
+            return;
+        }
+        float2 cs[IW], sn[IW];
         if (which < 2) {
 #pragma unroll
             for (int ii = 0; ii < IW; ++ii) {
@@ -474,16 +535,21 @@ __global__ __launch_bounds__(64 * KS, KS == 8 && (MT == 2 || EPI != EPI_PLAIN ||
     KS_STAMP(7);
 }
 
-template <int EPI, int MT, bool WIDE, int KS>
+template <int EPI, int MT, bool WIDE, int KS, bool PAIRED = false>
 int launch_one(const MatmulArgs &a, int tiles, hipStream_t stream) {
     dim3 grid((unsigned)tiles, (unsigned)a.splitk), block(64 * KS);
     if (a.tail_split > 1) grid = dim3((unsigned)(a.tail_first + (tiles - a.tail_first) * a.tail_split), 1u);
-    hipLaunchKernelGGL((gptq4_kslice_kernel<EPI, MT, WIDE, KS>), grid, block, 0, stream, a);
+    hipLaunchKernelGGL((gptq4_kslice_kernel<EPI, MT, WIDE, KS, PAIRED>), grid, block, 0, stream, a);
     return (int)hipGetLastError();
 }
 
 template <int EPI, int KS>
 int launch_waves(const MatmulArgs &a, const KslicePlan &pl, hipStream_t stream) {
+    if constexpr (EPI == EPI_ROPE) {
+        if (pl.paired)
+            return pl.mt == 1 ? launch_one<EPI_ROPE, 1, false, KS, true>(a, pl.tiles, stream)
+                              : launch_one<EPI_ROPE, 2, false, KS, true>(a, pl.tiles, stream);
+    }
     if constexpr (KS == 8) {
         // 32-row tiles with two column blocks per wave tile are never planned with eight waves (kslice_plan)
         if (EPI == EPI_PLAIN && !pl.wide)
@@ -505,26 +571,30 @@ int launch_epi(const MatmulArgs &a, const KslicePlan &pl, hipStream_t stream) {
 
 }  // namespace
 
-KsliceTuning g_kslice_tuning = {1, 0, 0, 0, 0};
+KsliceTuning g_kslice_tuning = {1, 0, 0, 0, 0, 0};
 
 // Row tile: 32 rows up to M = 32, else 64 - or 32 for plain projections where that scores higher, see below.  (128-row tiles decode each weight once instead of twice at M = 128 and
 // halve the instructions per MFMA, but came out no faster: 17.3 against 15.1 us on 4096 x 4096, level on
 // 11008 x 4096.  Four activation tiles per wave instead of two - the tile three K tiles on requested while one is
 // multiplied - gained nothing that eight waves do not gain as well.)  How far K is split across workgroups on top is
 // scored below.
-KslicePlan kslice_plan(int epi, int M, int N, int K, bool has_perm) {
+// One variant of the plan: the rotary epilogue on whole heads or on paired quarter heads.  *score: that of the split it
+// chose (0 with a forced split).
+static KslicePlan plan_variant(int epi, int M, int N, int K, bool has_perm, bool paired, double *score) {
     KslicePlan pl = {};
     // eight waves for plain projections wherever they fit (checked below): ahead of four waves by 4 - 18 % at
     // LLaMA-7B / 30B shapes from 17 to 256 rows, level at 512; the gate/up pair and the rotary epilogue take eight up to
     // 32 rows (one workgroup per CU then: two column blocks per wave tile need the registers of a whole SIMD; 7B QKV
     // 16.9 -> 15.6 us, gate/up 19.6 -> 18.6, 13B QKV 19.3 -> 18.0) and stay at four beyond (level or 3 % behind)
-    pl.waves = g_kslice_tuning.waves ? g_kslice_tuning.waves : ((epi == EPI_PLAIN || M <= 32) ? 8 : 4);
+    // (paired quarter heads: one column block per wave tile like a plain strip, so eight waves fit as they do there)
+    pl.paired = paired;
+    pl.waves = g_kslice_tuning.waves ? g_kslice_tuning.waves : ((epi == EPI_PLAIN || pl.paired || M <= 32) ? 8 : 4);
     int ks = pl.waves;
     // plain projections: 128-column strips (half the activation traffic per weight byte, half the tiles) pay
     // from 256 rows on when K is long (LLaMA-7B down_proj: 39.8 -> 37.3 us at 256 rows, 66.2 -> 61.1 at 512;
     // o_proj with K = 4096 loses below 512 rows)
     pl.wide = epi == EPI_PLAIN && (g_kslice_tuning.wide > 0 || (g_kslice_tuning.wide == 0 && M >= 256 && K >= 8192));
-    const int bn = (epi == EPI_ROPE || pl.wide) ? 128 : 64;
+    const int bn = ((epi == EPI_ROPE && !pl.paired) || pl.wide) ? 128 : 64;
     const int nk = K / 64;
     pl.mt = g_kslice_tuning.mt ? g_kslice_tuning.mt : (M <= 32 ? 1 : 2);
     int bm = 32 * pl.mt;
@@ -585,7 +655,7 @@ KslicePlan kslice_plan(int epi, int M, int N, int K, bool has_perm) {
     // column block per wave tile only, so two blocks also need the CU to themselves; and every wave needs a K tile
     // or two
     if (pl.waves == 8) {
-        const int nb = (epi == EPI_PLAIN && !pl.wide) ? 1 : 2;
+        const int nb = ((epi == EPI_PLAIN && !pl.wide) || pl.paired) ? 1 : 2;
         if (((pl.mt == 2 || nb == 2) && (long)pl.tiles * s > cus) || (pl.mt == 1 && nb == 2 && epi == EPI_PLAIN) || nk / s < 16) {
             pl.waves = ks = 4;
             s = choose_split(ks);
@@ -615,12 +685,30 @@ KslicePlan kslice_plan(int epi, int M, int N, int K, bool has_perm) {
     }
     // the wave loop needs the activations unpermuted and at least one K tile per wave
     pl.ok = !has_perm && (N % bn) == 0 && nk / s >= ks;
+    *score = split_score;
     return pl;
+}
+
+// Rotary epilogue: whole heads (tiles of 128 columns) or tiles of 32 columns of a head and their 32 rotation partners -
+// twice as many tiles, so that few rows fill the chip without splitting K across workgroups (an exchange of partial
+// sums through memory, 3 us), at the price of two 4-byte loads per row and lane instead of one 8-byte load and half as
+// many MFMAs per activation fragment (priced at 0.85 of the rate).  Each variant is planned by itself and the better
+// split score wins (never with a larger split than whole heads take).  LLaMA-7B QKV: 15.7 -> 13.0 us at 17 rows, 16.2 -> 13.4 at 32 (16 rows: 12.4), 21.1 -> 16.9 at 64,
+// 42.4 -> 37.0 at 192; 13B 18.7 -> 16.2 at 32, 24.6 -> 20.6 at 64; 30B 60 -> 54 at 96 rows and whole heads below that
+// (312 paired tiles do not fit one round of 256 CUs).
+KslicePlan kslice_plan(int epi, int M, int N, int K, bool has_perm) {
+    double score = 0.0;
+    if (epi != EPI_ROPE || g_kslice_tuning.paired == 2) return plan_variant(epi, M, N, K, has_perm, false, &score);
+    if (g_kslice_tuning.paired == 1) return plan_variant(epi, M, N, K, has_perm, true, &score);
+    double score_p = 0.0;
+    const KslicePlan heads = plan_variant(epi, M, N, K, has_perm, false, &score);
+    const KslicePlan pairs = plan_variant(epi, M, N, K, has_perm, true, &score_p);
+    return (pairs.ok && score > 0.0 && pairs.splitk <= heads.splitk && 0.85 * score_p > score + 1e-9) ? pairs : heads;
 }
 
 size_t kslice_partial_bytes(int epi, const KslicePlan &pl) {
     // (the same with four or eight waves: eight split the 32 values per lane and block over two owner waves)
-    const int nset = (epi == EPI_PLAIN && !pl.wide) ? 1 : 2;
+    const int nset = ((epi == EPI_PLAIN && !pl.wide) || pl.paired) ? 1 : 2;
     if (pl.tail_split > 1) return (size_t)(pl.tiles - pl.tail_first) * pl.tail_split * pl.mt * nset * 32 * 64 * sizeof(float);
     return pl.splitk > 1 ? (size_t)pl.tiles * pl.splitk * pl.mt * nset * 32 * 64 * sizeof(float) : 0;
 }

@@ -310,8 +310,9 @@ void gptq4_set_gemm_tuning(int mt, int splitk);
  * across the four or eight waves of a workgroup): mode 0 = never use it, 1 = where it is the faster
  * kernel, 2 = wherever it can run; 32-row blocks per row tile (1, 2; 10 + that, or 10 alone, also
  * selects 128-column strips for plain projections, a plain 1 or 2 the 64-column strips; 100 + any of
- * these: four waves per workgroup, 200 +: eight where they fit) and the split-K factor across
- * workgroups; 0 = automatic. */
+ * these: four waves per workgroup, 200 +: eight where they fit; 1000 + any of these: the rotary epilogue on tiles
+ * of 32 columns of a head plus their 32 rotation partners instead of whole heads, 2000 +: never) and the split-K
+ * factor across workgroups; 0 = automatic. */
 void gptq4_set_midm_tuning(int mode, int mt, int splitk);
 
 /* Same for the balanced decode GEMV (M <= 4): mode 0 = never use it, 1 = where it is the

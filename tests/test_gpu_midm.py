@@ -15,10 +15,12 @@ pytestmark = pytest.mark.gpu
 # (32-row blocks per row tile, split-K across workgroups); 0 = automatic; + 10: 128-column strips for plain
 # projections; + 100: four waves per workgroup, + 200: eight (where they fit: 64-row tiles, and 32-row tiles with two
 # column blocks per wave tile, only in launches of at most one workgroup per CU); automatic: eight for plain projections
-# and, up to 32 rows, for the fused epilogues
+# and, up to 32 rows, for the fused epilogues; + 1000: the rotary epilogue on tiles of 32 columns of a head plus their 32
+# rotation partners (automatic: up to 64 rows), + 2000: never
 CONFIGS = [(0, 0), (1, 1), (2, 1), (1, 2), (2, 3), (10, 0), (11, 1), (12, 3),
            (100, 0), (101, 1), (102, 1), (101, 3), (102, 2), (111, 2), (112, 1),
-           (200, 0), (201, 1), (202, 1), (201, 2), (202, 2), (211, 1), (212, 1)]
+           (200, 0), (201, 1), (202, 1), (201, 2), (202, 2), (211, 1), (212, 1),
+           (1000, 0), (1001, 1), (1002, 2), (1101, 2), (1102, 1), (1201, 1), (1202, 1), (2000, 0)]
 
 @pytest.fixture(params=CONFIGS, ids=lambda c: "mt%d_s%d" % c)
 def forced_midm(request):
