@@ -555,6 +555,8 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
         const int row_shift = (which == 0 || r.kv_offset < 0) ? 0 : r.kv_offset;
         if constexpr (ROPE_TAB) {
             if (PERM) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // table blocks 0 and 1 (the plain path has waited already)
+            uint32_t outw[MT][16];  // the rotated values, stored at the end
+            int crow_at[MT][16];    // (cache rows, when they are the tokens' positions)
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
                 if (need_tab) {
@@ -596,15 +598,26 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
                             o1 = o1 * cs.y + p1 * sn.y;
                         }
                     }
+                    const h2_t o = {(half_t)o0, (half_t)o1};
+                    outw[mt][i] = as_u32(o);
+                    if (at_position) crow_at[mt][i] = min(pos[i], r.kv_capacity - 1);
+                }
+            }
+            // All stores come behind the last wait for a table block: loads and stores share one counter, so a wait
+            // for a block's table loads would wait for the stores of the blocks before it as well (LLaMA-7B QKV at
+            // 1024 rows 118.6 -> 113.5 us, at 2048 rows 204.9 -> 198.2).
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int row = wrow0 + mt * 32 + 8 * (i >> 2) + 4 * lhi + (i & 3);
                     if (row < M) {
                         int bb, srow;
                         split_row(r, row, bb, srow);
-                        const int crow = at_position ? min(pos[i], r.kv_capacity - 1) : srow + row_shift;
-                        const h2_t o = {(half_t)o0, (half_t)o1};
-                        *reinterpret_cast<uint32_t *>(dst + (size_t)bb * seq_stride + (size_t)crow * 128) = as_u32(o);
+                        const int crow = at_position ? crow_at[mt][i] : srow + row_shift;
+                        *reinterpret_cast<uint32_t *>(dst + (size_t)bb * seq_stride + (size_t)crow * 128) = outw[mt][i];
                     }
                 }
-            }
             return;
         }
 #pragma unroll
