@@ -703,7 +703,11 @@ KslicePlan kslice_plan(int epi, int M, int N, int K, bool has_perm) {
     double score_p = 0.0;
     const KslicePlan heads = plan_variant(epi, M, N, K, has_perm, false, &score);
     const KslicePlan pairs = plan_variant(epi, M, N, K, has_perm, true, &score_p);
-    return (pairs.ok && score > 0.0 && pairs.splitk <= heads.splitk && 0.85 * score_p > score + 1e-9) ? pairs : heads;
+    // (only where whole heads leave the chip short of two workgroups per CU: beyond that the score's steps at whole
+    // rounds say nothing about twice as many, smaller tiles - 7B QKV at 512 rows: 768 whole heads 72.6 us, 1536 paired
+    // tiles 87.8)
+    const bool few = (long)heads.tiles < 2 * device_shape().cus;
+    return (pairs.ok && few && score > 0.0 && pairs.splitk <= heads.splitk && 0.85 * score_p > score + 1e-9) ? pairs : heads;
 }
 
 size_t kslice_partial_bytes(int epi, const KslicePlan &pl) {
