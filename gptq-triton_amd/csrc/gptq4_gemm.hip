@@ -406,12 +406,14 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
                 for (int mt = 0; mt < MT; ++mt) acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt], bf[1], acc[mt][1], 0, 0, 0);
                 bf[1] = decode_word_natural(nw.y, cn[1]);
                 // The decode of the next step's words (32 VALU instructions) spread between this step's MFMAs, three
-                // after each, instead of four MFMAs back to back and the decode behind them: 1 - 4 % (LLaMA-7B
-                // down_proj at 2048 rows 184 -> 177 us, o_proj 76.8 -> 74.5, gate/up 353 -> 347).
+                // after each of the wide tile's eight (six after each of the narrow tile's four), instead of four MFMAs
+                // back to back and the decode behind them: 1 - 4 % (LLaMA-7B down_proj at 2048 rows 184 -> 177 us,
+                // o_proj 76.8 -> 74.5, gate/up 353 -> 347; narrow tile: 13B o_proj at 640 rows 57.4 -> 53.8 with six,
+                // 30B o_proj at 512 rows 70.5 -> 65.8).
 #pragma unroll
                 for (int i = 0; i < 2 * MT; ++i) {
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, MT == 4 ? 3 : 6, 0);
                 }
             }
         };
