@@ -153,8 +153,10 @@ int setup_norm(MatmulArgs &a, const void *delta, const void *norm_weight, void *
 
 // M > 16: the mid-M kernel where it is the faster one, else the tiled kernel.  Measured at LLaMA-7B /
 // 13B / 30B shapes, 256..768 rows: the tiled kernel takes over once it has enough wide tiles (72 for a plain
-// projection, 160 for the gate/up pair, more than 192 with the rotary epilogue: LLaMA-7B QKV at 512 rows, 192 tiles, 75 -> 68 us) - with the rotary epilogue not while
-// their number fills the chip badly (just over one per CU with a short K, where splitting does not pay either).
+// projection, 160 for the gate/up pair, more than 192 with the rotary epilogue: LLaMA-7B QKV at 512 rows, 192 tiles, 75 -> 68 us).
+// (Tile counts just over one per CU used to stay with the mid-M kernel for the rotary epilogue; since the tiled kernel
+// cuts the panels past a whole round along K it is ahead there too: 7B QKV at 768 rows 93.5 against 101.6 us, 13B at
+// 640 rows 110.4 against 123.4.)
 bool prefer_kslice(const KslicePlan &kp, int epi, int M, int N, int K) {
     if (!kp.ok || g_kslice_tuning.mode == 0) return false;
     if (g_kslice_tuning.mode == 2) return true;
@@ -164,7 +166,7 @@ bool prefer_kslice(const KslicePlan &kp, int epi, int M, int N, int K) {
     const long cus = device_shape().cus;  // the crossovers were measured on 256 CUs: 72, 160 and 192 wide tiles
     if (epi == EPI_PLAIN) return wide < 9 * cus / 32;
     if (epi == EPI_SILU_MUL) return wide < 5 * cus / 8;
-    return wide <= 3 * cus / 4 || gemm_plan(epi, M, N, K).score < 0.65;
+    return wide <= 3 * cus / 4;
 }
 
 // Which kernel computes columns [.., .. + n) of an M > 16 call, with what plan, and the partial sums it exchanges.
