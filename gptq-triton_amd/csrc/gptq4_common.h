@@ -24,6 +24,29 @@ typedef float f16_t __attribute__((ext_vector_type(16)));
 __device__ __forceinline__ h2_t as_h2(uint32_t u) { return __builtin_bit_cast(h2_t, u); }
 __device__ __forceinline__ uint32_t as_u32(h2_t h) { return __builtin_bit_cast(uint32_t, h); }
 
+// 2*IW rows of 64 output columns in the register layout of the 32x32 MFMA result - word i of lane (l32 = lane % 32,
+// lhi = lane / 32) holds columns 2*l32 and 2*l32 + 1 of row 8*(i/4) + 4*lhi + i%4 - are turned through 8*IW*32 bytes
+// of LDS that belong to this wave into rows of 128 bytes and stored 16 bytes per lane: 8 lanes per row, 8 rows per
+// instruction, a quarter of the instructions.  A CU hands a 4-byte-per-lane store to the L2 as 64-byte requests
+// (16 lanes each); the 128 x 256 outputs of a tile went out as 1024 of them per wave, all at the end of the kernel,
+// and the chip waited for them: 16 MiB of outputs cost 7 - 9 us that way, about 3 us like this.
+// row_ptr(j, r): where the 64 halves of row r = 8*j + lane/8 of the block go (j is a constant after unrolling), or
+// nullptr for a row that is not stored.
+template <int IW, typename RowPtr>
+__device__ __forceinline__ void store_block_rows(uint32_t *tr, const uint32_t (&w)[IW], int lane, RowPtr row_ptr) {
+    const int l32 = lane & 31, lhi = lane >> 5;
+#pragma unroll
+    for (int i = 0; i < IW; ++i) tr[(8 * (i >> 2) + 4 * lhi + (i & 3)) * 32 + l32] = w[i];
+    // (the wave's own LDS writes and reads are carried out in order: no barrier)
+#pragma unroll
+    for (int j = 0; j < IW / 4; ++j) {
+        const int rr = 8 * j + (lane >> 3);
+        const uint4 v = *reinterpret_cast<const uint4 *>(tr + rr * 32 + 4 * (lane & 7));
+        half_t *const dst = row_ptr(j, rr);
+        if (dst != nullptr) *reinterpret_cast<uint4 *>(dst + 8 * (lane & 7)) = v;
+    }
+}
+
 // Per-column decode constants (both halves of each pair hold the same value).
 struct ColDecode {
     h2_t neg_lo;  // -(1024 + z + 1)

@@ -491,17 +491,22 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
     if (EPI == EPI_PLAIN) {
         h2_t bias2 = {(half_t)0.f, (half_t)0.f};
         if (p.bias != nullptr) bias2 = as_h2(*reinterpret_cast<const uint32_t *>(p.bias + ncol));
+        if (PERM) __syncthreads();  // (the plain K loop ends with a barrier; here the last tile may still be read)
+        uint32_t *const tr = reinterpret_cast<uint32_t *>(region(wave));
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
+        for (int mt = 0; mt < MT; ++mt) {
+            uint32_t w[16];
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                const int row = wrow0 + mt * 32 + 8 * (i >> 2) + 4 * lhi + (i & 3);
-                if (row < M) {
-                    h2_t o = {(half_t)acc[mt][0][i], (half_t)acc[mt][1][i]};
-                    if (p.bias != nullptr) o = o + bias2;
-                    *reinterpret_cast<uint32_t *>(p.y + (size_t)row * N + ncol) = as_u32(o);
-                }
+                h2_t o = {(half_t)acc[mt][0][i], (half_t)acc[mt][1][i]};
+                if (p.bias != nullptr) o = o + bias2;
+                w[i] = as_u32(o);
             }
+            store_block_rows<16>(tr, w, lane, [&](int, int rr) -> half_t * {
+                const int row = wrow0 + mt * 32 + rr;
+                return row < M ? p.y + (size_t)row * N + nw0 : nullptr;
+            });
+        }
     } else if (EPI == EPI_SILU_MUL) {
         // The gate wave (even) and the up wave (odd) of a pair hold the same output tile.
         // They split it by row blocks: in round r the up wave hands over block r and the
@@ -522,9 +527,9 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
                         to_up[(t * 16 + i) * 64 + lane] = acc[MT / 2 + r][t][i];
                 }
             __syncthreads();
+            uint32_t w[16];
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                const int row = wrow0 + mt * 32 + 8 * (i >> 2) + 4 * lhi + (i & 3);
                 float o0, o1;
                 if (wn_odd) {
                     o0 = silu_f32(to_up[(0 * 16 + i) * 64 + lane]) * acc[MT / 2 + r][0][i];
@@ -533,11 +538,14 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
                     o0 = silu_f32(acc[r][0][i]) * to_gate[(0 * 16 + i) * 64 + lane];
                     o1 = silu_f32(acc[r][1][i]) * to_gate[(1 * 16 + i) * 64 + lane];
                 }
-                if (row < M) {
-                    const h2_t o = {(half_t)o0, (half_t)o1};
-                    *reinterpret_cast<uint32_t *>(p.y + (size_t)row * N + ncol) = as_u32(o);
-                }
+                const h2_t o = {(half_t)o0, (half_t)o1};
+                w[i] = as_u32(o);
             }
+            // turned through the region this wave has just read (the partner writes there again behind the next barrier)
+            store_block_rows<16>(reinterpret_cast<uint32_t *>(wn_odd ? to_up : to_gate), w, lane, [&](int, int rr) -> half_t * {
+                const int row = wrow0 + mt * 32 + rr;
+                return row < M ? p.y + (size_t)row * N + nw0 : nullptr;
+            });
         }
     } else {
         // the workgroup's 128 columns are one head of q, k or v; this wave holds d in
@@ -551,14 +559,38 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
         const float *const theirs = region(WM == 2 ? (wave ^ 2) : (wave ^ 1));
         // destination of this wave's head: q [B,H,S,128], k and v [B,H,kv_capacity,128]
         const int cap = (which == 0) ? r.S : r.kv_capacity;
-        half_t *const dst = ((which == 0) ? r.q : (which == 1) ? r.k : r.v) + (size_t)head * cap * 128 + 64 * wn_odd + 2 * l32;
+        half_t *const dst = ((which == 0) ? r.q : (which == 1) ? r.k : r.v) + (size_t)head * cap * 128 + 64 * wn_odd;  // the wave's 64 values of cache row 0
         const size_t seq_stride = (size_t)r.H * cap * 128;
         const bool at_position = (which != 0) && r.kv_offset < 0;  // cache row = the token's position
         const int row_shift = (which == 0 || r.kv_offset < 0) ? 0 : r.kv_offset;
+        // The rotated values of all row blocks are kept in registers and stored at the end, 16 bytes per lane
+        // (store_block_rows): behind the last wait for table values - loads and stores share one counter, so a wait
+        // for a block's table loads would wait for the stores of the blocks before it as well (LLaMA-7B QKV at 1024
+        // rows 118.6 -> 113.5 us, at 2048 rows 204.9 -> 198.2) - and behind a barrier, since the LDS they are turned
+        // through is the region the partner wave read this wave's sums from.
+        uint32_t outw[MT][16];
+        int crow_at[MT][16];  // (cache rows, when they are the tokens' positions)
+        auto store_all = [&]() {
+            __syncthreads();
+            uint32_t *const tr = reinterpret_cast<uint32_t *>(mine);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+                store_block_rows<16>(tr, outw[mt], lane, [&](int j, int rr) -> half_t * {
+                    const int row = wrow0 + mt * 32 + rr;
+                    if (row >= M) return nullptr;
+                    int bb, srow;
+                    split_row(r, row, bb, srow);
+                    // the lane that stores row 8*j + 4*lhi + q holds that row's cache row itself, in word 4*j + q
+                    int crow = srow + row_shift;
+                    if (at_position) {
+                        const int q = (lane >> 3) & 3;
+                        crow = q == 0 ? crow_at[mt][4 * j] : q == 1 ? crow_at[mt][4 * j + 1] : q == 2 ? crow_at[mt][4 * j + 2] : crow_at[mt][4 * j + 3];
+                    }
+                    return dst + (size_t)bb * seq_stride + (size_t)crow * 128;
+                });
+        };
         if constexpr (ROPE_TAB) {
             if (PERM) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // table blocks 0 and 1 (the plain path has waited already)
-            uint32_t outw[MT][16];  // the rotated values, stored at the end
-            int crow_at[MT][16];    // (cache rows, when they are the tokens' positions)
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
                 if (need_tab) {
@@ -586,7 +618,6 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
                 const float *const tcos = rope_tab + (mt & 1) * (2 * 32 * 64) + (4 * lhi) * 64 + 2 * l32;
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
-                    const int row = wrow0 + mt * 32 + 8 * (i >> 2) + 4 * lhi + (i & 3);
                     float o0 = acc[mt][0][i], o1 = acc[mt][1][i];
                     if (which < 2) {
                         const float2 cs = *reinterpret_cast<const float2 *>(tcos + (8 * (i >> 2) + (i & 3)) * 64);
@@ -605,21 +636,7 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
                     if (at_position) crow_at[mt][i] = min(pos[i], r.kv_capacity - 1);
                 }
             }
-            // All stores come behind the last wait for a table block: loads and stores share one counter, so a wait
-            // for a block's table loads would wait for the stores of the blocks before it as well (LLaMA-7B QKV at
-            // 1024 rows 118.6 -> 113.5 us, at 2048 rows 204.9 -> 198.2).
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const int row = wrow0 + mt * 32 + 8 * (i >> 2) + 4 * lhi + (i & 3);
-                    if (row < M) {
-                        int bb, srow;
-                        split_row(r, row, bb, srow);
-                        const int crow = at_position ? crow_at[mt][i] : srow + row_shift;
-                        *reinterpret_cast<uint32_t *>(dst + (size_t)bb * seq_stride + (size_t)crow * 128) = outw[mt][i];
-                    }
-                }
+            store_all();
             return;
         }
 #pragma unroll
@@ -654,7 +671,6 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
             }
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                const int row = wrow0 + mt * 32 + 8 * (i >> 2) + 4 * lhi + (i & 3);
                 float o0 = acc[mt][0][i], o1 = acc[mt][1][i];
                 if (which < 2) {
                     const float p0 = theirs[(0 * 16 + i) * 64 + lane], p1 = theirs[(1 * 16 + i) * 64 + lane];
@@ -666,15 +682,12 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
                         o1 = o1 * cs[i].y + p1 * sn[i].y;
                     }
                 }
-                if (row < M) {
-                    int bb, srow;
-                    split_row(r, row, bb, srow);
-                    const int crow = at_position ? min(pos[i], r.kv_capacity - 1) : srow + row_shift;
-                    const h2_t o = {(half_t)o0, (half_t)o1};
-                    *reinterpret_cast<uint32_t *>(dst + (size_t)bb * seq_stride + (size_t)crow * 128) = as_u32(o);
-                }
+                const h2_t o = {(half_t)o0, (half_t)o1};
+                outw[mt][i] = as_u32(o);
+                if (at_position) crow_at[mt][i] = min(pos[i], r.kv_capacity - 1);
             }
         }
+        store_all();
     }
     };  // run_part
 
