@@ -126,6 +126,10 @@ int setup_gemm(int epi, MatmulArgs &a, const GemmPlan &pl, void *workspace, size
     a.slot_rem = nk % pl.splitk;
     a.tail_first = pl.tail_first;
     a.tail_split = pl.tail_split;
+#ifdef GPTQ4_PHASE_TIMERS
+    // (development build: the phase stamps go 32 MiB into the workspace, also of launches that exchange nothing)
+    if (workspace != nullptr && workspace_bytes >= (size_t)(33 << 20)) a.counters = reinterpret_cast<int *>(workspace);
+#endif
     // the tiles cut along K are the last column panels: the whole tiles cover the columns before them
     if (pl.tail_split > 1) a.n_count = (pl.tail_first / ((a.M + 127) / 128)) * ((epi == EPI_SILU_MUL) ? 128 : 256);
     if (pl.splitk > 1 || pl.streamed || pl.tail_split > 1) {

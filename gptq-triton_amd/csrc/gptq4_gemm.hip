@@ -38,6 +38,19 @@
 // panels in its L2.
 #include "gptq4_internal.h"
 
+// Development aid, compiled out of the product build: per-workgroup stamps of the 100 MHz clock at the phase
+// boundaries of the kernel, written 32 MiB into the workspace (size it so).
+#ifdef GPTQ4_PHASE_TIMERS
+#define GM_STAMP(i)                                                                                             \
+    do {                                                                                                        \
+        if (threadIdx.x == 0 && p.counters != nullptr)                                                          \
+            reinterpret_cast<unsigned long long *>(reinterpret_cast<char *>(p.counters) + (32 << 20))[(blockIdx.y * gridDim.x + blockIdx.x) * 8 + (i)] = \
+                wall_clock64();                                                                                 \
+    } while (0)
+#else
+#define GM_STAMP(i)
+#endif
+
 namespace {
 
 constexpr int BK = 64;
@@ -100,6 +113,7 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
     // One (part of a) tile: K tiles [k_begin, nk) of tile `logical`, which `nsplit` workgroups share; this one is
     // number `idx` of them in K order.  part_slot(c): where sharer c keeps its partial sums.
     auto run_part = [&](const int logical, const int k_begin, const int nk, const int nsplit, const int idx, auto part_slot) {
+    GM_STAMP(0);
     // XCD-contiguous logical tile index: workgroups that run at the same time on one XCD (one
     // L2) have consecutive logical indices.  These walk GROUP_M row tiles, then move to the
     // next column panel, and only after the last panel to the next GROUP_M row tiles: the
@@ -425,6 +439,7 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
         }
         // pairs of tiles without a branch between them (a join there would make the compiler
         // move packed words that are still in flight, and wait for them), then the odd one
+        GM_STAMP(1);
         int kt = k_begin;
         for (; kt + 1 < nk; kt += 2) {
             k_tile(As0, As1, kt, 0);
@@ -436,6 +451,7 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     }
 
+    GM_STAMP(2);
     if (nsplit > 1) {
         // Split-K for problems with too few tiles to fill the chip (or a tile cut by the streamed schedule): every
         // sharer publishes its fp32 accumulators (agent-scope atomics, no cache maintenance - see the small-M
@@ -689,6 +705,11 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
         }
         store_all();
     }
+#ifdef GPTQ4_PHASE_TIMERS
+    GM_STAMP(3);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    GM_STAMP(4);
+#endif
     };  // run_part
 
     if constexpr (!STREAM) {

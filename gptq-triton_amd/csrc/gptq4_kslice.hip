@@ -28,7 +28,7 @@
 #ifdef GPTQ4_PHASE_TIMERS
 #define KS_STAMP(i)                                                                                             \
     do {                                                                                                        \
-        if (threadIdx.x == 0)                                                                                   \
+        if (threadIdx.x == 0 && p.counters != nullptr)                                                          \
             reinterpret_cast<unsigned long long *>(reinterpret_cast<char *>(p.counters) + (32 << 20))[(blockIdx.y * gridDim.x + blockIdx.x) * 8 + (i)] = \
                 wall_clock64();                                                                                 \
     } while (0)
