@@ -429,12 +429,11 @@ __global__ __launch_bounds__(64 * KS, KS == 8 && (MT == 2 || (EPI != EPI_PLAIN &
     // ---- epilogue of registers i0 .. i0 + IW - 1 of row block own_mt
     const int row0 = m0 + own_mt * 32 + 4 * lhi;
     auto row_of = [&](int ii) { return row0 + 8 * ((i0 + ii) >> 2) + ((i0 + ii) & 3); };
-    // Stores go out 16 bytes per lane (store_block_rows), turned through the part of this wave's exchange region that
-    // only this wave read: its own registers' slots of the first column, 64 floats per register.
-    uint32_t *const tr = reinterpret_cast<uint32_t *>(region(own_mt, wave)) + i0 * 64;
-    const int block_row0 = m0 + own_mt * 32 + 2 * i0;  // first row of the 2 * IW rows this wave finishes
-    (void)tr, (void)block_row0;
     if (EPI == EPI_PLAIN) {
+        // Stores go out 16 bytes per lane (store_block_rows), turned through the part of this wave's exchange region
+        // that only this wave read: its own registers' slots of the first column, 64 floats per register.
+        uint32_t *const tr = reinterpret_cast<uint32_t *>(region(own_mt, wave)) + i0 * 64;
+        const int block_row0 = m0 + own_mt * 32 + 2 * i0;  // first row of the 2 * IW rows this wave finishes
 #pragma unroll
         for (int j = 0; j < NSET; ++j) {
             h2_t bias2 = {(half_t)0.f, (half_t)0.f};
@@ -521,38 +520,27 @@ __global__ __launch_bounds__(64 * KS, KS == 8 && (MT == 2 || (EPI != EPI_PLAIN &
                 sn[ii] = *reinterpret_cast<const float2 *>(r.sin_table + (size_t)tp * 64 + 2 * l32);
             }
         }
-        uint32_t wlo[IW], whi[IW];
 #pragma unroll
         for (int ii = 0; ii < IW; ++ii) {
+            const int row = row_of(ii);
             float lo0 = vals[0][0][ii], lo1 = vals[0][1][ii], hi0 = vals[NSET - 1][0][ii], hi1 = vals[NSET - 1][1][ii];
             if (which < 2) {
                 const float a0 = lo0 * cs[ii].x - hi0 * sn[ii].x, a1 = lo1 * cs[ii].y - hi1 * sn[ii].y;
                 const float b0 = hi0 * cs[ii].x + lo0 * sn[ii].x, b1 = hi1 * cs[ii].y + lo1 * sn[ii].y;
                 lo0 = a0, lo1 = a1, hi0 = b0, hi1 = b1;
             }
-            const h2_t olo = {(half_t)lo0, (half_t)lo1}, ohi = {(half_t)hi0, (half_t)hi1};
-            wlo[ii] = as_u32(olo);
-            whi[ii] = as_u32(ohi);
-        }
-        // the lane that stores row 8*j + 4*lhi + q of the block holds that row's position itself, in word 4*j + q
-        auto cache_row = [&](int j, int rr) -> half_t * {
-            const int row = block_row0 + rr;
-            if (row >= M) return nullptr;
-            int bb, srow;
-            split_row(r, row, bb, srow);
-            int crow = srow + row_shift;
-            if (at_position) {
-                const int q = (lane >> 3) & 3;
-                const int ps = q == 0 ? pos[4 * j] : q == 1 ? pos[4 * j + 1] : q == 2 ? pos[4 * j + 2] : pos[4 * j + 3];
-                crow = min(ps, r.kv_capacity - 1);
+            // (4 bytes per lane, as for gate/up: with 16-byte stores this epilogue was 2 - 6 % slower at 256 and 512 rows
+            // with the weights from HBM, and the 64-row variants spilled two more values)
+            if (row < M) {
+                int bb, srow;
+                split_row(r, row, bb, srow);
+                const int crow = at_position ? min(pos[ii], r.kv_capacity - 1) : srow + row_shift;
+                half_t *const at = dst + (size_t)bb * seq_stride + (size_t)crow * 128;
+                const h2_t olo = {(half_t)lo0, (half_t)lo1}, ohi = {(half_t)hi0, (half_t)hi1};
+                *reinterpret_cast<uint32_t *>(at) = as_u32(olo);
+                *reinterpret_cast<uint32_t *>(at + 64) = as_u32(ohi);
             }
-            return dst - 2 * l32 + (size_t)bb * seq_stride + (size_t)crow * 128;
-        };
-        store_block_rows<IW>(tr, wlo, lane, cache_row);
-        store_block_rows<IW>(tr, whi, lane, [&](int j, int rr) -> half_t * {
-            half_t *const at = cache_row(j, rr);
-            return at != nullptr ? at + 64 : nullptr;
-        });
+        }
     }
     KS_STAMP(7);
 }
