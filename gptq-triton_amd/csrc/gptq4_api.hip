@@ -297,6 +297,9 @@ int run_tiled(int epi, MatmulArgs &a, void *workspace, size_t workspace_bytes, h
                 a.counters = reinterpret_cast<int *>(workspace);
                 a.partials = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_HEAD_BYTES);
             }
+#ifdef GPTQ4_PHASE_TIMERS
+            if (workspace != nullptr && workspace_bytes >= (size_t)(33 << 20)) a.counters = reinterpret_cast<int *>(workspace);
+#endif
             rc = launch_kslice(epi, a, c.kp, s);
         } else {
             rc = setup_gemm(epi, a, c.gp, workspace, workspace_bytes);

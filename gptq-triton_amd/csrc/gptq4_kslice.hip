@@ -320,6 +320,7 @@ __global__ __launch_bounds__(64 * KS, KS == 8 && (MT == 2 || (EPI != EPI_PLAIN &
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     KS_STAMP(3);
     __syncthreads();
+    KS_STAMP(2);
 
     // ---- the KS accumulator sets meet, one column block at a time.  Row block mt is finished by PARTS waves
     // (one with four waves, two with eight): wave mt * PARTS + part takes registers i = part * IW .. + IW - 1.
@@ -344,6 +345,9 @@ __global__ __launch_bounds__(64 * KS, KS == 8 && (MT == 2 || (EPI != EPI_PLAIN &
                 for (int i = 0; i < 16; ++i) dst[(t * 16 + i) * 64 + lane] = acc[j][mt][t][i];
         }
         __syncthreads();
+#ifdef GPTQ4_PHASE_TIMERS
+        if (j == 0 && nsplit == 1) KS_STAMP(6);
+#endif
         if (owner) {
             const float *src[KS];
 #pragma unroll
