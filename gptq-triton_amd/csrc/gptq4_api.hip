@@ -169,6 +169,10 @@ bool prefer_kslice(const KslicePlan &kp, int epi, int M, int N, int K) {
     const long wide = (long)((M + 127) / 128) * (N / wide_bn);
     const long cus = device_shape().cus;  // the crossovers were measured on 256 CUs: 72, 160 and 192 wide tiles
     if (epi == EPI_PLAIN) return wide < 9 * cus / 32;
+    // (gate/up at 129 .. 192 rows: the tiled kernel's second row tile is at most half full - a quarter or more of its
+    // work is padding - while the mid-M kernel's 64-row tiles fit: 17920 x 6656 at 192 rows 148 against 114 us, 280 wide
+    // tiles; 11008 x 4096 57.2 against 54.4; 13824 x 5120 level; 22016 x 8192 172 against 158; 28672 x 8192 214 against 205)
+    if (epi == EPI_SILU_MUL && M > 128 && M <= 192) return true;
     if (epi == EPI_SILU_MUL) return wide < 5 * cus / 8;
     return wide <= 3 * cus / 4;
 }
