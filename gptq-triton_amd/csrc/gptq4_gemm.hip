@@ -387,6 +387,7 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
             // Every wave has issued at least 4 vector-memory loads after its LDS-direct loads
             // of this tile (the scale/zero words and the packed words of 4 K steps), and
             // loads complete in order: at most 4 outstanding means the tile has landed.
+            // (tests/test_wait_counts.py counts the loads behind the tile's in the compiled code of every variant.)
             asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");
             dma_a(nxt, min(kt + 1, nk - 1));
             load_group2(par);

@@ -273,6 +273,7 @@ __global__ __launch_bounds__(64 * KS, KS == 8 && (MT == 2 || (EPI != EPI_PLAIN &
             // Loads complete in order and this wave issued 4 * NB packed-word loads after the
             // scale/zero words that followed its LDS-direct loads of this tile: at most that
             // many outstanding means the tile has landed.  It is this wave's own tile: no barrier.
+            // (tests/test_wait_counts.py counts the loads behind the tile's in the compiled code of every variant.)
             // (lgkmcnt: the fragment reads of the tile before are done before its buffer is requested again.)
             asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(4 * NB * (PAIRED ? 2 : 1)) : "memory");
             dma_a(nxt, min(kt + 1, nk - 1));
