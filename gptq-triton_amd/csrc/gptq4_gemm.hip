@@ -441,6 +441,10 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
         // pairs of tiles without a branch between them (a join there would make the compiler
         // move packed words that are still in flight, and wait for them), then the odd one
         GM_STAMP(1);
+#ifdef GPTQ4_PHASE_TIMERS
+        if (threadIdx.x == 0 && p.counters != nullptr)
+            reinterpret_cast<unsigned long long *>(reinterpret_cast<char *>(p.counters) + (32 << 20))[(blockIdx.y * gridDim.x + blockIdx.x) * 8 + 5] = __builtin_readcyclecounter();
+#endif
         int kt = k_begin;
         for (; kt + 1 < nk; kt += 2) {
             k_tile(As0, As1, kt, 0);
@@ -453,6 +457,10 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
     }
 
     GM_STAMP(2);
+#ifdef GPTQ4_PHASE_TIMERS
+    if (threadIdx.x == 0 && p.counters != nullptr)
+        reinterpret_cast<unsigned long long *>(reinterpret_cast<char *>(p.counters) + (32 << 20))[(blockIdx.y * gridDim.x + blockIdx.x) * 8 + 6] = __builtin_readcyclecounter();
+#endif
     if (nsplit > 1) {
         // Split-K for problems with too few tiles to fill the chip (or a tile cut by the streamed schedule): every
         // sharer publishes its fp32 accumulators (agent-scope atomics, no cache maintenance - see the small-M
