@@ -52,6 +52,16 @@ SIGNATURES = {
     "gptq4_rmsnorm": (c_int, [c_void_p] * 4 + [c_int, c_int, c_float, c_void_p]),
     "gptq4_add_rmsnorm": (c_int, [c_void_p] * 6 + [c_int, c_int, c_float, c_void_p]),
     "gptq4_decode_attention": (c_int, [c_void_p] * 6 + [c_int] * 4 + [c_float, c_void_p, c_size_t, c_void_p]),
+    "gptq4_stream_rows": (c_int, [c_int, c_int, c_int, c_int]),
+    "gptq4_stream_pack": (c_int, [c_void_p] * 5 + [c_int, c_int, c_int, c_void_p]),
+    "gptq4_stream_unpack": (c_int, [c_void_p] * 5 + [c_int, c_int, c_int, c_void_p]),
+    "gptq4_stream_dequant": (c_int, [c_void_p] * 3 + [c_int, c_int, c_int, c_void_p]),
+    "gptq4_stream_matmul": (c_int, [c_void_p] * 6 + [c_int] * 4 + [c_void_p, c_size_t, c_void_p]),
+    "gptq4_stream_mlp_gateup": (c_int, [c_void_p] * 3 + [c_float] + [c_void_p] * 7 + [c_int] * 4 + [c_void_p, c_size_t, c_void_p]),
+    "gptq4_stream_qkv_rotary": (c_int, [c_void_p] * 3 + [c_float] + [c_void_p] * 7 + [c_int] + [c_void_p] * 3 + [c_int] * 8
+                                + [c_void_p, c_size_t, c_void_p]),
+    "gptq4_set_stream_tuning": (None, [c_int, c_int]),
+    "gptq4_stream_probe": (c_int, [c_int] + [c_void_p] * 6 + [c_int] * 4 + [c_void_p, c_size_t, c_void_p]),
     "gptq4_chain_workspace_bytes": (c_size_t, [POINTER(Phase), c_int, c_int]),
     "gptq4_decode_chain": (c_int, [POINTER(Phase), c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "gptq4_set_chain_tuning": (None, [c_int, c_int, c_uint, c_int]),

@@ -61,6 +61,18 @@ def build_library(verbose: bool = False, extra_flags=()) -> Path:
     return LIB_PATH
 
 
+PROBE_SRC = CSRC / "probe" / "floor_probe.hip"
+PROBE_PATH = CSRC / "probe" / "floor_probe"
+
+
+def build_probe(verbose: bool = False) -> Path:
+    """Compile the stand-alone floor probe (launch floor, plain-read rate; `bench.py --floor-probe` runs it)."""
+    _run([_hipcc(), "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+          str(PROBE_SRC), "-o", str(PROBE_PATH)], verbose)
+    return PROBE_PATH
+
+
 if __name__ == "__main__":
     path = build_library(verbose=True, extra_flags=sys.argv[1:])
     print("built", path)
+    print("built", build_probe(verbose=True))

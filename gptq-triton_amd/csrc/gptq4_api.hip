@@ -703,4 +703,202 @@ int gptq4_decode_attention(const void *q, const void *k_cache, const void *v_cac
                               reinterpret_cast<hipStream_t>(stream));
 }
 
+
+// ---- streaming-order layout ---------------------------------------------------------------------------------------
+
+static int stream_fill(StreamArgs &a, int epi, int groupsize, void *workspace, size_t workspace_bytes, StreamPlan &pl, bool norm) {
+    pl = stream_plan(epi, a.M, a.N, a.K, norm);
+    if (!pl.ok) return -GPTQ4_E_SHAPE;
+    if (workspace == nullptr || workspace_bytes < GPTQ4_WS_HEAD_BYTES) return -GPTQ4_E_WORKSPACE;
+    a.counters = reinterpret_cast<int *>(workspace);
+    a.tagged = reinterpret_cast<uint64_t *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_COUNTER_BYTES);
+    a.spin_limit = g_gemv_tuning.spin_limit ? g_gemv_tuning.spin_limit : (1u << 22);
+    a.groups = a.K / groupsize;
+    a.batches_per_group = groupsize / 128;
+    a.group_magic = a.batches_per_group > 1 ? (uint32_t)(0x100000000ull / (unsigned)a.batches_per_group + 1) : 0u;
+    return 0;
+}
+
+static int stream_norm(StreamArgs &a, const void *delta, const void *norm_weight, void *sum_out, float eps) {
+    if (delta && !sum_out) return -GPTQ4_E_NULL;
+    if (a.M > NORM_MAX_M || a.K > NORM_MAX_H || !(eps >= 0.f)) return -GPTQ4_E_SHAPE;
+    if (delta && (sum_out == static_cast<const void *>(a.x) || sum_out == delta)) return -GPTQ4_E_SHAPE;
+    if (misaligned16(norm_weight) || (delta && (misaligned16(delta) || misaligned16(sum_out)))) return -GPTQ4_E_ALIGN;
+    a.nrm_delta = reinterpret_cast<const half_t *>(delta);
+    a.nrm_weight = reinterpret_cast<const half_t *>(norm_weight);
+    a.nrm_sum_out = delta ? reinterpret_cast<half_t *>(sum_out) : nullptr;
+    a.nrm_eps = eps;
+    return 0;
+}
+
+int gptq4_stream_rows(int op, int K, int N, int groupsize) {
+    op &= ~GPTQ4_OP_WITH_PERM;
+    if (op < GPTQ4_OP_MATMUL || op > GPTQ4_OP_QKV_ROTARY) return 0;
+    int g = groupsize;
+    if (check_dims(K, N, &g)) return 0;
+    const int epi = (op == GPTQ4_OP_MLP_GATEUP) ? EPI_SILU_MUL : (op == GPTQ4_OP_QKV_ROTARY ? EPI_ROPE : EPI_PLAIN);
+    int rows = 0;
+    for (int m = 1; m <= STREAM_MAX_M; ++m)
+        if (stream_plan(epi, m, N, K, false).ok) rows = m;
+    return rows;
+}
+
+int gptq4_stream_pack(const int32_t *qweight, const int32_t *qzeros, const void *scales, int32_t *sweight, int32_t *smeta, int K,
+                      int N, int groupsize, void *stream) {
+    if (!qweight || !sweight || (smeta && (!qzeros || !scales))) return -GPTQ4_E_NULL;
+    int rc = check_dims(K, N, &groupsize);
+    if (rc) return rc;
+    if (static_cast<const void *>(qweight) == static_cast<const void *>(sweight)) return -GPTQ4_E_SHAPE;
+    return launch_stream_pack(reinterpret_cast<const uint32_t *>(qweight), reinterpret_cast<const uint32_t *>(qzeros),
+                              reinterpret_cast<const half_t *>(scales), reinterpret_cast<uint32_t *>(sweight),
+                              reinterpret_cast<uint32_t *>(smeta), K, N, groupsize, reinterpret_cast<hipStream_t>(stream));
+}
+
+int gptq4_stream_unpack(const int32_t *sweight, const int32_t *smeta, int32_t *qweight, int32_t *qzeros, void *scales, int K, int N,
+                        int groupsize, void *stream) {
+    if (!sweight || !qweight || (smeta && (!qzeros || !scales))) return -GPTQ4_E_NULL;
+    int rc = check_dims(K, N, &groupsize);
+    if (rc) return rc;
+    if (static_cast<const void *>(qweight) == static_cast<const void *>(sweight)) return -GPTQ4_E_SHAPE;
+    return launch_stream_unpack(reinterpret_cast<const uint32_t *>(sweight), reinterpret_cast<const uint32_t *>(smeta),
+                                reinterpret_cast<uint32_t *>(qweight), reinterpret_cast<uint32_t *>(qzeros),
+                                reinterpret_cast<half_t *>(scales), K, N, groupsize, reinterpret_cast<hipStream_t>(stream));
+}
+
+int gptq4_stream_dequant(const int32_t *sweight, const int32_t *smeta, void *W_out, int K, int N, int groupsize, void *stream) {
+    if (!sweight || !smeta || !W_out) return -GPTQ4_E_NULL;
+    int rc = check_dims(K, N, &groupsize);
+    if (rc) return rc;
+    return launch_stream_dequant(reinterpret_cast<const uint32_t *>(sweight), reinterpret_cast<const uint32_t *>(smeta),
+                                 reinterpret_cast<half_t *>(W_out), K, N, groupsize, reinterpret_cast<hipStream_t>(stream));
+}
+
+static int stream_matmul_impl(const void *x, const int32_t *sweight, const int32_t *smeta, const int32_t *perm, const void *bias,
+                              void *y, int M, int K, int N, int groupsize, void *workspace, size_t workspace_bytes, void *stream,
+                              bool nomath) {
+    if (!x || !sweight || !smeta || !y) return -GPTQ4_E_NULL;
+    if (M < 1) return -GPTQ4_E_SHAPE;
+    int rc = check_dims(K, N, &groupsize);
+    if (rc) return rc;
+    if (misaligned16(x) || misaligned16(sweight) || misaligned16(smeta) || misaligned16(y) || (perm && misaligned16(perm)) ||
+        (bias && misaligned16(bias)))
+        return -GPTQ4_E_ALIGN;
+    StreamArgs a = {};
+    a.x = reinterpret_cast<const half_t *>(x);
+    a.m[0] = SMat{reinterpret_cast<const uint32_t *>(sweight), reinterpret_cast<const uint32_t *>(smeta)};
+    a.m[1] = a.m[0];
+    a.perm = perm;
+    a.bias = reinterpret_cast<const half_t *>(bias);
+    a.y = reinterpret_cast<half_t *>(y);
+    a.M = M;
+    a.K = K;
+    a.N = N;
+    StreamPlan pl;
+    rc = stream_fill(a, EPI_PLAIN, groupsize, workspace, workspace_bytes, pl, false);
+    if (rc) return rc;
+    return launch_stream(EPI_PLAIN, a, pl, nomath, reinterpret_cast<hipStream_t>(stream));
+}
+
+int gptq4_stream_matmul(const void *x, const int32_t *sweight, const int32_t *smeta, const int32_t *perm, const void *bias, void *y,
+                        int M, int K, int N, int groupsize, void *workspace, size_t workspace_bytes, void *stream) {
+    return stream_matmul_impl(x, sweight, smeta, perm, bias, y, M, K, N, groupsize, workspace, workspace_bytes, stream, false);
+}
+
+static int stream_gateup_impl(const void *x, const void *delta, const void *norm_weight, float eps, void *sum_out,
+                              const int32_t *gate_sweight, const int32_t *gate_smeta, const int32_t *up_sweight,
+                              const int32_t *up_smeta, const int32_t *perm, void *h, int M, int K, int I, int groupsize,
+                              void *workspace, size_t workspace_bytes, void *stream, bool nomath) {
+    if (!x || !gate_sweight || !gate_smeta || !up_sweight || !up_smeta || !h) return -GPTQ4_E_NULL;
+    if (M < 1) return -GPTQ4_E_SHAPE;
+    int rc = check_dims(K, I, &groupsize);
+    if (rc) return rc;
+    if (misaligned16(x) || misaligned16(gate_sweight) || misaligned16(up_sweight) || misaligned16(gate_smeta) ||
+        misaligned16(up_smeta) || misaligned16(h) || (perm && misaligned16(perm)))
+        return -GPTQ4_E_ALIGN;
+    StreamArgs a = {};
+    a.x = reinterpret_cast<const half_t *>(x);
+    a.m[0] = SMat{reinterpret_cast<const uint32_t *>(gate_sweight), reinterpret_cast<const uint32_t *>(gate_smeta)};
+    a.m[1] = SMat{reinterpret_cast<const uint32_t *>(up_sweight), reinterpret_cast<const uint32_t *>(up_smeta)};
+    a.perm = perm;
+    a.y = reinterpret_cast<half_t *>(h);
+    a.M = M;
+    a.K = K;
+    a.N = I;
+    if (norm_weight) {
+        rc = stream_norm(a, delta, norm_weight, sum_out, eps);
+        if (rc) return rc;
+    }
+    StreamPlan pl;
+    rc = stream_fill(a, EPI_SILU_MUL, groupsize, workspace, workspace_bytes, pl, norm_weight != nullptr);
+    if (rc) return rc;
+    return launch_stream(EPI_SILU_MUL, a, pl, nomath, reinterpret_cast<hipStream_t>(stream));
+}
+
+int gptq4_stream_mlp_gateup(const void *x, const void *delta, const void *norm_weight, float eps, void *sum_out,
+                            const int32_t *gate_sweight, const int32_t *gate_smeta, const int32_t *up_sweight,
+                            const int32_t *up_smeta, const int32_t *perm, void *h, int M, int K, int I, int groupsize,
+                            void *workspace, size_t workspace_bytes, void *stream) {
+    return stream_gateup_impl(x, delta, norm_weight, eps, sum_out, gate_sweight, gate_smeta, up_sweight, up_smeta, perm, h, M, K, I,
+                              groupsize, workspace, workspace_bytes, stream, false);
+}
+
+int gptq4_stream_qkv_rotary(const void *x, const void *delta, const void *norm_weight, float eps, void *sum_out,
+                            const int32_t *sweight, const int32_t *smeta, const int32_t *perm, const int32_t *position_ids,
+                            const float *cos_table, const float *sin_table, int max_pos, void *q, void *k, void *v, int B, int S,
+                            int H, int D, int K, int groupsize, int kv_capacity, int kv_offset, void *workspace,
+                            size_t workspace_bytes, void *stream) {
+    if (!x || !sweight || !smeta || !position_ids || !cos_table || !sin_table || !q || !k || !v) return -GPTQ4_E_NULL;
+    if (B < 1 || S < 1 || H < 1 || D != 128 || max_pos < 1) return -GPTQ4_E_SHAPE;
+    if (kv_offset < GPTQ4_KV_AT_POSITION || kv_capacity < 1 || (kv_offset >= 0 && kv_capacity < kv_offset + S)) return -GPTQ4_E_SHAPE;
+    if ((long)B * S > STREAM_MAX_M) return -GPTQ4_E_SHAPE;
+    const int N = 3 * H * D;
+    int rc = check_dims(K, N, &groupsize);
+    if (rc) return rc;
+    if (misaligned16(x) || misaligned16(sweight) || misaligned16(smeta) || misaligned16(q) || misaligned16(k) || misaligned16(v) ||
+        misaligned16(cos_table) || misaligned16(sin_table) || (perm && misaligned16(perm)))
+        return -GPTQ4_E_ALIGN;
+    StreamArgs a = {};
+    a.x = reinterpret_cast<const half_t *>(x);
+    a.m[0] = SMat{reinterpret_cast<const uint32_t *>(sweight), reinterpret_cast<const uint32_t *>(smeta)};
+    a.m[1] = a.m[0];
+    a.perm = perm;
+    a.M = B * S;
+    a.K = K;
+    a.N = N;
+    a.rope.position_ids = position_ids;
+    a.rope.cos_table = cos_table;
+    a.rope.sin_table = sin_table;
+    a.rope.q = reinterpret_cast<half_t *>(q);
+    a.rope.k = reinterpret_cast<half_t *>(k);
+    a.rope.v = reinterpret_cast<half_t *>(v);
+    a.rope.S = S;
+    a.rope.H = H;
+    a.rope.kv_capacity = kv_capacity;
+    a.rope.kv_offset = kv_offset;
+    a.rope.max_pos = max_pos;
+    a.rope.s_magic = 0;  // at most STREAM_MAX_M rows: a plain division
+    if (norm_weight) {
+        rc = stream_norm(a, delta, norm_weight, sum_out, eps);
+        if (rc) return rc;
+    }
+    StreamPlan pl;
+    rc = stream_fill(a, EPI_ROPE, groupsize, workspace, workspace_bytes, pl, norm_weight != nullptr);
+    if (rc) return rc;
+    return launch_stream(EPI_ROPE, a, pl, false, reinterpret_cast<hipStream_t>(stream));
+}
+
+void gptq4_set_stream_tuning(int waves, int depth) {
+    g_stream_tuning.waves = (waves == 8 || waves == 16) ? waves : 0;
+    g_stream_tuning.depth = (depth >= 1 && depth <= 4) ? depth : 0;
+}
+
+int gptq4_stream_probe(int op, const void *x, const int32_t *sweight, const int32_t *smeta, const int32_t *up_sweight,
+                       const int32_t *up_smeta, void *y, int M, int K, int N, int groupsize, void *workspace, size_t workspace_bytes,
+                       void *stream) {
+    if (op == GPTQ4_OP_MLP_GATEUP)
+        return stream_gateup_impl(x, nullptr, nullptr, 0.f, nullptr, sweight, smeta, up_sweight, up_smeta, nullptr, y, M, K, N, groupsize,
+                                  workspace, workspace_bytes, stream, true);
+    return stream_matmul_impl(x, sweight, smeta, nullptr, nullptr, y, M, K, N, groupsize, workspace, workspace_bytes, stream, true);
+}
+
 }  // extern "C"

@@ -155,6 +155,69 @@ KslicePlan kslice_plan(int epi, int M, int N, int K, bool has_perm);
 size_t kslice_partial_bytes(int epi, const KslicePlan &plan);
 int launch_kslice(int epi, const MatmulArgs &a, const KslicePlan &plan, hipStream_t stream);
 
+// ---- Streaming-order layout (gptq4_stream.hip) ------------------------------------------------------------------
+// One quantised projection in streaming order: per strip of 16 output columns and per unit of 128 input rows one
+// contiguous 1 KiB block; lane l = 16 * r + c of a wave (r = 0..3, c = 0..15) owns bytes [16 * l, 16 * l + 16) of
+// the block: the packed words of the 8-row blocks 4 * r + j (j = 0..3) of the unit, column c of the strip - the B
+// operands of four v_mfma_f32_16x16x32_f16 steps.  Blocks are ordered [strip][unit].  `meta` holds one word per
+// (strip, group, column): fp16 scale bits | stored zero << 16, ordered [strip][group][column].
+struct SMat {
+    const uint32_t *w;
+    const uint32_t *meta;
+};
+
+struct StreamArgs {
+    // (what a wave needs before its first load comes first)
+    const half_t *x;  // [M, K]
+    SMat m[2];        // m[1]: the up projection (EPI_SILU_MUL) or m[0] again (EPI_ROPE: the rotation partners' strips)
+    int M, K, N;
+    int nb;      // units per strip: K / 128
+    int groups;  // K / groupsize
+    int batches_per_group;
+    uint32_t group_magic;
+    int q, r;  // units per workgroup, and how many workgroups take one more
+    uint32_t nb_magic;
+    int xrow;     // 16-byte chunks per row of the activations in LDS
+    int red_off;  // 16-byte chunks of LDS in front of the partial-sum slots
+    int m_magic;  // ceil(2^16 / M)
+    uint64_t *tagged;  // marked partial sums, one slot per workgroup
+    uint32_t q_magic, q1_magic;
+    int nat_off;  // NORM: 16-byte chunks of LDS in front of the normalised rows in natural order
+    uint32_t spin_limit;
+    int *counters;     // the workspace's counter region (error word)
+    half_t *y;
+    const half_t *bias;
+    const int32_t *perm;
+    RopeArgs rope;
+    const half_t *nrm_delta;
+    const half_t *nrm_weight;
+    half_t *nrm_sum_out;
+    float nrm_eps;
+};
+
+struct StreamPlan {
+    int waves, depth;  // waves per workgroup (8 or 16), units in flight per wave
+    int workgroups;
+    int tiles, nb;
+    int q, r;
+    int pieces;  // most strips a workgroup's range touches
+    int xrow, red_off, nat_off;
+    size_t lds_bytes;
+    bool ok;
+};
+struct StreamTuning {
+    int waves, depth;  // 0 = automatic
+};
+extern StreamTuning g_stream_tuning;
+enum { STREAM_MAX_M = 4 };
+StreamPlan stream_plan(int epi, int M, int N, int K, bool norm);
+int launch_stream(int epi, StreamArgs &a, const StreamPlan &plan, bool nomath, hipStream_t stream);
+int launch_stream_pack(const uint32_t *qweight, const uint32_t *qzeros, const half_t *scales, uint32_t *sw, uint32_t *meta,
+                       int K, int N, int groupsize, hipStream_t stream);
+int launch_stream_unpack(const uint32_t *sw, const uint32_t *meta, uint32_t *qweight, uint32_t *qzeros, half_t *scales,
+                         int K, int N, int groupsize, hipStream_t stream);
+int launch_stream_dequant(const uint32_t *sw, const uint32_t *meta, half_t *out, int K, int N, int groupsize, hipStream_t stream);
+
 int launch_dequant(const uint32_t *qweight, const uint32_t *qzeros, const half_t *scales,
                    const int32_t *g_idx, half_t *out, int K, int N, int groupsize,
                    hipStream_t stream);

@@ -30,10 +30,10 @@ __device__ __forceinline__ uint4 norm_take(uint4 v, uint4 d, float &ss) {
 }
 
 // 1/rms of the row from the per-thread sums of squares; part4 = 4 floats of LDS.  Contains a
-// workgroup barrier: all 256 threads call it.
-__device__ __forceinline__ float norm_inv_rms(float ss, float *part4, int tid, int H, float eps) {
+// workgroup barrier: every thread of the workgroup calls it; `active` marks the 256 that hold sums.
+__device__ __forceinline__ float norm_inv_rms(float ss, float *part4, int tid, int H, float eps, bool active = true) {
     ss = norm_wave_sum(ss);
-    if ((tid & 63) == 0) part4[tid >> 6] = ss;
+    if (active && (tid & 63) == 0) part4[tid >> 6] = ss;
     __syncthreads();
     return rsqrtf((part4[0] + part4[1] + part4[2] + part4[3]) / (float)H + eps);
 }
@@ -79,11 +79,12 @@ __device__ __forceinline__ void norm_issue_row0(const half_t *x, const half_t *d
 // Rows 0..M-1 of weight * rmsnorm(x (+ delta)) into xs[row * (H/8) + chunk] (LDS, natural k order);
 // row 0 from the registers norm_issue_row0 filled, further rows loaded here.  If sum_out is not
 // null the sums x + delta are written there as well (one workgroup of the launch does that).
-// 256 threads, part = NORM_MAX_M * 4 floats of LDS.  Ends with a barrier.
+// 256 threads, part = NORM_MAX_M * 4 floats of LDS.  Ends with a barrier.  In a workgroup of more than 256
+// threads all of them call it (the barriers are the workgroup's) and `active` is true for threads 0..255 only.
 template <bool ADD, int KEEP>
 __device__ __forceinline__ void norm_rows_to_lds(const half_t *x, const half_t *delta, const half_t *w, half_t *sum_out,
                                                  uint4 *xs, float *part, int M, int H, float eps, int tid,
-                                                 const NormLoads<KEEP> &r0) {
+                                                 const NormLoads<KEEP> &r0, bool active = true) {
     const int chunks = H >> 3;
     for (int row = 0; row < M; ++row) {
         const uint4 *xr = reinterpret_cast<const uint4 *>(x + (size_t)row * H);
@@ -93,18 +94,18 @@ __device__ __forceinline__ void norm_rows_to_lds(const half_t *x, const half_t *
 #pragma unroll
         for (int n = 0; n < KEEP; ++n) {
             const int c = tid + 256 * n;
-            if (c < chunks) {
+            if (active && c < chunks) {
                 const uint4 v = (row == 0) ? r0.x[n] : xr[c];
                 const uint4 d = (row == 0) ? r0.d[n] : (ADD ? dr[c] : v);
                 held[n] = norm_take<ADD>(v, d, ss);
                 if (ADD && sum_out != nullptr) reinterpret_cast<uint4 *>(sum_out + (size_t)row * H)[c] = held[n];
             }
         }
-        const float inv = norm_inv_rms(ss, part + 4 * row, tid, H, eps);
+        const float inv = norm_inv_rms(ss, part + 4 * row, tid, H, eps, active);
 #pragma unroll
         for (int n = 0; n < KEEP; ++n) {
             const int c = tid + 256 * n;
-            if (c < chunks) xs[row * chunks + c] = norm_put(held[n], r0.g[n], inv);
+            if (active && c < chunks) xs[row * chunks + c] = norm_put(held[n], r0.g[n], inv);
         }
     }
     __syncthreads();
