@@ -1,4 +1,5 @@
-"""ctypes binding of csrc/libgptq4.so (the C ABI declared in include/gptq4.h).
+"""ctypes binding of csrc/libgptq4.so (the C ABI declared in include/gptq4.h; tuning and test hooks in
+include/gptq4_experimental.h).
 
 The HIP library is the only compute path: if it is missing, load() raises, and every
 operator that needs it raises with it.  There is no CPU fallback.
@@ -12,7 +13,7 @@ from pathlib import Path
 import torch
 
 LIB_PATH = Path(__file__).resolve().parent / "csrc" / "libgptq4.so"
-ABI_VERSION = 2
+ABI_VERSION = 3
 WS_COUNTER_BYTES = 524288            # arrival counters
 WS_HEAD_BYTES = WS_COUNTER_BYTES + (16 << 20)  # GPTQ4_WS_HEAD_BYTES: counters + marked partial sums, zero between calls
 WS_ERROR_WORD = 1                     # GPTQ4_WS_ERROR_WORD

@@ -2,6 +2,7 @@
 // host, then one kernel launch on the caller's stream.  No allocation, no
 // synchronisation, no exceptions.
 #include "../../include/gptq4.h"
+#include "../../include/gptq4_experimental.h"
 
 #include "gptq4_internal.h"
 #include "gptq4_norm.h"
@@ -889,7 +890,7 @@ int gptq4_stream_qkv_rotary(const void *x, const void *delta, const void *norm_w
 
 void gptq4_set_stream_tuning(int waves, int depth) {
     g_stream_tuning.waves = (waves == 8 || waves == 16) ? waves : 0;
-    g_stream_tuning.depth = (depth >= 1 && depth <= 4) ? depth : 0;
+    g_stream_tuning.depth = (depth >= 1 && depth <= 3) ? depth : 0;
 }
 
 int gptq4_stream_probe(int op, const void *x, const int32_t *sweight, const int32_t *smeta, const int32_t *up_sweight,

@@ -37,6 +37,7 @@
 #include "gptq4_chain.h"
 
 #include "../../include/gptq4.h"
+#include "../../include/gptq4_experimental.h"
 #include "gptq4_norm.h"
 
 #include <mutex>

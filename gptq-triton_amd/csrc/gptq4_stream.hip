@@ -535,10 +535,8 @@ int launch_epi(const StreamArgs &a, const StreamPlan &pl, bool nomath, hipStream
         case 81: return launch_shape<EPI, 8, 1>(a, pl, nomath, stream);
         case 82: return launch_shape<EPI, 8, 2>(a, pl, nomath, stream);
         case 83: return launch_shape<EPI, 8, 3>(a, pl, nomath, stream);
-        case 84: return launch_shape<EPI, 8, 4>(a, pl, nomath, stream);
         case 161: return launch_shape<EPI, 16, 1>(a, pl, nomath, stream);
         case 162: return launch_shape<EPI, 16, 2>(a, pl, nomath, stream);
-        case 163: return launch_shape<EPI, 16, 3>(a, pl, nomath, stream);
         default: return (int)hipErrorInvalidValue;
     }
 }
@@ -551,9 +549,7 @@ StreamTuning g_stream_tuning = {0, 0};
 
 StreamPlan stream_plan(int epi, int M, int N, int K, bool norm) {
     StreamPlan pl = {};
-    pl.waves = g_stream_tuning.waves ? g_stream_tuning.waves : 16;
     pl.depth = g_stream_tuning.depth ? g_stream_tuning.depth : 2;
-    if (pl.waves == 16 && pl.depth > 3) pl.depth = 3;
     const int nv = (epi == EPI_PLAIN) ? 1 : 2;
     pl.tiles = (epi == EPI_ROPE) ? N / 32 : N / 16;
     pl.nb = K / 128;
@@ -563,6 +559,12 @@ StreamPlan stream_plan(int epi, int M, int N, int K, bool norm) {
     if (pl.workgroups < 1) return pl;
     pl.q = (int)(units / pl.workgroups);
     pl.r = (int)(units % pl.workgroups);
+    // Launch shape, from sweeps at LLaMA-7B shapes with the weights coming from HBM (one row): two units in flight per
+    // wave; eight waves per workgroup, sixteen for a plain projection with long ranges (down_proj: 8.1 against 8.6 us),
+    // where a wave of eight would walk through a dozen units one after the other.
+    pl.waves = g_stream_tuning.waves ? g_stream_tuning.waves : ((nv == 1 && pl.q >= 48) ? 16 : 8);
+    if (!g_stream_tuning.waves && pl.nb < pl.waves) pl.waves = 8;
+    if (pl.waves == 16 && pl.depth > 2) pl.depth = 2;
     pl.pieces = (pl.q + 1 + pl.nb - 1) / pl.nb + 1;
     pl.xrow = K / 8 + 1;
     pl.red_off = M * pl.xrow;

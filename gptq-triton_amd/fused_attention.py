@@ -126,6 +126,53 @@ def qkv_rotary(groupsize: int, hidden_states: torch.Tensor, qweight: torch.Tenso
     return q, kk, vv
 
 
+def qkv_rotary_stream(groupsize: int, hidden_states: torch.Tensor, sweight: torch.Tensor, smeta: torch.Tensor,
+                      position_ids: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, num_heads: int, head_dim: int = 128,
+                      perm: Optional[torch.Tensor] = None, kv_out: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+                      kv_offset: int = 0, norm=None):
+    """qkv_rotary on a projection in streaming order (quant_linear.stream_pack), for up to stream_rows() tokens in all;
+    same arguments otherwise, same results to the last bit of the fp32 sums' order."""
+    k_in, n = _check_matmul_args(hidden_states, sweight, groupsize)
+    _check_device_tensors(hidden_states, sweight, smeta, perm, cos, sin)
+    if hidden_states.dim() != 3:
+        raise ValueError(f"hidden_states must be [B, S, hidden], got {tuple(hidden_states.shape)}")
+    bsz, q_len, _ = hidden_states.shape
+    if n != 3 * num_heads * head_dim:
+        raise ValueError(f"packed QKV has {n} columns, expected 3*{num_heads}*{head_dim}")
+    dev = hidden_states.device
+    pos = position_ids
+    if pos.dtype != torch.int32 or pos.device != dev or tuple(pos.shape) != (bsz, q_len) or not pos.is_contiguous():
+        pos = position_ids.to(device=dev, dtype=torch.int32).expand(bsz, q_len).contiguous()
+    q = torch.empty((bsz, num_heads, q_len, head_dim), dtype=torch.float16, device=dev)
+    if kv_out is None:
+        kk, vv = torch.empty_like(q), torch.empty_like(q)
+        cap, off = q_len, 0
+    else:
+        kk, vv = kv_out
+        cap, off = kk.shape[2], kv_offset
+        if kk.shape != vv.shape or kk.shape[0] != bsz or kk.shape[1] != num_heads or kk.shape[3] != head_dim \
+                or not kk.is_contiguous() or not vv.is_contiguous() or off < KV_AT_POSITION or off + q_len > cap:
+            raise ValueError("kv_out buffers must be contiguous [B, H, capacity, D] with room for the new rows")
+    delta_p = nw_p = sum_p = None
+    eps, s = 0.0, None
+    x2d = hidden_states.view(-1, k_in)
+    if norm is not None:
+        from .decoder_ops import check_norm_args
+        delta, norm_weight, eps = norm
+        x2d, d2, s = check_norm_args(hidden_states, delta, norm_weight)
+        delta_p, nw_p, sum_p = _lib.ptr(d2), norm_weight.data_ptr(), _lib.ptr(s)
+    lib = _lib.load()
+    ws = _lib.workspace(dev, _lib.WS_HEAD_BYTES)
+    rc = lib.gptq4_stream_qkv_rotary(x2d.data_ptr(), delta_p, nw_p, float(eps), sum_p, sweight.data_ptr(), smeta.data_ptr(),
+                                     _lib.ptr(perm), pos.data_ptr(), cos.data_ptr(), sin.data_ptr(), cos.shape[0], q.data_ptr(),
+                                     kk.data_ptr(), vv.data_ptr(), bsz, q_len, num_heads, head_dim, k_in, groupsize, cap, off,
+                                     ws.data_ptr(), ws.numel(), _lib.current_stream(dev))
+    _lib.check(rc, "gptq4_stream_qkv_rotary")
+    if norm is None:
+        return q, kk, vv
+    return q, kk, vv, (hidden_states if s is None else s.view(hidden_states.shape))
+
+
 def _fuse_qkv(q_proj: QuantLinear, k_proj: QuantLinear, v_proj: QuantLinear) -> QuantLinear:
     gq, gk, gv = (getattr(p, 'g_idx', None) for p in (q_proj, k_proj, v_proj))
     have = [g is not None for g in (gq, gk, gv)]
@@ -134,7 +181,8 @@ def _fuse_qkv(q_proj: QuantLinear, k_proj: QuantLinear, v_proj: QuantLinear) -> 
     layer = QuantLinear(q_proj.bits, q_proj.groupsize, q_proj.infeatures,
                         q_proj.outfeatures + k_proj.outfeatures + v_proj.outfeatures, bias=False,
                         act_order=all(have))
-    layer.qweight = torch.cat([q_proj.qweight, k_proj.qweight, v_proj.qweight], dim=1)
+    # (checkpoint_qweight: a compacted or streamed projection hands over the checkpoint's layout, not what its buffer holds)
+    layer.qweight = torch.cat([q_proj.checkpoint_qweight(), k_proj.checkpoint_qweight(), v_proj.checkpoint_qweight()], dim=1)
     layer.qzeros = torch.cat([q_proj.qzeros, k_proj.qzeros, v_proj.qzeros], dim=1)
     layer.scales = torch.cat([q_proj.scales, k_proj.scales, v_proj.scales], dim=1)
     layer.bias = None
@@ -218,6 +266,10 @@ class QuantLlamaAttention(nn.Module):
         else:
             need = max(kv_offset, 0) + hidden_states.shape[1]
         cos, sin = self.rope.get(hidden_states.device, max(need, self.max_position_embeddings))
+        sw = self.qkv_proj.stream_weights(hidden_states.shape[0] * hidden_states.shape[1])
+        if sw is not None:
+            return qkv_rotary_stream(self.qkv_proj.groupsize, hidden_states, sw[0], sw[1], position_ids, cos, sin, self.num_heads,
+                                     self.head_dim, perm=None if ordered else sw[2], kv_out=kv_out, kv_offset=kv_offset, norm=norm)
         qweight, perm = self.qkv_proj.kernel_weights()
         return qkv_rotary(self.qkv_proj.groupsize, hidden_states, qweight, self.qkv_proj.scales,
                           self.qkv_proj.qzeros, position_ids, cos, sin, self.num_heads, self.head_dim,
@@ -227,7 +279,7 @@ class QuantLlamaAttention(nn.Module):
         """Where each feature of the attention output should be stored so that an act-order o_proj reads
         it in the order of its sorted rows (int32 [hidden], the inverse of o_proj's permutation), or
         None without act-order.  decode_attention(out_index=...) writes in that order."""
-        _, perm = self.o_proj.kernel_weights()
+        perm = self.o_proj.row_permutation()
         if perm is None:
             return None
         if self._context_order is None or self._context_order[0] != tensor_key(perm):
@@ -237,7 +289,7 @@ class QuantLlamaAttention(nn.Module):
     def input_order(self):
         """The same for the input of the fused QKV projection: rms_norm / add_rms_norm(out_index=...) write in
         that order, and project_qkv(ordered=True) then runs without a gather.  None without act-order."""
-        _, perm = self.qkv_proj.kernel_weights()
+        perm = self.qkv_proj.row_permutation()
         if perm is None:
             return None
         if self._input_order is None or self._input_order[0] != tensor_key(perm):
@@ -246,11 +298,7 @@ class QuantLlamaAttention(nn.Module):
 
     def project_out(self, context: torch.Tensor, ordered: bool = False) -> torch.Tensor:
         """o_proj(context); ordered: the context already is in the order of context_order()."""
-        if not ordered:
-            return self.o_proj(context)
-        o = self.o_proj
-        qweight, _ = o.kernel_weights()
-        return matmul4(o.groupsize, context, qweight, o.scales, o.qzeros, o.bias, None)
+        return self.o_proj.multiply(context, ordered=ordered)
 
     def norm_fusable(self, rows: int) -> bool:
         """Whether project_qkv(norm=...) is the faster way for this many rows."""

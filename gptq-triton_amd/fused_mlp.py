@@ -13,7 +13,8 @@ import torch
 import torch.nn as nn
 
 from . import _lib
-from .quant_linear import QuantLinear, _check_device_tensors, _check_matmul_args, matmul4, tensor_key
+from .quant_linear import (QuantLinear, _check_device_tensors, _check_matmul_args, matmul4, stream_pack, stream_rows,
+                           stream_unpack, tensor_key)
 
 
 def llama_mlp_4(groupsize: int, a: torch.Tensor,
@@ -73,6 +74,37 @@ def norm_llama_mlp_4(groupsize: int, h: torch.Tensor, delta: Optional[torch.Tens
     return (h if s is None else s.view(h.shape)), c.view(h.shape[:-1] + (n,))
 
 
+def llama_mlp_4_stream(groupsize: int, a: torch.Tensor, gate_sweight: torch.Tensor, gate_smeta: torch.Tensor,
+                       up_sweight: torch.Tensor, up_smeta: torch.Tensor, perm: Optional[torch.Tensor] = None, norm=None):
+    """llama_mlp_4 on projections in streaming order (quant_linear.stream_pack), for up to stream_rows() rows.
+    norm = (delta or None, norm_weight, eps): `a` is the residual stream h and the kernel multiplies with
+    RMSNorm(h + delta) * norm_weight; returns (h + delta, result) then."""
+    assert gate_sweight.shape == up_sweight.shape and gate_smeta.shape == up_smeta.shape, "All weights must have the same shape"
+    k, n = _check_matmul_args(a, gate_sweight, groupsize)
+    _check_device_tensors(a, gate_sweight, gate_smeta, up_sweight, up_smeta, perm)
+    lib = _lib.load()
+    delta_p = nw_p = sum_p = None
+    eps = 0.0
+    x, s = a.view(-1, k), None
+    if norm is not None:
+        from .decoder_ops import check_norm_args
+        delta, norm_weight, eps = norm
+        x, d2, s = check_norm_args(a, delta, norm_weight)
+        delta_p, nw_p, sum_p = _lib.ptr(d2), norm_weight.data_ptr(), _lib.ptr(s)
+    m = x.shape[0]
+    c = torch.empty((m, n), device=a.device, dtype=torch.float16)
+    if m:
+        ws = _lib.workspace(a.device, _lib.WS_HEAD_BYTES)
+        rc = lib.gptq4_stream_mlp_gateup(x.data_ptr(), delta_p, nw_p, float(eps), sum_p, gate_sweight.data_ptr(), gate_smeta.data_ptr(),
+                                         up_sweight.data_ptr(), up_smeta.data_ptr(), _lib.ptr(perm), c.data_ptr(), m, k, n, groupsize,
+                                         ws.data_ptr(), ws.numel(), _lib.current_stream(a.device))
+        _lib.check(rc, "gptq4_stream_mlp_gateup")
+    out = c.view(a.shape[:-1] + (n,))
+    if norm is None:
+        return out
+    return (a if s is None else s.view(a.shape)), out
+
+
 def _move_zero_columns(qzeros: torch.Tensor, cols: torch.Tensor) -> torch.Tensor:
     """qzeros [G, N/8] (eight 4-bit stored zeros per word, column 8c+t in bits [4t, 4t+4)) with its
     columns gathered: column j of the result = column cols[j] of the input."""
@@ -92,10 +124,10 @@ class QuantLlamaMLP(nn.Module):
     def __init__(self, gate_proj: QuantLinear, down_proj: QuantLinear, up_proj: QuantLinear):
         super().__init__()
         assert gate_proj.groupsize == up_proj.groupsize
-        self.register_buffer('gate_proj_qweight', gate_proj.qweight)
+        self.register_buffer('gate_proj_qweight', gate_proj.checkpoint_qweight())
         self.register_buffer('gate_proj_scales', gate_proj.scales)
         self.register_buffer('gate_proj_qzeros', gate_proj.qzeros)
-        self.register_buffer('up_proj_qweight', up_proj.qweight)
+        self.register_buffer('up_proj_qweight', up_proj.checkpoint_qweight())
         self.register_buffer('up_proj_scales', up_proj.scales)
         self.register_buffer('up_proj_qzeros', up_proj.qzeros)
         self.groupsize = gate_proj.groupsize
@@ -118,6 +150,11 @@ class QuantLlamaMLP(nn.Module):
         self._is_compact = False
         self.register_buffer('_compact_rows', None, persistent=False)   # row permutation (act-order input), or None
         self.register_buffer('_compact_cols', None, persistent=False)   # column order (act-order down_proj), or None
+        # to_stream(): the two qweight buffers hold streaming-order words (of the layout above) and these the {scale, zero}
+        # words that go with them
+        self.register_buffer('_gate_meta', None, persistent=False)
+        self.register_buffer('_up_meta', None, persistent=False)
+        self._stream_rows = 0
 
     _SIX = ('gate_proj_qweight', 'gate_proj_scales', 'gate_proj_qzeros', 'up_proj_qweight', 'up_proj_scales', 'up_proj_qzeros')
 
@@ -126,11 +163,11 @@ class QuantLlamaMLP(nn.Module):
         by group, columns in the order of an act-order down_proj's rows), in the module's own buffers - otherwise that
         layout lives beside the checkpoint tensors.  state_dict() still gives the checkpoint layout (rows and columns
         put back on the way out) and load_state_dict() brings the module back to it."""
-        if self._is_compact or not self.gate_proj_qweight.is_cuda:
+        if self._is_compact or self._gate_meta is not None or not self.gate_proj_qweight.is_cuda:
             return
         self.down_proj.compact()
         w, perm, _ = self._chained_weights()
-        _, down_perm = self.down_proj.kernel_weights()
+        down_perm = self.down_proj.row_permutation()
         if perm is None and down_perm is None:
             return
         for name, t in zip(self._SIX, w):
@@ -140,9 +177,44 @@ class QuantLlamaMLP(nn.Module):
         self._is_compact = True
         self._sorted = self._chained = None
 
+    def to_stream(self) -> bool:
+        """On the GPU: gate, up (and down_proj) keep their packed weights in streaming order, which the decode kernel
+        for up to `_stream_rows` rows reads - still one copy (see QuantLinear.to_stream; an act-order block is
+        compacted first).  Returns whether gate and up now are in streaming order."""
+        if self._gate_meta is not None:
+            return True
+        if not self.gate_proj_qweight.is_cuda:
+            return False
+        self.compact()  # (act-order: rows sorted, columns in down_proj's order, while down_proj still is in the checkpoint's word layout)
+        self.down_proj.to_stream()
+        rows = stream_rows(_lib.OP_MLP_GATEUP, self.infeatures, self.gate_proj_qweight.shape[1], self.groupsize)
+        if rows == 0 or ((self.g_idx is not None or self.down_proj.g_idx is not None) and not self._is_compact):
+            return False
+        self.gate_proj_qweight, self._gate_meta = stream_pack(self.gate_proj_qweight, self.gate_proj_qzeros, self.gate_proj_scales, self.groupsize)
+        self.up_proj_qweight, self._up_meta = stream_pack(self.up_proj_qweight, self.up_proj_qzeros, self.up_proj_scales, self.groupsize)
+        self._stream_rows = rows
+        self._sorted = self._chained = None
+        return True
+
+    def to_checkpoint(self) -> None:
+        """Undo to_stream() (a compacted act-order block stays compacted)."""
+        self.down_proj.to_checkpoint()
+        if self._gate_meta is not None:
+            self.gate_proj_qweight = stream_unpack(self.gate_proj_qweight)
+            self.up_proj_qweight = stream_unpack(self.up_proj_qweight)
+            self._gate_meta = self._up_meta = None
+            self._stream_rows = 0
+
+    def _six(self) -> tuple:
+        """The six gate / up tensors in the checkpoint's word layout (rows and columns as the kernels read them)."""
+        out = [getattr(self, name) for name in self._SIX]
+        if self._gate_meta is not None:
+            out[0], out[3] = stream_unpack(out[0]), stream_unpack(out[3])
+        return tuple(out)
+
     def checkpoint_tensors(self) -> dict:
         """The six gate / up tensors in the checkpoint's layout, by buffer name."""
-        out = {name: getattr(self, name) for name in self._SIX}
+        out = dict(zip(self._SIX, self._six()))
         if not self._is_compact:
             return out
         from .quant_linear import inverse_permutation, sort_rows
@@ -158,16 +230,18 @@ class QuantLlamaMLP(nn.Module):
 
     def _save_to_state_dict(self, destination, prefix, keep_vars):
         super()._save_to_state_dict(destination, prefix, keep_vars)
-        if self._is_compact:
+        if self._is_compact or self._gate_meta is not None:
             for name, t in self.checkpoint_tensors().items():
                 destination[prefix + name] = t
 
     def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
-        if self._is_compact:
+        if self._is_compact or self._gate_meta is not None:
             for name, t in self.checkpoint_tensors().items():
                 setattr(self, name, t)
             self._is_compact = False
             self._compact_rows = self._compact_cols = None
+            self._gate_meta = self._up_meta = None
+            self._stream_rows = 0
         super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
 
     def _kernel_weights(self):
@@ -185,11 +259,13 @@ class QuantLlamaMLP(nn.Module):
 
     def gate_up(self, x: torch.Tensor) -> torch.Tensor:
         if self._is_compact:
-            mid = llama_mlp_4(self.groupsize, x, *(getattr(self, n) for n in self._SIX), self._compact_rows)
+            mid = llama_mlp_4(self.groupsize, x, *self._six(), self._compact_rows)
             if self._compact_cols is None:
                 return mid
             from .quant_linear import inverse_permutation
             return mid.index_select(-1, inverse_permutation(self._compact_cols))
+        if self._gate_meta is not None:
+            return llama_mlp_4(self.groupsize, x, *self._six(), None)
         gq, uq, perm = self._kernel_weights()
         return llama_mlp_4(self.groupsize, x, gq, self.gate_proj_scales, self.gate_proj_qzeros,
                            uq, self.up_proj_scales, self.up_proj_qzeros, perm)
@@ -202,8 +278,8 @@ class QuantLlamaMLP(nn.Module):
         column only moves, its values do not change).  The intermediate then comes out of the gate/up
         launch already in the order down_proj's kernel reads, and down_proj runs without a gather."""
         down_q, down_perm = self.down_proj.kernel_weights()
-        if self._is_compact:
-            return tuple(getattr(self, n) for n in self._SIX), self._compact_rows, down_q
+        if self._is_compact or self._gate_meta is not None:
+            return self._six(), self._compact_rows, down_q
         if down_perm is None:
             gq, uq, perm = self._kernel_weights()
             return (gq, self.gate_proj_scales, self.gate_proj_qzeros, uq, self.up_proj_scales, self.up_proj_qzeros), perm, down_q
@@ -237,7 +313,7 @@ class QuantLlamaMLP(nn.Module):
         (int32 [infeatures], the inverse of their shared permutation; None without act-order):
         rms_norm / add_rms_norm(out_index=...) write in that order and forward(x, ordered=True) runs
         without a gather."""
-        perm = self._chained_weights()[1]
+        perm = self._compact_rows if (self._is_compact or self._gate_meta is not None) else self._chained_weights()[1]
         if perm is None:
             return None
         if self._input_order is None or self._input_order[0] != tensor_key(perm):
@@ -245,7 +321,14 @@ class QuantLlamaMLP(nn.Module):
             self._input_order = (tensor_key(perm), inverse_permutation(perm))
         return self._input_order[1]
 
+    def _stream_ready(self, x: torch.Tensor) -> bool:
+        return self._gate_meta is not None and x.numel() // max(self.infeatures, 1) <= self._stream_rows
+
     def forward(self, x: torch.Tensor, ordered: bool = False) -> torch.Tensor:
+        if self._stream_ready(x):
+            mid = llama_mlp_4_stream(self.groupsize, x, self.gate_proj_qweight, self._gate_meta, self.up_proj_qweight, self._up_meta,
+                                     None if ordered else self._compact_rows)
+            return self.down_proj.multiply(mid, ordered=True)  # the columns of gate and up are laid out in the order down_proj reads
         w, perm, down_q = self._chained_weights()
         return self._down(llama_mlp_4(self.groupsize, x, *w, None if ordered else perm), down_q)
 
@@ -256,6 +339,10 @@ class QuantLlamaMLP(nn.Module):
 
     def forward_normed(self, h: torch.Tensor, delta: Optional[torch.Tensor], norm_weight: torch.Tensor, eps: float):
         """(h + delta, forward(RMSNorm(h + delta))): the residual add and the norm run inside the gate/up launch."""
+        if self._stream_ready(h):
+            s, mid = llama_mlp_4_stream(self.groupsize, h, self.gate_proj_qweight, self._gate_meta, self.up_proj_qweight, self._up_meta,
+                                        self._compact_rows, norm=(delta, norm_weight, eps))
+            return s, self.down_proj.multiply(mid, ordered=True)
         w, perm, down_q = self._chained_weights()
         s, mid = norm_llama_mlp_4(self.groupsize, h, delta, norm_weight, eps, *w, perm)
         return s, self._down(mid, down_q)

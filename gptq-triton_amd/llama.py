@@ -23,6 +23,8 @@ from .fused_attention import LlamaConfigLite
 
 # up to this many rows the decoder's norms write act-order inputs in their consumer's order
 ORDERED_NORM_ROWS = 16
+# up to this many sequences a GreedyDecoder asks for the streaming-order weight layout (the rows its kernel takes)
+STREAM_BATCH = 4
 
 
 def config_from_json(path) -> LlamaConfigLite:
@@ -166,10 +168,18 @@ class GreedyDecoder:
     K and V by position id, the attention kernel reads how far to attend from the position
     buffer), so the step can be captured once as a HIP graph and replayed."""
 
-    def __init__(self, model: LlamaForCausalLM, bsz: int, capacity: int):
+    def __init__(self, model: LlamaForCausalLM, bsz: int, capacity: int, layout: str = 'auto'):
+        """layout: 'stream' / 'checkpoint' put the model's packed weights into that layout first (quant_linear.set_layout;
+        one copy either way), 'keep' leaves them as they are, 'auto' = 'stream' for up to STREAM_BATCH sequences - what
+        the decode kernel for a handful of rows reads - and 'checkpoint' beyond."""
         cfg = model.config
         self.model, self.bsz, self.capacity = model, bsz, capacity
         dev = model.lm_head.weight.device
+        if layout == 'auto':
+            layout = 'stream' if bsz <= STREAM_BATCH else 'checkpoint'
+        if layout != 'keep' and dev.type == 'cuda':
+            from .quant_linear import set_layout
+            set_layout(model, layout)
         heads, hd = cfg.num_attention_heads, cfg.hidden_size // cfg.num_attention_heads
         self.caches = [(torch.zeros((bsz, heads, capacity, hd), dtype=torch.float16, device=dev),
                         torch.zeros((bsz, heads, capacity, hd), dtype=torch.float16, device=dev))

@@ -22,7 +22,8 @@ from .quant_linear import QuantLinear, make_quant
 
 
 def load_quant(checkpoint: str, warmup_autotune: bool = True, device: Optional[str] = 'cuda',
-               fuse_mlp: Optional[bool] = None, use_transformers: bool = False, compact: bool = True):
+               fuse_mlp: Optional[bool] = None, use_transformers: bool = False, compact: bool = True,
+               layout: str = 'stream'):
     """Load a quantised model from a checkpoint directory.
 
     use_transformers: build the skeleton as the reference does (src/gptq_triton/__init__.py:32-52): a
@@ -33,6 +34,12 @@ def load_quant(checkpoint: str, warmup_autotune: bool = True, device: Optional[s
     compact: act-order checkpoints on a GPU keep ONE copy of every packed weight, in the layout the kernels read
     (QuantLinear.compact, QuantLlamaMLP.compact); state_dict() / save_quant() still produce the checkpoint layout.
     With False the kernel layout is built at first use beside the checkpoint tensors (twice the weight memory).
+
+    layout: 'stream' (default; GPU only) keeps every packed weight in streaming order, the layout the decode kernel for
+    up to four rows reads (quant_linear.set_layout, QuantLinear.to_stream) - one copy of the weights either way, and
+    state_dict() / save_quant() produce the checkpoint layout.  Calls with more rows (a prompt pass) unpack a projection's
+    words into a scratch tensor for the duration of the call; a model that mostly serves such calls, or decodes more than
+    four sequences at a time, is better kept in the 'checkpoint' layout.
 
     warmup_autotune is accepted for compatibility: launch shapes are static, there is
     nothing to tune (the reference spends 18-49 s here).  It still requires a device, as
@@ -100,6 +107,10 @@ def load_quant(checkpoint: str, warmup_autotune: bool = True, device: Optional[s
         model = model.to(device)
         if compact and act_order and torch.device(device).type == 'cuda':
             quant_linear.compact_act_order(model)
+        if layout == 'stream' and torch.device(device).type == 'cuda':
+            quant_linear.set_layout(model, 'stream')
+        elif layout not in ('stream', 'checkpoint'):
+            raise ValueError("layout must be 'stream' or 'checkpoint'")
     if warmup_autotune:
         if device is None:
             raise ValueError("You must specify a device when warmup_autotune is True.")

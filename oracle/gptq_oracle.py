@@ -358,3 +358,53 @@ def decode_attention_ref(q: np.ndarray, k_cache: np.ndarray, v_cache: np.ndarray
             w = np.exp(s - s.max())
             out[b, 0, h * hd:(h + 1) * hd] = (w / w.sum()) @ v
     return out
+
+
+# ---- streaming order of the packed words (the build's own load-time re-layout; no reference counterpart) ----------
+# Pinned by: stream_order_loops (the definition, word by word) == stream_order (index arithmetic) on small shapes;
+# unstream(stream_order(q)) == q; and the library's dequantisation FROM the streaming order must reproduce
+# dequant_fp16 bit for bit (tests/test_gpu_stream.py), which fails for any wrong index.
+def stream_order_loops(qweight: np.ndarray) -> np.ndarray:
+    """Definition, word by word: per strip of 16 columns and unit of 128 rows (16 packed rows) one block of 256 words;
+    lane l = 16 * r + c owns words 4 * l + j, j = 0..3: packed row unit * 16 + 4 * r + j, column strip * 16 + c."""
+    rows, n = qweight.shape
+    nb = rows // 16
+    out = np.empty(rows * n, dtype=qweight.dtype)
+    o = 0
+    for strip in range(n // 16):
+        for unit in range(nb):
+            for r in range(4):
+                for c in range(16):
+                    for j in range(4):
+                        out[o] = qweight[unit * 16 + 4 * r + j, strip * 16 + c]
+                        o += 1
+    return out.reshape(rows, n)
+
+
+def stream_order(qweight: np.ndarray, qzeros=None, scales=None):
+    """(sweight, smeta): the same permutation by index arithmetic, and the {scale, zero} words
+    smeta[(strip * G + g) * 16 + c] = fp16 bits of scales[g, 16 * strip + c] | stored zero << 16."""
+    rows, n = qweight.shape
+    nb = rows // 16
+    o = np.arange(rows * n, dtype=np.int64)
+    j, lane, blk = o & 3, (o >> 2) & 63, o >> 8
+    strip, unit = blk // nb, blk % nb
+    sw = qweight.reshape(-1)[(unit * 16 + 4 * (lane >> 4) + j) * n + strip * 16 + (lane & 15)].reshape(rows, n)
+    if scales is None:
+        return sw, None
+    g = scales.shape[0]
+    word = scales.view(np.uint16).astype(np.uint32) | (unpack_qzeros(qzeros).astype(np.uint32) << 16)   # [G, N]
+    meta = word.reshape(g, n // 16, 16).transpose(1, 0, 2).reshape(-1).view(np.int32)
+    return sw, meta
+
+
+def unstream(sweight: np.ndarray) -> np.ndarray:
+    """The inverse permutation."""
+    rows, n = sweight.shape
+    nb = rows // 16
+    o = np.arange(rows * n, dtype=np.int64)
+    j, lane, blk = o & 3, (o >> 2) & 63, o >> 8
+    strip, unit = blk // nb, blk % nb
+    out = np.empty(rows * n, dtype=sweight.dtype)
+    out[(unit * 16 + 4 * (lane >> 4) + j) * n + strip * 16 + (lane & 15)] = sweight.reshape(-1)
+    return out.reshape(rows, n)

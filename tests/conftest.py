@@ -51,3 +51,4 @@ def _automatic_launch_plans_after_every_test():
     lib.gptq4_set_gemm_tuning(0, 0)
     lib.gptq4_set_exchange_spin_limit(0)
     lib.gptq4_set_chain_tuning(0, 0, 0, -1)
+    lib.gptq4_set_stream_tuning(0, 0)

@@ -16,20 +16,22 @@ from gptq_triton_amd import _lib
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def declared_symbols():
-    text = open(os.path.join(ROOT, "include", "gptq4.h")).read()
+def declared_symbols(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(gptq4_[a-z0-9_]+)\s*\(", text)))
 
 
 def test_library_exports_every_declared_symbol():
     lib = _lib.load()
-    names = declared_symbols()
-    assert len(names) >= 10
-    for name in names:
-        assert hasattr(lib, name), f"{name} declared in include/gptq4.h but not exported"
-    assert set(names) == set(_lib.SIGNATURES), "ctypes binding and header disagree"
-    assert lib.gptq4_abi_version() == 2
+    stable, experimental = declared_symbols("gptq4.h"), declared_symbols("gptq4_experimental.h")
+    assert len(stable) >= 20
+    for name in stable + experimental:
+        assert hasattr(lib, name), f"{name} declared in include/ but not exported"
+    assert set(stable + experimental) == set(_lib.SIGNATURES), "ctypes binding and headers disagree"
+    # the stable header carries no tuning, probe or test hook
+    assert not [n for n in stable if "_set_" in n or "probe" in n or "chain" in n or "column_parts" in n]
+    assert lib.gptq4_abi_version() == 3
 
 
 def test_error_codes_are_returned_before_any_launch():
