@@ -1,20 +1,25 @@
 #!/usr/bin/env python3
 """Benchmark of the 4-bit GPTQ hot path on one MI355X.
 
-Workload (config.workload): one batch-1 decode token through the quantised linears of a
-LLaMA-7B-shape decoder - 32 layers x [fused QKV + rotary (4096 -> 12288), o_proj
-(4096 -> 4096), fused gate/up + SiLU*mul (4096 -> 2 x 11008), down_proj (11008 -> 4096)],
-4-bit, groupsize 128, every layer with its own synthetic weights (3.2 GB, so each
-launch streams its weights from HBM, not from the 256 MB Infinity Cache).  The 128
-launches of a step are captured once in a HIP graph and replayed; a "step" is one
-replay.  value = tokens/s = 1 / step time.  The attention core, norms and lm_head are
-not part of this path and are not in the step.
+Workload (config.workload): greedy decode of a random-init LLaMA-7B-shape decoder at batch 1
+behind a 2048-token prompt - 32 layers x [RMSNorm + fused QKV + rotary into the KV cache
+(4096 -> 12288), one-token attention over the cache, o_proj (4096 -> 4096), RMSNorm + fused
+gate/up + SiLU*mul (4096 -> 2 x 11008), down_proj (11008 -> 4096)], final norm, fp16 lm_head,
+argmax; 4-bit, groupsize 128, every layer with its own synthetic weights (3.2 GB, so each launch
+streams its weights from HBM, not from the 256 MB Infinity Cache), packed weights in streaming
+order (what the decode kernel reads).  The launches of a step are captured once in a HIP graph
+and replayed; a "step" is one replay = one token.  value = tokens/s = 1 / step time.
+
+`linears_only` (top level): the same step with nothing but its 128 quantised-linear launches - the
+hot path by itself, what `value` was in earlier builds.
 
 Also reported on the same line:
-  roofline      the dominant kernel (small-M gate/up GEMV, 46.9 MB per launch): its
-                average duration over back-to-back launches on distinct weights
+  roofline      the dominant kernel (gate/up GEMV on streaming-order weights, 46.9 MB per
+                launch): its average duration over back-to-back launches on distinct weights
                 (HIP events on the launch stream), as algorithmic bytes / time against
-                the 8 TB/s HBM peak
+                the 8 TB/s HBM peak; floor_us / frac_of_floor: the same bytes read by a plain
+                16-byte-per-lane kernel, launch included (the stand-alone floor probe, when it
+                is built); attention: the one-token attention kernel's own fraction
   cpu_baseline  the PyTorch CPU dequantise-then-fp32-matmul path (oracle/torch_cpu.py)
                 on the host cores for 1 of the 32 layers, extrapolated to a token
                 (+ step_frac: the weights of the whole 128-launch step over the step time;
@@ -34,6 +39,10 @@ Also reported on the same line:
                 M = 2048 shapes
   --chain-probe / --chain-timeline: the chained decode launch (gptq4_decode_chain) against the
                 separate launches it would replace
+  --floor-probe what a launch costs before it computes anything: empty launches and plain reads of
+                the four decode operators' bytes (csrc/probe/floor_probe, a stand-alone program),
+                then each decode operator's own access pattern with the arithmetic left out
+                (gptq4_stream_probe) beside the operator itself; prints text and one JSON line
 
 Other workloads (--workload llama7b | llama13b | llama30b): a full random-init decoder of
 that shape (embedding, RMSNorm, fused QKV + rotary into a preallocated KV cache, torch
@@ -80,9 +89,14 @@ DECODERS = {
 }
 
 
-def decoder_figures(workload, bsz, prompt, new):
+def decoder_figures(workload, bsz, prompt, new, steps=None, warmup=None):
     """Full-decoder workload: prefill + graph-replayed greedy decode on a random-init model.  Returns the result
-    record (the JSON line of `--workload llamaNNb`)."""
+    record (the JSON line of `--workload llamaNNb`).  steps / warmup: exactly that many timed / untimed graph replays
+    (new is then derived from them)."""
+    eager_steps = 8 if steps is None else 4
+    if steps is not None:
+        warmup = 0 if warmup is None else warmup
+        new = 1 + eager_steps + 2 + warmup + steps
     import gc
 
     import torch
@@ -159,14 +173,17 @@ def decoder_figures(workload, bsz, prompt, new):
     prefill_tf = 2.0 * bsz * prompt * per_token_kn / prefill_s / 1e12
     log(f"prefill: {prefill_s * 1e3:.1f} ms for {bsz} x {prompt} tokens = {prefill_tf:.0f} TFLOP/s in the quantised linears")
 
-    eager_steps = min(8, new - 1)
+    eager_steps = min(eager_steps, new - 1)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     generated = [first, dec.decode(eager_steps)]
     torch.cuda.synchronize()
     eager_s = (time.perf_counter() - t0) / max(eager_steps, 1)
     generated.append(dec.decode(2, use_graph=True))  # captures the step
-    steps = new - 1 - eager_steps - 2
+    if steps is None:
+        steps = new - 1 - eager_steps - 2
+    elif warmup:
+        generated.append(dec.decode(warmup, use_graph=True))
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     toks = dec.decode(steps, use_graph=True)
@@ -190,11 +207,12 @@ def decoder_figures(workload, bsz, prompt, new):
         f"{step_bytes / 1e9:.2f} GB per step -> {gbs:.0f} GB/s")
     result = {
         "metric": f"{workload}-shape 4-bit greedy decode tok/s (full decoder)", "value": round(bsz / step_s, 2),
-        "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": eager_steps + 2, "ms_per_step": round(step_s * 1e3, 4),
+        "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": eager_steps + 2 + (warmup or 0), "ms_per_step": round(step_s * 1e3, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp16", "data": "synthetic",
         "config": {"workload": f"random-init {workload}-shape decoder, batch {bsz}, {prompt}-token prompt prefill then "
                                f"{new} greedy tokens, 4-bit groupsize {groupsize}{' act-order' if act_order else ''}, "
-                               "fp16 lm_head, one HIP-graph replay per token",
+                               f"fp16 lm_head, one HIP-graph replay per token, packed weights in "
+                               f"{'streaming order' if bsz <= 4 else 'the checkpoint layout'}",
                    "layers": layers, "hidden": hidden, "intermediate": inter, "heads": heads, "batch": bsz,
                    "prompt": prompt, "new_tokens": new},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -215,6 +233,83 @@ def decoder_figures(workload, bsz, prompt, new):
 
 def run_decoder(args):
     print(json.dumps(decoder_figures(args.workload, args.batch, args.prompt, args.new_tokens)), flush=True)
+
+
+# HBM bytes one launch of the dominant kernel moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see roofline.traffic_source)
+TRAFFIC_GATEUP_STREAM = None
+
+FLOOR_BINARY = os.path.join(ROOT, "gptq-triton_amd", "csrc", "probe", "floor_probe")
+
+
+def run_floor_binary():
+    """Figures of the stand-alone floor probe (csrc/probe/floor_probe.hip) as {name: value}, or None when it is not built.
+    Runs as a child process, before this process has many launches in flight; about ten seconds."""
+    import subprocess
+    if not os.path.exists(FLOOR_BINARY):
+        log("floor probe not built (python gptq-triton_amd/build.py builds it): no floor figures")
+        return None
+    try:
+        out = subprocess.run([FLOOR_BINARY], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120).stdout
+    except Exception as e:
+        log(f"floor probe failed: {e!r}")
+        return None
+    figures = {}
+    for line in out.splitlines():
+        parts = line.split()
+        if len(parts) == 3:
+            try:
+                figures[parts[0]] = float(parts[1])
+            except ValueError:
+                pass
+    return figures or None
+
+
+def floor_probe(args, layers, x1, dev, capture, time_graph, s_o_op, s_gateup_op, s_down_op, s_qkv_op, pos1):
+    """`--floor-probe`: per decode operator of the 7B shape, at one row and with the weights coming from HBM - the launch
+    floor, a plain read of the operator's bytes, the operator's own access pattern with the arithmetic left out, the
+    operator.  Text on stderr, one JSON line on stdout."""
+    import torch
+
+    import gptq_triton_amd as G
+    from gptq_triton_amd import _lib
+
+    lib = _lib.load()
+    figures = run_floor_binary() or {}
+    for k, v in figures.items():
+        log(f"  {k:44s} {v:10.3f}")
+    ws = _lib.workspace(dev, _lib.WS_HEAD_BYTES)
+    h1 = torch.randn((1, INTER), device=dev).half()
+    x = x1.view(1, HIDDEN)
+    y = torch.empty((1, max(INTER, 3 * HIDDEN)), device=dev).half()
+
+    def pattern(op, xin, k, n, a, b=None):
+        def run():
+            st = _lib.current_stream(dev)
+            for L in layers:
+                (sw, mt), up = L[a], (L[b] if b else (None, None))
+                rc = lib.gptq4_stream_probe(op, xin.data_ptr(), sw.data_ptr(), mt.data_ptr(), _lib.ptr(up[0]), _lib.ptr(up[1]), y.data_ptr(),
+                                            1, k, n, GROUPSIZE, ws.data_ptr(), ws.numel(), st)
+                _lib.check(rc, "gptq4_stream_probe")
+        return run
+
+    rows = {}
+    plain = {"o_proj": "plain_read_8.7MB", "down_proj": "plain_read_23.4MB", "qkv+rotary": "plain_read_26.1MB", "gate/up+silu*mul": "plain_read_46.9MB"}
+    ops = {"o_proj": (lambda: [s_o_op(x, L) for L in layers], pattern(0, x, HIDDEN, HIDDEN, "s_o")),
+           "down_proj": (lambda: [s_down_op(h1, L) for L in layers], pattern(0, h1, INTER, HIDDEN, "s_down")),
+           # (the rotary epilogue has no variant without arithmetic: the plain projection's pattern on the same bytes stands in)
+           "qkv+rotary": (lambda: [s_qkv_op(x1, L, pos1) for L in layers], pattern(0, x, HIDDEN, 3 * HIDDEN, "s_qkv")),
+           "gate/up+silu*mul": (lambda: [s_gateup_op(x, L) for L in layers], pattern(1, x, HIDDEN, INTER, "s_gate", "s_up"))}
+    log(f"  {'operator (M = 1, 7B shape, weights from HBM)':46s} {'launch floor':>12s} {'plain read':>11s} {'pattern only':>13s} {'operator':>9s}   us")
+    for name, (full, loads_only) in ops.items():
+        g1, _ = capture(full)
+        g2, _ = capture(loads_only)
+        t_full = statistics.median(time_graph(g1, 10)) * 1e3 / LAYERS
+        t_loads = statistics.median(time_graph(g2, 10)) * 1e3 / LAYERS
+        del g1, g2
+        rows[name] = {"operator_us": round(t_full, 2), "access_pattern_without_arithmetic_us": round(t_loads, 2),
+                      "plain_read_us": figures.get(plain[name]), "launch_floor_us": figures.get("launch_floor_1wg_per_cu_512t_81k")}
+        log(f"  {name:46s} {rows[name]['launch_floor_us'] or float('nan'):12.2f} {rows[name]['plain_read_us'] or float('nan'):11.2f} {t_loads:13.2f} {t_full:9.2f}")
+    print(json.dumps({"floor_probe": rows, "device_figures": figures}), flush=True)
 
 
 def chain_probe(args):
@@ -334,6 +429,9 @@ def main():
     ap.add_argument("--traffic-probe", action="store_true",
                     help="for rocprofv3 --pmc runs: a 256 MiB device copy (calibration) followed by plain launches of "
                          "each decode operator on distinct weights; prints no JSON")
+    ap.add_argument("--floor-probe", action="store_true",
+                    help="launch floor, plain reads and each decode operator's access pattern without its arithmetic beside the "
+                         "operator itself (7B shapes, one row); prints text and one JSON line")
     ap.add_argument("--chain-probe", action="store_true",
                     help="time gptq4_decode_chain against the separate launches (7B shapes, --batch rows); prints text, no JSON")
     ap.add_argument("--chain-timeline", action="store_true",
@@ -377,7 +475,24 @@ def main():
     log("building 32 layers of synthetic 4-bit weights ...")
     layers = [dict(qkv=make(HIDDEN, 3 * HIDDEN), o=make(HIDDEN, HIDDEN), gate=make(HIDDEN, INTER),
                    up=make(HIDDEN, INTER), down=make(INTER, HIDDEN)) for _ in range(LAYERS)]
+    # the same weights in streaming order, the resident layout of a model that decodes up to four sequences
+    for L in layers:
+        for name in ("qkv", "o", "gate", "up", "down"):
+            qw, qz, sc = L[name]
+            L["s_" + name] = G.stream_pack(qw, qz, sc, GROUPSIZE)
     cos, sin = G.RotaryTable(128, 2048).get(dev, 2048)
+
+    def s_qkv_op(x, L, pos):
+        return G.qkv_rotary_stream(GROUPSIZE, x, *L["s_qkv"], pos, cos, sin, HEADS)
+
+    def s_o_op(x, L):
+        return G.matmul4_stream(GROUPSIZE, x, *L["s_o"])
+
+    def s_gateup_op(x, L):
+        return G.llama_mlp_4_stream(GROUPSIZE, x, *L["s_gate"], *L["s_up"])
+
+    def s_down_op(h, L):
+        return G.matmul4_stream(GROUPSIZE, h, *L["s_down"])
 
     def qkv_op(x, L, pos):
         qw, qz, sc = L["qkv"]
@@ -443,17 +558,27 @@ def main():
         hs = [gateup_op(x1, L) for L in layers]
         for h, L in zip(hs, layers):
             down_op(h, L)
+        for L in layers:
+            s_qkv_op(x1, L, pos1)
+        for L in layers:
+            s_o_op(x1, L)
+        hs = [s_gateup_op(x1, L) for L in layers]
+        for h, L in zip(hs, layers):
+            s_down_op(h, L)
         torch.cuda.synchronize()
         log("traffic probe done")
         return
 
+    if args.floor_probe:
+        return floor_probe(args, layers, x1, dev, capture, time_graph, s_o_op, s_gateup_op, s_down_op, s_qkv_op, pos1)
+
     def decode_step():
         outs = []
         for L in layers:
-            q, k, v = qkv_op(x1, L, pos1)
-            o = o_op(x1, L)
-            h = gateup_op(x1, L)
-            y = down_op(h, L)
+            q, k, v = s_qkv_op(x1, L, pos1)
+            o = s_o_op(x1.view(1, HIDDEN), L)
+            h = s_gateup_op(x1.view(1, HIDDEN), L)
+            y = s_down_op(h, L)
             outs.append((q, k, v, o, y))
         return outs
 
@@ -472,28 +597,36 @@ def main():
     tok_s = 1000.0 / ms_per_step
     layer_bytes = (weight_bytes(HIDDEN, 3 * HIDDEN, GROUPSIZE) + weight_bytes(HIDDEN, HIDDEN, GROUPSIZE)
                    + 2 * weight_bytes(HIDDEN, INTER, GROUPSIZE) + weight_bytes(INTER, HIDDEN, GROUPSIZE))
-    log(f"decode step: {ms_per_step * 1e3:.1f} us -> {tok_s:.1f} tok/s "
+    log(f"decode step, quantised linears only: {ms_per_step * 1e3:.1f} us -> {tok_s:.1f} tok/s "
         f"({LAYERS * layer_bytes / ms_per_step / 1e6:.0f} GB/s of weights over the whole step)")
 
     # ----------------------------------------------- roofline of the dominant kernel
     def gateup_all():
-        return [gateup_op(x1, L) for L in layers]
+        return [s_gateup_op(x1.view(1, HIDDEN), L) for L in layers]
 
     gu_graph, _ = capture(gateup_all)
     gu_ms = time_graph(gu_graph, reps=max(10, args.steps // 2))
     gu_us = statistics.median(gu_ms) * 1e3 / LAYERS
+    # algorithmic bytes of one launch = one unit of work: the two projections' packed words, zeros and scales as the
+    # checkpoint holds them, the input row and the output row
     gu_bytes = 2 * weight_bytes(HIDDEN, INTER, GROUPSIZE) + HIDDEN * 2 + INTER * 2
     gu_gbs = gu_bytes / gu_us / 1e3
+    floor = run_floor_binary()
     roofline = {"bound": "hbm", "achieved": round(gu_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(gu_gbs / HBM_PEAK_GBS, 4),
                 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-                # `bench.py --traffic-probe`, scaled by a 256 MiB copy (x2.000 / x1.000)
-                "traffic": 51_322_000 + 3_561_000,
-                "traffic_source": "constant: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this kernel, profiles/decode_gemv_llama7b_m1.md",
+                # `bench.py --traffic-probe`, scaled by a 256 MiB copy
+                "traffic": TRAFFIC_GATEUP_STREAM,
+                "traffic_source": "constant: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this kernel, profiles/decode_stream_llama7b_m1.md",
                 "step_frac": round(LAYERS * layer_bytes / ms_per_step / 1e6 / HBM_PEAK_GBS, 4),
                 "step_GBps": round(LAYERS * layer_bytes / ms_per_step / 1e6, 1),
-                "kernel": "gptq4_gemv_kernel<SILU_MUL> (gate/up GEMV, M=1, K=4096, I=11008, g=128)",
+                "kernel": "gptq4_stream_kernel<SILU_MUL> (gate/up GEMV on streaming-order weights, M=1, K=4096, I=11008, g=128)",
                 "bytes_per_launch": gu_bytes, "avg_launch_us": round(gu_us, 2)}
+    if floor and "plain_read_46.9MB" in floor:
+        # what ANY launch pays to read these bytes: the launch floor plus a plain 16-byte-per-lane read of 46.9 MB from HBM
+        roofline["floor_us"] = floor["plain_read_46.9MB"]
+        roofline["frac_of_floor"] = round(floor["plain_read_46.9MB"] / gu_us, 4)
+        roofline["launch_floor_us"] = floor.get("launch_floor_1wg_per_cu_512t_81k")
     log(f"gate/up GEMV: {gu_us:.2f} us/launch, {gu_gbs:.0f} GB/s = {100 * gu_gbs / HBM_PEAK_GBS:.1f}% of HBM peak")
 
     # --------------------------------------------------------------------------- extras
@@ -510,10 +643,39 @@ def main():
         wq, wo, wg, wd = (weight_bytes(HIDDEN, 3 * HIDDEN, GROUPSIZE), weight_bytes(HIDDEN, HIDDEN, GROUPSIZE),
                           weight_bytes(HIDDEN, INTER, GROUPSIZE), weight_bytes(INTER, HIDDEN, GROUPSIZE))
         h1 = torch.randn((1, INTER), device=dev, generator=gen).half()
-        per_op("decode M=1 qkv+rotary", lambda L: qkv_op(x1, L, pos1), wq + 2 * HIDDEN + 6 * HIDDEN, 2 * HIDDEN * 3 * HIDDEN)
-        per_op("decode M=1 o_proj", lambda L: o_op(x1, L), wo + 4 * HIDDEN, 2 * HIDDEN * HIDDEN)
-        per_op("decode M=1 gate/up+silu*mul", lambda L: gateup_op(x1, L), gu_bytes, 4 * HIDDEN * INTER)
-        per_op("decode M=1 down_proj", lambda L: down_op(h1, L), wd + 2 * INTER + 2 * HIDDEN, 2 * HIDDEN * INTER)
+        x1f = x1.view(1, HIDDEN)
+        per_op("decode M=1 qkv+rotary", lambda L: s_qkv_op(x1, L, pos1), wq + 2 * HIDDEN + 6 * HIDDEN, 2 * HIDDEN * 3 * HIDDEN)
+        per_op("decode M=1 o_proj", lambda L: s_o_op(x1f, L), wo + 4 * HIDDEN, 2 * HIDDEN * HIDDEN)
+        per_op("decode M=1 gate/up+silu*mul", lambda L: s_gateup_op(x1f, L), gu_bytes, 4 * HIDDEN * INTER)
+        per_op("decode M=1 down_proj", lambda L: s_down_op(h1, L), wd + 2 * INTER + 2 * HIDDEN, 2 * HIDDEN * INTER)
+        for mm in (2, 4):
+            xm = torch.randn((mm, 1, HIDDEN), device=dev, generator=gen).half()
+            hm = torch.randn((mm, INTER), device=dev, generator=gen).half()
+            posm = torch.full((mm, 1), 2047, device=dev, dtype=torch.int32)
+            per_op(f"decode M={mm} qkv+rotary", lambda L: s_qkv_op(xm, L, posm), wq + 8 * mm * HIDDEN, 2 * mm * HIDDEN * 3 * HIDDEN)
+            per_op(f"decode M={mm} o_proj", lambda L: s_o_op(xm.view(mm, HIDDEN), L), wo + 4 * mm * HIDDEN, 2 * mm * HIDDEN * HIDDEN)
+            per_op(f"decode M={mm} gate/up+silu*mul", lambda L: s_gateup_op(xm.view(mm, HIDDEN), L), 2 * wg + 2 * mm * (HIDDEN + INTER), 4 * mm * HIDDEN * INTER)
+            per_op(f"decode M={mm} down_proj", lambda L: s_down_op(hm, L), wd + 2 * mm * (INTER + HIDDEN), 2 * mm * HIDDEN * INTER)
+        # the kernels for the checkpoint layout on the same shapes (what a model kept in that layout runs at one row)
+        per_op("checkpoint layout M=1 qkv+rotary", lambda L: qkv_op(x1, L, pos1), wq + 2 * HIDDEN + 6 * HIDDEN, 2 * HIDDEN * 3 * HIDDEN)
+        per_op("checkpoint layout M=1 o_proj", lambda L: o_op(x1, L), wo + 4 * HIDDEN, 2 * HIDDEN * HIDDEN)
+        per_op("checkpoint layout M=1 gate/up+silu*mul", lambda L: gateup_op(x1, L), gu_bytes, 4 * HIDDEN * INTER)
+        per_op("checkpoint layout M=1 down_proj", lambda L: down_op(h1, L), wd + 2 * INTER + 2 * HIDDEN, 2 * HIDDEN * INTER)
+        # one-token attention over a 2048-row cache: 32 caches of 33.5 MB, one per layer, so that every launch reads HBM
+        from gptq_triton_amd.decoder_ops import decode_attention
+        caches = [(torch.randn((1, HEADS, 2048, 128), device=dev, generator=gen).half(), torch.randn((1, HEADS, 2048, 128), device=dev, generator=gen).half())
+                  for _ in range(LAYERS)]
+        qa = torch.randn((1, HEADS, 1, 128), device=dev, generator=gen).half()
+        pa = torch.tensor([2047], device=dev, dtype=torch.int32)
+        att_bytes = 2 * HEADS * 2048 * 128 * 2 + 4 * HEADS * 128
+        ga, _ = capture(lambda: [decode_attention(qa, kc, vc, pa) for kc, vc in caches])
+        att_us = statistics.median(time_graph(ga, 10)) * 1e3 / LAYERS
+        del ga, caches
+        extra["decode attention, 2048 cached tokens"] = {"us": round(att_us, 2), "GBps": round(att_bytes / att_us / 1e3, 1)}
+        roofline["attention"] = {"kernel": "gptq4_decode_attention (32 heads x 128, 2048 cached tokens, one query token)",
+                                 "bytes_per_launch": att_bytes, "avg_launch_us": round(att_us, 2),
+                                 "frac": round(att_bytes / att_us / 1e3 / HBM_PEAK_GBS, 4)}
+        log(f"  {'decode attention, 2048 tokens':34s} {att_us:9.2f} us  {att_bytes / att_us / 1e3:8.0f} GB/s")
         # "hot": the same launches on ONE layer's weights over and over, so that they come out of the
         # 256 MB Infinity Cache instead of HBM.  Not an HBM figure; it shows what the memory side costs.
         def per_op_hot(name, fn, nbytes, flops, reps=10):
@@ -522,10 +684,10 @@ def main():
             extra[name] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1), "TFLOPs": round(flops / us / 1e6, 2)}
             log(f"  {name:34s} {us:9.2f} us  {nbytes / us / 1e3:8.0f} GB/s  {flops / us / 1e6:8.1f} TFLOP/s")
             del g
-        per_op_hot("hot M=1 qkv+rotary", lambda L: qkv_op(x1, L, pos1), wq + 2 * HIDDEN + 6 * HIDDEN, 2 * HIDDEN * 3 * HIDDEN)
-        per_op_hot("hot M=1 o_proj", lambda L: o_op(x1, L), wo + 4 * HIDDEN, 2 * HIDDEN * HIDDEN)
-        per_op_hot("hot M=1 gate/up+silu*mul", lambda L: gateup_op(x1, L), gu_bytes, 4 * HIDDEN * INTER)
-        per_op_hot("hot M=1 down_proj", lambda L: down_op(h1, L), wd + 2 * INTER + 2 * HIDDEN, 2 * HIDDEN * INTER)
+        per_op_hot("hot M=1 qkv+rotary", lambda L: s_qkv_op(x1, L, pos1), wq + 2 * HIDDEN + 6 * HIDDEN, 2 * HIDDEN * 3 * HIDDEN)
+        per_op_hot("hot M=1 o_proj", lambda L: s_o_op(x1f, L), wo + 4 * HIDDEN, 2 * HIDDEN * HIDDEN)
+        per_op_hot("hot M=1 gate/up+silu*mul", lambda L: s_gateup_op(x1f, L), gu_bytes, 4 * HIDDEN * INTER)
+        per_op_hot("hot M=1 down_proj", lambda L: s_down_op(h1, L), wd + 2 * INTER + 2 * HIDDEN, 2 * HIDDEN * INTER)
         for m in (16, 64, 128, 256, 512, 2048, 8192):
             xm = torch.randn((1, m, HIDDEN), device=dev, generator=gen).half()
             hm = torch.randn((m, INTER), device=dev, generator=gen).half()
@@ -562,12 +724,19 @@ def main():
             xm = torch.randn((m, HIDDEN), device=dev, generator=gen).half()
             config_row("C1", "QuantLinear 4096x4096 g=-1", m, lambda w: G.matmul4(HIDDEN, xm, w[0], w[2], w[1]), c1,
                        w1 + 4 * m * HIDDEN, 2 * m * HIDDEN * HIDDEN)
-        del c1
+        c1s = [G.stream_pack(w[0], w[1], w[2], HIDDEN) for w in c1]
+        xm = torch.randn((1, HIDDEN), device=dev, generator=gen).half()
+        config_row("C1", "QuantLinear 4096x4096 g=-1, streaming order", 1, lambda w: G.matmul4_stream(HIDDEN, xm, w[0], w[1]), c1s,
+                   w1 + 4 * HIDDEN, 2 * HIDDEN * HIDDEN)
+        del c1, c1s
         # C2: the fused MLP module, gate/up + SiLU*mul then down, groupsize 128, M in {1, 16, 512}
         for m in (1, 16, 512):
             xm = torch.randn((m, HIDDEN), device=dev, generator=gen).half()
             config_row("C2", "MLP gate/up+silu*mul, down g=128", m, lambda L: down_op(gateup_op(xm, L), L), layers,
                        2 * wg + wd + 4 * m * HIDDEN + 4 * m * INTER, 6 * m * HIDDEN * INTER, reps=5)
+        xm = torch.randn((1, HIDDEN), device=dev, generator=gen).half()
+        config_row("C2", "MLP gate/up+silu*mul, down g=128, streaming order", 1, lambda L: s_down_op(s_gateup_op(xm, L), L), layers,
+                   2 * wg + wd + 4 * HIDDEN + 4 * INTER, 6 * HIDDEN * INTER, reps=5)
         # C3: fused QKV + rotary 4096 -> 12288, one group, M = 1 at position 2047 and a 2048-token prefill
         c3 = [make(HIDDEN, 3 * HIDDEN, -1) for _ in range(12)]
         w3 = weight_bytes(HIDDEN, 3 * HIDDEN, HIDDEN)
@@ -575,6 +744,10 @@ def main():
         x1r = torch.randn((1, 1, HIDDEN), device=dev, generator=gen).half()
         config_row("C3", "QKV+rotary 4096x12288 g=-1", 1, lambda w: G.qkv_rotary(HIDDEN, x1r, w[0], w[2], w[1], pos2047, cos, sin, HEADS), c3,
                    w3 + 2 * HIDDEN + 6 * HIDDEN, 2 * HIDDEN * 3 * HIDDEN)
+        c3s = [G.stream_pack(w[0], w[1], w[2], HIDDEN) for w in c3]
+        config_row("C3", "QKV+rotary 4096x12288 g=-1, streaming order", 1, lambda w: G.qkv_rotary_stream(HIDDEN, x1r, w[0], w[1], pos2047, cos, sin, HEADS), c3s,
+                   w3 + 2 * HIDDEN + 6 * HIDDEN, 2 * HIDDEN * 3 * HIDDEN)
+        del c3s
         xp = torch.randn((1, 2048, HIDDEN), device=dev, generator=gen).half()
         posp = torch.arange(2048, device=dev, dtype=torch.int32).unsqueeze(0)
         config_row("C3", "QKV+rotary 4096x12288 g=-1", 2048, lambda w: G.qkv_rotary(HIDDEN, xp, w[0], w[2], w[1], posp, cos, sin, HEADS), c3[:4],
@@ -622,15 +795,21 @@ def main():
         extra["prefill_best_TFLOPs"] = best_prefill
         extra["prefill_frac_of_fp16_mfma_peak"] = round(best_prefill / MFMA_FP16_PEAK_TFLOPS, 4)
 
-    L0 = None if args.no_cpu else {k: tuple(t.cpu() for t in v) for k, v in layers[0].items()}
-    # ------------------------------------------------- C4 / C5: the full decoders (prefill + greedy decode)
+    L0 = None if args.no_cpu else {k: tuple(t.cpu() for t in v) for k, v in layers[0].items() if not k.startswith("s_")}
+    # ------------------------------------------------- the headline: the whole 7B decoder, then C4 / C5 (prefill + greedy decode)
+    del layers, step_graph, gu_graph
+    import gc
+    gc.collect()
+    torch.cuda.empty_cache()
+    head = decoder_figures("llama7b", 1, 2048, None, steps=args.steps, warmup=args.warmup)
+    extra["llama7b_b1"] = {"prefill_ms": head["extra"]["prefill_ms"], "prefill_linear_TFLOPs": head["extra"]["prefill_linear_TFLOPs"],
+                           "eager_decode_ms_per_step": head["extra"]["eager_decode_ms_per_step"],
+                           "step_GBps": head["roofline"]["achieved"], "step_frac_hbm": head["roofline"]["frac"],
+                           "prefill_path_agrees_with_decode_path_on_next_tokens":
+                               head["extra"]["prefill_path_agrees_with_decode_path_on_next_tokens"]}
     if not args.no_extra and not args.no_decoders:
-        del layers, step_graph, gu_graph
-        import gc
-        gc.collect()
-        torch.cuda.empty_cache()
         decs = {}
-        for name, bsz in (("llama7b", 1), ("llama13b", 1), ("llama30b", 1), ("llama30b", 8)):
+        for name, bsz in (("llama13b", 1), ("llama30b", 1), ("llama30b", 8)):
             try:
                 r = decoder_figures(name, bsz, 2048, 128 if name != "llama30b" else 256)
             except Exception as e:  # report, do not lose the line
@@ -695,15 +874,19 @@ def main():
                         "quantlinear_4096x4096": c1}
         log(f"cpu baseline: {t_layer:.3f} s per layer dequantise + matmul, {t_mm:.4f} s matmul alone, on {torch.get_num_threads()} threads")
 
+    roofline["decoder_step_frac"] = head["roofline"]["frac"]
+    roofline["decoder_step_GBps"] = head["roofline"]["achieved"]
     result = {
-        "metric": "LLaMA-7B-shape 4-bit decode tok/s", "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
+        "metric": "LLaMA-7B-shape 4-bit decode tok/s", "value": head["value"], "unit": "tok/s", "n_gpus": 1,
+        "steps": head["steps"], "warmup": head["warmup"], "ms_per_step": head["ms_per_step"], "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "fp16", "data": "synthetic",
-        "config": {"workload": "llama7b-shape decode, batch 1, position 2047: 32 layers x [fused qkv+rotary, o_proj, "
-                               "fused gate/up+silu*mul, down_proj], 4-bit, groupsize 128, distinct weights per layer, "
-                               "one HIP-graph replay per token (quantised-linear hot path only)",
-                   "hidden": HIDDEN, "intermediate": INTER, "layers": LAYERS, "groupsize": GROUPSIZE,
-                   "weight_bytes_per_token": LAYERS * layer_bytes},
+        "config": {"workload": head["config"]["workload"], "hidden": HIDDEN, "intermediate": INTER, "layers": LAYERS,
+                   "groupsize": GROUPSIZE, "weight_bytes_per_token": LAYERS * layer_bytes,
+                   "bytes_per_token": head["roofline"]["bytes_per_launch"]},
+        # the step with nothing but its 128 quantised-linear launches (no attention, norms, lm_head): the hot path alone
+        "linears_only": {"tok_s": round(tok_s, 2), "ms_per_step": round(ms_per_step, 5), "steps": args.steps, "warmup": args.warmup,
+                         "workload": "32 layers x [fused qkv+rotary, o_proj, fused gate/up+silu*mul, down_proj] at batch 1, position 2047, "
+                                     "streaming-order weights, one HIP-graph replay per token"},
         "roofline": roofline, "cpu_baseline": cpu_baseline, "extra": extra,
     }
     print(json.dumps(result))
