@@ -434,13 +434,21 @@ __global__ __launch_bounds__(256) void gptq4_stream_pack_kernel(const uint32_t *
     sw[o] = qweight[(size_t)kb * N + n];
 }
 
+// (on the path of every call with more rows than the streaming-order kernel takes, so written for whole lines both
+// ways: a wave moves the packed rows 4 * r .. 4 * r + 3 of one unit for 64 columns - it reads one 16-byte chunk per lane,
+// 256 contiguous bytes per strip, and writes 256 contiguous bytes of each of the four rows)
 __global__ __launch_bounds__(256) void gptq4_stream_unpack_kernel(const uint32_t *__restrict__ sw, uint32_t *__restrict__ qweight,
                                                                   int K, int N) {
-    const size_t o = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (o >= (size_t)(K >> 3) * N) return;
-    int kb, n;
-    stream_coords(o, K >> 7, kb, n);
-    qweight[(size_t)kb * N + n] = sw[o];
+    const int nb = K >> 7;
+    const int r = threadIdx.x >> 6, cc = threadIdx.x & 63;
+    const int col = blockIdx.x * 64 + cc;  // N % 64 == 0
+    const int unit = blockIdx.y;
+    const uint4 w = reinterpret_cast<const uint4 *>(sw)[((size_t)(col >> 4) * nb + unit) * 64 + r * 16 + (col & 15)];
+    uint32_t *dst = qweight + (size_t)(unit * 16 + 4 * r) * N + col;
+    dst[0] = w.x;
+    dst[(size_t)N] = w.y;
+    dst[2 * (size_t)N] = w.z;
+    dst[3 * (size_t)N] = w.w;
 }
 
 // meta[(strip * G + g) * 16 + c] = scale bits | stored zero << 16 of column 16 * strip + c in group g
@@ -613,7 +621,8 @@ int launch_stream_pack(const uint32_t *qweight, const uint32_t *qzeros, const ha
 int launch_stream_unpack(const uint32_t *sw, const uint32_t *meta, uint32_t *qweight, uint32_t *qzeros, half_t *scales, int K, int N,
                          int groupsize, hipStream_t stream) {
     const size_t words = (size_t)(K >> 3) * N;
-    hipLaunchKernelGGL(gptq4_stream_unpack_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream, sw, qweight, K, N);
+    (void)words;
+    hipLaunchKernelGGL(gptq4_stream_unpack_kernel, dim3((unsigned)(N / 64), (unsigned)(K / 128)), dim3(256), 0, stream, sw, qweight, K, N);
     if (meta != nullptr) {
         const int G = K / groupsize;
         const size_t zwords = (size_t)G * (N >> 3);

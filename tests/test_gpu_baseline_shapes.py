@@ -269,6 +269,86 @@ def test_30b_qkv_rotary(b, s, pos0):
         assert_close(got[:, :, rows].cpu().numpy(), ref, f"30B qkv {name} b={b} s={s}")
 
 
+# ------------------------------------------- workload 4 at its full batch: 8 sequences x 2048 tokens = 16384 rows
+# The largest call any benchmark workload makes: 128 row tiles x 70 - 78 column panels of the tiled kernel, its banded
+# tile order and the panels cut along K.  The oracle is evaluated on a sample of rows (first, last, tile boundaries,
+# seeded); the rest is covered by the row-permutation property (bit-equal) and by one-hot rows (exact weight rows).
+BIG = 16384
+
+
+def big_rows(m, seed):
+    fixed = [0, 1, 127, 128, 129, 1023, 1024, 2047, 2048, 8191, 8192, m - 129, m - 128, m - 2, m - 1]
+    return np.unique(np.concatenate([np.array(fixed), np.random.default_rng(seed).choice(m, size=12, replace=False)]))
+
+
+@pytest.mark.parametrize("k,n", [(6656, 6656), (17920, 6656)])
+def test_30b_linear_at_16384_rows(k, n):
+    g = 512
+    L, W = layer_and_weights(k, n, g, 1400 + k // 128)
+    D = to_dev(L)
+    x = O.make_x(BIG, k, seed=1450)
+    x[5] = 0
+    x[5, 4321] = 1.0          # a one-hot row: the result is row 4321 of the weight, exactly
+    xd = torch.from_numpy(x).cuda()
+    y = gptq().matmul4(g, xd, D["qweight"], D["scales"], D["qzeros"])
+    rows = big_rows(BIG, seed=n)
+    assert_close(y[rows].cpu().numpy(), O.matmul_ref(x[rows], W), f"30B K={k} N={n} M={BIG}")
+    assert (bits(y[5].cpu().numpy()) == bits(W[4321])).all()
+    p = torch.from_numpy(np.random.default_rng(11).permutation(BIG)).cuda()
+    assert torch.equal(gptq().matmul4(g, xd[p], D["qweight"], D["scales"], D["qzeros"]), y[p])
+
+
+def test_30b_mlp_gateup_at_16384_rows():
+    k, n, g = 6656, 17920, 512
+    (gate, Wg), (up, Wu) = layer_and_weights(k, n, g, 1410), layer_and_weights(k, n, g, 1411)
+    Dg, Du = to_dev(gate), to_dev(up)
+    x = O.make_x(BIG, k, seed=1451)
+    xd = torch.from_numpy(x).cuda()
+    args = (Dg["qweight"], Dg["scales"], Dg["qzeros"], Du["qweight"], Du["scales"], Du["qzeros"])
+    h = gptq().llama_mlp_4(g, xd, *args)
+    rows = big_rows(BIG, seed=3)
+    ref = O.silu_mul_ref(O.matmul_ref(x[rows], Wg), O.matmul_ref(x[rows], Wu))
+    assert_close(h[rows].cpu().numpy(), ref, f"30B gate/up M={BIG}")
+    p = torch.from_numpy(np.random.default_rng(12).permutation(BIG)).cuda()
+    assert torch.equal(gptq().llama_mlp_4(g, xd[p], *args), h[p])
+
+
+def test_30b_qkv_rotary_at_8_sequences_of_2048_tokens():
+    hidden, H, Dh, g, b, s = 6656, 52, 128, 512, 8, 2048
+    L = O.make_layer(hidden, 3 * hidden, g, seed=1420)
+    D = to_dev(L)
+    G = gptq()
+    cos, sin = G.RotaryTable(Dh, 2304).get(torch.device("cuda"), 2304)
+    x = O.make_x(b * s, hidden, seed=1452).reshape(b, s, hidden)
+    pos = np.arange(s, dtype=np.int64)[None, :].repeat(b, 0) + np.arange(b)[:, None]
+    xd, posd = torch.from_numpy(x).cuda(), torch.from_numpy(pos).cuda()
+    q, k, v = G.qkv_rotary(g, xd, D["qweight"], D["scales"], D["qzeros"], posd, cos, sin, H, Dh)
+    rows = np.array([0, 1, 127, 128, 1023, 1024, 2046, 2047])
+    qr, kr, vr = O.qkv_rotary_ref(x[:, rows], L["qweight"], L["qzeros"], L["scales"], g, pos[:, rows], H, Dh, max_pos=2304)
+    for got, ref, name in ((q, qr, "q"), (k, kr, "k"), (v, vr, "v")):
+        assert got.shape == (b, H, s, Dh)
+        assert_close(got[:, :, rows].cpu().numpy(), ref, f"30B qkv {name} b={b} s={s}")
+    # the sequences in another order (positions go with them): the same bits, sequence by sequence
+    p = torch.tensor([3, 0, 7, 1, 6, 2, 5, 4], device="cuda")
+    q2, k2, v2 = G.qkv_rotary(g, xd[p].contiguous(), D["qweight"], D["scales"], D["qzeros"], posd[p].contiguous(), cos, sin, H, Dh)
+    assert torch.equal(q2, q[p]) and torch.equal(k2, k[p]) and torch.equal(v2, v[p])
+
+
+def test_7b_gate_up_at_8192_rows():
+    k, n, g, m = 4096, 11008, 128, 8192
+    (gate, Wg), (up, Wu) = layer_and_weights(k, n, g, 1460), layer_and_weights(k, n, g, 1461)
+    Dg, Du = to_dev(gate), to_dev(up)
+    x = O.make_x(m, k, seed=1462)
+    xd = torch.from_numpy(x).cuda()
+    args = (Dg["qweight"], Dg["scales"], Dg["qzeros"], Du["qweight"], Du["scales"], Du["qzeros"])
+    h = gptq().llama_mlp_4(g, xd, *args)
+    rows = big_rows(m, seed=4)
+    ref = O.silu_mul_ref(O.matmul_ref(x[rows], Wg), O.matmul_ref(x[rows], Wu))
+    assert_close(h[rows].cpu().numpy(), ref, f"7B gate/up M={m}")
+    p = torch.from_numpy(np.random.default_rng(13).permutation(m)).cuda()
+    assert torch.equal(gptq().llama_mlp_4(g, xd[p], *args), h[p])
+
+
 # ------------------------------------------------------------- size-independent: one-hot rows
 def test_one_hot_rows_at_full_size():
     """2048 one-hot rows through the 7B down_proj shape: every output row equals the
