@@ -24,7 +24,7 @@ Also reported on the same line:
                 on the host cores for 1 of the 32 layers, extrapolated to a token
                 (+ step_frac: the weights of the whole 128-launch step over the step time;
                 traffic: HBM bytes per launch from rocprofv3 counters, a constant taken from
-                profiles/decode_gemv_llama7b_m1.md, see traffic_source)
+                profiles/decode_stream_llama7b_m1.md, see traffic_source)
   extra         baseline_configs: one row per configuration of BASELINE.json that fits this
                 path - C1 QuantLinear 4096 x 4096 (one group) at M = 1 and 128, C2 the fused
                 MLP (gate/up + SiLU*mul, then down; groupsize 128) at M = 1, 16 and 512, C3
@@ -236,7 +236,7 @@ def run_decoder(args):
 
 
 # HBM bytes one launch of the dominant kernel moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see roofline.traffic_source)
-TRAFFIC_GATEUP_STREAM = None
+TRAFFIC_GATEUP_STREAM = 48316000  # 48.17 MB fetched + 0.14 MB written
 
 FLOOR_BINARY = os.path.join(ROOT, "gptq-triton_amd", "csrc", "probe", "floor_probe")
 
@@ -261,6 +261,8 @@ def run_floor_binary():
                 figures[parts[0]] = float(parts[1])
             except ValueError:
                 pass
+    if not figures:
+        log("floor probe printed no figures (it does not run under a profiler): no floor figures")
     return figures or None
 
 
