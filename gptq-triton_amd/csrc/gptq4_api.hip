@@ -186,11 +186,11 @@ struct TiledChoice {
     size_t partial;
 };
 
-TiledChoice choose_tiled(int epi, int M, int n, int K, bool kernel_gathers) {
+TiledChoice choose_tiled(int epi, int M, int n, int K, bool kernel_gathers, bool allow_streamed = true) {
     TiledChoice c = {};
     c.kp = kslice_plan(epi, M, n, K, kernel_gathers);
     c.kslice = prefer_kslice(c.kp, epi, M, n, K);
-    c.gp = gemm_plan(epi, M, n, K, kernel_gathers);
+    c.gp = gemm_plan(epi, M, n, K, kernel_gathers, allow_streamed);
     c.partial = c.kslice ? kslice_partial_bytes(epi, c.kp) : gemm_partial_bytes(c.gp);
     return c;
 }
@@ -233,7 +233,7 @@ ColumnParts tiled_parts(int epi, int M, int N, int K, bool kernel_gathers) {
     return parts;
 }
 
-TiledChoice choose_part(int epi, int M, int K, const ColumnParts &parts, int i, bool kernel_gathers) {
+TiledChoice choose_part(int epi, int M, int K, const ColumnParts &parts, int i, bool kernel_gathers, bool allow_streamed = true) {
     if (i == 0 && parts.first_is_wide) {
         TiledChoice c = {};
         c.kslice = false;
@@ -247,7 +247,7 @@ TiledChoice choose_part(int epi, int M, int K, const ColumnParts &parts, int i, 
         c.partial = 0;
         return c;
     }
-    return choose_tiled(epi, M, parts.cols[i], K, kernel_gathers);
+    return choose_tiled(epi, M, parts.cols[i], K, kernel_gathers, allow_streamed);
 }
 
 int run_tiled(int epi, MatmulArgs &a, void *workspace, size_t workspace_bytes, hipStream_t s) {
@@ -258,12 +258,13 @@ int run_tiled(int epi, MatmulArgs &a, void *workspace, size_t workspace_bytes, h
     ColumnParts parts;
     TiledChoice choice[2];
     size_t partial = 0;
+    bool allow_streamed = true;
     auto plan_all = [&]() {
         const bool kernel_gathers = a.perm != nullptr && !stage;
         parts = tiled_parts(epi, a.M, a.N, a.K, kernel_gathers);
         partial = 0;
         for (int i = 0; i < parts.count; ++i) {
-            choice[i] = choose_part(epi, a.M, a.K, parts, i, kernel_gathers);
+            choice[i] = choose_part(epi, a.M, a.K, parts, i, kernel_gathers, allow_streamed);
             if (choice[i].partial > partial) partial = choice[i].partial;
         }
     };
@@ -271,9 +272,8 @@ int run_tiled(int epi, MatmulArgs &a, void *workspace, size_t workspace_bytes, h
     // the streamed schedule keeps 128 MiB of partial sums: without the room for them, the unstreamed plan
     if (parts.count == 1 && !choice[0].kslice && choice[0].gp.streamed &&
         (workspace == nullptr || workspace_bytes < GPTQ4_WS_HEAD_BYTES + partial + (stage ? rows_bytes : 0))) {
-        g_stream_off = true;
+        allow_streamed = false;
         plan_all();
-        g_stream_off = false;
     }
     if (stage && (workspace == nullptr || workspace_bytes < GPTQ4_WS_HEAD_BYTES + partial + rows_bytes)) {
         stage = false;
@@ -334,6 +334,8 @@ const char *gptq4_strerror(int code) {
             return "groupsize must be -1, K, or a multiple of 128 dividing K";
         case GPTQ4_E_WORKSPACE:
             return "workspace is NULL or too small (see gptq4_workspace_bytes)";
+        case GPTQ4_E_EXCHANGE:
+            return "a kernel's bounded wait for another workgroup's partial sums ran out: results of that call are invalid";
         case GPTQ4_E_ALIGN:
             return "a pointer is not 16-byte aligned";
         case GPTQ4_E_STATIC_LIMIT:
@@ -393,7 +395,9 @@ void gptq4_set_tuning(int words, int depth, int splitk) {
     g_skinny_tuning.splitk = splitk > 0 ? splitk : 0;
 }
 
-size_t gptq4_workspace_bytes(int op, int M, int K, int N) {
+// allow_streamed = false: the need of the same call planned without the tiled kernel's streamed schedule (a
+// measurement mode whose partial sums alone are 128 MiB)
+static size_t workspace_need(int op, int M, int K, int N, bool allow_streamed) {
     size_t bytes = GPTQ4_WS_HEAD_BYTES;
     const bool with_perm = (op & GPTQ4_OP_WITH_PERM) != 0;
     op &= ~GPTQ4_OP_WITH_PERM;
@@ -407,12 +411,12 @@ size_t gptq4_workspace_bytes(int op, int M, int K, int N) {
         const int epi = (op == GPTQ4_OP_MLP_GATEUP) ? EPI_SILU_MUL : (op == GPTQ4_OP_QKV_ROTARY ? EPI_ROPE : EPI_PLAIN);
         // whichever kernel the current (automatic or forced) plans pick, with or without act-order, for the whole
         // matrix and for each of the column ranges a call may be cut into
-        size_t need = gemm_partial_bytes(gemm_plan(epi, M, N, K));
+        size_t need = gemm_partial_bytes(gemm_plan(epi, M, N, K, false, allow_streamed));
         const KslicePlan kp = kslice_plan(epi, M, N, K, false);
         if (kp.ok && kslice_partial_bytes(epi, kp) > need) need = kslice_partial_bytes(epi, kp);
         const ColumnParts parts = tiled_parts(epi, M, N, K, false);
         for (int i = 0; i < parts.count; ++i) {
-            const TiledChoice c = choose_part(epi, M, K, parts, i, false);
+            const TiledChoice c = choose_part(epi, M, K, parts, i, false, allow_streamed);
             if (c.partial > need) need = c.partial;
             const KslicePlan pk = kslice_plan(epi, M, parts.cols[i], K, false);
             if (pk.ok && kslice_partial_bytes(epi, pk) > need) need = kslice_partial_bytes(epi, pk);
@@ -423,6 +427,8 @@ size_t gptq4_workspace_bytes(int op, int M, int K, int N) {
     }
     return bytes;
 }
+
+size_t gptq4_workspace_bytes(int op, int M, int K, int N) { return workspace_need(op, M, K, N, true); }
 
 int gptq4_column_parts(int op, int M, int K, int N, int *begin, int *cols) {
     op &= ~GPTQ4_OP_WITH_PERM;
@@ -519,14 +525,32 @@ int gptq4_matmul_static(const void *x, const int32_t *qweight, const int32_t *qz
     if (rc) return rc;
     // what the same call would ask of a caller's workspace - planned without the streamed schedule of the tiled
     // kernel, whose partial sums alone are 128 MiB - has to fit the static array
-    g_stream_off = true;
-    const size_t need = gptq4_workspace_bytes(GPTQ4_OP_MATMUL, M, K, N);
-    g_stream_off = false;
+    const size_t need = workspace_need(GPTQ4_OP_MATMUL, M, K, N, false);
     if (need > (size_t)GPTQ4_STATIC_SCRATCH_BYTES) return -GPTQ4_E_STATIC_LIMIT;
     void *ws = nullptr;
     rc = static_scratch(&ws);
     if (rc) return rc;
     return gptq4_matmul(x, qweight, qzeros, scales, nullptr, bias, y, M, K, N, groupsize, ws, GPTQ4_STATIC_SCRATCH_BYTES, stream);
+}
+
+int gptq4_static_status(void *stream) {
+    void *ws = nullptr;
+    int rc = static_scratch(&ws);
+    if (rc) return rc;
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    int word = 0;
+    hipError_t e = hipMemcpyAsync(&word, reinterpret_cast<const int *>(ws) + GPTQ4_WS_ERROR_WORD, sizeof(int), hipMemcpyDeviceToHost, s);
+    if (e != hipSuccess) return (int)e;
+    e = hipStreamSynchronize(s);
+    if (e != hipSuccess) return (int)e;
+    return word != 0 ? -GPTQ4_E_EXCHANGE : 0;
+}
+
+int gptq4_static_reset(void *stream) {
+    void *ws = nullptr;
+    int rc = static_scratch(&ws);
+    if (rc) return rc;
+    return (int)hipMemsetAsync(ws, 0, GPTQ4_WS_HEAD_BYTES, reinterpret_cast<hipStream_t>(stream));
 }
 
 static int mlp_gateup_impl(const void *x, const void *delta, const void *norm_weight, void *sum_out, float eps,

@@ -781,7 +781,9 @@ ChainPlan plan_chain(const gptq4_phase_t *phases, int nphases, int M, int grid) 
     ChainArgs &a = pl.a;
     a.nphases = nphases;
     a.M = M;
-    a.spin_limit = g_chain_tuning.spin_limit ? g_chain_tuning.spin_limit : (4u << 20);
+    // a poll is one round trip to memory (1 - 2 us) and a hop between phases takes a few of them: 16384 polls give up
+    // within tens of milliseconds on a grid that is not fully resident (another stream holding CUs), not seconds
+    a.spin_limit = g_chain_tuning.spin_limit ? g_chain_tuning.spin_limit : (1u << 14);
     a.skip_flag_wg = g_chain_tuning.skip_flag_wg;
     size_t partial_elems = 0;
     int stage_chunks = 16, red_tiles = 1, keep_chunks = 0;

@@ -837,7 +837,6 @@ int launch_epi(const MatmulArgs &a, const GemmPlan &pl, hipStream_t stream) {
 }  // namespace
 
 GemmTuning g_gemm_tuning = {0, 0, 0, 0, 0, 0};
-thread_local bool g_stream_off = false;
 
 // Tile shape and split-K factor of the tiled kernel.  The wide tile (128 x 256, half as
 // wide for SiLU*mul) is the faster one as soon as there are enough of them to give three
@@ -854,7 +853,7 @@ static double fill_efficiency(long w) {
     return (double)w / ((double)(2 * cus) * (double)((w + 2 * cus - 1) / (2 * cus)));
 }
 
-GemmPlan gemm_plan(int epi, int M, int N, int K, bool has_perm) {
+GemmPlan gemm_plan(int epi, int M, int N, int K, bool has_perm, bool allow_streamed) {
     GemmPlan pl;
     pl.score = 1.0;
     pl.streamed = 0;
@@ -936,7 +935,7 @@ GemmPlan gemm_plan(int epi, int M, int N, int K, bool has_perm) {
     // 2048 rows 216 -> 240), ahead only where K is long and the tile count large (30B down_proj at 4096 rows
     // 970 -> 942 us).  gptq4_set_gemm_tuning(200, 0) runs it wherever it can run.
     const long slots = 2 * cus;
-    const bool can_stream = !has_perm && !g_stream_off && g_gemm_tuning.streamed == 2 && g_gemm_tuning.mt == 0 && g_gemm_tuning.splitk == 0 &&
+    const bool can_stream = !has_perm && allow_streamed && g_gemm_tuning.streamed == 2 && g_gemm_tuning.mt == 0 && g_gemm_tuning.splitk == 0 &&
                             wide >= 1 && wide <= SKINNY_MAX_TILES;
     if (can_stream) {
         // every workgroup of the grid needs at least one K tile (the sharers of a tile are counted from the

@@ -122,10 +122,9 @@ struct GemmTuning {
     int tail;        // 0 = automatic, 1 = never cut the tiles past a whole number of rounds along K
 };
 extern GemmTuning g_gemm_tuning;
-// set around a call that must not plan the streamed schedule (its partial sums would not fit the caller's scratch memory)
-extern thread_local bool g_stream_off;
-// has_perm: the kernel will gather act-order activations itself (no streamed schedule then)
-GemmPlan gemm_plan(int epi, int M, int N, int K, bool has_perm = false);
+// has_perm: the kernel will gather act-order activations itself (no streamed schedule then); allow_streamed = false:
+// the call must not plan the streamed schedule (its partial sums would not fit the caller's scratch memory)
+GemmPlan gemm_plan(int epi, int M, int N, int K, bool has_perm = false, bool allow_streamed = true);
 size_t gemm_partial_bytes(const GemmPlan &plan);
 // Tiled matrix-core GEMM for any M.  Returns hipError_t.
 int launch_gemm(int epi, const MatmulArgs &a, const GemmPlan &plan, hipStream_t stream);

@@ -32,15 +32,6 @@
 
 #include <mutex>
 
-#ifdef STREAM_STAMPS
-#define STAMP(i)                                                                                                       \
-    do {                                                                                                               \
-        if (lane == 0) reinterpret_cast<unsigned long long *>(reinterpret_cast<char *>(p.counters) + (40 << 20))[(wg * NW + wave) * 8 + (i)] = wall_clock64(); \
-    } while (0)
-#else
-#define STAMP(i)
-#endif
-
 namespace {
 
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -85,7 +76,6 @@ __global__ __launch_bounds__(64 * NW) void gptq4_stream_kernel(StreamArgs p) {
 
     const int M = p.M, K = p.K, N = p.N, nb = p.nb, G = p.groups;
     const int wg = blockIdx.x;
-    STAMP(0);
     const int a0 = wg * p.q + min(wg, p.r);      // first unit of this workgroup
     const int L = p.q + (wg < p.r ? 1 : 0);      // its units
     const int b0 = a0 + L;
@@ -162,7 +152,6 @@ __global__ __launch_bounds__(64 * NW) void gptq4_stream_kernel(StreamArgs p) {
     SUnit<NV> ring[DEPTH];
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) issue(ring[d], d < n);
-    STAMP(1);
 
     const int tile_lo = sdiv_magic(a0, nb, p.nb_magic);
     const int npieces = tile_hi - tile_lo + 1;
@@ -248,7 +237,6 @@ __global__ __launch_bounds__(64 * NW) void gptq4_stream_kernel(StreamArgs p) {
         rope_sn = p.rope.sin_table[(size_t)pos * 64 + rope_dd];
     }
     __syncthreads();
-    STAMP(2);
 
     // ---- a wave's sums of a piece -> its slot; the top piece of a range whose strip goes on in the next workgroup
     //      is added up and published by the last wave to leave it
@@ -328,7 +316,6 @@ __global__ __launch_bounds__(64 * NW) void gptq4_stream_kernel(StreamArgs p) {
             issue(ring[d], i + d + DEPTH < n);
         }
     }
-    STAMP(4);
     if (n > 0) dump(tile_hi - cur_tile);
 
     // ---- the lower workgroups' sums of the bottom strip, published when they were a few units into their ranges:
@@ -369,7 +356,6 @@ __global__ __launch_bounds__(64 * NW) void gptq4_stream_kernel(StreamArgs p) {
         }
     }
     __syncthreads();
-    STAMP(5);
 
     if (owner) {
         const int pc = npieces - 1 - e_pb;
@@ -410,7 +396,6 @@ __global__ __launch_bounds__(64 * NW) void gptq4_stream_kernel(StreamArgs p) {
             dst[off + 64 + rope_dd] = (half_t)o2;
         }
     }
-    STAMP(6);
 }
 
 // ---- layout conversion ------------------------------------------------------------------------------------------

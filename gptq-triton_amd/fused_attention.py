@@ -388,12 +388,22 @@ def _forward_with_cache(self, hidden_states, attention_mask, position_ids, cache
             position_ids = torch.arange(past, past + q_len, device=hidden_states.device).unsqueeze(0)
     if position_ids.shape[0] != bsz:
         position_ids = position_ids.expand(bsz, -1)
+    if cache is not None and self.layer_idx is None:
+        raise ValueError("this attention block does not know its layer index and cannot update a Cache")
+    # tokens the cache holds before this call; read only when no mask says what to attend to
+    past = int(cache.get_seq_length(self.layer_idx)) if cache is not None and attention_mask is None else 0
     query_states, key_states, value_states = self.project_qkv(hidden_states, position_ids.contiguous())
     if cache is not None:
-        if self.layer_idx is None:
-            raise ValueError("this attention block does not know its layer index and cannot update a Cache")
         key_states, value_states = cache.update(key_states, value_states, self.layer_idx)
     kv_len = key_states.shape[-2]
+    if attention_mask is None and kv_len > past + q_len:
+        # a preallocated cache hands back its whole capacity: without a mask only the slots written so far count
+        kv_len = past + q_len
+        key_states, value_states = key_states[:, :, :kv_len], value_states[:, :, :kv_len]
+    causal = None
+    if attention_mask is None and q_len > 1 and kv_len != q_len:
+        # a prompt chunk behind cached tokens: token i sees the cached tokens and the chunk up to itself
+        causal = torch.ones(q_len, kv_len, dtype=torch.bool, device=hidden_states.device).tril(kv_len - q_len)
     attn_weights = None
     if output_attentions:
         attn_weights = torch.matmul(query_states, key_states.transpose(2, 3)) / math.sqrt(self.head_dim)
@@ -403,18 +413,16 @@ def _forward_with_cache(self, hidden_states, attention_mask, position_ids, cache
             else:
                 attn_weights = torch.clamp_min(attn_weights + attention_mask[..., :kv_len], torch.finfo(attn_weights.dtype).min)
         elif q_len > 1:
-            causal = torch.ones(q_len, kv_len, dtype=torch.bool, device=attn_weights.device).tril(kv_len - q_len)
-            attn_weights = attn_weights.masked_fill(~causal, torch.finfo(attn_weights.dtype).min)
+            full = causal if causal is not None else torch.ones(q_len, kv_len, dtype=torch.bool, device=attn_weights.device).tril()
+            attn_weights = attn_weights.masked_fill(~full, torch.finfo(attn_weights.dtype).min)
         attn_weights = nn.functional.softmax(attn_weights, dim=-1, dtype=torch.float32).to(query_states.dtype)
         attn_output = torch.matmul(attn_weights, value_states)
     else:
         # as transformers' own scaled-dot-product path: a given mask is used as it is, none means causal for a prompt
         # and full attention for a single token
-        mask = None if attention_mask is None else attention_mask[..., :kv_len]
+        mask = causal if attention_mask is None else attention_mask[..., :kv_len]
         attn_output = nn.functional.scaled_dot_product_attention(query_states, key_states, value_states, attn_mask=mask,
-                                                                 is_causal=(mask is None and q_len > 1 and kv_len == q_len))
-        if mask is None and q_len > 1 and kv_len != q_len:
-            raise ValueError("a prompt chunk behind cached tokens needs an attention mask")
+                                                                 is_causal=(mask is None and q_len > 1))
     attn_output = attn_output.transpose(1, 2).reshape(bsz, q_len, self.hidden_size)
     return self.o_proj(attn_output), attn_weights
 

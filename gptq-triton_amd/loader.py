@@ -14,7 +14,7 @@ from typing import Optional
 
 import torch
 
-from . import fused_mlp, quant_linear
+from . import _lib, fused_mlp, quant_linear
 from .fused_attention import make_quant_attn
 from .fused_mlp import make_fused_mlp
 from .llama import LlamaForCausalLM, config_from_json
@@ -116,6 +116,14 @@ def load_quant(checkpoint: str, warmup_autotune: bool = True, device: Optional[s
             raise ValueError("You must specify a device when warmup_autotune is True.")
         autotune_warmup(model)
     model.seqlen = 2048
+    if use_transformers and device is not None and torch.device(device).type == 'cuda':
+        # transformers' generate() reads every step's logits on the host anyway; the same point checks the error word
+        # of the workspaces, so that a kernel's bounded wait that ran out raises instead of yielding wrong tokens
+        # (GreedyDecoder.decode does the same for this package's own decoder)
+        def _check(module, args, output):
+            if not torch.cuda.is_current_stream_capturing():
+                _lib.check_exchange_errors()
+        model.register_forward_hook(_check)
     return model
 
 

@@ -56,6 +56,7 @@ extern "C" {
 #define GPTQ4_E_WORKSPACE 4  /* workspace NULL or smaller than required          */
 #define GPTQ4_E_ALIGN 5      /* a pointer is not 16-byte aligned                 */
 #define GPTQ4_E_STATIC_LIMIT 6 /* gptq4_matmul_static: the call needs more scratch than the library holds */
+#define GPTQ4_E_EXCHANGE 7   /* gptq4_static_status: a bounded wait between workgroups ran out (error word set) */
 
 /* head of a workspace, kept zero between calls: arrival counters, then marked partial sums (8 bytes each) */
 #define GPTQ4_WS_COUNTER_BYTES 524288
@@ -121,6 +122,14 @@ int gptq4_matmul(const void *x, const int32_t *qweight, const int32_t *qzeros,
 int gptq4_matmul_static(const void *x, const int32_t *qweight, const int32_t *qzeros,
                         const void *scales, const void *bias, void *y, int M, int K, int N,
                         int groupsize, void *stream);
+/* The library's array is private, so these two do for it what a caller does with its own workspace (no reference
+ * counterpart either).  gptq4_static_status waits for `stream` and returns 0, or -GPTQ4_E_EXCHANGE when a
+ * gptq4_matmul_static call on this GPU gave up its bounded wait (GPTQ4_WS_ERROR_WORD set: that call's result is
+ * invalid, and late partial sums may spoil later calls until the head is zeroed).  gptq4_static_reset zeroes the
+ * head of the array on `stream` (a memset node: not under stream capture).  Neither allocates.  After an error:
+ * let the GPU drain (gptq4_static_status did), then gptq4_static_reset. */
+int gptq4_static_status(void *stream);
+int gptq4_static_reset(void *stream);
 
 /* h fp16 [M, I] = silu(x @ Wgate) * (x @ Wup); SiLU and the product are taken on the
  * fp32 accumulators, one rounding to fp16.

@@ -117,7 +117,7 @@ size_t gptq4_chain_workspace_bytes(const gptq4_phase_t *phases, int nphases, int
 int gptq4_decode_chain(const gptq4_phase_t *phases, int nphases, int M, void *workspace,
                        size_t workspace_bytes, void *stream);
 /* Measurement and test knobs of the chained launch: units of LDS ring per streaming wave (2..4, 0 = as many as
- * fit), a reserved value, polls before a wait gives up (0 = default, about seconds), and a workgroup that never
+ * fit), a reserved value, polls before a wait gives up (0 = default: 16384, tens of milliseconds), and a workgroup that never
  * stores its partial sums (-1 = none; lets a test see the bounded waits give up with every kernel exiting normally). */
 void gptq4_set_chain_tuning(int ring_slots, int reserved, unsigned spin_limit, int skip_flag_wg);
 

@@ -88,3 +88,44 @@ def test_reference_signature_still_answers(tmp_path):
     assert out.shape == (2, 5, 256) and weights is None and present[0].shape == (2, 2, 5, 128)
     out2, _, present2 = attn(x[:, :1].contiguous(), past_key_value=present, use_cache=True)
     assert out2.shape == (2, 1, 256) and present2[0].shape == (2, 2, 6, 128)
+
+
+def test_preallocated_cache_without_a_mask_attends_to_written_slots_only(tmp_path):
+    """A StaticCache hands back tensors of its whole capacity.  Called without a mask, the block attends to the slots
+    written so far - a prompt, a chunk behind it, single tokens - exactly as with a DynamicCache."""
+    make_checkpoint(tmp_path, 128, seed=14)
+    hf = G.load_quant(str(tmp_path), device="cuda", fuse_mlp=True, use_transformers=True)
+    attn = hf.model.layers[0].self_attn
+    torch.manual_seed(4)
+    x = (0.5 * torch.randn(2, 12, 256, device="cuda")).half()
+    chunks = ((0, 6), (6, 10), (10, 11), (11, 12))
+
+    def run(cache):
+        outs = []
+        with torch.no_grad():
+            for a, b in chunks:
+                pos = torch.arange(a, b, device="cuda").unsqueeze(0)
+                out, _ = attn(x[:, a:b].contiguous(), position_ids=pos, past_key_values=cache,
+                              position_embeddings=(None, None), cache_position=pos[0])
+                outs.append(out)
+        return torch.cat(outs, dim=1)
+
+    dyn = run(transformers.DynamicCache())
+    static = run(transformers.StaticCache(config=hf.config, max_cache_len=32))
+    assert torch.equal(dyn, static)
+    with torch.no_grad():
+        whole, _ = attn(x, position_ids=torch.arange(12, device="cuda").unsqueeze(0), past_key_values=None,
+                        position_embeddings=(None, None))
+    assert (whole.float() - dyn.float()).abs().max() < 2e-3 + 1e-2 * whole.float().abs().max()
+
+
+def test_generate_with_a_static_cache(tmp_path):
+    """transformers builds the mask for a preallocated cache itself; greedy tokens equal those of the default cache."""
+    cfg = make_checkpoint(tmp_path, 128, seed=15)
+    hf = G.load_quant(str(tmp_path), device="cuda", fuse_mlp=True, use_transformers=True)
+    torch.manual_seed(5)
+    prompt = torch.randint(1, cfg.vocab_size, (2, 8)).cuda()
+    with torch.no_grad():
+        a = hf.generate(prompt, max_new_tokens=6, do_sample=False, pad_token_id=0)
+        b = hf.generate(prompt, max_new_tokens=6, do_sample=False, pad_token_id=0, cache_implementation="static")
+    assert torch.equal(a, b)

@@ -77,3 +77,35 @@ def test_static_scratch_rejects_what_does_not_fit():
     # the ordinary argument errors come first
     assert lib.gptq4_matmul_static(None, fake, fake, fake, None, fake, 1, 4096, 4096, -1, None) == -1
     assert lib.gptq4_matmul_static(fake, fake, fake, fake, None, fake, 1, 4000, 4096, -1, None) == -2
+
+
+def test_static_scratch_status_and_reset():
+    """The library's array is private: gptq4_static_status reports a bounded wait that ran out (forced from the
+    host with the spin-limit hook; every kernel exits normally), gptq4_static_reset zeroes the head, and the next
+    call is right again."""
+    from gptq_triton_amd import _lib
+    lib = _lib.load()
+    m, k, n, g = 1, 4096, 4096, 128
+    L = O.make_layer(k, n, g, seed=31)
+    D = to_dev(L)
+    xd = torch.from_numpy(O.make_x(m, k, seed=32)).cuda()
+    stream = _lib.current_stream(xd.device)
+    y = torch.empty((m, n), dtype=torch.float16, device="cuda")
+
+    def call():
+        return lib.gptq4_matmul_static(xd.data_ptr(), D["qweight"].data_ptr(), D["qzeros"].data_ptr(), D["scales"].data_ptr(),
+                                       None, y.data_ptr(), m, k, n, g, stream)
+
+    assert call() == 0 and lib.gptq4_static_status(stream) == 0
+    try:
+        lib.gptq4_set_exchange_spin_limit(0xFFFFFFFF)
+        assert call() == 0
+        assert lib.gptq4_static_status(stream) == -7
+        assert b"wait" in lib.gptq4_strerror(-7)
+    finally:
+        lib.gptq4_set_exchange_spin_limit(0)
+        torch.cuda.synchronize()
+        assert lib.gptq4_static_reset(stream) == 0
+    assert lib.gptq4_static_status(stream) == 0
+    y_ws, y_st = _both(lib, xd, D, k, n, g)
+    assert torch.equal(y_ws, y_st)
