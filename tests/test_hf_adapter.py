@@ -120,12 +120,14 @@ def test_preallocated_cache_without_a_mask_attends_to_written_slots_only(tmp_pat
 
 
 def test_generate_with_a_static_cache(tmp_path):
-    """transformers builds the mask for a preallocated cache itself; greedy tokens equal those of the default cache."""
+    """transformers builds the mask for a preallocated cache itself; greedy tokens equal those of the default cache.
+    (disable_compile: with a preallocated cache generate() would otherwise hand the forward pass to torch.compile,
+    which cannot trace calls into a C library.)"""
     cfg = make_checkpoint(tmp_path, 128, seed=15)
     hf = G.load_quant(str(tmp_path), device="cuda", fuse_mlp=True, use_transformers=True)
     torch.manual_seed(5)
     prompt = torch.randint(1, cfg.vocab_size, (2, 8)).cuda()
     with torch.no_grad():
         a = hf.generate(prompt, max_new_tokens=6, do_sample=False, pad_token_id=0)
-        b = hf.generate(prompt, max_new_tokens=6, do_sample=False, pad_token_id=0, cache_implementation="static")
+        b = hf.generate(prompt, max_new_tokens=6, do_sample=False, pad_token_id=0, cache_implementation="static", disable_compile=True)
     assert torch.equal(a, b)
