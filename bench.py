@@ -212,7 +212,7 @@ def decoder_figures(workload, bsz, prompt, new, steps=None, warmup=None):
         "config": {"workload": f"random-init {workload}-shape decoder, batch {bsz}, {prompt}-token prompt prefill then "
                                f"{new} greedy tokens, 4-bit groupsize {groupsize}{' act-order' if act_order else ''}, "
                                f"fp16 lm_head, one HIP-graph replay per token, packed weights in "
-                               f"{'streaming order' if bsz <= 4 else 'the checkpoint layout'}",
+                               f"{'streaming order' if bsz <= 16 else 'the checkpoint layout'}",
                    "layers": layers, "hidden": hidden, "intermediate": inter, "heads": heads, "batch": bsz,
                    "prompt": prompt, "new_tokens": new},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -477,7 +477,7 @@ def main():
     log("building 32 layers of synthetic 4-bit weights ...")
     layers = [dict(qkv=make(HIDDEN, 3 * HIDDEN), o=make(HIDDEN, HIDDEN), gate=make(HIDDEN, INTER),
                    up=make(HIDDEN, INTER), down=make(INTER, HIDDEN)) for _ in range(LAYERS)]
-    # the same weights in streaming order, the resident layout of a model that decodes up to four sequences
+    # the same weights in streaming order, the resident layout of a model that decodes up to sixteen sequences
     for L in layers:
         for name in ("qkv", "o", "gate", "up", "down"):
             qw, qz, sc = L[name]
@@ -650,7 +650,7 @@ def main():
         per_op("decode M=1 o_proj", lambda L: s_o_op(x1f, L), wo + 4 * HIDDEN, 2 * HIDDEN * HIDDEN)
         per_op("decode M=1 gate/up+silu*mul", lambda L: s_gateup_op(x1f, L), gu_bytes, 4 * HIDDEN * INTER)
         per_op("decode M=1 down_proj", lambda L: s_down_op(h1, L), wd + 2 * INTER + 2 * HIDDEN, 2 * HIDDEN * INTER)
-        for mm in (2, 4):
+        for mm in (2, 4, 8, 16):  # (from five rows on: the variant that fetches the rows with every unit)
             xm = torch.randn((mm, 1, HIDDEN), device=dev, generator=gen).half()
             hm = torch.randn((mm, INTER), device=dev, generator=gen).half()
             posm = torch.full((mm, 1), 2047, device=dev, dtype=torch.int32)
@@ -736,9 +736,10 @@ def main():
             xm = torch.randn((m, HIDDEN), device=dev, generator=gen).half()
             config_row("C2", "MLP gate/up+silu*mul, down g=128", m, lambda L: down_op(gateup_op(xm, L), L), layers,
                        2 * wg + wd + 4 * m * HIDDEN + 4 * m * INTER, 6 * m * HIDDEN * INTER, reps=5)
-        xm = torch.randn((1, HIDDEN), device=dev, generator=gen).half()
-        config_row("C2", "MLP gate/up+silu*mul, down g=128, streaming order", 1, lambda L: s_down_op(s_gateup_op(xm, L), L), layers,
-                   2 * wg + wd + 4 * HIDDEN + 4 * INTER, 6 * HIDDEN * INTER, reps=5)
+        for m in (1, 16):
+            xm = torch.randn((m, HIDDEN), device=dev, generator=gen).half()
+            config_row("C2", "MLP gate/up+silu*mul, down g=128, streaming order", m, lambda L: s_down_op(s_gateup_op(xm, L), L), layers,
+                       2 * wg + wd + 4 * m * HIDDEN + 4 * m * INTER, 6 * m * HIDDEN * INTER, reps=5)
         # C3: fused QKV + rotary 4096 -> 12288, one group, M = 1 at position 2047 and a 2048-token prefill
         c3 = [make(HIDDEN, 3 * HIDDEN, -1) for _ in range(12)]
         w3 = weight_bytes(HIDDEN, 3 * HIDDEN, HIDDEN)

@@ -731,10 +731,21 @@ int gptq4_decode_attention(const void *q, const void *k_cache, const void *v_cac
 
 // ---- streaming-order layout ---------------------------------------------------------------------------------------
 
-static int stream_fill(StreamArgs &a, int epi, int groupsize, void *workspace, size_t workspace_bytes, StreamPlan &pl, bool norm) {
+static int stream_fill(StreamArgs &a, int epi, int groupsize, void *workspace, size_t workspace_bytes, StreamPlan &pl, bool norm,
+                       void *stream) {
     pl = stream_plan(epi, a.M, a.N, a.K, norm);
     if (!pl.ok) return -GPTQ4_E_SHAPE;
     if (workspace == nullptr || workspace_bytes < GPTQ4_WS_HEAD_BYTES) return -GPTQ4_E_WORKSPACE;
+    if (pl.tall && a.perm != nullptr) {
+        // the kernel for more than STREAM_MAX_M rows does not gather: one small launch does, into the workspace behind the head
+        const size_t bytes = (size_t)a.M * a.K * sizeof(half_t);
+        if (workspace_bytes < GPTQ4_WS_HEAD_BYTES + bytes) return -GPTQ4_E_WORKSPACE;
+        half_t *xg = reinterpret_cast<half_t *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_HEAD_BYTES);
+        const int rc = launch_gather_cols(a.x, a.perm, xg, a.M, a.K, reinterpret_cast<hipStream_t>(stream));
+        if (rc) return rc;
+        a.x = xg;
+        a.perm = nullptr;
+    }
     a.counters = reinterpret_cast<int *>(workspace);
     a.tagged = reinterpret_cast<uint64_t *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_COUNTER_BYTES);
     a.spin_limit = g_gemv_tuning.spin_limit ? g_gemv_tuning.spin_limit : (1u << 22);
@@ -763,7 +774,7 @@ int gptq4_stream_rows(int op, int K, int N, int groupsize) {
     if (check_dims(K, N, &g)) return 0;
     const int epi = (op == GPTQ4_OP_MLP_GATEUP) ? EPI_SILU_MUL : (op == GPTQ4_OP_QKV_ROTARY ? EPI_ROPE : EPI_PLAIN);
     int rows = 0;
-    for (int m = 1; m <= STREAM_MAX_M; ++m)
+    for (int m = 1; m <= STREAM_TALL_MAX_M; ++m)
         if (stream_plan(epi, m, N, K, false).ok) rows = m;
     return rows;
 }
@@ -819,7 +830,7 @@ static int stream_matmul_impl(const void *x, const int32_t *sweight, const int32
     a.K = K;
     a.N = N;
     StreamPlan pl;
-    rc = stream_fill(a, EPI_PLAIN, groupsize, workspace, workspace_bytes, pl, false);
+    rc = stream_fill(a, EPI_PLAIN, groupsize, workspace, workspace_bytes, pl, false, stream);
     if (rc) return rc;
     return launch_stream(EPI_PLAIN, a, pl, nomath, reinterpret_cast<hipStream_t>(stream));
 }
@@ -854,7 +865,7 @@ static int stream_gateup_impl(const void *x, const void *delta, const void *norm
         if (rc) return rc;
     }
     StreamPlan pl;
-    rc = stream_fill(a, EPI_SILU_MUL, groupsize, workspace, workspace_bytes, pl, norm_weight != nullptr);
+    rc = stream_fill(a, EPI_SILU_MUL, groupsize, workspace, workspace_bytes, pl, norm_weight != nullptr, stream);
     if (rc) return rc;
     return launch_stream(EPI_SILU_MUL, a, pl, nomath, reinterpret_cast<hipStream_t>(stream));
 }
@@ -875,7 +886,7 @@ int gptq4_stream_qkv_rotary(const void *x, const void *delta, const void *norm_w
     if (!x || !sweight || !smeta || !position_ids || !cos_table || !sin_table || !q || !k || !v) return -GPTQ4_E_NULL;
     if (B < 1 || S < 1 || H < 1 || D != 128 || max_pos < 1) return -GPTQ4_E_SHAPE;
     if (kv_offset < GPTQ4_KV_AT_POSITION || kv_capacity < 1 || (kv_offset >= 0 && kv_capacity < kv_offset + S)) return -GPTQ4_E_SHAPE;
-    if ((long)B * S > STREAM_MAX_M) return -GPTQ4_E_SHAPE;
+    if ((long)B * S > STREAM_TALL_MAX_M) return -GPTQ4_E_SHAPE;
     const int N = 3 * H * D;
     int rc = check_dims(K, N, &groupsize);
     if (rc) return rc;
@@ -901,13 +912,13 @@ int gptq4_stream_qkv_rotary(const void *x, const void *delta, const void *norm_w
     a.rope.kv_capacity = kv_capacity;
     a.rope.kv_offset = kv_offset;
     a.rope.max_pos = max_pos;
-    a.rope.s_magic = 0;  // at most STREAM_MAX_M rows: a plain division
+    a.rope.s_magic = 0;  // a handful of rows: a plain division
     if (norm_weight) {
         rc = stream_norm(a, delta, norm_weight, sum_out, eps);
         if (rc) return rc;
     }
     StreamPlan pl;
-    rc = stream_fill(a, EPI_ROPE, groupsize, workspace, workspace_bytes, pl, norm_weight != nullptr);
+    rc = stream_fill(a, EPI_ROPE, groupsize, workspace, workspace_bytes, pl, norm_weight != nullptr, stream);
     if (rc) return rc;
     return launch_stream(EPI_ROPE, a, pl, false, reinterpret_cast<hipStream_t>(stream));
 }

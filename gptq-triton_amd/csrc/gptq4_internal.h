@@ -203,12 +203,13 @@ struct StreamPlan {
     int xrow, red_off, nat_off;
     size_t lds_bytes;
     bool ok;
+    bool tall;  // 5 .. 16 rows: the kernel that fetches its A operand with every unit
 };
 struct StreamTuning {
     int waves, depth;  // 0 = automatic
 };
 extern StreamTuning g_stream_tuning;
-enum { STREAM_MAX_M = 4 };
+enum { STREAM_MAX_M = 4, STREAM_TALL_MAX_M = 16 };  // rows with the activations in LDS (and the norm inside); rows at all
 StreamPlan stream_plan(int epi, int M, int N, int K, bool norm);
 int launch_stream(int epi, StreamArgs &a, const StreamPlan &plan, bool nomath, hipStream_t stream);
 int launch_stream_pack(const uint32_t *qweight, const uint32_t *qzeros, const half_t *scales, uint32_t *sw, uint32_t *meta,

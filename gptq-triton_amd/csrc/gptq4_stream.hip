@@ -398,6 +398,305 @@ __global__ __launch_bounds__(64 * NW) void gptq4_stream_kernel(StreamArgs p) {
     }
 }
 
+// ---- 5 .. 16 rows ------------------------------------------------------------------------------------------------
+// The same walk over the same layout for more rows than fit LDS with all of K (16 rows of K = 11008 are 344 KiB): a
+// wave fetches the rows' values of a unit WITH the unit, from memory (the rows are a few hundred KiB that every
+// workgroup reads: they live in L2) - four loads of four rows each, 256 contiguous bytes per row, so that a load
+// touches eight cache lines and uses all of them (fetching the A operand as the matrix core wants it - lane (r4, c):
+// row c, chunks 4 * r4 + j - would touch 32 lines per load and use a quarter of each; measured, that made the time grow
+// with the number of rows: 14.4 us at 5 rows, 20.6 at 16 for the LLaMA-7B gate/up pair).  The wave turns the block
+// into operand order through a 4.25 KiB LDS slot of its own (rows 17 chunks apart: both directions free of bank
+// conflicts; no barrier, a wave's LDS accesses are in order), in the k order of the decoded weights.  All 64 lanes of
+// an accumulator hold rows below M now (lane (r4, c): rows 4 * r4 .. 4 * r4 + 3 of column c), so a wave's slot of
+// partial sums is 1 KiB per strip, and a thread may finish several output elements.  No variant with the norm inside
+// or with the act-order gather: callers with more than four rows run the norm launch (which can store in the
+// projection's row order) and the entry points gather beforehand.
+template <int NV>
+struct TUnit {
+    u32x4_t w[NV];
+    uint32_t meta[NV];
+    u32x4_t a[4];
+};
+
+template <int EPI, int NW, int DEPTH>
+__global__ __launch_bounds__(64 * NW) void gptq4_stream_tall_kernel(StreamArgs p) {
+    constexpr int NV = (EPI == EPI_PLAIN) ? 1 : 2;
+    constexpr int NT = 64 * NW;
+    constexpr int RE = (16 * 64 + NT - 1) / NT;  // (row, column of a head's half) pairs of the rotary table per thread
+    extern __shared__ uint4 smem[];
+    __shared__ int arrivals;
+    __shared__ int pos_s[16];
+
+    asm volatile("" ::"s"(p.x), "s"(p.m[0].w), "s"(p.m[0].meta), "s"(p.m[1].w), "s"(p.m[1].meta), "s"(p.M), "s"(p.K), "s"(p.N), "s"(p.nb),
+                 "s"(p.groups), "s"(p.batches_per_group), "s"(p.group_magic), "s"(p.q), "s"(p.r), "s"(p.nb_magic), "s"(p.red_off),
+                 "s"(p.nat_off), "s"(p.m_magic), "s"(p.tagged));
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r4 = lane >> 4;
+    const int c = lane & 15;
+
+    const int M = p.M, K = p.K, N = p.N, nb = p.nb, G = p.groups;
+    const int wg = blockIdx.x;
+    const int a0 = wg * p.q + min(wg, p.r);
+    const int L = p.q + (wg < p.r ? 1 : 0);
+    const int b0 = a0 + L;
+    const int tile_hi = sdiv_magic(b0 - 1, nb, p.nb_magic);
+    const int n = wave < L ? (L - wave + NW - 1) / NW : 0;
+
+    // ---- rotary: the table rows of the M tokens, requested ahead of everything (two dependent loads), parked in
+    //      registers until the loop is done
+    int rp_pos[RE];
+    float rp_cs[RE], rp_sn[RE];
+    if (EPI == EPI_ROPE) {
+#pragma unroll
+        for (int i = 0; i < RE; ++i) {
+            const int idx = tid + i * NT;
+            rp_pos[i] = idx < M * 64 ? p.rope.position_ids[idx >> 6] : 0;
+        }
+    }
+
+    const __amdgpu_buffer_rsrc_t rs_x = srsrc(p.x, (uint32_t)M * K * 2u);
+    // load i of a unit: row 4 * i + r4, chunk c of the unit's sixteen; rows from M on are never read
+    uint32_t xoff[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) xoff[i] = (4 * i + r4 < M) ? (uint32_t)(4 * i + r4) * (uint32_t)K * 2u + (uint32_t)c * 16u : S_OFF_RANGE;
+    const uint32_t wbytes = (uint32_t)(((size_t)K * (size_t)N) >> 1);
+    const uint32_t mbytes = (uint32_t)G * (uint32_t)N * 4u;
+    __amdgpu_buffer_rsrc_t rs_w[NV], rs_m[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        rs_w[v] = srsrc(p.m[v].w, wbytes);
+        rs_m[v] = srsrc(p.m[v].meta, mbytes);
+    }
+    const int bpg = p.batches_per_group;
+    int ld_tile = tile_hi, ld_batch = 0;
+    if (n > 0) {
+        const int u = b0 - 1 - wave;
+        ld_tile = sdiv_magic(u, nb, p.nb_magic);
+        ld_batch = u - ld_tile * nb;
+    }
+    int cp_tile = ld_tile, cp_batch = ld_batch;
+    auto strip_of = [&](int tile, int v) { return (EPI == EPI_ROPE) ? ((tile >> 2) << 3) + (tile & 3) + 4 * v : tile; };
+    auto issue = [&](TUnit<NV> &U, bool live) {
+        const uint32_t dead = live ? 0u : S_OFF_RANGE;
+        const int g = (bpg == 1) ? ld_batch : (int)__umulhi((unsigned)ld_batch, p.group_magic);
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int strip = strip_of(ld_tile, v);
+            U.w[v] = __builtin_amdgcn_raw_buffer_load_b128(rs_w[v], ((uint32_t)lane * 16u) | dead, (uint32_t)(strip * nb + ld_batch) * 1024u, 2);
+            U.meta[v] = __builtin_amdgcn_raw_buffer_load_b32(rs_m[v], ((uint32_t)c * 4u) | dead, (uint32_t)(strip * G + g) * 64u, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) U.a[i] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, xoff[i] | dead, (uint32_t)ld_batch * 256u, 0);
+        ld_batch -= NW;
+        if (ld_batch < 0) {
+            ld_batch += nb;
+            ld_tile -= 1;
+        }
+    };
+    TUnit<NV> ring[DEPTH];
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) issue(ring[d], d < n);
+
+    if (EPI == EPI_ROPE) {
+#pragma unroll
+        for (int i = 0; i < RE; ++i) {
+            const int idx = tid + i * NT;
+            const int pos = min(max(rp_pos[i], 0), p.rope.max_pos - 1);
+            rp_cs[i] = idx < M * 64 ? p.rope.cos_table[(size_t)pos * 64 + (idx & 63)] : 1.f;
+            rp_sn[i] = idx < M * 64 ? p.rope.sin_table[(size_t)pos * 64 + (idx & 63)] : 0.f;
+        }
+    }
+
+    const int tile_lo = sdiv_magic(a0, nb, p.nb_magic);
+    const int npieces = tile_hi - tile_lo + 1;
+    const int top_len = min(L, b0 - tile_hi * nb);
+    const bool publishes = (b0 - tile_hi * nb) != nb;
+    const bool shared_lo = (a0 - tile_lo * nb) != 0;
+    const int fin0 = publishes ? 1 : 0;
+    const int total = (npieces - fin0) * M * 16;
+
+    // element e = (piece from the bottom, row, column); thread t finishes e = NT - 1 - t, + NT, ...: the bottom piece,
+    // whose other part comes from memory, falls to lanes of the last wave, which never has the most units
+    const int e_mine = NT - 1 - tid;
+    const bool gets_partials = shared_lo && e_mine < min(total, M * 16);
+
+    f4_t *const red = reinterpret_cast<f4_t *>(smem);  // [piece][wave][NV][lane]
+    const float *const redf = reinterpret_cast<const float *>(red);
+    for (int pc = 0; pc < npieces; ++pc)
+#pragma unroll
+        for (int v = 0; v < NV; ++v) red[((pc * NW + wave) * NV + v) * 64 + lane] = (f4_t){0.f, 0.f, 0.f, 0.f};
+    if (tid == 0) arrivals = 0;
+    __syncthreads();
+
+    const int slot_elems = NV * 16 * M;
+    auto arrive_top = [&]() {
+        int old = 0;
+        if (lane == 0) old = __hip_atomic_fetch_add(&arrivals, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_WORKGROUP);
+        old = __builtin_amdgcn_readfirstlane(old);
+        if (old != NW - 1) return;
+        uint64_t *const mine = p.tagged + (size_t)wg * slot_elems;
+        for (int e = lane; e < slot_elems; e += 64) {  // e = (v * M + row) * 16 + column
+            const int col = e & 15, t = e >> 4;
+            const int v = (t >= M) ? 1 : 0;
+            const int row = t - v * M;
+            float s = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) s += redf[((w * NV + v) * 64 + (row >> 2) * 16 + col) * 4 + (row & 3)];
+            __hip_atomic_store(&mine[e], S_MARK | (uint64_t)__float_as_uint(s), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    };
+    f4_t acc[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) acc[v] = (f4_t){0.f, 0.f, 0.f, 0.f};
+    auto dump = [&](int pc) {
+#pragma unroll
+        for (int v = 0; v < NV; ++v) red[((pc * NW + wave) * NV + v) * 64 + lane] = acc[v];
+        if (pc == 0 && publishes) arrive_top();
+    };
+    if (publishes && wave >= top_len) arrive_top();
+
+    int cur_tile = cp_tile;
+    uint4 *const turn = smem + p.nat_off + wave * (16 * 17);  // the wave's own 16 x 17 chunks
+    auto compute = [&](const TUnit<NV> &U) {
+        if (cp_tile != cur_tile) {
+            dump(tile_hi - cur_tile);
+            cur_tile = cp_tile;
+#pragma unroll
+            for (int v = 0; v < NV; ++v) acc[v] = (f4_t){0.f, 0.f, 0.f, 0.f};
+        }
+        // rows x chunks in, (row c, chunks 4 * r4 + j) out
+#pragma unroll
+        for (int i = 0; i < 4; ++i) turn[(4 * i + r4) * 17 + c] = pair_order_u4(__builtin_bit_cast(uint4, U.a[i]));
+        h8_t a[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) a[j] = __builtin_bit_cast(h8_t, turn[c * 17 + 4 * r4 + j]);
+        ColDecode cd[NV];
+#pragma unroll
+        for (int v = 0; v < NV; ++v) cd[v] = make_col_decode(U.meta[v] >> 16, U.meta[v]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int v = 0; v < NV; ++v)
+                acc[v] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j], decode_word_h8(U.w[v][j], cd[v]), acc[v], 0, 0, 0);
+        cp_batch -= NW;
+        if (cp_batch < 0) {
+            cp_batch += nb;
+            cp_tile -= 1;
+        }
+    };
+
+    for (int i = 0; i < n; i += DEPTH) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            if (i + d < n) compute(ring[d]);
+            issue(ring[d], i + d + DEPTH < n);
+        }
+    }
+    if (n > 0) dump(tile_hi - cur_tile);
+
+    // ---- the rotary table rows reach LDS (behind the partial sums)
+    float *const cs_s = reinterpret_cast<float *>(smem + p.red_off);  // [M][64], then the sines
+    float *const sn_s = cs_s + 16 * 64;
+    if (EPI == EPI_ROPE) {
+#pragma unroll
+        for (int i = 0; i < RE; ++i) {
+            const int idx = tid + i * NT;
+            if (idx < M * 64) {
+                cs_s[idx] = rp_cs[i];
+                sn_s[idx] = rp_sn[i];
+                if ((idx & 63) == 0) pos_s[idx >> 6] = rp_pos[i];
+            }
+        }
+    }
+
+    // ---- the lower workgroups' sums of the bottom strip
+    float part[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) part[v] = 0.f;
+    if (gets_partials) {
+        const int e_col = e_mine & 15, e_row = e_mine >> 4;  // piece 0: e = row * 16 + column
+        const int u_first = tile_lo * nb;
+        const int big = p.r * (p.q + 1);
+        const int first = u_first < big ? sdiv_magic(u_first, p.q + 1, p.q1_magic) : p.r + sdiv_magic(u_first - big, p.q, p.q_magic);
+        for (int src = first; src < wg; ++src) {
+            uint64_t *const slot = p.tagged + (size_t)src * slot_elems;
+            uint64_t got[NV];
+            uint32_t tries = p.spin_limit;
+            for (;;) {
+                uint64_t all = S_MARK;
+#pragma unroll
+                for (int v = 0; v < NV; ++v) {
+                    got[v] = __hip_atomic_load(&slot[(v * M + e_row) * 16 + e_col], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    all &= got[v];
+                }
+                if (p.spin_limit != 0xFFFFFFFFu && all != 0) break;
+                if (p.spin_limit == 0xFFFFFFFFu || --tries == 0) {
+                    __hip_atomic_store(&p.counters[EXCHANGE_ERROR_WORD], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(1);
+            }
+#pragma unroll
+            for (int v = 0; v < NV; ++v) {
+                part[v] += __uint_as_float((uint32_t)got[v]);
+                __hip_atomic_store(&slot[(v * M + e_row) * 16 + e_col], (uint64_t)0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+    }
+    __syncthreads();
+
+    for (int e = e_mine; e < total; e += NT) {
+        const int e_col = e & 15;
+        const int e_t = e >> 4;
+        const int e_pb = (e_t * p.m_magic) >> 16;
+        const int e_row = e_t - e_pb * M;
+        const int e_tile = tile_lo + e_pb;
+        const int pc = npieces - 1 - e_pb;
+        float s[NV];
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            s[v] = (e == e_mine) ? part[v] : 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) s[v] += redf[(((pc * NW + w) * NV + v) * 64 + (e_row >> 2) * 16 + e_col) * 4 + (e_row & 3)];
+        }
+        if (EPI == EPI_PLAIN) {
+            half_t o = (half_t)s[0];
+            if (p.bias != nullptr) o = o + p.bias[e_tile * 16 + e_col];
+            p.y[(size_t)e_row * N + e_tile * 16 + e_col] = o;
+        } else if (EPI == EPI_SILU_MUL) {
+            p.y[(size_t)e_row * N + e_tile * 16 + e_col] = (half_t)(silu_f32(s[0]) * s[NV - 1]);
+        } else {
+            const RopeArgs &ra = p.rope;
+            const int head_col = e_tile >> 2;
+            const int dd = ((e_tile & 3) << 4) + e_col;
+            const int which = head_col / ra.H;
+            const int head = head_col - which * ra.H;
+            int bb, ss;
+            split_row(ra, e_row, bb, ss);
+            float o1 = s[0], o2 = s[NV - 1];
+            if (which < 2) {
+                const float cs = cs_s[e_row * 64 + dd], sn = sn_s[e_row * 64 + dd];
+                o1 = s[0] * cs - s[NV - 1] * sn;
+                o2 = s[NV - 1] * cs + s[0] * sn;
+            }
+            half_t *dst;
+            size_t off;
+            if (which == 0) {
+                dst = ra.q;
+                off = ((size_t)(bb * ra.H + head) * ra.S + ss) * 128;
+            } else {
+                dst = (which == 1) ? ra.k : ra.v;
+                const int crow = ra.kv_offset >= 0 ? ra.kv_offset + ss : min(max(pos_s[e_row], 0), ra.kv_capacity - 1);
+                off = ((size_t)(bb * ra.H + head) * ra.kv_capacity + crow) * 128;
+            }
+            dst[off + dd] = (half_t)o1;
+            dst[off + 64 + dd] = (half_t)o2;
+        }
+    }
+}
+
 // ---- layout conversion ------------------------------------------------------------------------------------------
 // word o of the streaming order <-> (8-row block kb, column n) of the checkpoint order
 __device__ __forceinline__ void stream_coords(size_t o, int nb, int &kb, int &n) {
@@ -522,8 +821,35 @@ int launch_shape(const StreamArgs &a, const StreamPlan &pl, bool nomath, hipStre
     return perm ? launch_kernel<EPI, NW, DEPTH, true, 0, false>(a, pl, stream) : launch_kernel<EPI, NW, DEPTH, false, 0, false>(a, pl, stream);
 }
 
+template <int EPI, int NW, int DEPTH>
+int launch_tall(const StreamArgs &a, const StreamPlan &pl, hipStream_t stream) {
+    static bool prepared = false;
+    static std::mutex lock;
+    {
+        std::lock_guard<std::mutex> guard(lock);
+        if (!prepared) {
+            const void *fn = reinterpret_cast<const void *>(&gptq4_stream_tall_kernel<EPI, NW, DEPTH>);
+            const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)STREAM_LDS_BUDGET);
+            if (e != hipSuccess) return (int)e;
+            prepared = true;
+        }
+    }
+    hipLaunchKernelGGL((gptq4_stream_tall_kernel<EPI, NW, DEPTH>), dim3((unsigned)pl.workgroups), dim3(64 * NW), pl.lds_bytes, stream, a);
+    return (int)hipGetLastError();
+}
+
 template <int EPI>
 int launch_epi(const StreamArgs &a, const StreamPlan &pl, bool nomath, hipStream_t stream) {
+    if (pl.tall) {
+        if (nomath || a.perm != nullptr || a.nrm_weight != nullptr) return (int)hipErrorInvalidValue;
+        switch (pl.waves * 10 + pl.depth) {
+            case 81: return launch_tall<EPI, 8, 1>(a, pl, stream);
+            case 82: return launch_tall<EPI, 8, 2>(a, pl, stream);
+            case 161: return launch_tall<EPI, 16, 1>(a, pl, stream);
+            case 162: return launch_tall<EPI, 16, 2>(a, pl, stream);
+            default: return (int)hipErrorInvalidValue;
+        }
+    }
     switch (pl.waves * 10 + pl.depth) {
         case 81: return launch_shape<EPI, 8, 1>(a, pl, nomath, stream);
         case 82: return launch_shape<EPI, 8, 2>(a, pl, nomath, stream);
@@ -559,6 +885,25 @@ StreamPlan stream_plan(int epi, int M, int N, int K, bool norm) {
     if (!g_stream_tuning.waves && pl.nb < pl.waves) pl.waves = 8;
     if (pl.waves == 16 && pl.depth > 2) pl.depth = 2;
     pl.pieces = (pl.q + 1 + pl.nb - 1) / pl.nb + 1;
+    if (M > STREAM_MAX_M) {
+        // 5 .. 16 rows: the A operand comes from memory with every unit, LDS holds the waves' partial sums (1 KiB per
+        // wave, matrix and strip) and the rotary table rows of the tokens
+        pl.tall = true;
+        if (pl.depth > 2) pl.depth = 2;
+        // eight waves for every shape here (LLaMA-7B down_proj at 16 rows: 11.2 us against 11.7 with sixteen)
+        if (!g_stream_tuning.waves) pl.waves = 8;
+        pl.xrow = 0;
+        pl.red_off = pl.pieces * pl.waves * nv * 64;
+        pl.nat_off = pl.red_off + 2 * 16 * 64 * (int)sizeof(float) / 16;  // behind the rotary table rows: a 16 x 17 chunk slot per wave
+        size_t lds = ((size_t)pl.nat_off + (size_t)pl.waves * 16 * 17) * 16;
+        if (lds < (size_t)81 * 1024) lds = (size_t)81 * 1024;
+        pl.lds_bytes = lds;
+        pl.ok = M <= STREAM_TALL_MAX_M && !norm && lds <= STREAM_LDS_BUDGET && (long)K * N < (1L << 32) && (long)M * K < (1L << 30) &&
+                units < (1L << 24) && units * (pl.nb > pl.q + 1 ? pl.nb : pl.q + 1) < (1L << 32) &&
+                (size_t)pl.workgroups * nv * 16 * M * sizeof(uint64_t) <= GPTQ4_WS_TAGGED_BYTES && pl.nb >= pl.waves &&
+                (epi != EPI_ROPE || (N % 128) == 0);
+        return pl;
+    }
     pl.xrow = K / 8 + 1;
     pl.red_off = M * pl.xrow;
     const size_t red_chunks = (size_t)pl.pieces * pl.waves * nv * 16;  // one 16-byte chunk (four rows) per column

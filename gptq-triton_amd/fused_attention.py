@@ -162,7 +162,8 @@ def qkv_rotary_stream(groupsize: int, hidden_states: torch.Tensor, sweight: torc
         x2d, d2, s = check_norm_args(hidden_states, delta, norm_weight)
         delta_p, nw_p, sum_p = _lib.ptr(d2), norm_weight.data_ptr(), _lib.ptr(s)
     lib = _lib.load()
-    ws = _lib.workspace(dev, _lib.WS_HEAD_BYTES)
+    rows = bsz * q_len
+    ws = _lib.workspace(dev, _lib.WS_HEAD_BYTES + (2 * rows * k_in if perm is not None and rows > 4 else 0))
     rc = lib.gptq4_stream_qkv_rotary(x2d.data_ptr(), delta_p, nw_p, float(eps), sum_p, sweight.data_ptr(), smeta.data_ptr(),
                                      _lib.ptr(perm), pos.data_ptr(), cos.data_ptr(), sin.data_ptr(), cos.shape[0], q.data_ptr(),
                                      kk.data_ptr(), vv.data_ptr(), bsz, q_len, num_heads, head_dim, k_in, groupsize, cap, off,
@@ -266,8 +267,10 @@ class QuantLlamaAttention(nn.Module):
         else:
             need = max(kv_offset, 0) + hidden_states.shape[1]
         cos, sin = self.rope.get(hidden_states.device, max(need, self.max_position_embeddings))
-        sw = self.qkv_proj.stream_weights(hidden_states.shape[0] * hidden_states.shape[1])
-        if sw is not None:
+        rows = hidden_states.shape[0] * hidden_states.shape[1]
+        sw = self.qkv_proj.stream_weights(rows)
+        from .decoder_ops import NORM_MAX_ROWS
+        if sw is not None and (norm is None or rows <= NORM_MAX_ROWS):
             return qkv_rotary_stream(self.qkv_proj.groupsize, hidden_states, sw[0], sw[1], position_ids, cos, sin, self.num_heads,
                                      self.head_dim, perm=None if ordered else sw[2], kv_out=kv_out, kv_offset=kv_offset, norm=norm)
         qweight, perm = self.qkv_proj.kernel_weights()

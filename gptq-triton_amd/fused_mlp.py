@@ -94,7 +94,7 @@ def llama_mlp_4_stream(groupsize: int, a: torch.Tensor, gate_sweight: torch.Tens
     m = x.shape[0]
     c = torch.empty((m, n), device=a.device, dtype=torch.float16)
     if m:
-        ws = _lib.workspace(a.device, _lib.WS_HEAD_BYTES)
+        ws = _lib.workspace(a.device, _lib.WS_HEAD_BYTES + (2 * m * k if perm is not None and m > 4 else 0))
         rc = lib.gptq4_stream_mlp_gateup(x.data_ptr(), delta_p, nw_p, float(eps), sum_p, gate_sweight.data_ptr(), gate_smeta.data_ptr(),
                                          up_sweight.data_ptr(), up_smeta.data_ptr(), _lib.ptr(perm), c.data_ptr(), m, k, n, groupsize,
                                          ws.data_ptr(), ws.numel(), _lib.current_stream(a.device))
@@ -339,7 +339,8 @@ class QuantLlamaMLP(nn.Module):
 
     def forward_normed(self, h: torch.Tensor, delta: Optional[torch.Tensor], norm_weight: torch.Tensor, eps: float):
         """(h + delta, forward(RMSNorm(h + delta))): the residual add and the norm run inside the gate/up launch."""
-        if self._stream_ready(h):
+        from .decoder_ops import NORM_MAX_ROWS
+        if self._stream_ready(h) and h.numel() // self.infeatures <= NORM_MAX_ROWS:
             s, mid = llama_mlp_4_stream(self.groupsize, h, self.gate_proj_qweight, self._gate_meta, self.up_proj_qweight, self._up_meta,
                                         self._compact_rows, norm=(delta, norm_weight, eps))
             return s, self.down_proj.multiply(mid, ordered=True)

@@ -24,7 +24,7 @@ from .fused_attention import LlamaConfigLite
 # up to this many rows the decoder's norms write act-order inputs in their consumer's order
 ORDERED_NORM_ROWS = 16
 # up to this many sequences a GreedyDecoder asks for the streaming-order weight layout (the rows its kernel takes)
-STREAM_BATCH = 4
+STREAM_BATCH = 16
 
 
 def config_from_json(path) -> LlamaConfigLite:

@@ -196,7 +196,8 @@ def matmul4_stream(groupsize: int, a: torch.Tensor, sweight: torch.Tensor, smeta
     c = torch.empty((m, n), device=a.device, dtype=torch.float16)
     if m == 0:
         return c.view(a.shape[:-1] + (n,))
-    ws = _lib.workspace(a.device, _lib.WS_HEAD_BYTES)
+    # (more than four rows of an act-order projection are gathered into the workspace first)
+    ws = _lib.workspace(a.device, _lib.WS_HEAD_BYTES + (2 * m * k if perm is not None and m > 4 else 0))
     rc = lib.gptq4_stream_matmul(x.data_ptr(), sweight.data_ptr(), smeta.data_ptr(), _lib.ptr(perm), _lib.ptr(bias), c.data_ptr(),
                                  m, k, n, groupsize, ws.data_ptr(), ws.numel(), _lib.current_stream(a.device))
     _lib.check(rc, "gptq4_stream_matmul")

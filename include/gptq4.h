@@ -239,8 +239,9 @@ int gptq4_decode_attention(const void *q, const void *k_cache, const void *v_cac
  * resident (the conversion is exact both ways).  For act-order, convert the row-sorted weight and pass `perm` as to
  * the plain entry points. */
 
-/* Most rows (M) the streaming-order entry points take for this operator and shape; 0: the shape is not supported
- * (K below 1024, or rows / partial sums that do not fit a CU's LDS).  `op` is a GPTQ4_OP_* matmul selector, N = I
+/* Most rows (M) the streaming-order entry points take for this operator and shape (at most 16); 0: the shape is not
+ * supported (K below 1024, or partial sums that do not fit a CU's LDS).  Up to 4 rows the kernel keeps the rows in LDS;
+ * from 5 rows on a variant fetches them with every block of weights.  `op` is a GPTQ4_OP_* matmul selector, N = I
  * for MLP_GATEUP, N = 3*H*D for QKV_ROTARY. */
 int gptq4_stream_rows(int op, int K, int N, int groupsize);
 
@@ -258,8 +259,9 @@ int gptq4_stream_dequant(const int32_t *sweight, const int32_t *smeta, void *W_o
  * (more rows: -GPTQ4_E_SHAPE).  Same arithmetic (fp16 weights of the formula above, fp32 accumulation, one rounding)
  * - only the order in which the fp32 partial sums are added differs, fixed for a shape and GPU.  The two fused
  * entry points take the residual add + RMSNorm of their input along when norm_weight is not NULL (delta, sum_out
- * as in gptq4_norm_qkv_rotary; bit-identical to gptq4_add_rmsnorm followed by the plain call; K <= 8192).
- * workspace: GPTQ4_WS_HEAD_BYTES, zero before the first call. */
+ * as in gptq4_norm_qkv_rotary; bit-identical to gptq4_add_rmsnorm followed by the plain call; K <= 8192, M <= 4).
+ * workspace: GPTQ4_WS_HEAD_BYTES, zero before the first call; a call with `perm` and more than 4 rows gathers the
+ * rows into the workspace first (one small launch) and needs M * K * 2 bytes behind the head. */
 int gptq4_stream_matmul(const void *x, const int32_t *sweight, const int32_t *smeta, const int32_t *perm,
                         const void *bias, void *y, int M, int K, int N, int groupsize, void *workspace,
                         size_t workspace_bytes, void *stream);

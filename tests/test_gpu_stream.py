@@ -99,7 +99,7 @@ def test_dequant_from_the_streaming_order_exhaustive_q_z_scale():
 
 # ------------------------------------------------------------------ the three operators
 @pytest.mark.parametrize("k,n,g", SHAPES)
-@pytest.mark.parametrize("m", [1, 2, 3, 4])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 8, 13, 16])
 def test_matmul(k, n, g, m):
     G = gptq()
     L = O.make_layer(k, n, g, seed=1000 + k + n, bias=(m == 2))
@@ -138,7 +138,7 @@ def test_matmul_in_every_launch_shape(waves, depth):
             L = O.make_layer(k, n, g, seed=1100 + k)
             D = to_dev(L)
             sw, meta = G.stream_pack(D["qweight"], D["qzeros"], D["scales"], g)
-            for m in (1, 4):
+            for m in (1, 4) + ((9, 16) if depth <= 2 else ()):
                 x = O.make_x(m, k, seed=m)
                 y = G.matmul4_stream(g, torch.from_numpy(x).cuda(), sw, meta)
                 assert_close(y.cpu().numpy(), O.quant_matmul_ref(x, L["qweight"], L["qzeros"], L["scales"], g), f"{waves}x{depth} {k}x{n} M={m}")
@@ -161,10 +161,17 @@ def test_one_hot_rows_return_weight_rows_exactly():
             x[i, r] = 1.0
         y = G.matmul4_stream(g, torch.from_numpy(x).cuda(), sw, meta)
         assert (bits(y.cpu().numpy()) == bits(w[rows])).all()
+    # sixteen rows: the kernel that fetches its rows with every unit
+    rows = [0, 1, 7, 8, 31, 32, 127, 128, 129, 1000, 2047, 2048, 3000, 4000, 4094, 4095]
+    x = np.zeros((16, k), dtype=np.float16)
+    for i, r in enumerate(rows):
+        x[i, r] = 1.0
+    y = G.matmul4_stream(g, torch.from_numpy(x).cuda(), sw, meta)
+    assert (bits(y.cpu().numpy()) == bits(w[rows])).all()
 
 
 @pytest.mark.parametrize("k,n,g", [(1024, 512, 128), (4096, 4096, 128), (5120, 5120, 128)])
-@pytest.mark.parametrize("m", [1, 3])
+@pytest.mark.parametrize("m", [1, 3, 6, 16])
 def test_matmul_act_order(k, n, g, m):
     """Rows sorted by group first (gptq4_actorder_sort_rows), then streaming order; x gathered through perm inside the kernel."""
     G = gptq()
@@ -179,7 +186,7 @@ def test_matmul_act_order(k, n, g, m):
 
 
 @pytest.mark.parametrize("k,inter,g", [(1024, 2816, 128), (4096, 11008, 128), (5120, 13824, 128), (6656, 17920, 512)])
-@pytest.mark.parametrize("m", [1, 2, 4])
+@pytest.mark.parametrize("m", [1, 2, 4, 5, 11, 16])
 def test_mlp_gateup(k, inter, g, m):
     G = gptq()
     gate, up = O.make_layer(k, inter, g, seed=1400 + k), O.make_layer(k, inter, g, seed=1401 + k)
@@ -196,7 +203,7 @@ def test_mlp_gateup(k, inter, g, m):
 
 
 @pytest.mark.parametrize("k,heads,g", [(1024, 8, -1), (4096, 32, -1), (4096, 32, 128), (5120, 40, 128), (6656, 52, 512)])
-@pytest.mark.parametrize("m", [1, 4])
+@pytest.mark.parametrize("m", [1, 4, 7, 16])
 def test_qkv_rotary_and_cache_rows(k, heads, g, m):
     G = gptq()
     n = 3 * heads * 128
@@ -207,7 +214,7 @@ def test_qkv_rotary_and_cache_rows(k, heads, g, m):
         pytest.skip("shape outside what the streaming-order kernel takes")
     sw, meta = G.stream_pack(D["qweight"], D["qzeros"], D["scales"], gs)
     x = O.make_x(m, k, seed=m + 60).reshape(m, 1, k)
-    pos = (np.arange(m)[:, None] * 37 + 2047 - 37 * (m - 1)).astype(np.int64)
+    pos = (np.arange(m)[:, None] * 37 + 2047 - 37 * (m - 1)).astype(np.int64)  # distinct, the last one at the table's end
     cos, sin = G.RotaryTable(128, 2048).get(torch.device("cuda"), 2048)
     xd, posd = torch.from_numpy(x).cuda(), torch.from_numpy(pos).cuda()
     q, kk, vv = G.qkv_rotary_stream(gs, xd, sw, meta, posd, cos, sin, heads)
@@ -317,12 +324,14 @@ def test_host_side_argument_errors():
     lib = _lib.load()
     fake, ws = 0x1000, _lib.WS_HEAD_BYTES
     assert lib.gptq4_stream_matmul(None, fake, fake, None, None, fake, 1, 4096, 4096, 128, fake, ws, None) == -1
-    assert lib.gptq4_stream_matmul(fake, fake, fake, None, None, fake, 5, 4096, 4096, 128, fake, ws, None) == -2     # more rows than the kernel takes
+    assert lib.gptq4_stream_matmul(fake, fake, fake, None, None, fake, 17, 4096, 4096, 128, fake, ws, None) == -2    # more rows than the kernels take
+    assert lib.gptq4_stream_matmul(fake, fake, fake, fake, None, fake, 5, 4096, 4096, 128, fake, ws, None) == -4     # act-order above four rows: room for the gathered rows
+    assert lib.gptq4_stream_mlp_gateup(fake, None, fake, 1e-6, None, fake, fake, fake, fake, None, fake, 5, 4096, 11008, 128, fake, ws, None) == -2  # norm inside: four rows
     assert lib.gptq4_stream_matmul(fake, fake, fake, None, None, fake, 1, 512, 4096, 128, fake, ws, None) == -2      # K too short for its waves
     assert lib.gptq4_stream_matmul(fake, fake, fake, None, None, fake, 1, 4096, 4096, 96, fake, ws, None) == -3
     assert lib.gptq4_stream_matmul(fake, fake, fake, None, None, fake, 1, 4096, 4096, 128, fake, 64, None) == -4
     assert lib.gptq4_stream_matmul(fake + 2, fake, fake, None, None, fake, 1, 4096, 4096, 128, fake, ws, None) == -5
-    assert lib.gptq4_stream_rows(0, 4096, 4096, 128) == 4 and lib.gptq4_stream_rows(0, 512, 4096, 128) == 0
+    assert lib.gptq4_stream_rows(0, 4096, 4096, 128) == 16 and lib.gptq4_stream_rows(0, 512, 4096, 128) == 0
     assert lib.gptq4_stream_rows(0, 4096, 4100, 128) == 0
 
 
@@ -351,9 +360,9 @@ def test_quant_linear_in_streaming_order(act):
     q = q.cuda()
     before = {name: t.clone() for name, t in q.state_dict().items()}
     w_before = q.dequantize()
-    assert q.to_stream() and q._stream_rows == 4
+    assert q.to_stream() and q._stream_rows == 16
     assert q.qweight.shape == before["qweight"].shape and not torch.equal(q.qweight, before["qweight"])
-    for m in (1, 4, 33):   # 33 rows: unpacked for the duration of the call, tiled kernels
+    for m in (1, 4, 9, 16, 33):   # 33 rows: unpacked for the duration of the call, tiled kernels
         x = O.make_x(m, k, seed=m)
         y = q(torch.from_numpy(x).cuda())
         ref = O.quant_matmul_ref(x, L["qweight"], L["qzeros"], L["scales"], g, bias=L["bias"], g_idx=L["g_idx"] if act else None)
@@ -387,8 +396,13 @@ def test_fused_mlp_in_streaming_order(act):
     x = O.make_x(3, k, seed=5)
     xd = torch.from_numpy(x).cuda()
     y_ckpt = mlp(xd)
+    x12 = torch.from_numpy(O.make_x(12, k, seed=7)).cuda()
+    y12_ckpt = mlp(x12)
     assert mlp.to_stream() and mlp.down_proj._stream_meta is not None
     y = mlp(xd)
+    # twelve rows: the streaming-order kernel for 5 .. 16 rows (an act-order block's rows are gathered by a launch before it)
+    ok, max_abs, _ = O.within_tolerance(mlp(x12).float().cpu().numpy(), y12_ckpt.float().cpu().numpy())
+    assert ok, max_abs
     # same fp16 intermediate up to the order of the fp32 sums: compare both against the oracle's composed result
     trip = lambda d: (d["qweight"], d["qzeros"], d["scales"])
     if not act:
