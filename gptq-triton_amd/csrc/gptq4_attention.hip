@@ -1,0 +1,207 @@
+// Causal attention over a prompt for gfx950 (head dimension 128): the pass between the fused QKV + rotary projection,
+// whose q and KV-cache rows it reads where they lie, and o_proj, whose input [B, S, H * 128] it writes directly.
+// (The reference hands this step to torch's scaled_dot_product_attention and transposes the result,
+// fused_attention.py:117-141; with a 2048-token prompt it is a sixth of the prompt pass.)
+//
+// One workgroup of four waves per 128 queries of one head, a wave per 32 queries; the keys come in blocks of 64
+// through LDS, shared by the four waves.  Both products run on v_mfma_f32_32x32x16_f16 in their TRANSPOSED form, so
+// that what one produces is what the next consumes without leaving the lane:
+//   S^T = K Q^T   A = 32 keys x 16 dims out of LDS (rows 256 bytes apart, 16-byte chunks XOR-swizzled by the key),
+//                 B = the wave's queries, in registers for the whole kernel; lane (h, q) then holds, for its query
+//                 column q, the scores of keys 8 * i + 4 * h + j of each half block (register 4 * i + j);
+//   O^T = V^T P^T A = 32 dims x 16 keys, B = 16 keys x 32 queries: the lane's own probabilities, registers 8 * u .. 8 * u + 7
+//                 of a half block for step u.  That fixes which key sits in which of the 16 contraction slots of a
+//                 step - slot 8 * h + t is key 4 * h + t (t < 4) or 8 + 4 * h + t - 4 - and V^T is written to LDS with
+//                 its keys in that order (the two middle groups of four swapped), rows of 64 keys = 128 bytes apart,
+//                 chunks swizzled by the dimension.
+// The softmax runs per lane on its own query column (one exchange per block with the other half-wave for the running
+// maximum; the row sums meet once, at the end), in base 2 with the scale folded in.  Blocks beyond a wave's last
+// visible key are skipped by that wave; the heaviest workgroups (last queries) are launched first.
+#include "../../include/gptq4.h"
+#include "gptq4_internal.h"
+
+namespace {
+
+typedef float f16x_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ int key_slot(int key) {  // position of a key of a 64-key block in V^T's row
+    const int o = key & 15;
+    return (key & ~15) | (o < 4 ? o : o < 8 ? o + 4 : o < 12 ? o - 4 : o);
+}
+
+__global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t *__restrict__ q, const half_t *__restrict__ kc,
+                                                                    const half_t *__restrict__ vc, half_t *__restrict__ out, int H,
+                                                                    int S, int capacity, int past, float scale_log2e) {
+    __shared__ uint4 k_s[64 * 16];  // [key][16 chunks of 8 dims], chunk c of key k at c ^ (k & 7)
+    __shared__ uint4 v_s[128 * 8];  // [dim][8 chunks of 8 key slots], chunk c of dim d at c ^ (d & 7)
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int h = lane >> 5, c32 = lane & 31;
+    const int qb = (int)gridDim.x - 1 - (int)blockIdx.x;
+    const int bh = blockIdx.y;
+    const int q0 = qb * 128 + wave * 32;  // first query of the wave
+    const int kv_len = past + S;
+
+    // ---- the wave's queries: B operand of S^T, lane (h, q): dims 16 * ks + 8 * h .. + 7
+    h8_t qf[8];
+    {
+        const int row = min(q0 + c32, S - 1);
+        const uint4 *qp = reinterpret_cast<const uint4 *>(q + ((size_t)bh * S + row) * 128);
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) qf[ks] = __builtin_bit_cast(h8_t, qp[2 * ks + h]);
+    }
+    f16x_t o[4];
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[db][i] = 0.f;
+    float m = -INFINITY, l = 0.f;
+
+    const int kmax = min(kv_len, past + (qb + 1) * 128);  // keys any query of the workgroup sees
+    const int nblk = (kmax + 63) >> 6;
+    const int my_last = past + min(q0 + 31, S - 1);      // last key the wave's last query sees
+    const int my_first = past + q0;                      // last key its first query sees
+    const half_t *kb = kc + (size_t)bh * capacity * 128;
+    const half_t *vb = vc + (size_t)bh * capacity * 128;
+
+    // ---- staging: K chunk id = tid + 256 * n -> (key id / 16, chunk id % 16): whole rows per 16 lanes;
+    //      V chunk (key tid % 64, chunk tid / 64 + 4 * n): a wave writes 64 consecutive key slots of one dimension
+    u32x4_t kr[4], vr[4];
+#define FETCH_BLOCK(blk)                                                                                             \
+    _Pragma("unroll") for (int n = 0; n < 4; ++n) {                                                                  \
+        const int id = tid + 256 * n;                                                                                \
+        const int key = min((blk) * 64 + (id >> 4), kv_len - 1);                                                     \
+        kr[n] = *reinterpret_cast<const u32x4_t *>(kb + (size_t)key * 128 + 8 * (id & 15));                            \
+        const int vkey = min((blk) * 64 + (tid & 63), kv_len - 1);                                                   \
+        vr[n] = *reinterpret_cast<const u32x4_t *>(vb + (size_t)vkey * 128 + 8 * ((tid >> 6) + 4 * n));                \
+    }
+    const int vslot = key_slot(tid & 63);
+    uint16_t *const v16 = reinterpret_cast<uint16_t *>(v_s);
+    FETCH_BLOCK(0)
+    for (int blk = 0; blk < nblk; ++blk) {
+        __syncthreads();  // the block before has been read
+#pragma unroll
+        for (int n = 0; n < 4; ++n) {
+            const int id = tid + 256 * n;
+            const int key = id >> 4, c = id & 15;
+            k_s[key * 16 + (c ^ (key & 7))] = __builtin_bit_cast(uint4, kr[n]);
+            const int dc = (tid >> 6) + 4 * n;
+            auto put = [&](int e, uint32_t w) {  // halves e and e + 1: dims 8 * dc + e, + 1 (d & 7 = e: dc * 8 is a multiple of 8)
+                const int d = 8 * dc + e;
+                v16[d * 64 + (((vslot >> 3) ^ e) << 3) + (vslot & 7)] = (uint16_t)w;
+                v16[(d + 1) * 64 + (((vslot >> 3) ^ (e + 1)) << 3) + (vslot & 7)] = (uint16_t)(w >> 16);
+            };
+            put(0, vr[n].x);
+            put(2, vr[n].y);
+            put(4, vr[n].z);
+            put(6, vr[n].w);
+        }
+        __syncthreads();
+        if (blk + 1 < nblk) {
+            FETCH_BLOCK(blk + 1)
+        }
+        const int key0 = blk * 64;
+        if (key0 > my_last) continue;  // nothing in this block is visible to the wave (it still takes part in the staging)
+
+        // ---- S^T = K Q^T for the two half blocks of 32 keys
+        f16x_t s[2];
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s[rb][i] = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) {
+                const int key = 32 * rb + c32;
+                const h8_t a = __builtin_bit_cast(h8_t, k_s[key * 16 + ((2 * ks + h) ^ (key & 7))]);
+                s[rb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[ks], s[rb], 0, 0, 0);
+            }
+        }
+        // ---- scale, mask, running maximum
+        const bool mask = key0 + 63 > my_first;
+        const int limit = past + q0 + c32;  // last key this lane's query sees
+        float mx = -INFINITY;
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                float val = s[rb][i] * scale_log2e;
+                if (mask) {
+                    const int key = key0 + 32 * rb + 8 * (i >> 2) + 4 * h + (i & 3);
+                    if (key > limit) val = -INFINITY;
+                }
+                s[rb][i] = val;
+                mx = fmaxf(mx, val);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m, mx);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // (a query beyond S in a clamped row: nothing visible yet)
+        const float corr = __builtin_amdgcn_exp2f(m - m_use);
+        float sum = 0.f;
+        h8_t pf[2][2];
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    const float pv = __builtin_amdgcn_exp2f(s[rb][8 * u + t] - m_use);
+                    sum += pv;
+                    pf[rb][u][t] = (_Float16)pv;
+                }
+        l = l * corr + sum;
+        m = m_new;
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) o[db][i] *= corr;
+        // ---- O^T += V^T P^T
+#pragma unroll
+        for (int db = 0; db < 4; ++db) {
+            const int d = 32 * db + c32;
+#pragma unroll
+            for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+                for (int u = 0; u < 2; ++u) {
+                    const h8_t a = __builtin_bit_cast(h8_t, v_s[d * 8 + ((4 * rb + 2 * u + h) ^ (d & 7))]);
+                    o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pf[rb][u], o[db], 0, 0, 0);
+                }
+        }
+    }
+
+    // ---- out[b, s, head * 128 + d] = O[s, d] / l: lane (h, q) holds dims 32 * db + 8 * i + 4 * h + j of its query
+    l += __shfl_xor(l, 32);
+    const int row = q0 + c32;
+    if (row < S) {
+        const float inv = 1.0f / l;
+        const int b = bh / H, head = bh - b * H;
+        half_t *dst = out + (((size_t)b * S + row) * H + head) * 128;
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                h2_t lo, hi;
+                lo.x = (half_t)(o[db][4 * i] * inv);
+                lo.y = (half_t)(o[db][4 * i + 1] * inv);
+                hi.x = (half_t)(o[db][4 * i + 2] * inv);
+                hi.y = (half_t)(o[db][4 * i + 3] * inv);
+                uint2 w;
+                w.x = __builtin_bit_cast(uint32_t, lo);
+                w.y = __builtin_bit_cast(uint32_t, hi);
+                *reinterpret_cast<uint2 *>(dst + 32 * db + 8 * i + 4 * h) = w;
+            }
+    }
+}
+
+#undef FETCH_BLOCK
+
+}  // namespace
+
+int launch_attn_prefill(const half_t *q, const half_t *kc, const half_t *vc, half_t *out, int B, int H, int S, int capacity, int past,
+                        float scale, hipStream_t stream) {
+    const int qblocks = (S + 127) / 128;
+    hipLaunchKernelGGL(gptq4_attn_prefill_kernel, dim3((unsigned)qblocks, (unsigned)(B * H)), dim3(256), 0, stream, q, kc, vc, out, H, S,
+                       capacity, past, scale * 1.4426950408889634f);
+    return (int)hipGetLastError();
+}

@@ -101,6 +101,31 @@ def add_rms_norm(x: torch.Tensor, delta: torch.Tensor, weight: torch.Tensor, eps
     return s.reshape(x.shape), y.reshape(x.shape)
 
 
+def prefill_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, past: int = 0) -> torch.Tensor:
+    """Causal attention of a prompt (or of a chunk behind `past` cached tokens): q fp16 [B, H, S, 128]; caches fp16
+    [B, H, capacity, 128] holding the S new tokens in rows past .. past + S - 1 (for a plain prompt: the k and v the QKV
+    projection returned); query i attends to rows 0 .. past + i.  Returns fp16 [B, S, H*128], what o_proj consumes."""
+    for t, name in ((q, "q"), (k_cache, "k_cache"), (v_cache, "v_cache")):
+        _lib.require_cuda(t, name)
+        if t.dtype != torch.float16:
+            raise TypeError("prefill_attention takes fp16 tensors")
+    bsz, heads, q_len, hd = q.shape
+    if hd != 128:
+        raise ValueError("prefill_attention needs head_dim 128")
+    if k_cache.shape != v_cache.shape or k_cache.shape[:2] != (bsz, heads) or k_cache.shape[3] != hd \
+            or not (q.is_contiguous() and k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise ValueError("caches must be contiguous [B, H, capacity, 128] tensors matching q")
+    cap = k_cache.shape[2]
+    if past < 0 or past + q_len > cap:
+        raise ValueError("the cache has no room for past + S rows")
+    out = torch.empty((bsz, q_len, heads * hd), dtype=torch.float16, device=q.device)
+    if q_len:
+        rc = _lib.load().gptq4_prefill_attention(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(), bsz, heads, q_len,
+                                                 hd, cap, past, 1.0 / math.sqrt(hd), _lib.current_stream(q.device))
+        _lib.check(rc, "gptq4_prefill_attention")
+    return out
+
+
 def decode_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, positions: torch.Tensor,
                      out_index: torch.Tensor = None) -> torch.Tensor:
     """q fp16 [B, H, 1, 128]; caches fp16 [B, H, capacity, 128]; positions int32 [B] or [B, 1]:

@@ -222,6 +222,16 @@ int gptq4_decode_attention(const void *q, const void *k_cache, const void *v_cac
                            int kv_capacity, float scale, void *workspace,
                            size_t workspace_bytes, void *stream);
 
+/* Causal attention of S query tokens per sequence (a prompt, or a chunk of one behind `past` cached tokens): query i
+ * attends to cache rows 0 .. past + i; softmax in fp32, output fp16 out [B, S, H*D] - the layout o_proj consumes, no
+ * transpose.  q fp16 [B, H, S, D] (as gptq4_qkv_rotary writes it); k_cache, v_cache fp16 [B, H, kv_capacity, D] with
+ * the S new tokens already in rows past .. past + S - 1 (gptq4_qkv_rotary with kv_offset = past puts them there; for
+ * a plain prompt its k / v outputs serve as caches of capacity S).  D must be 128, past + S <= kv_capacity.  No
+ * workspace.  Replaces the attention core of QuantLlamaAttention.forward for a prompt (fused_attention.py:117-141:
+ * scores, causal mask, fp32 softmax, weighted sum, transpose + reshape). */
+int gptq4_prefill_attention(const void *q, const void *k_cache, const void *v_cache, void *out, int B, int H, int S,
+                            int D, int kv_capacity, int past, float scale, void *stream);
+
 /* ---- Streaming-order weight layout: what the decode kernel for a handful of rows reads -------------------------
  * A decode GEMV streams every weight once; what bounds it on this GPU is how long a launch runs with nothing in
  * flight and how many separate requests a CU has to make per byte.  In streaming order the packed words of one strip

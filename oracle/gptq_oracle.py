@@ -360,6 +360,26 @@ def decode_attention_ref(q: np.ndarray, k_cache: np.ndarray, v_cache: np.ndarray
     return out
 
 
+def prefill_attention_ref(q: np.ndarray, k_cache: np.ndarray, v_cache: np.ndarray, past: int = 0) -> np.ndarray:
+    """Causal attention of S query tokens behind `past` cached ones, in float64: query i of (b, h) attends to cache
+    rows 0 .. past + i; returns [B, S, H*D] (src/gptq_triton/fused_attention.py:117-141 with the causal mask of
+    modeling_llama: scores, mask, fp32 softmax, weighted sum, transpose + reshape).  Pinned by: every query row
+    equals decode_attention_ref at position past + i, and torch's scaled_dot_product_attention(is_causal=True) on
+    the CPU (tests/test_oracle.py)."""
+    q = np.asarray(q, dtype=np.float64)
+    bsz, heads, s_len, hd = q.shape
+    out = np.zeros((bsz, s_len, heads * hd))
+    for b in range(bsz):
+        for h in range(heads):
+            k = np.asarray(k_cache[b, h, :past + s_len], dtype=np.float64)
+            v = np.asarray(v_cache[b, h, :past + s_len], dtype=np.float64)
+            sc = q[b, h] @ k.T / np.sqrt(hd)                                       # [S, past + S]
+            sc = np.where(np.arange(past + s_len)[None, :] <= past + np.arange(s_len)[:, None], sc, -np.inf)
+            w = np.exp(sc - sc.max(axis=1, keepdims=True))
+            out[b, :, h * hd:(h + 1) * hd] = (w / w.sum(axis=1, keepdims=True)) @ v
+    return out
+
+
 # ---- streaming order of the packed words (the build's own load-time re-layout; no reference counterpart) ----------
 # Pinned by: stream_order_loops (the definition, word by word) == stream_order (index arithmetic) on small shapes;
 # unstream(stream_order(q)) == q; and the library's dequantisation FROM the streaming order must reproduce

@@ -298,3 +298,21 @@ def test_decode_attention_oracle_special_cases():
     # rows beyond the position are invisible
     v2 = v.copy(); v2[:, :, 5:] = 1e4
     assert np.array_equal(O.decode_attention_ref(q, k, v, [4, 4]), O.decode_attention_ref(q, k, v2, [4, 4]))
+
+
+def test_prefill_attention_ref_is_the_single_query_form_row_by_row_and_torchs_causal_attention():
+    import torch
+    rng = np.random.default_rng(7)
+    b, h, s, past, d = 2, 3, 9, 4, 128
+    q = rng.standard_normal((b, h, s, d)).astype(np.float16)
+    k = rng.standard_normal((b, h, past + s + 2, d)).astype(np.float16)
+    v = rng.standard_normal((b, h, past + s + 2, d)).astype(np.float16)
+    out = O.prefill_attention_ref(q, k, v, past)
+    for i in range(s):
+        one = O.decode_attention_ref(q[:, :, i:i + 1], k, v, [past + i] * b)
+        assert np.allclose(out[:, i], one[:, 0], rtol=0, atol=1e-12)
+    # no past: the library routine with its own causal mask
+    out0 = O.prefill_attention_ref(q, k, v, 0)
+    tq, tk, tv = (torch.from_numpy(a.astype(np.float64)) for a in (q, k[:, :, :s], v[:, :, :s]))
+    ref = torch.nn.functional.scaled_dot_product_attention(tq, tk, tv, is_causal=True).transpose(1, 2).reshape(b, s, h * d)
+    assert np.allclose(out0, ref.numpy(), rtol=0, atol=1e-10)
