@@ -167,11 +167,13 @@ def decoder_figures(workload, bsz, prompt, new, steps=None, warmup=None):
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     first = dec.prefill(ids)
+    enqueue_s = time.perf_counter() - t0  # the host's share: every launch of the prompt pass is issued from Python
     torch.cuda.synchronize()
     prefill_s = time.perf_counter() - t0
     per_token_kn = layers * (hidden * 3 * hidden + hidden * hidden + 2 * hidden * inter + inter * hidden)
     prefill_tf = 2.0 * bsz * prompt * per_token_kn / prefill_s / 1e12
-    log(f"prefill: {prefill_s * 1e3:.1f} ms for {bsz} x {prompt} tokens = {prefill_tf:.0f} TFLOP/s in the quantised linears")
+    log(f"prefill: {prefill_s * 1e3:.1f} ms for {bsz} x {prompt} tokens = {prefill_tf:.0f} TFLOP/s in the quantised linears "
+        f"(the host needed {enqueue_s * 1e3:.1f} ms to issue its launches)")
 
     eager_steps = min(eager_steps, new - 1)
     torch.cuda.synchronize()
@@ -220,7 +222,8 @@ def decoder_figures(workload, bsz, prompt, new, steps=None, warmup=None):
                      "kernel": "whole decode step: packed weights + fp16 lm_head + the full-capacity KV cache, read once",
                      "bytes_per_launch": step_bytes, "avg_launch_us": round(step_s * 1e6, 1)},
         "cpu_baseline": None,
-        "extra": {"prefill_ms": round(prefill_s * 1e3, 2), "prefill_linear_TFLOPs": round(prefill_tf, 1),
+        "extra": {"prefill_ms": round(prefill_s * 1e3, 2), "prefill_host_issue_ms": round(enqueue_s * 1e3, 2),
+                  "prefill_linear_TFLOPs": round(prefill_tf, 1),
                   "prefill_frac_of_fp16_mfma_peak": round(prefill_tf / MFMA_FP16_PEAK_TFLOPS, 4),
                   "eager_decode_ms_per_step": round(eager_s * 1e3, 3), "last_tokens": toks[0, -4:].tolist(),
                   "prefill_path_agrees_with_decode_path_on_next_tokens": agreement},

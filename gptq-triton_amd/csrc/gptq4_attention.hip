@@ -16,7 +16,7 @@
 //                 chunks swizzled by the dimension.
 // The softmax runs per lane on its own query column (one exchange per block with the other half-wave for the running
 // maximum; the row sums meet once, at the end), in base 2 with the scale folded in.  Blocks beyond a wave's last
-// visible key are skipped by that wave; the heaviest workgroups (last queries) are launched first.
+// visible key are skipped by that wave; heavy and light query blocks are paired up by workgroup id (see the kernel).
 #include "../../include/gptq4.h"
 #include "gptq4_internal.h"
 
@@ -25,6 +25,14 @@ namespace {
 typedef float f16x_t __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
+// (fmaxf makes the compiler quiet possible signalling NaNs first, one more instruction per operand; the scores are
+// matrix-core outputs or -inf)
+__device__ __forceinline__ float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
 __device__ __forceinline__ int key_slot(int key) {  // position of a key of a 64-key block in V^T's row
     const int o = key & 15;
     return (key & ~15) | (o < 4 ? o : o < 8 ? o + 4 : o < 12 ? o - 4 : o);
@@ -32,15 +40,29 @@ __device__ __forceinline__ int key_slot(int key) {  // position of a key of a 64
 
 __global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t *__restrict__ q, const half_t *__restrict__ kc,
                                                                     const half_t *__restrict__ vc, half_t *__restrict__ out, int H,
-                                                                    int S, int capacity, int past, float scale_log2e) {
-    __shared__ uint4 k_s[64 * 16];  // [key][16 chunks of 8 dims], chunk c of key k at c ^ (k & 7)
-    __shared__ uint4 v_s[128 * 8];  // [dim][8 chunks of 8 key slots], chunk c of dim d at c ^ (d & 7)
+                                                                    int S, int capacity, int past, float scale_log2e, int nq, int nbh) {
+    // (the LDS serves a 16-byte read of 16 lanes at a time from 64 banks: the 16 chunks must fall into different 16-byte slots of 256)
+    __shared__ uint4 k_s[64 * 16];  // [key][16 chunks of 8 dims], chunk c of key k at c ^ (k & 15)
+    __shared__ uint4 v_s[128 * 8];  // [dim][8 chunks of 8 key slots], chunk c of dim d at c ^ ((d >> 1) & 7)
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int h = lane >> 5, c32 = lane & 31;
-    const int qb = (int)gridDim.x - 1 - (int)blockIdx.x;
-    const int bh = blockIdx.y;
+    // Workgroup id -> (head, query block).  A query block's work grows with its index, and the grid's first half lands
+    // one workgroup per CU, the second half beside them: ids i and i + T/2 take blocks nq - 1 - j and j of the same head, so
+    // that the two a CU holds together add up to the same work everywhere (and share the head's keys in L2).
+    int qb, bh;
+    {
+        const int id = blockIdx.x, half = (nq + 1) >> 1, first = nbh * half;
+        if (id < first) {
+            bh = id / half;
+            qb = nq - 1 - (id - bh * half);
+        } else {
+            const int k = id - first, low = nq - half;
+            bh = k / low;
+            qb = k - bh * low;
+        }
+    }
     const int q0 = qb * 128 + wave * 32;  // first query of the wave
     const int kv_len = past + S;
 
@@ -86,12 +108,13 @@ __global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t
         for (int n = 0; n < 4; ++n) {
             const int id = tid + 256 * n;
             const int key = id >> 4, c = id & 15;
-            k_s[key * 16 + (c ^ (key & 7))] = __builtin_bit_cast(uint4, kr[n]);
+            k_s[key * 16 + (c ^ (key & 15))] = __builtin_bit_cast(uint4, kr[n]);
             const int dc = (tid >> 6) + 4 * n;
-            auto put = [&](int e, uint32_t w) {  // halves e and e + 1: dims 8 * dc + e, + 1 (d & 7 = e: dc * 8 is a multiple of 8)
+            auto put = [&](int e, uint32_t w) {  // halves e and e + 1 of the chunk: dims d = 8 * dc + e and d + 1 (same d >> 1)
                 const int d = 8 * dc + e;
-                v16[d * 64 + (((vslot >> 3) ^ e) << 3) + (vslot & 7)] = (uint16_t)w;
-                v16[(d + 1) * 64 + (((vslot >> 3) ^ (e + 1)) << 3) + (vslot & 7)] = (uint16_t)(w >> 16);
+                const int at = (((vslot >> 3) ^ ((d >> 1) & 7)) << 3) + (vslot & 7);
+                v16[d * 64 + at] = (uint16_t)w;
+                v16[(d + 1) * 64 + at] = (uint16_t)(w >> 16);
             };
             put(0, vr[n].x);
             put(2, vr[n].y);
@@ -114,30 +137,26 @@ __global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t
 #pragma unroll
             for (int ks = 0; ks < 8; ++ks) {
                 const int key = 32 * rb + c32;
-                const h8_t a = __builtin_bit_cast(h8_t, k_s[key * 16 + ((2 * ks + h) ^ (key & 7))]);
+                const h8_t a = __builtin_bit_cast(h8_t, k_s[key * 16 + ((2 * ks + h) ^ (key & 15))]);
                 s[rb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[ks], s[rb], 0, 0, 0);
             }
         }
-        // ---- scale, mask, running maximum
-        const bool mask = key0 + 63 > my_first;
-        const int limit = past + q0 + c32;  // last key this lane's query sees
+        // ---- masking (only a block that reaches past the wave's first query's last key), running maximum,
+        //      probabilities; the accumulators are rescaled only when some lane's maximum moved
+        if (key0 + 63 > my_first) {
+            const int limit = past + q0 + c32 - key0 - 4 * h;  // last visible key of this lane's query, in the lane's numbering
+#pragma unroll
+            for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+                    if (32 * rb + 8 * (i >> 2) + (i & 3) > limit) s[rb][i] = -INFINITY;
+        }
         float mx = -INFINITY;
 #pragma unroll
-        for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                float val = s[rb][i] * scale_log2e;
-                if (mask) {
-                    const int key = key0 + 32 * rb + 8 * (i >> 2) + 4 * h + (i & 3);
-                    if (key > limit) val = -INFINITY;
-                }
-                s[rb][i] = val;
-                mx = fmaxf(mx, val);
-            }
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        for (int i = 0; i < 16; ++i) mx = max3(mx, s[0][i], s[1][i]);
+        mx = fmaxf(mx, __shfl_xor(mx, 32)) * scale_log2e;  // (the scale is positive: the maximum commutes with it)
         const float m_new = fmaxf(m, mx);
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // (a query beyond S in a clamped row: nothing visible yet)
-        const float corr = __builtin_amdgcn_exp2f(m - m_use);
         float sum = 0.f;
         h8_t pf[2][2];
 #pragma unroll
@@ -146,16 +165,20 @@ __global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t
             for (int u = 0; u < 2; ++u)
 #pragma unroll
                 for (int t = 0; t < 8; ++t) {
-                    const float pv = __builtin_amdgcn_exp2f(s[rb][8 * u + t] - m_use);
+                    const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(s[rb][8 * u + t], scale_log2e, -m_use));
                     sum += pv;
                     pf[rb][u][t] = (_Float16)pv;
                 }
-        l = l * corr + sum;
-        m = m_new;
+        if (__any(m_new != m)) {
+            const float corr = __builtin_amdgcn_exp2f(m - m_use);
+            l *= corr;
 #pragma unroll
-        for (int db = 0; db < 4; ++db)
+            for (int db = 0; db < 4; ++db)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) o[db][i] *= corr;
+                for (int i = 0; i < 16; ++i) o[db][i] *= corr;
+            m = m_new;
+        }
+        l += sum;
         // ---- O^T += V^T P^T
 #pragma unroll
         for (int db = 0; db < 4; ++db) {
@@ -164,7 +187,7 @@ __global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t
             for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
                 for (int u = 0; u < 2; ++u) {
-                    const h8_t a = __builtin_bit_cast(h8_t, v_s[d * 8 + ((4 * rb + 2 * u + h) ^ (d & 7))]);
+                    const h8_t a = __builtin_bit_cast(h8_t, v_s[d * 8 + ((4 * rb + 2 * u + h) ^ ((d >> 1) & 7))]);
                     o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pf[rb][u], o[db], 0, 0, 0);
                 }
         }
@@ -201,7 +224,7 @@ __global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t
 int launch_attn_prefill(const half_t *q, const half_t *kc, const half_t *vc, half_t *out, int B, int H, int S, int capacity, int past,
                         float scale, hipStream_t stream) {
     const int qblocks = (S + 127) / 128;
-    hipLaunchKernelGGL(gptq4_attn_prefill_kernel, dim3((unsigned)qblocks, (unsigned)(B * H)), dim3(256), 0, stream, q, kc, vc, out, H, S,
-                       capacity, past, scale * 1.4426950408889634f);
+    hipLaunchKernelGGL(gptq4_attn_prefill_kernel, dim3((unsigned)(qblocks * B * H)), dim3(256), 0, stream, q, kc, vc, out, H, S, capacity,
+                       past, scale * 1.4426950408889634f, qblocks, B * H);
     return (int)hipGetLastError();
 }

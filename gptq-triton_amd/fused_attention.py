@@ -318,6 +318,7 @@ class QuantLlamaAttention(nn.Module):
         use_cache: bool = False,
         past_key_values=None,
         position_embeddings=None,
+        causal: bool = False,
         **kwargs,
     ) -> Tuple[torch.Tensor, Optional[torch.Tensor], Optional[Tuple[torch.Tensor]]]:
         """Input shape: Batch x Time x Channel.
@@ -326,7 +327,11 @@ class QuantLlamaAttention(nn.Module):
         (key, value) pair or None, the result is (output, weights or None, (key, value) or None).  Called the way the
         decoder layer of current transformers calls its attention block - `past_key_values` (a Cache object or None)
         and / or `position_embeddings` given - it updates the Cache in slot `layer_idx` and returns (output, weights or
-        None); the cos / sin handed in are not used: the kernel turns q and k itself, from `position_ids`."""
+        None); the cos / sin handed in are not used: the kernel turns q and k itself, from `position_ids`.
+
+        causal (not in the reference, whose callers hand over an additive mask): with no attention_mask, query i attends to
+        the past and to the new tokens up to itself - the prompt pass of this package's own decoder, which runs on the
+        library's attention kernel instead of a materialised mask."""
         if past_key_values is not None or position_embeddings is not None:
             return self._forward_with_cache(hidden_states, attention_mask, position_ids, past_key_values,
                                             output_attentions or bool(kwargs.get('output_attentions', False)),
@@ -353,6 +358,14 @@ class QuantLlamaAttention(nn.Module):
         if attention_mask is not None and attention_mask.size() != (bsz, 1, q_len, kv_seq_len):
             raise ValueError(
                 f"Attention mask should be of size {(bsz, 1, q_len, kv_seq_len)}, but is {attention_mask.size()}")
+
+        if causal and attention_mask is None and not output_attentions and q_len > 1 and self.head_dim == 128:
+            from .decoder_ops import prefill_attention
+            attn_output = prefill_attention(query_states, key_states, value_states, past_len)  # [B, S, hidden]
+            return self.o_proj(attn_output), None, past_key_value
+        if causal and attention_mask is None and q_len > 1:
+            from .llama import causal_mask
+            attention_mask = causal_mask(q_len, kv_seq_len, hidden_states.device).expand(bsz, 1, q_len, kv_seq_len)
 
         attn_weights = None
         if output_attentions:
@@ -420,6 +433,9 @@ def _forward_with_cache(self, hidden_states, attention_mask, position_ids, cache
             attn_weights = attn_weights.masked_fill(~full, torch.finfo(attn_weights.dtype).min)
         attn_weights = nn.functional.softmax(attn_weights, dim=-1, dtype=torch.float32).to(query_states.dtype)
         attn_output = torch.matmul(attn_weights, value_states)
+    elif attention_mask is None and q_len > 1 and self.head_dim == 128 and key_states.is_contiguous() and value_states.is_contiguous():
+        from .decoder_ops import prefill_attention
+        return self.o_proj(prefill_attention(query_states, key_states, value_states, kv_len - q_len)), None
     else:
         # as transformers' own scaled-dot-product path: a given mask is used as it is, none means causal for a prompt
         # and full attention for a single token

@@ -90,10 +90,10 @@ class LlamaDecoderLayer(nn.Module):
         self.input_layernorm = LlamaRMSNorm(config.hidden_size, config.rms_norm_eps)
         self.post_attention_layernorm = LlamaRMSNorm(config.hidden_size, config.rms_norm_eps)
 
-    def forward(self, hidden_states, attention_mask=None, position_ids=None, past_key_value=None, use_cache=False):
+    def forward(self, hidden_states, attention_mask=None, position_ids=None, past_key_value=None, use_cache=False, causal=False):
         attn_out, _, present = self.self_attn(hidden_states=self.input_layernorm(hidden_states),
                                               attention_mask=attention_mask, position_ids=position_ids,
-                                              past_key_value=past_key_value, use_cache=use_cache)
+                                              past_key_value=past_key_value, use_cache=use_cache, causal=causal)
         hidden_states = hidden_states + attn_out
         hidden_states = hidden_states + self.mlp(self.post_attention_layernorm(hidden_states))
         return hidden_states, present
@@ -134,14 +134,13 @@ class LlamaForCausalLM(nn.Module):
         bsz, q_len = input_ids.shape
         past_len = 0 if past_key_values is None else past_key_values[0][0].shape[2]
         position_ids = torch.arange(past_len, past_len + q_len, device=input_ids.device).unsqueeze(0)
-        mask = causal_mask(q_len, past_len + q_len, input_ids.device)
-        if mask is not None:
-            mask = mask.expand(bsz, 1, q_len, past_len + q_len)
         h = self.model.embed_tokens(input_ids)
         presents = []
         for i, layer in enumerate(self.model.layers):
-            h, present = layer(h, attention_mask=mask, position_ids=position_ids,
-                               past_key_value=None if past_key_values is None else past_key_values[i], use_cache=use_cache)
+            # (causal: the attention block masks by position itself - on the GPU inside the attention kernel)
+            h, present = layer(h, attention_mask=None, position_ids=position_ids,
+                               past_key_value=None if past_key_values is None else past_key_values[i], use_cache=use_cache,
+                               causal=True)
             presents.append(present)
         h = self.model.norm(h)
         if last_token_only:
@@ -243,11 +242,11 @@ class GreedyDecoder:
             raise ValueError("prompt does not fit this decoder's batch size / capacity")
         dev = input_ids.device
         position_ids = torch.arange(prompt, device=dev, dtype=torch.int32).unsqueeze(0).expand(bsz, prompt).contiguous()
-        sdpa = torch.nn.functional.scaled_dot_product_attention
+        from .decoder_ops import prefill_attention
 
         def attend(q, kc, vc, attn):
-            o = sdpa(q, kc[:, :, :prompt], vc[:, :, :prompt], is_causal=prompt > 1)
-            return o.transpose(1, 2).reshape(bsz, prompt, self.model.config.hidden_size), False
+            # the prompt's K and V are in cache rows 0 .. prompt - 1 already; the result comes in o_proj's input layout
+            return prefill_attention(q, kc, vc, 0), False
 
         nxt = self._layers(self.model.model.embed_tokens(input_ids), position_ids, 0, attend)
         self.tokens.copy_(nxt)
