@@ -42,8 +42,8 @@ __global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t
                                                                     const half_t *__restrict__ vc, half_t *__restrict__ out, int H,
                                                                     int S, int capacity, int past, float scale_log2e, int nq, int nbh) {
     // (the LDS serves a 16-byte read of 16 lanes at a time from 64 banks: the 16 chunks must fall into different 16-byte slots of 256)
-    __shared__ uint4 k_s[64 * 16];  // [key][16 chunks of 8 dims], chunk c of key k at c ^ (k & 15)
-    __shared__ uint4 v_s[128 * 8];  // [dim][8 chunks of 8 key slots], chunk c of dim d at c ^ ((d >> 1) & 7)
+    __shared__ uint4 k_s[2 * 64 * 16];  // two buffers of [key][16 chunks of 8 dims], chunk c of key k at c ^ (k & 15)
+    __shared__ uint4 v_s[2 * 128 * 8];  // two buffers of [dim][8 chunks of 8 key slots], chunk c of dim d at c ^ ((d >> 1) & 7)
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -88,43 +88,61 @@ __global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t
     const half_t *kb = kc + (size_t)bh * capacity * 128;
     const half_t *vb = vc + (size_t)bh * capacity * 128;
 
-    // ---- staging: K chunk id = tid + 256 * n -> (key id / 16, chunk id % 16): whole rows per 16 lanes;
-    //      V chunk (key tid % 64, chunk tid / 64 + 4 * n): a wave writes 64 consecutive key slots of one dimension
-    u32x4_t kr[4], vr[4];
+    // ---- staging, two LDS buffers: while block i is multiplied, block i + 1 goes from registers into the other buffer
+    //      and block i + 2 is on its way from memory; one barrier per block.
+    //      K chunk id = tid + 256 * n -> (key id / 16, chunk id % 16): whole rows per 16 lanes.
+    //      V: thread (pair p = tid % 32, dc = tid / 32 + 8 * n) holds chunk dc of keys 2p and 2p + 1 - neighbours in V^T's
+    //      slot order too - and writes, per dimension, one dword {key 2p, key 2p + 1}: half a wave fills 128 bytes of a row.
+    u32x4_t kr[4], vr[2][2];
 #define FETCH_BLOCK(blk)                                                                                             \
     _Pragma("unroll") for (int n = 0; n < 4; ++n) {                                                                  \
         const int id = tid + 256 * n;                                                                                \
         const int key = min((blk) * 64 + (id >> 4), kv_len - 1);                                                     \
-        kr[n] = *reinterpret_cast<const u32x4_t *>(kb + (size_t)key * 128 + 8 * (id & 15));                            \
-        const int vkey = min((blk) * 64 + (tid & 63), kv_len - 1);                                                   \
-        vr[n] = *reinterpret_cast<const u32x4_t *>(vb + (size_t)vkey * 128 + 8 * ((tid >> 6) + 4 * n));                \
+        kr[n] = *reinterpret_cast<const u32x4_t *>(kb + (size_t)key * 128 + 8 * (id & 15));                          \
+    }                                                                                                                \
+    _Pragma("unroll") for (int n = 0; n < 2; ++n) _Pragma("unroll") for (int kk = 0; kk < 2; ++kk) {                 \
+        const int vkey = min((blk) * 64 + 2 * (tid & 31) + kk, kv_len - 1);                                          \
+        vr[n][kk] = *reinterpret_cast<const u32x4_t *>(vb + (size_t)vkey * 128 + 8 * ((tid >> 5) + 8 * n));          \
     }
-    const int vslot = key_slot(tid & 63);
-    uint16_t *const v16 = reinterpret_cast<uint16_t *>(v_s);
-    FETCH_BLOCK(0)
-    for (int blk = 0; blk < nblk; ++blk) {
-        __syncthreads();  // the block before has been read
+    const int vslot = key_slot(2 * (tid & 31));  // even: the pair's dword
+    auto stage = [&](int buf) {
+        uint4 *const kd = k_s + buf * (64 * 16);
+        uint32_t *const vd = reinterpret_cast<uint32_t *>(v_s + buf * (128 * 8));
 #pragma unroll
         for (int n = 0; n < 4; ++n) {
             const int id = tid + 256 * n;
             const int key = id >> 4, c = id & 15;
-            k_s[key * 16 + (c ^ (key & 15))] = __builtin_bit_cast(uint4, kr[n]);
-            const int dc = (tid >> 6) + 4 * n;
-            auto put = [&](int e, uint32_t w) {  // halves e and e + 1 of the chunk: dims d = 8 * dc + e and d + 1 (same d >> 1)
+            kd[key * 16 + (c ^ (key & 15))] = __builtin_bit_cast(uint4, kr[n]);
+        }
+#pragma unroll
+        for (int n = 0; n < 2; ++n) {
+            const int dc = (tid >> 5) + 8 * n;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
                 const int d = 8 * dc + e;
-                const int at = (((vslot >> 3) ^ ((d >> 1) & 7)) << 3) + (vslot & 7);
-                v16[d * 64 + at] = (uint16_t)w;
-                v16[(d + 1) * 64 + at] = (uint16_t)(w >> 16);
-            };
-            put(0, vr[n].x);
-            put(2, vr[n].y);
-            put(4, vr[n].z);
-            put(6, vr[n].w);
+                const uint32_t lo = vr[n][0][e >> 1], hi = vr[n][1][e >> 1];
+                // halves e of the two keys: bytes (0, 1) or (2, 3) of each word
+                const uint32_t w = (e & 1) ? __builtin_amdgcn_perm(hi, lo, 0x07060302u) : __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+                vd[d * 32 + ((((vslot >> 3) ^ ((d >> 1) & 7)) << 3) + (vslot & 7)) / 2] = w;
+            }
         }
-        __syncthreads();
+    };
+    FETCH_BLOCK(0)
+    stage(0);
+    if (nblk > 1) {
+        FETCH_BLOCK(1)
+    }
+    for (int blk = 0; blk < nblk; ++blk) {
+        const int buf = blk & 1;
+        __syncthreads();  // block blk is in its buffer; the other buffer (block blk - 1) has been read by every wave
         if (blk + 1 < nblk) {
-            FETCH_BLOCK(blk + 1)
+            stage(buf ^ 1);
+            if (blk + 2 < nblk) {
+                FETCH_BLOCK(blk + 2)
+            }
         }
+        const uint4 *const kt = k_s + buf * (64 * 16);
+        const uint4 *const vt = v_s + buf * (128 * 8);
         const int key0 = blk * 64;
         if (key0 > my_last) continue;  // nothing in this block is visible to the wave (it still takes part in the staging)
 
@@ -137,7 +155,7 @@ __global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t
 #pragma unroll
             for (int ks = 0; ks < 8; ++ks) {
                 const int key = 32 * rb + c32;
-                const h8_t a = __builtin_bit_cast(h8_t, k_s[key * 16 + ((2 * ks + h) ^ (key & 15))]);
+                const h8_t a = __builtin_bit_cast(h8_t, kt[key * 16 + ((2 * ks + h) ^ (key & 15))]);
                 s[rb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[ks], s[rb], 0, 0, 0);
             }
         }
@@ -179,17 +197,23 @@ __global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t
             m = m_new;
         }
         l += sum;
-        // ---- O^T += V^T P^T
+        // ---- O^T += V^T P^T: per step of 16 keys four independent products (the four blocks of 32 dims), the V^T
+        //      fragments of the next step requested before this step's products are issued
+        h8_t va[2][4];
+        auto read_v = [&](int step, int slot) {
 #pragma unroll
-        for (int db = 0; db < 4; ++db) {
-            const int d = 32 * db + c32;
+            for (int db = 0; db < 4; ++db) {
+                const int d = 32 * db + c32;
+                va[slot][db] = __builtin_bit_cast(h8_t, vt[d * 8 + ((2 * step + h) ^ ((d >> 1) & 7))]);
+            }
+        };
+        read_v(0, 0);
 #pragma unroll
-            for (int rb = 0; rb < 2; ++rb)
+        for (int step = 0; step < 4; ++step) {
+            if (step < 3) read_v(step + 1, (step + 1) & 1);
 #pragma unroll
-                for (int u = 0; u < 2; ++u) {
-                    const h8_t a = __builtin_bit_cast(h8_t, v_s[d * 8 + ((4 * rb + 2 * u + h) ^ ((d >> 1) & 7))]);
-                    o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pf[rb][u], o[db], 0, 0, 0);
-                }
+            for (int db = 0; db < 4; ++db)
+                o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[step & 1][db], pf[step >> 1][step & 1], o[db], 0, 0, 0);
         }
     }
 
