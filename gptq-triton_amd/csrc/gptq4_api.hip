@@ -265,6 +265,10 @@ int run_tiled(int epi, MatmulArgs &a, void *workspace, size_t workspace_bytes, h
         partial = 0;
         for (int i = 0; i < parts.count; ++i) {
             choice[i] = choose_part(epi, a.M, a.K, parts, i, kernel_gathers, allow_streamed);
+            if (a.stream_b && choice[i].kslice) {  // the mid-M kernel reads the checkpoint order only
+                choice[i].kslice = false;
+                choice[i].partial = gemm_partial_bytes(choice[i].gp);
+            }
             if (choice[i].partial > partial) partial = choice[i].partial;
         }
     };
@@ -614,6 +618,14 @@ int gptq4_rope_table(float *cos_out, float *sin_out, int max_pos, int D, float b
     return launch_rope_table(cos_out, sin_out, max_pos, D, base, reinterpret_cast<hipStream_t>(stream));
 }
 
+// round-up reciprocal of S for row -> (sequence, token): exact for every row < M when (M - 1) * (magic * S - 2^32) < 2^32; 0: divide
+static uint32_t rope_s_magic(int S, int M) {
+    if (S <= 1) return 0;
+    const uint64_t magic = (1ull << 32) / (uint64_t)S + 1;
+    const uint64_t err = magic * (uint64_t)S - (1ull << 32);
+    return (magic < (1ull << 32) && (uint64_t)(M - 1) * err < (1ull << 32)) ? (uint32_t)magic : 0u;
+}
+
 static int qkv_rotary_impl(const void *x, const void *delta, const void *norm_weight, void *sum_out, float eps,
                            const int32_t *qweight, const int32_t *qzeros, const void *scales, const int32_t *perm,
                            const int32_t *position_ids, const float *cos_table, const float *sin_table, int max_pos,
@@ -653,13 +665,7 @@ static int qkv_rotary_impl(const void *x, const void *delta, const void *norm_we
     a.rope.kv_capacity = kv_capacity;
     a.rope.kv_offset = kv_offset;
     a.rope.max_pos = max_pos;
-    a.rope.s_magic = 0;
-    if (S > 1) {
-        // round-up reciprocal: exact for every row < M when (M - 1) * (magic * S - 2^32) < 2^32
-        const uint64_t magic = (1ull << 32) / (uint64_t)S + 1;
-        const uint64_t err = magic * (uint64_t)S - (1ull << 32);
-        if (magic < (1ull << 32) && (uint64_t)(a.M - 1) * err < (1ull << 32)) a.rope.s_magic = (uint32_t)magic;
-    }
+    a.rope.s_magic = rope_s_magic(S, a.M);
     if (norm) {
         rc = setup_norm(a, delta, norm_weight, sum_out, eps);
         if (rc) return rc;
@@ -766,6 +772,18 @@ static int stream_fill(StreamArgs &a, int epi, int groupsize, void *workspace, s
     return 0;
 }
 
+// More rows than the streaming-order kernels take: the tiled kernel reads the same words (its SB variant).
+static int stream_tiled(int epi, MatmulArgs &t, int M, int K, int N, int groupsize, void *workspace, size_t workspace_bytes, void *stream) {
+    t.M = M;
+    t.K = K;
+    t.N = N;
+    t.n_begin = 0;
+    t.n_count = N;
+    t.groupsize = groupsize;
+    t.stream_b = 1;
+    return run_tiled(epi, t, workspace, workspace_bytes, reinterpret_cast<hipStream_t>(stream));
+}
+
 static int stream_norm(StreamArgs &a, const void *delta, const void *norm_weight, void *sum_out, float eps) {
     if (delta && !sum_out) return -GPTQ4_E_NULL;
     if (a.M > NORM_MAX_M || a.K > NORM_MAX_H || !(eps >= 0.f)) return -GPTQ4_E_SHAPE;
@@ -840,6 +858,16 @@ static int stream_matmul_impl(const void *x, const int32_t *sweight, const int32
     a.M = M;
     a.K = K;
     a.N = N;
+    if (M > STREAM_TALL_MAX_M) {
+        if (nomath) return -GPTQ4_E_SHAPE;
+        MatmulArgs t = {};
+        t.x = a.x;
+        t.w[0] = QMat{a.m[0].w, a.m[0].meta, nullptr};
+        t.perm = perm;
+        t.bias = a.bias;
+        t.y = a.y;
+        return stream_tiled(EPI_PLAIN, t, M, K, N, groupsize, workspace, workspace_bytes, stream);
+    }
     StreamPlan pl;
     rc = stream_fill(a, EPI_PLAIN, groupsize, workspace, workspace_bytes, pl, false, stream);
     if (rc) return rc;
@@ -871,6 +899,16 @@ static int stream_gateup_impl(const void *x, const void *delta, const void *norm
     a.M = M;
     a.K = K;
     a.N = I;
+    if (M > STREAM_TALL_MAX_M) {
+        if (nomath || norm_weight) return -GPTQ4_E_SHAPE;
+        MatmulArgs t = {};
+        t.x = a.x;
+        t.w[0] = QMat{a.m[0].w, a.m[0].meta, nullptr};
+        t.w[1] = QMat{a.m[1].w, a.m[1].meta, nullptr};
+        t.perm = perm;
+        t.y = a.y;
+        return stream_tiled(EPI_SILU_MUL, t, M, K, I, groupsize, workspace, workspace_bytes, stream);
+    }
     if (norm_weight) {
         rc = stream_norm(a, delta, norm_weight, sum_out, eps);
         if (rc) return rc;
@@ -897,13 +935,33 @@ int gptq4_stream_qkv_rotary(const void *x, const void *delta, const void *norm_w
     if (!x || !sweight || !smeta || !position_ids || !cos_table || !sin_table || !q || !k || !v) return -GPTQ4_E_NULL;
     if (B < 1 || S < 1 || H < 1 || D != 128 || max_pos < 1) return -GPTQ4_E_SHAPE;
     if (kv_offset < GPTQ4_KV_AT_POSITION || kv_capacity < 1 || (kv_offset >= 0 && kv_capacity < kv_offset + S)) return -GPTQ4_E_SHAPE;
-    if ((long)B * S > STREAM_TALL_MAX_M) return -GPTQ4_E_SHAPE;
+    if ((long)B * S > 0x7fffffffL) return -GPTQ4_E_SHAPE;
     const int N = 3 * H * D;
     int rc = check_dims(K, N, &groupsize);
     if (rc) return rc;
     if (misaligned16(x) || misaligned16(sweight) || misaligned16(smeta) || misaligned16(q) || misaligned16(k) || misaligned16(v) ||
         misaligned16(cos_table) || misaligned16(sin_table) || (perm && misaligned16(perm)))
         return -GPTQ4_E_ALIGN;
+    if ((long)B * S > STREAM_TALL_MAX_M) {
+        if (norm_weight) return -GPTQ4_E_SHAPE;
+        MatmulArgs t = {};
+        t.x = reinterpret_cast<const half_t *>(x);
+        t.w[0] = QMat{reinterpret_cast<const uint32_t *>(sweight), reinterpret_cast<const uint32_t *>(smeta), nullptr};
+        t.perm = perm;
+        t.rope.position_ids = position_ids;
+        t.rope.cos_table = cos_table;
+        t.rope.sin_table = sin_table;
+        t.rope.q = reinterpret_cast<half_t *>(q);
+        t.rope.k = reinterpret_cast<half_t *>(k);
+        t.rope.v = reinterpret_cast<half_t *>(v);
+        t.rope.S = S;
+        t.rope.H = H;
+        t.rope.kv_capacity = kv_capacity;
+        t.rope.kv_offset = kv_offset;
+        t.rope.max_pos = max_pos;
+        t.rope.s_magic = rope_s_magic(S, B * S);
+        return stream_tiled(EPI_ROPE, t, B * S, K, N, groupsize, workspace, workspace_bytes, stream);
+    }
     StreamArgs a = {};
     a.x = reinterpret_cast<const half_t *>(x);
     a.m[0] = SMat{reinterpret_cast<const uint32_t *>(sweight), reinterpret_cast<const uint32_t *>(smeta)};

@@ -64,9 +64,14 @@ constexpr int LDS_ROW = BK + 8;  // halves; 144-byte rows keep 128-bit reads con
 // boundary is finished like a split-K tile: its parts are exchanged through the workspace, the last to arrive
 // adds them in K order and runs the epilogue; nobody waits for anybody.  (Measured slower than whole tiles at the
 // shapes of the plan's comment, so only the tuning hook selects it.)
-template <int EPI, int MT, bool PERM, bool STREAM = false>
+// SB: the packed words are in streaming order (see gptq4_stream.hip): the 8 packed rows of a K tile are two 64-byte
+// chunks of four rows per column, so a lane fetches, per column, rows 2 * lhi and 2 * lhi + 1 of a chunk with one 8-byte
+// load - as many loads of the same width as from the checkpoint order - and K step ks multiplies packed row
+// 4 * (ks / 2) + 2 * lhi + ks % 2 of the tile instead of 2 * ks + lhi (the activation fragments follow: only an index).
+template <int EPI, int MT, bool PERM, bool STREAM = false, bool SB = false>
 __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
     static_assert(!STREAM || !PERM, "act-order calls reach the streamed schedule with gathered activations");
+    static_assert(!SB || (!PERM && !STREAM), "streaming-order words: plain path only");
     constexpr int NW = 4;        // waves
     constexpr int NT = 64 * NW;  // threads
     constexpr int WM = (MT == 4) ? 1 : 2;  // waves along M
@@ -340,9 +345,33 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
         // Packed words of two K tiles: slot [par][ks] holds step ks of a tile of parity par.  It
         // is decoded during step ks - 1 and refilled during step ks - once its old contents
         // are dead, so the load can land in place - with the same step two tiles on.
+        // (SB: slot [par][2 * m + t] holds, for column t, the words of steps 2 * m and 2 * m + 1; both are refilled during
+        // step 2 * m + 1, when the later of the two has been decoded)
         uint2 b2[2][4];
+        const uint32_t *sbptr = nullptr, *sb_meta = nullptr;
+        if constexpr (SB) {
+            sbptr = p.w[mat].qweight + ((size_t)(ncol >> 4) * (size_t)(K >> 7)) * 256 + (ncol & 15) * 4 + 2 * lhi;
+            sb_meta = p.w[mat].qzeros + (size_t)(ncol >> 4) * (size_t)(K / p.groupsize) * 16 + (ncol & 15);  // (the meta words travel in the qzeros field)
+        }
         auto load_b2 = [&](int par, int kt, int ks) {
-            b2[par][ks] = *reinterpret_cast<const uint2 *>(bptr + ((size_t)min(kt, nk - 1) * (BK / 8) + 2 * ks) * N);
+            if constexpr (SB) {
+                if (ks & 1) {
+                    const uint32_t *src = sbptr + ((size_t)(2 * min(kt, nk - 1) + (ks >> 1))) * 64;
+                    b2[par][ks - 1] = *reinterpret_cast<const uint2 *>(src);
+                    b2[par][ks] = *reinterpret_cast<const uint2 *>(src + 4);
+                }
+            } else {
+                b2[par][ks] = *reinterpret_cast<const uint2 *>(bptr + ((size_t)min(kt, nk - 1) * (BK / 8) + 2 * ks) * N);
+            }
+        };
+        // the packed word of column t for step `step` of the tile of parity par
+        auto word_of = [&](int par, int step, int t) -> uint32_t {
+            if constexpr (SB) {
+                const uint2 w = b2[par][(step & ~1) + t];
+                return (step & 1) ? w.y : w.x;
+            } else {
+                return t ? b2[par][step].y : b2[par][step].x;
+            }
         };
         dma_a(As0, k_begin);
 #pragma unroll
@@ -357,8 +386,15 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
         int group2 = group, left2 = left_in_group;
         auto load_group2 = [&](int par) {
             const int g = min(group2, last_group);
-            g_s[par] = *reinterpret_cast<const uint32_t *>(sc + (size_t)g * N);
-            g_z[par] = qz[(size_t)g * (N >> 3)];
+            if constexpr (SB) {
+                // {scale | zero << 16} of the lane's two columns: neighbours in the strip's row of the group
+                const uint2 m2 = *reinterpret_cast<const uint2 *>(sb_meta + (size_t)g * 16);
+                g_s[par] = m2.x;
+                g_z[par] = m2.y;
+            } else {
+                g_s[par] = *reinterpret_cast<const uint32_t *>(sc + (size_t)g * N);
+                g_z[par] = qz[(size_t)g * (N >> 3)];
+            }
             if (left2 == 1) {
                 ++group2;
                 left2 = tiles_per_group;
@@ -370,16 +406,21 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
         // decoded in natural order too
         ColDecodeNat cn[2];
         auto make_cn = [&](int par) {
-            const uint32_t z2 = g_z[par] >> (((2 * l32) & 7) * 4);
-            cn[0] = make_col_decode_nat(z2 & 0xFu, g_s[par]);
-            cn[1] = make_col_decode_nat((z2 >> 4) & 0xFu, g_s[par] >> 16);
+            if constexpr (SB) {
+                cn[0] = make_col_decode_nat((g_s[par] >> 16) & 0xFu, g_s[par]);
+                cn[1] = make_col_decode_nat((g_z[par] >> 16) & 0xFu, g_z[par]);
+            } else {
+                const uint32_t z2 = g_z[par] >> (((2 * l32) & 7) * 4);
+                cn[0] = make_col_decode_nat(z2 & 0xFu, g_s[par]);
+                cn[1] = make_col_decode_nat((z2 >> 4) & 0xFu, g_s[par] >> 16);
+            }
         };
         load_group2(0);  // group of tile k_begin
         make_cn(0);
         load_group2(1);  // group of tile k_begin + 1, made into constants at the end of tile k_begin
         h8_t bf[2];
-        bf[0] = decode_word_natural(b2[0][0].x, cn[0]);
-        bf[1] = decode_word_natural(b2[0][0].y, cn[1]);
+        bf[0] = decode_word_natural(word_of(0, 0, 0), cn[0]);
+        bf[1] = decode_word_natural(word_of(0, 0, 1), cn[1]);
 
         // one K tile (of parity `par` counted from k_begin) from buffer `cur`, while the next
         // tile streams into `nxt`
@@ -397,7 +438,8 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) {
                     const int row = wm * (32 * MT) + mt * 32 + l32;
-                    araw[mt] = *reinterpret_cast<const h8_t *>(cur + row * BK + 8 * ((2 * ks + lhi) ^ sw));
+                    const int chunk = SB ? 4 * (ks >> 1) + 2 * lhi + (ks & 1) : 2 * ks + lhi;
+                    araw[mt] = *reinterpret_cast<const h8_t *>(cur + row * BK + 8 * (chunk ^ sw));
                 }
             };
             read_a(0);
@@ -413,13 +455,14 @@ __global__ __launch_bounds__(256, 2) void gptq4_gemm_kernel(MatmulArgs p) {
                 load_b2(par, kt + 2, ks);  // this step's words were decoded during the previous step
                 __builtin_amdgcn_sched_barrier(0);  // keep the loads above the MFMAs that hide them
                 // words of the next step (step 0 of the next tile when ks == 3)
-                const uint2 nw = (ks < 3) ? b2[par][ks + 1] : b2[par ^ 1][0];
+                const uint32_t next0 = (ks < 3) ? word_of(par, ks + 1, 0) : word_of(par ^ 1, 0, 0);
+                const uint32_t next1 = (ks < 3) ? word_of(par, ks + 1, 1) : word_of(par ^ 1, 0, 1);
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt], bf[0], acc[mt][0], 0, 0, 0);
-                bf[0] = decode_word_natural(nw.x, cn[0]);
+                bf[0] = decode_word_natural(next0, cn[0]);
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt], bf[1], acc[mt][1], 0, 0, 0);
-                bf[1] = decode_word_natural(nw.y, cn[1]);
+                bf[1] = decode_word_natural(next1, cn[1]);
                 // The decode of the next step's words (32 VALU instructions) spread between this step's MFMAs, three
                 // after each of the wide tile's eight (six after each of the narrow tile's four), instead of four MFMAs
                 // back to back and the decode behind them: 1 - 4 % (LLaMA-7B down_proj at 2048 rows 184 -> 177 us,
@@ -791,17 +834,22 @@ int launch_one(const MatmulArgs &a, int tiles, hipStream_t stream) {
     // the wide rotary tile stages its cos / sin rows in 32 KiB of LDS on top of the activation tiles: more than
     // the 64 KiB a launch may ask for unless the kernel is marked for it (once per variant)
     const size_t lds = (EPI == EPI_ROPE && MT == 4) ? 2 * 2 * 32 * 64 * sizeof(float) : 0;
+    if (a.stream_b && perm) return (int)hipErrorInvalidValue;  // (the entry points gather beforehand)
+    const int variant = a.stream_b ? 2 : (perm ? 1 : 0);
     if (lds) {
-        static bool allowed[2] = {false, false};
-        if (!allowed[perm]) {
-            const void *fn = perm ? reinterpret_cast<const void *>(&gptq4_gemm_kernel<EPI, MT, true>)
-                                  : reinterpret_cast<const void *>(&gptq4_gemm_kernel<EPI, MT, false>);
+        static bool allowed[3] = {false, false, false};
+        if (!allowed[variant]) {
+            const void *fn = variant == 2   ? reinterpret_cast<const void *>(&gptq4_gemm_kernel<EPI, MT, false, false, true>)
+                             : variant == 1 ? reinterpret_cast<const void *>(&gptq4_gemm_kernel<EPI, MT, true>)
+                                            : reinterpret_cast<const void *>(&gptq4_gemm_kernel<EPI, MT, false>);
             const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
             if (e != hipSuccess) return (int)e;
-            allowed[perm] = true;
+            allowed[variant] = true;
         }
     }
-    if (!perm)
+    if (variant == 2)
+        hipLaunchKernelGGL((gptq4_gemm_kernel<EPI, MT, false, false, true>), grid, block, lds, stream, a);
+    else if (variant == 0)
         hipLaunchKernelGGL((gptq4_gemm_kernel<EPI, MT, false>), grid, block, lds, stream, a);
     else
         hipLaunchKernelGGL((gptq4_gemm_kernel<EPI, MT, true>), grid, block, lds, stream, a);

@@ -38,6 +38,7 @@ struct MatmulArgs {
     int groupsize;  // normalised: K when the caller passed -1
     int splitk;
     int tiles;
+    int stream_b;  // tiled kernel: the packed words are in streaming order and w[].qzeros holds the {scale, zero} words (w[].scales unused)
     // small-M kernel: K batches (128 k each) dealt to splitk * 4 wave slots - slot i
     // gets slot_q batches, the first slot_rem slots one more.  Tiled kernel: K tiles
     // (64 k each) dealt to splitk splits the same way.

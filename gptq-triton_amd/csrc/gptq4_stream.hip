@@ -1,4 +1,4 @@
-// Decode GEMV (1..4 rows) for gfx950 on weights in streaming order.
+// Decode GEMV (1..4 rows; a variant for 5..16 follows it) for gfx950 on weights in streaming order.
 //
 // What bounds a decode GEMV on this chip is not arithmetic and not the memory's rate but how many bytes a CU can
 // have in flight and how long a launch runs with nothing in flight: its start (arguments, addresses, first-load
@@ -718,9 +718,8 @@ __global__ __launch_bounds__(256) void gptq4_stream_pack_kernel(const uint32_t *
     sw[o] = qweight[(size_t)kb * N + n];
 }
 
-// (on the path of every call with more rows than the streaming-order kernel takes, so written for whole lines both
-// ways: a wave moves the packed rows 4 * r .. 4 * r + 3 of one unit for 64 columns - it reads one 16-byte chunk per lane,
-// 256 contiguous bytes per strip, and writes 256 contiguous bytes of each of the four rows)
+// (whole lines both ways: a wave moves the packed rows 4 * r .. 4 * r + 3 of one unit for 64 columns - it reads one
+// 16-byte chunk per lane, 256 contiguous bytes per strip, and writes 256 contiguous bytes of each of the four rows)
 __global__ __launch_bounds__(256) void gptq4_stream_unpack_kernel(const uint32_t *__restrict__ sw, uint32_t *__restrict__ qweight,
                                                                   int K, int N) {
     const int nb = K >> 7;

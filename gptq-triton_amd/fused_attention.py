@@ -162,8 +162,8 @@ def qkv_rotary_stream(groupsize: int, hidden_states: torch.Tensor, sweight: torc
         x2d, d2, s = check_norm_args(hidden_states, delta, norm_weight)
         delta_p, nw_p, sum_p = _lib.ptr(d2), norm_weight.data_ptr(), _lib.ptr(s)
     lib = _lib.load()
-    rows = bsz * q_len
-    ws = _lib.workspace(dev, _lib.WS_HEAD_BYTES + (2 * rows * k_in if perm is not None and rows > 4 else 0))
+    from .quant_linear import stream_workspace_bytes
+    ws = _lib.workspace(dev, stream_workspace_bytes(_lib.OP_QKV_ROTARY, bsz * q_len, k_in, n, perm is not None))
     rc = lib.gptq4_stream_qkv_rotary(x2d.data_ptr(), delta_p, nw_p, float(eps), sum_p, sweight.data_ptr(), smeta.data_ptr(),
                                      _lib.ptr(perm), pos.data_ptr(), cos.data_ptr(), sin.data_ptr(), cos.shape[0], q.data_ptr(),
                                      kk.data_ptr(), vv.data_ptr(), bsz, q_len, num_heads, head_dim, k_in, groupsize, cap, off,

@@ -13,7 +13,7 @@ import torch
 import torch.nn as nn
 
 from . import _lib
-from .quant_linear import (QuantLinear, _check_device_tensors, _check_matmul_args, matmul4, stream_pack, stream_rows,
+from .quant_linear import (QuantLinear, _check_device_tensors, _check_matmul_args, matmul4, stream_pack, stream_rows, stream_workspace_bytes,
                            stream_unpack, tensor_key)
 
 
@@ -94,7 +94,7 @@ def llama_mlp_4_stream(groupsize: int, a: torch.Tensor, gate_sweight: torch.Tens
     m = x.shape[0]
     c = torch.empty((m, n), device=a.device, dtype=torch.float16)
     if m:
-        ws = _lib.workspace(a.device, _lib.WS_HEAD_BYTES + (2 * m * k if perm is not None and m > 4 else 0))
+        ws = _lib.workspace(a.device, stream_workspace_bytes(_lib.OP_MLP_GATEUP, m, k, n, perm is not None))
         rc = lib.gptq4_stream_mlp_gateup(x.data_ptr(), delta_p, nw_p, float(eps), sum_p, gate_sweight.data_ptr(), gate_smeta.data_ptr(),
                                          up_sweight.data_ptr(), up_smeta.data_ptr(), _lib.ptr(perm), c.data_ptr(), m, k, n, groupsize,
                                          ws.data_ptr(), ws.numel(), _lib.current_stream(a.device))
@@ -322,7 +322,9 @@ class QuantLlamaMLP(nn.Module):
         return self._input_order[1]
 
     def _stream_ready(self, x: torch.Tensor) -> bool:
-        return self._gate_meta is not None and x.numel() // max(self.infeatures, 1) <= self._stream_rows
+        # (any number of rows: the decode kernels up to _stream_rows, the tiled kernel above 16)
+        rows = x.numel() // max(self.infeatures, 1)
+        return self._gate_meta is not None and not (self._stream_rows < rows <= 16)
 
     def forward(self, x: torch.Tensor, ordered: bool = False) -> torch.Tensor:
         if self._stream_ready(x):

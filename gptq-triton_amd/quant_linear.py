@@ -139,6 +139,14 @@ def stream_rows(op: int, k: int, n: int, groupsize: int) -> int:
     return int(_lib.load().gptq4_stream_rows(op, k, n, groupsize))
 
 
+def stream_workspace_bytes(op: int, m: int, k: int, n: int, with_perm: bool) -> int:
+    """Workspace a streaming-order call needs: the zeroed head; for more than four rows of an act-order projection room for
+    the gathered rows; above 16 rows what the tiled kernel asks for (it reads the same words)."""
+    if m > 16:
+        return int(_lib.load().gptq4_workspace_bytes(op | (_lib.OP_WITH_PERM if with_perm else 0), m, k, n))
+    return _lib.WS_HEAD_BYTES + (2 * m * k if with_perm and m > 4 else 0)
+
+
 def _stream_source_index(k: int, n: int, device) -> torch.Tensor:
     """For every word o of the streaming order, its index kb * N + n in the checkpoint order (int64 [K/8 * N])."""
     nb = k // 128
@@ -196,8 +204,7 @@ def matmul4_stream(groupsize: int, a: torch.Tensor, sweight: torch.Tensor, smeta
     c = torch.empty((m, n), device=a.device, dtype=torch.float16)
     if m == 0:
         return c.view(a.shape[:-1] + (n,))
-    # (more than four rows of an act-order projection are gathered into the workspace first)
-    ws = _lib.workspace(a.device, _lib.WS_HEAD_BYTES + (2 * m * k if perm is not None and m > 4 else 0))
+    ws = _lib.workspace(a.device, stream_workspace_bytes(_lib.OP_MATMUL, m, k, n, perm is not None))
     rc = lib.gptq4_stream_matmul(x.data_ptr(), sweight.data_ptr(), smeta.data_ptr(), _lib.ptr(perm), _lib.ptr(bias), c.data_ptr(),
                                  m, k, n, groupsize, ws.data_ptr(), ws.numel(), _lib.current_stream(a.device))
     _lib.check(rc, "gptq4_stream_matmul")
@@ -274,9 +281,9 @@ class QuantLinear(nn.Module):
 
     def to_stream(self) -> bool:
         """On the GPU: keep the packed weight in streaming order - still ONE copy, in the `qweight` buffer - which is
-        what the decode kernel for up to `_stream_rows` rows reads (an act-order module is compacted first).  Calls
-        with more rows unpack the words into a scratch tensor for the duration of the call and run the kernels for the
-        checkpoint order on it.  state_dict(), dequantize() and checkpoint_qweight() still give the checkpoint layout;
+        what the decode kernels for up to `_stream_rows` rows read (an act-order module is compacted first); calls
+        with more than 16 rows go to the tiled kernel, which reads the same words.  state_dict(), dequantize() and
+        checkpoint_qweight() still give the checkpoint layout (converted on the way out);
         load_state_dict() and to_checkpoint() bring the module back to it.  Returns whether the module now is in
         streaming order (shapes the kernel does not take stay as they are)."""
         if self._stream_meta is not None:
@@ -347,9 +354,10 @@ class QuantLinear(nn.Module):
             return None
         return self._compact_perm if self._compact_perm is not None else self._act_order()[1]
 
-    def stream_weights(self, rows: int):
-        """(sweight, smeta, perm) if the module is in streaming order and its kernel takes `rows` rows, else None."""
-        if self._stream_meta is None or rows > self._stream_rows:
+    def stream_weights(self, rows: int = 1):
+        """(sweight, smeta, perm) if the module is in streaming order, else None (any number of rows: up to `_stream_rows`
+        the decode kernels read these words, above that the tiled kernel does)."""
+        if self._stream_meta is None or self._stream_rows < rows <= 16:
             return None
         return self.qweight, self._stream_meta, self._compact_perm
 

@@ -265,13 +265,15 @@ int gptq4_stream_unpack(const int32_t *sweight, const int32_t *smeta, int32_t *q
 int gptq4_stream_dequant(const int32_t *sweight, const int32_t *smeta, void *W_out, int K, int N, int groupsize,
                          void *stream);
 
-/* gptq4_matmul / gptq4_mlp_gateup / gptq4_qkv_rotary on projections in streaming order, for M <= gptq4_stream_rows()
- * (more rows: -GPTQ4_E_SHAPE).  Same arithmetic (fp16 weights of the formula above, fp32 accumulation, one rounding)
+/* gptq4_matmul / gptq4_mlp_gateup / gptq4_qkv_rotary on projections in streaming order: the decode kernels for
+ * M <= gptq4_stream_rows(); for M > 16 the tiled kernel of the plain entry points, which reads the same words (a
+ * shape with 0 < gptq4_stream_rows() < M <= 16: -GPTQ4_E_SHAPE).  Same arithmetic (fp16 weights of the formula above, fp32 accumulation, one rounding)
  * - only the order in which the fp32 partial sums are added differs, fixed for a shape and GPU.  The two fused
  * entry points take the residual add + RMSNorm of their input along when norm_weight is not NULL (delta, sum_out
  * as in gptq4_norm_qkv_rotary; bit-identical to gptq4_add_rmsnorm followed by the plain call; K <= 8192, M <= 4).
  * workspace: GPTQ4_WS_HEAD_BYTES, zero before the first call; a call with `perm` and more than 4 rows gathers the
- * rows into the workspace first (one small launch) and needs M * K * 2 bytes behind the head. */
+ * rows into the workspace first (one small launch) and needs M * K * 2 bytes behind the head; above 16 rows
+ * gptq4_workspace_bytes() of the plain operator (the tiled kernel's split-K sums). */
 int gptq4_stream_matmul(const void *x, const int32_t *sweight, const int32_t *smeta, const int32_t *perm,
                         const void *bias, void *y, int M, int K, int N, int groupsize, void *workspace,
                         size_t workspace_bytes, void *stream);

@@ -127,6 +127,57 @@ def test_matmul(k, n, g, m):
     assert head_is_zero()
 
 
+@pytest.mark.parametrize("k,n,g", [(1024, 512, 128), (4096, 4096, -1), (11008, 4096, 128), (4096, 12288, 128)])
+@pytest.mark.parametrize("m", [17, 100, 640, 2048])
+def test_matmul_with_more_rows_reads_the_same_words(k, n, g, m):
+    """Above 16 rows the tiled kernel reads the streaming order itself (no copy in the checkpoint order is made)."""
+    G = gptq()
+    L = O.make_layer(k, n, g, seed=1600 + k + m, bias=(m == 100))
+    D = to_dev(L)
+    gs = k if g == -1 else g
+    sw, meta = G.stream_pack(D["qweight"], D["qzeros"], D["scales"], gs)
+    x = O.make_x(m, k, seed=m)
+    y = G.matmul4_stream(gs, torch.from_numpy(x).cuda(), sw, meta, D.get("bias"))
+    rows = np.unique(np.concatenate([[r for r in (0, 1, 16, 31, 32, m - 1) if r < m], np.random.default_rng(m).choice(m, size=min(m, 12), replace=False)]))
+    ref = O.quant_matmul_ref(x[rows], L["qweight"], L["qzeros"], L["scales"], g, bias=L.get("bias"))
+    ok, max_abs, _ = O.within_tolerance(y[rows].cpu().numpy(), ref)
+    assert ok, max_abs
+    if L.get("bias") is None:
+        assert_close(y[rows].cpu().numpy(), ref, f"tiled kernel on streaming order {k}x{n} M={m}")
+    assert head_is_zero()
+
+
+@pytest.mark.parametrize("m", [48, 2048])
+def test_fused_operators_with_more_rows_read_the_same_words(m):
+    G = gptq()
+    k, inter, heads, g = 1024, 2816, 8, 128
+    gate, up = O.make_layer(k, inter, g, seed=1700), O.make_layer(k, inter, g, seed=1701)
+    Dg, Du = to_dev(gate), to_dev(up)
+    gsw, gm = G.stream_pack(Dg["qweight"], Dg["qzeros"], Dg["scales"], g)
+    usw, um = G.stream_pack(Du["qweight"], Du["qzeros"], Du["scales"], g)
+    x = O.make_x(m, k, seed=m + 1)
+    xd = torch.from_numpy(x).cuda()
+    rows = np.unique(np.concatenate([[0, 31, 32, m - 1], np.random.default_rng(m).choice(m, size=10, replace=False)]))
+    y = G.llama_mlp_4_stream(g, xd, gsw, gm, usw, um)
+    trip = lambda d: (d["qweight"], d["qzeros"], d["scales"])
+    assert_close(y[rows].cpu().numpy(), O.mlp_gateup_ref(x[rows], trip(gate), trip(up), g), f"tiled gate/up on streaming order M={m}")
+    # fused QKV + rotary, two sequences
+    L = O.make_layer(k, 3 * heads * 128, g, seed=1702)
+    D = to_dev(L)
+    sw, meta = G.stream_pack(D["qweight"], D["qzeros"], D["scales"], g)
+    b, s = 2, m // 2
+    x3 = x.reshape(b, s, k)
+    pos = (np.arange(s, dtype=np.int64)[None, :] + np.array([[3], [40]]))
+    cos, sin = G.RotaryTable(128, 4096).get(torch.device("cuda"), 4096)
+    q, kk, vv = G.qkv_rotary_stream(g, torch.from_numpy(x3).cuda(), sw, meta, torch.from_numpy(pos).cuda(), cos, sin, heads)
+    q2, k2, v2 = G.qkv_rotary(g, torch.from_numpy(x3).cuda(), D["qweight"], D["scales"], D["qzeros"], torch.from_numpy(pos).cuda(), cos, sin, heads)
+    toks = np.unique(np.concatenate([[0, s - 1], np.random.default_rng(s).choice(s, size=6, replace=False)]))
+    qr, kr, vr = O.qkv_rotary_ref(x3[:, toks], L["qweight"], L["qzeros"], L["scales"], g, pos[:, toks], heads, max_pos=4096)
+    for got, ref, name in ((q, qr, "q"), (kk, kr, "k"), (vv, vr, "v")):
+        assert_close(got[:, :, toks].cpu().numpy(), ref, f"tiled qkv {name} on streaming order M={m}")
+    assert head_is_zero()
+
+
 @pytest.mark.parametrize("waves,depth", [(8, 1), (8, 3), (16, 1), (16, 2)])
 def test_matmul_in_every_launch_shape(waves, depth):
     G = gptq()
@@ -324,7 +375,6 @@ def test_host_side_argument_errors():
     lib = _lib.load()
     fake, ws = 0x1000, _lib.WS_HEAD_BYTES
     assert lib.gptq4_stream_matmul(None, fake, fake, None, None, fake, 1, 4096, 4096, 128, fake, ws, None) == -1
-    assert lib.gptq4_stream_matmul(fake, fake, fake, None, None, fake, 17, 4096, 4096, 128, fake, ws, None) == -2    # more rows than the kernels take
     assert lib.gptq4_stream_matmul(fake, fake, fake, fake, None, fake, 5, 4096, 4096, 128, fake, ws, None) == -4     # act-order above four rows: room for the gathered rows
     assert lib.gptq4_stream_mlp_gateup(fake, None, fake, 1e-6, None, fake, fake, fake, fake, None, fake, 5, 4096, 11008, 128, fake, ws, None) == -2  # norm inside: four rows
     assert lib.gptq4_stream_matmul(fake, fake, fake, None, None, fake, 1, 512, 4096, 128, fake, ws, None) == -2      # K too short for its waves
