@@ -39,6 +39,7 @@ Also reported on the same line:
                 M = 2048 shapes
   --chain-probe / --chain-timeline: the chained decode launch (gptq4_decode_chain) against the
                 separate launches it would replace
+  --attention-probe: the causal prompt-attention kernel beside torch's fused attention + transpose
   --floor-probe what a launch costs before it computes anything: empty launches and plain reads of
                 the four decode operators' bytes (csrc/probe/floor_probe, a stand-alone program),
                 then each decode operator's own access pattern with the arithmetic left out
@@ -423,6 +424,42 @@ def chain_probe(args):
             print(f"    {name:10s} {what:34s} {col.min():7.2f} {np.median(col):7.2f} {col.max():7.2f}")
 
 
+def attention_probe():
+    """`--attention-probe`: gptq4_prefill_attention against torch.nn.functional.scaled_dot_product_attention(is_causal=True)
+    followed by the transpose into o_proj's input layout, HIP events around single launches, median of 20."""
+    import torch
+
+    from gptq_triton_amd import _lib, decoder_ops
+
+    _lib.load()
+    dev = torch.device("cuda:0")
+    rows = {}
+    for (b, h, s) in ((1, 32, 2048), (1, 40, 2048), (8, 52, 2048), (1, 32, 512)):
+        q = torch.randn((b, h, s, 128), device=dev).half()
+        k, v = torch.randn_like(q), torch.randn_like(q)
+
+        def timed(fn, reps=20):
+            for _ in range(3):
+                fn()
+            torch.cuda.synchronize()
+            ts = []
+            for _ in range(reps):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                fn()
+                e1.record()
+                torch.cuda.synchronize()
+                ts.append(e0.elapsed_time(e1) * 1e3)
+            return statistics.median(ts)
+
+        mine = timed(lambda: decoder_ops.prefill_attention(q, k, v))
+        ref = timed(lambda: torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True).transpose(1, 2).reshape(b, s, h * 128))
+        flops = 4 * b * h * s * s * 128 / 2
+        rows[f"B={b} H={h} S={s}"] = {"us": round(mine, 1), "causal_TFLOPs": round(flops / mine / 1e6, 1), "torch_sdpa_plus_transpose_us": round(ref, 1)}
+        log(f"  B={b} H={h} S={s}: {mine:8.1f} us ({flops / mine / 1e6:.0f} TFLOP/s causal)   torch: {ref:8.1f} us")
+    print(json.dumps({"attention_probe": rows}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -434,6 +471,8 @@ def main():
     ap.add_argument("--traffic-probe", action="store_true",
                     help="for rocprofv3 --pmc runs: a 256 MiB device copy (calibration) followed by plain launches of "
                          "each decode operator on distinct weights; prints no JSON")
+    ap.add_argument("--attention-probe", action="store_true",
+                    help="the causal prompt-attention kernel against torch's fused attention + transpose at LLaMA shapes")
     ap.add_argument("--floor-probe", action="store_true",
                     help="launch floor, plain reads and each decode operator's access pattern without its arithmetic beside the "
                          "operator itself (7B shapes, one row); prints text and one JSON line")
@@ -455,6 +494,8 @@ def main():
 
     if args.chain_probe:
         return chain_probe(args)
+    if args.attention_probe:
+        return attention_probe()
     if args.workload != "linears7b":
         return run_decoder(args)
 
