@@ -45,6 +45,15 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t srsrc(const void *p, uint32_t 
 constexpr uint32_t S_OFF_RANGE = 0x80000000u;
 constexpr uint64_t S_MARK = 1ull << 32;
 
+// What a wave needs for the address of its first loads, as kernel arguments of their own in front of the struct, and
+// buffer sizes that do not wait for K and N: LLaMA-7B QKV + rotary at one row 8.49 -> 8.03 us, down_proj 7.88 -> 7.59
+// (having the compiler ask for these arguments in registers at wave start, -amdgpu-kernarg-preload-count, measured
+// no further gain: 7.98 / 7.54)
+#define STREAM_HOT_PARAMS                                                                                                   \
+    const uint32_t *hw0, const uint32_t *hm0, const uint32_t *hw1, const uint32_t *hm1, int hq, int hr, int hnb, uint32_t hnb_magic, \
+        int hgroups, int hbpg, uint32_t hgroup_magic
+#define STREAM_HOT_ARGS(a) (a).m[0].w, (a).m[0].meta, (a).m[1].w, (a).m[1].meta, (a).q, (a).r, (a).nb, (a).nb_magic, (a).groups, (a).batches_per_group, (a).group_magic
+
 template <int NV>
 struct SUnit {
     u32x4_t w[NV];      // the lane's four packed words of the unit, per matrix
@@ -56,7 +65,7 @@ struct SUnit {
 // the residual stream and the workgroup multiplies with weight * rmsnorm(x (+ delta)); NOMATH: the same loads, waits
 // and stores with the decode and the matrix-core instructions left out (measurement only).
 template <int EPI, int NW, int DEPTH, bool PERM, int NORM, bool NOMATH>
-__global__ __launch_bounds__(64 * NW) void gptq4_stream_kernel(StreamArgs p) {
+__global__ __launch_bounds__(64 * NW) void gptq4_stream_kernel(STREAM_HOT_PARAMS, StreamArgs p) {
     constexpr int NV = (EPI == EPI_PLAIN) ? 1 : 2;
     constexpr int NT = 64 * NW;
     extern __shared__ uint4 smem[];
@@ -65,21 +74,19 @@ __global__ __launch_bounds__(64 * NW) void gptq4_stream_kernel(StreamArgs p) {
 
     // (the compiler fetches kernel arguments where it first needs them, in dependent round trips of 0.2 - 0.3 us each
     // with nothing else in flight: naming them here makes it one)
-    asm volatile("" ::"s"(p.x), "s"(p.m[0].w), "s"(p.m[0].meta), "s"(p.m[1].w), "s"(p.m[1].meta), "s"(p.M), "s"(p.K), "s"(p.N), "s"(p.nb),
-                 "s"(p.groups), "s"(p.batches_per_group), "s"(p.group_magic), "s"(p.q), "s"(p.r), "s"(p.nb_magic), "s"(p.xrow),
-                 "s"(p.red_off), "s"(p.m_magic), "s"(p.tagged));
+    asm volatile("" ::"s"(p.x), "s"(p.M), "s"(p.K), "s"(p.N), "s"(p.xrow), "s"(p.red_off), "s"(p.m_magic), "s"(p.tagged));
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r4 = lane >> 4;
     const int c = lane & 15;
 
-    const int M = p.M, K = p.K, N = p.N, nb = p.nb, G = p.groups;
+    const int M = p.M, K = p.K, N = p.N, nb = hnb, G = hgroups;
     const int wg = blockIdx.x;
-    const int a0 = wg * p.q + min(wg, p.r);      // first unit of this workgroup
-    const int L = p.q + (wg < p.r ? 1 : 0);      // its units
+    const int a0 = wg * hq + min(wg, hr);      // first unit of this workgroup
+    const int L = hq + (wg < hr ? 1 : 0);      // its units
     const int b0 = a0 + L;
-    const int tile_hi = sdiv_magic(b0 - 1, nb, p.nb_magic);
+    const int tile_hi = sdiv_magic(b0 - 1, nb, hnb_magic);
     const int n = wave < L ? (L - wave + NW - 1) / NW : 0;   // units of this wave: positions wave, wave + NW, ...
 
     // ---- which output element this thread finishes, if any: e = (piece from the bottom, row, column) belongs to
@@ -116,26 +123,26 @@ __global__ __launch_bounds__(64 * NW) void gptq4_stream_kernel(StreamArgs p) {
 
     // ---- weights: the unit the next load / the next multiplication is for, (tile, 128-k batch), walking down from
     //      the top of the range
-    const uint32_t wbytes = (uint32_t)(((size_t)K * (size_t)N) >> 1);
-    const uint32_t mbytes = (uint32_t)G * (uint32_t)N * 4u;
+    // (both below the plan's limit of 2 GiB and below the offset that switches a load off; exact sizes would wait for K and N)
+    constexpr uint32_t wbytes = 0x7FFFFFF0u, mbytes = 0x7FFFFFF0u;
     __amdgpu_buffer_rsrc_t rs_w[NV], rs_m[NV];
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
-        rs_w[v] = srsrc(p.m[v].w, wbytes);
-        rs_m[v] = srsrc(p.m[v].meta, mbytes);
+        rs_w[v] = srsrc(v ? hw1 : hw0, wbytes);
+        rs_m[v] = srsrc(v ? hm1 : hm0, mbytes);
     }
-    const int bpg = p.batches_per_group;
+    const int bpg = hbpg;
     int ld_tile = tile_hi, ld_batch = 0;
     if (n > 0) {
         const int u = b0 - 1 - wave;
-        ld_tile = sdiv_magic(u, nb, p.nb_magic);
+        ld_tile = sdiv_magic(u, nb, hnb_magic);
         ld_batch = u - ld_tile * nb;
     }
     int cp_tile = ld_tile, cp_batch = ld_batch;
     auto strip_of = [&](int tile, int v) { return (EPI == EPI_ROPE) ? ((tile >> 2) << 3) + (tile & 3) + 4 * v : tile; };
     auto issue = [&](SUnit<NV> &U, bool live) {
         const uint32_t dead = live ? 0u : S_OFF_RANGE;
-        const int g = (bpg == 1) ? ld_batch : (int)__umulhi((unsigned)ld_batch, p.group_magic);
+        const int g = (bpg == 1) ? ld_batch : (int)__umulhi((unsigned)ld_batch, hgroup_magic);
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             const int strip = strip_of(ld_tile, v);
@@ -153,7 +160,7 @@ __global__ __launch_bounds__(64 * NW) void gptq4_stream_kernel(StreamArgs p) {
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) issue(ring[d], d < n);
 
-    const int tile_lo = sdiv_magic(a0, nb, p.nb_magic);
+    const int tile_lo = sdiv_magic(a0, nb, hnb_magic);
     const int npieces = tile_hi - tile_lo + 1;
     const int top_len = min(L, b0 - tile_hi * nb);           // units of the top piece
     const bool publishes = (b0 - tile_hi * nb) != nb;        // its strip goes on in the next workgroup
@@ -325,8 +332,8 @@ __global__ __launch_bounds__(64 * NW) void gptq4_stream_kernel(StreamArgs p) {
     for (int v = 0; v < NV; ++v) part[v] = 0.f;
     if (gets_partials && owner && e_pb == 0) {
         const int u_first = tile_lo * nb;
-        const int big = p.r * (p.q + 1);
-        const int first = u_first < big ? sdiv_magic(u_first, p.q + 1, p.q1_magic) : p.r + sdiv_magic(u_first - big, p.q, p.q_magic);
+        const int big = hr * (hq + 1);
+        const int first = u_first < big ? sdiv_magic(u_first, hq + 1, p.q1_magic) : hr + sdiv_magic(u_first - big, hq, p.q_magic);
         for (int src = first; src < wg; ++src) {
             uint64_t *const slot = p.tagged + (size_t)src * slot_elems;
             uint64_t got[NV];
@@ -419,7 +426,7 @@ struct TUnit {
 };
 
 template <int EPI, int NW, int DEPTH>
-__global__ __launch_bounds__(64 * NW) void gptq4_stream_tall_kernel(StreamArgs p) {
+__global__ __launch_bounds__(64 * NW) void gptq4_stream_tall_kernel(STREAM_HOT_PARAMS, StreamArgs p) {
     constexpr int NV = (EPI == EPI_PLAIN) ? 1 : 2;
     constexpr int NT = 64 * NW;
     constexpr int RE = (16 * 64 + NT - 1) / NT;  // (row, column of a head's half) pairs of the rotary table per thread
@@ -427,21 +434,19 @@ __global__ __launch_bounds__(64 * NW) void gptq4_stream_tall_kernel(StreamArgs p
     __shared__ int arrivals;
     __shared__ int pos_s[16];
 
-    asm volatile("" ::"s"(p.x), "s"(p.m[0].w), "s"(p.m[0].meta), "s"(p.m[1].w), "s"(p.m[1].meta), "s"(p.M), "s"(p.K), "s"(p.N), "s"(p.nb),
-                 "s"(p.groups), "s"(p.batches_per_group), "s"(p.group_magic), "s"(p.q), "s"(p.r), "s"(p.nb_magic), "s"(p.red_off),
-                 "s"(p.nat_off), "s"(p.m_magic), "s"(p.tagged));
+    asm volatile("" ::"s"(p.x), "s"(p.M), "s"(p.K), "s"(p.N), "s"(p.red_off), "s"(p.nat_off), "s"(p.m_magic), "s"(p.tagged));
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r4 = lane >> 4;
     const int c = lane & 15;
 
-    const int M = p.M, K = p.K, N = p.N, nb = p.nb, G = p.groups;
+    const int M = p.M, K = p.K, N = p.N, nb = hnb, G = hgroups;
     const int wg = blockIdx.x;
-    const int a0 = wg * p.q + min(wg, p.r);
-    const int L = p.q + (wg < p.r ? 1 : 0);
+    const int a0 = wg * hq + min(wg, hr);
+    const int L = hq + (wg < hr ? 1 : 0);
     const int b0 = a0 + L;
-    const int tile_hi = sdiv_magic(b0 - 1, nb, p.nb_magic);
+    const int tile_hi = sdiv_magic(b0 - 1, nb, hnb_magic);
     const int n = wave < L ? (L - wave + NW - 1) / NW : 0;
 
     // ---- rotary: the table rows of the M tokens, requested ahead of everything (two dependent loads), parked in
@@ -461,26 +466,25 @@ __global__ __launch_bounds__(64 * NW) void gptq4_stream_tall_kernel(StreamArgs p
     uint32_t xoff[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) xoff[i] = (4 * i + r4 < M) ? (uint32_t)(4 * i + r4) * (uint32_t)K * 2u + (uint32_t)c * 16u : S_OFF_RANGE;
-    const uint32_t wbytes = (uint32_t)(((size_t)K * (size_t)N) >> 1);
-    const uint32_t mbytes = (uint32_t)G * (uint32_t)N * 4u;
+    constexpr uint32_t wbytes = 0x7FFFFFF0u, mbytes = 0x7FFFFFF0u;  // (see the kernel above)
     __amdgpu_buffer_rsrc_t rs_w[NV], rs_m[NV];
 #pragma unroll
     for (int v = 0; v < NV; ++v) {
-        rs_w[v] = srsrc(p.m[v].w, wbytes);
-        rs_m[v] = srsrc(p.m[v].meta, mbytes);
+        rs_w[v] = srsrc(v ? hw1 : hw0, wbytes);
+        rs_m[v] = srsrc(v ? hm1 : hm0, mbytes);
     }
-    const int bpg = p.batches_per_group;
+    const int bpg = hbpg;
     int ld_tile = tile_hi, ld_batch = 0;
     if (n > 0) {
         const int u = b0 - 1 - wave;
-        ld_tile = sdiv_magic(u, nb, p.nb_magic);
+        ld_tile = sdiv_magic(u, nb, hnb_magic);
         ld_batch = u - ld_tile * nb;
     }
     int cp_tile = ld_tile, cp_batch = ld_batch;
     auto strip_of = [&](int tile, int v) { return (EPI == EPI_ROPE) ? ((tile >> 2) << 3) + (tile & 3) + 4 * v : tile; };
     auto issue = [&](TUnit<NV> &U, bool live) {
         const uint32_t dead = live ? 0u : S_OFF_RANGE;
-        const int g = (bpg == 1) ? ld_batch : (int)__umulhi((unsigned)ld_batch, p.group_magic);
+        const int g = (bpg == 1) ? ld_batch : (int)__umulhi((unsigned)ld_batch, hgroup_magic);
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             const int strip = strip_of(ld_tile, v);
@@ -509,7 +513,7 @@ __global__ __launch_bounds__(64 * NW) void gptq4_stream_tall_kernel(StreamArgs p
         }
     }
 
-    const int tile_lo = sdiv_magic(a0, nb, p.nb_magic);
+    const int tile_lo = sdiv_magic(a0, nb, hnb_magic);
     const int npieces = tile_hi - tile_lo + 1;
     const int top_len = min(L, b0 - tile_hi * nb);
     const bool publishes = (b0 - tile_hi * nb) != nb;
@@ -618,8 +622,8 @@ __global__ __launch_bounds__(64 * NW) void gptq4_stream_tall_kernel(StreamArgs p
     if (gets_partials) {
         const int e_col = e_mine & 15, e_row = e_mine >> 4;  // piece 0: e = row * 16 + column
         const int u_first = tile_lo * nb;
-        const int big = p.r * (p.q + 1);
-        const int first = u_first < big ? sdiv_magic(u_first, p.q + 1, p.q1_magic) : p.r + sdiv_magic(u_first - big, p.q, p.q_magic);
+        const int big = hr * (hq + 1);
+        const int first = u_first < big ? sdiv_magic(u_first, hq + 1, p.q1_magic) : hr + sdiv_magic(u_first - big, hq, p.q_magic);
         for (int src = first; src < wg; ++src) {
             uint64_t *const slot = p.tagged + (size_t)src * slot_elems;
             uint64_t got[NV];
@@ -803,7 +807,7 @@ int launch_kernel(const StreamArgs &a, const StreamPlan &pl, hipStream_t stream)
         }
     }
     hipLaunchKernelGGL((gptq4_stream_kernel<EPI, NW, DEPTH, PERM, NORM, NOMATH>), dim3((unsigned)pl.workgroups), dim3(64 * NW), pl.lds_bytes,
-                       stream, a);
+                       stream, STREAM_HOT_ARGS(a), a);
     return (int)hipGetLastError();
 }
 
@@ -833,7 +837,8 @@ int launch_tall(const StreamArgs &a, const StreamPlan &pl, hipStream_t stream) {
             prepared = true;
         }
     }
-    hipLaunchKernelGGL((gptq4_stream_tall_kernel<EPI, NW, DEPTH>), dim3((unsigned)pl.workgroups), dim3(64 * NW), pl.lds_bytes, stream, a);
+    hipLaunchKernelGGL((gptq4_stream_tall_kernel<EPI, NW, DEPTH>), dim3((unsigned)pl.workgroups), dim3(64 * NW), pl.lds_bytes, stream,
+                       STREAM_HOT_ARGS(a), a);
     return (int)hipGetLastError();
 }
 
