@@ -81,10 +81,12 @@ __device__ __forceinline__ void norm_issue_row0(const half_t *x, const half_t *d
 // null the sums x + delta are written there as well (one workgroup of the launch does that).
 // 256 threads, part = NORM_MAX_M * 4 floats of LDS.  Ends with a barrier.  In a workgroup of more than 256
 // threads all of them call it (the barriers are the workgroup's) and `active` is true for threads 0..255 only.
-template <bool ADD, int KEEP>
-__device__ __forceinline__ void norm_rows_to_lds(const half_t *x, const half_t *delta, const half_t *w, half_t *sum_out,
-                                                 uint4 *xs, float *part, int M, int H, float eps, int tid,
-                                                 const NormLoads<KEEP> &r0, bool active = true) {
+// (`put(row, chunk, value)` places a normalised chunk: natural order into an LDS array for most callers, straight into
+// the k order of the decoded weights for the kernel that keeps its activations that way)
+template <bool ADD, int KEEP, typename Put>
+__device__ __forceinline__ void norm_rows_put(const half_t *x, const half_t *delta, const half_t *w, half_t *sum_out, Put put,
+                                              float *part, int M, int H, float eps, int tid, const NormLoads<KEEP> &r0,
+                                              bool active = true) {
     const int chunks = H >> 3;
     for (int row = 0; row < M; ++row) {
         const uint4 *xr = reinterpret_cast<const uint4 *>(x + (size_t)row * H);
@@ -105,8 +107,17 @@ __device__ __forceinline__ void norm_rows_to_lds(const half_t *x, const half_t *
 #pragma unroll
         for (int n = 0; n < KEEP; ++n) {
             const int c = tid + 256 * n;
-            if (active && c < chunks) xs[row * chunks + c] = norm_put(held[n], r0.g[n], inv);
+            if (active && c < chunks) put(row, c, norm_put(held[n], r0.g[n], inv));
         }
     }
     __syncthreads();
+}
+
+template <bool ADD, int KEEP>
+__device__ __forceinline__ void norm_rows_to_lds(const half_t *x, const half_t *delta, const half_t *w, half_t *sum_out,
+                                                 uint4 *xs, float *part, int M, int H, float eps, int tid,
+                                                 const NormLoads<KEEP> &r0, bool active = true) {
+    const int chunks = H >> 3;
+    norm_rows_put<ADD, KEEP>(x, delta, w, sum_out, [&](int row, int c, uint4 v) { xs[row * chunks + c] = v; }, part, M, H, eps, tid, r0,
+                             active);
 }

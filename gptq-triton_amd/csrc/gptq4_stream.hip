@@ -215,17 +215,21 @@ __global__ __launch_bounds__(64 * NW) void gptq4_stream_kernel(STREAM_HOT_PARAMS
         xs[row * p.xrow + (ch - row * chunks)] = val;
     };
     if (NORM) {
-        uint4 *const xn = smem + p.nat_off;  // [M][chunks], natural order
         half_t *const sums = (wg == 0) ? p.nrm_sum_out : nullptr;
-        if (p.nrm_delta != nullptr)
-            norm_rows_to_lds<true>(p.x, p.nrm_delta, p.nrm_weight, sums, xn, norm_part, M, K, p.nrm_eps, tid, nl, wave < 4);
-        else
-            norm_rows_to_lds<false>(p.x, p.x, p.nrm_weight, nullptr, xn, norm_part, M, K, p.nrm_eps, tid, nl, wave < 4);
-        for (int ch = tid; ch < M * chunks; ch += NT) {
-            if (!PERM)
-                put_x(ch, xn[ch]);
+        if (!PERM) {
+            // the normalised chunks go straight into the k order of the decoded weights
+            auto put = [&](int row, int c, uint4 v) { xs[row * p.xrow + c] = pair_order_u4(v); };
+            if (p.nrm_delta != nullptr)
+                norm_rows_put<true>(p.x, p.nrm_delta, p.nrm_weight, sums, put, norm_part, M, K, p.nrm_eps, tid, nl, wave < 4);
             else
-                gather_x(reinterpret_cast<const uint16_t *>(xn), ch);
+                norm_rows_put<false>(p.x, p.x, p.nrm_weight, nullptr, put, norm_part, M, K, p.nrm_eps, tid, nl, wave < 4);
+        } else {
+            uint4 *const xn = smem + p.nat_off;  // [M][chunks], natural order: the gather reads single values of it
+            if (p.nrm_delta != nullptr)
+                norm_rows_to_lds<true>(p.x, p.nrm_delta, p.nrm_weight, sums, xn, norm_part, M, K, p.nrm_eps, tid, nl, wave < 4);
+            else
+                norm_rows_to_lds<false>(p.x, p.x, p.nrm_weight, nullptr, xn, norm_part, M, K, p.nrm_eps, tid, nl, wave < 4);
+            for (int ch = tid; ch < M * chunks; ch += NT) gather_x(reinterpret_cast<const uint16_t *>(xn), ch);
         }
     } else if (!PERM) {
 #pragma unroll
