@@ -215,7 +215,7 @@ def decoder_figures(workload, bsz, prompt, new, steps=None, warmup=None):
         "config": {"workload": f"random-init {workload}-shape decoder, batch {bsz}, {prompt}-token prompt prefill then "
                                f"{new} greedy tokens, 4-bit groupsize {groupsize}{' act-order' if act_order else ''}, "
                                f"fp16 lm_head, one HIP-graph replay per token, packed weights in "
-                               f"{'streaming order' if bsz <= 16 else 'the checkpoint layout'}",
+                               "streaming order",
                    "layers": layers, "hidden": hidden, "intermediate": inter, "heads": heads, "batch": bsz,
                    "prompt": prompt, "new_tokens": new},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",

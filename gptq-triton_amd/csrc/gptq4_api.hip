@@ -265,10 +265,6 @@ int run_tiled(int epi, MatmulArgs &a, void *workspace, size_t workspace_bytes, h
         partial = 0;
         for (int i = 0; i < parts.count; ++i) {
             choice[i] = choose_part(epi, a.M, a.K, parts, i, kernel_gathers, allow_streamed);
-            if (a.stream_b && choice[i].kslice) {  // the mid-M kernel reads the checkpoint order only
-                choice[i].kslice = false;
-                choice[i].partial = gemm_partial_bytes(choice[i].gp);
-            }
             if (choice[i].partial > partial) partial = choice[i].partial;
         }
     };

@@ -49,7 +49,10 @@ constexpr int BK = 64;
 // instead of the whole head.  The two columns of a lane are then d and d + 64 - two 4-byte loads per row instead of one
 // 8-byte load of adjacent columns - so the wave tile has ONE column block, like a plain strip, twice as many workgroups
 // share the projection without splitting K, and the lane that finishes a value holds its rotation partner itself.
-template <int EPI, int MT, bool WIDE, int KS, bool PAIRED = false>
+// SB: the packed words are in streaming order and w[].qzeros holds the {scale, zero} words, as in the tiled kernel's
+// variant of the same name: per column one 8-byte load of rows 2 * lhi, 2 * lhi + 1 of a four-row chunk, K step ks
+// multiplies packed row 4 * (ks / 2) + 2 * lhi + ks % 2 of the tile.
+template <int EPI, int MT, bool WIDE, int KS, bool PAIRED = false, bool SB = false>
 // (eight waves: one workgroup per CU - all its registers - wherever the wave tile has two column blocks or two row blocks)
 __global__ __launch_bounds__(64 * KS, KS == 8 && (MT == 2 || (EPI != EPI_PLAIN && !PAIRED) || WIDE) ? 1 : 2) void gptq4_kslice_kernel(MatmulArgs p) {
     static_assert(KS == 4 || KS == 8, "four or eight waves");
@@ -138,6 +141,14 @@ __global__ __launch_bounds__(64 * KS, KS == 8 && (MT == 2 || (EPI != EPI_PLAIN &
         sc_[j] = p.w[j].scales + ncol;
     }
     auto bptr = [&](int j) { return ADJ ? bptr_[0] + 64 * j : bptr_[j < NPTR ? j : 0]; };
+    // SB: word offset of the lane's rows 2 * lhi, 2 * lhi + 1 of chunk 0 of column ncol, and of its {scale, zero} word of
+    // group 0; 64 columns on are four strips on
+    const uint32_t sb_strip = (uint32_t)(K >> 7) * 256u;            // words of a strip
+    const uint32_t sb_groups16 = (uint32_t)(K / p.groupsize) * 16u;  // {scale, zero} words of a strip
+    const uint32_t sb_off = (uint32_t)(ncol >> 4) * sb_strip + (uint32_t)(ncol & 15) * 4u + 2u * lhi;
+    const uint32_t sb_moff = (uint32_t)(ncol >> 4) * sb_groups16 + (uint32_t)(ncol & 15);
+    auto sb_words = [&](int j) { return p.w[(EPI == EPI_SILU_MUL) ? j : 0].qweight + ((ADJ && j) ? 4 * sb_strip : 0u); };
+    auto sb_meta = [&](int j) { return p.w[(EPI == EPI_SILU_MUL) ? j : 0].qzeros + ((ADJ && j) ? 4 * sb_groups16 : 0u); };
     auto qz = [&](int j) { return ADJ ? qz_[0] + 8 * j : qz_[j < NPTR ? j : 0]; };
     auto sc = [&](int j) { return ADJ ? sc_[0] + 64 * j : sc_[j < NPTR ? j : 0]; };
     const int tiles_per_group = p.groupsize / BK;
@@ -198,7 +209,21 @@ __global__ __launch_bounds__(64 * KS, KS == 8 && (MT == 2 || (EPI != EPI_PLAIN &
         // is decoded during step ks - 1 and refilled during step ks - once its old contents
         // are dead, so the load can land in place - with the same step two tiles on.
         uint2 b2[NB][2][4];
+        // (SB: slot [par][2 * m + t] holds, for column t, the words of steps 2 * m and 2 * m + 1; both are refilled during step
+        // 2 * m + 1)
         auto load_b2 = [&](int par, int kt, int ks) {
+            if constexpr (SB) {
+                if (ks & 1) {
+                    const uint32_t off = sb_off + (uint32_t)(2 * min(kt, nk - 1) + (ks >> 1)) * 64u;
+#pragma unroll
+                    for (int j = 0; j < NB; ++j) {
+                        const uint32_t *src = sb_words(j) + off;
+                        b2[j][par][ks - 1] = *reinterpret_cast<const uint2 *>(src);
+                        b2[j][par][ks] = *reinterpret_cast<const uint2 *>(src + (PAIRED ? 4 * sb_strip : 4u));
+                    }
+                }
+                return;
+            }
             const size_t off = ((size_t)min(kt, nk - 1) * (BK / 8) + 2 * ks) * N;
             if constexpr (PAIRED) {
                 b2[0][par][ks].x = bptr_[0][off];
@@ -214,9 +239,31 @@ __global__ __launch_bounds__(64 * KS, KS == 8 && (MT == 2 || (EPI != EPI_PLAIN &
         int left2 = tiles_per_group - (k_begin - group2 * tiles_per_group);
         uint32_t g_s[NB][2], g_z[NB][2];
         uint32_t g_s_hi[2], g_z_hi[2];  // PAIRED: scale and zero word of the lane's second column
+        auto word_of = [&](int j, int par, int step, int t) -> uint32_t {
+            if constexpr (SB) {
+                const uint2 w = b2[j][par][(step & ~1) + t];
+                return (step & 1) ? w.y : w.x;
+            } else {
+                return t ? b2[j][par][step].y : b2[j][par][step].x;
+            }
+        };
         auto load_group2 = [&](int par) {
             const int g = min(group2, last_group);
-            if constexpr (PAIRED) {
+            if constexpr (SB) {
+                // {scale | zero << 16} of the lane's two columns of each block, in g_s and g_z
+#pragma unroll
+                for (int j = 0; j < NB; ++j) {
+                    const uint32_t *src = sb_meta(j) + sb_moff + (uint32_t)g * 16u;
+                    if constexpr (PAIRED) {
+                        g_s[j][par] = src[0];
+                        g_z[j][par] = src[4 * sb_groups16];
+                    } else {
+                        const uint2 m2 = *reinterpret_cast<const uint2 *>(src);
+                        g_s[j][par] = m2.x;
+                        g_z[j][par] = m2.y;
+                    }
+                }
+            } else if constexpr (PAIRED) {
                 const uint16_t *const sp = reinterpret_cast<const uint16_t *>(sc_[0] + (size_t)g * N);
                 g_s[0][par] = sp[0];
                 g_s_hi[par] = sp[64];
@@ -238,6 +285,14 @@ __global__ __launch_bounds__(64 * KS, KS == 8 && (MT == 2 || (EPI != EPI_PLAIN &
         };
         ColDecodeNat cn[NB][2];
         auto make_cn = [&](int par) {
+            if constexpr (SB) {
+#pragma unroll
+                for (int j = 0; j < NB; ++j) {
+                    cn[j][0] = make_col_decode_nat((g_s[j][par] >> 16) & 0xFu, g_s[j][par]);
+                    cn[j][1] = make_col_decode_nat((g_z[j][par] >> 16) & 0xFu, g_z[j][par]);
+                }
+                return;
+            }
             if constexpr (PAIRED) {
                 const int sh = (l32 & 7) * 4;
                 cn[0][0] = make_col_decode_nat((g_z[0][par] >> sh) & 0xFu, g_s[0][par]);
@@ -263,8 +318,8 @@ __global__ __launch_bounds__(64 * KS, KS == 8 && (MT == 2 || (EPI != EPI_PLAIN &
         h8_t bf[NB][2];
 #pragma unroll
         for (int j = 0; j < NB; ++j) {
-            bf[j][0] = decode_word_natural(b2[j][0][0].x, cn[j][0]);
-            bf[j][1] = decode_word_natural(b2[j][0][0].y, cn[j][1]);
+            bf[j][0] = decode_word_natural(word_of(j, 0, 0, 0), cn[j][0]);
+            bf[j][1] = decode_word_natural(word_of(j, 0, 0, 1), cn[j][1]);
         }
 
         // one K tile (of parity `par` counted from k_begin) from buffer `cur`, while the next
@@ -275,14 +330,15 @@ __global__ __launch_bounds__(64 * KS, KS == 8 && (MT == 2 || (EPI != EPI_PLAIN &
             // many outstanding means the tile has landed.  It is this wave's own tile: no barrier.
             // (tests/test_wait_counts.py counts the loads behind the tile's in the compiled code of every variant.)
             // (lgkmcnt: the fragment reads of the tile before are done before its buffer is requested again.)
-            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(4 * NB * (PAIRED ? 2 : 1)) : "memory");
+            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(4 * NB * ((PAIRED && !SB) ? 2 : 1)) : "memory");
             dma_a(nxt, min(kt + 1, nk - 1));
             load_group2(par);
             h8_t araw[MT];
             auto read_a = [&](int ks) {
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt)
-                    araw[mt] = *reinterpret_cast<const h8_t *>(cur + (mt * 32 + l32) * BK + 8 * ((2 * ks + lhi) ^ sw));
+                    araw[mt] = *reinterpret_cast<const h8_t *>(cur + (mt * 32 + l32) * BK +
+                                                               8 * ((SB ? 4 * (ks >> 1) + 2 * lhi + (ks & 1) : 2 * ks + lhi) ^ sw));
             };
             read_a(0);
 #pragma unroll
@@ -296,15 +352,16 @@ __global__ __launch_bounds__(64 * KS, KS == 8 && (MT == 2 || (EPI != EPI_PLAIN &
                 __builtin_amdgcn_sched_barrier(0);  // keep the loads above the MFMAs that hide them
 #pragma unroll
                 for (int j = 0; j < NB; ++j) {
-                    const uint2 nw = (ks < 3) ? b2[j][par][ks + 1] : b2[j][par ^ 1][0];
+                    const uint32_t next0 = (ks < 3) ? word_of(j, par, ks + 1, 0) : word_of(j, par ^ 1, 0, 0);
+                    const uint32_t next1 = (ks < 3) ? word_of(j, par, ks + 1, 1) : word_of(j, par ^ 1, 0, 1);
 #pragma unroll
                     for (int mt = 0; mt < MT; ++mt)
                         acc[j][mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt], bf[j][0], acc[j][mt][0], 0, 0, 0);
-                    bf[j][0] = decode_word_natural(nw.x, cn[j][0]);
+                    bf[j][0] = decode_word_natural(next0, cn[j][0]);
 #pragma unroll
                     for (int mt = 0; mt < MT; ++mt)
                         acc[j][mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[mt], bf[j][1], acc[j][mt][1], 0, 0, 0);
-                    bf[j][1] = decode_word_natural(nw.y, cn[j][1]);
+                    bf[j][1] = decode_word_natural(next1, cn[j][1]);
                 }
             }
         };
@@ -554,7 +611,10 @@ template <int EPI, int MT, bool WIDE, int KS, bool PAIRED = false>
 int launch_one(const MatmulArgs &a, int tiles, hipStream_t stream) {
     dim3 grid((unsigned)tiles, (unsigned)a.splitk), block(64 * KS);
     if (a.tail_split > 1) grid = dim3((unsigned)(a.tail_first + (tiles - a.tail_first) * a.tail_split), 1u);
-    hipLaunchKernelGGL((gptq4_kslice_kernel<EPI, MT, WIDE, KS, PAIRED>), grid, block, 0, stream, a);
+    if (a.stream_b)
+        hipLaunchKernelGGL((gptq4_kslice_kernel<EPI, MT, WIDE, KS, PAIRED, true>), grid, block, 0, stream, a);
+    else
+        hipLaunchKernelGGL((gptq4_kslice_kernel<EPI, MT, WIDE, KS, PAIRED>), grid, block, 0, stream, a);
     return (int)hipGetLastError();
 }
 

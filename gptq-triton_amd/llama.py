@@ -23,7 +23,7 @@ from .fused_attention import LlamaConfigLite
 
 # up to this many rows the decoder's norms write act-order inputs in their consumer's order
 ORDERED_NORM_ROWS = 16
-# up to this many sequences a GreedyDecoder asks for the streaming-order weight layout (the rows its kernel takes)
+# the rows the decode kernels built on the streaming-order weight layout take (more rows: the mid-M and tiled kernels)
 STREAM_BATCH = 16
 
 
@@ -169,13 +169,13 @@ class GreedyDecoder:
 
     def __init__(self, model: LlamaForCausalLM, bsz: int, capacity: int, layout: str = 'auto'):
         """layout: 'stream' / 'checkpoint' put the model's packed weights into that layout first (quant_linear.set_layout;
-        one copy either way), 'keep' leaves them as they are, 'auto' = 'stream' for up to STREAM_BATCH sequences - what
-        the decode kernel for a handful of rows reads - and 'checkpoint' beyond."""
+        one copy either way), 'keep' leaves them as they are, 'auto' = 'stream': every kernel reads that layout, and the
+        decode kernels for up to STREAM_BATCH rows are built on it."""
         cfg = model.config
         self.model, self.bsz, self.capacity = model, bsz, capacity
         dev = model.lm_head.weight.device
         if layout == 'auto':
-            layout = 'stream' if bsz <= STREAM_BATCH else 'checkpoint'
+            layout = 'stream'
         if layout != 'keep' and dev.type == 'cuda':
             from .quant_linear import set_layout
             set_layout(model, layout)

@@ -38,9 +38,9 @@ def load_quant(checkpoint: str, warmup_autotune: bool = True, device: Optional[s
     layout: 'stream' (default; GPU only) keeps every packed weight in streaming order, the layout the decode kernels for
     up to sixteen rows are built on (quant_linear.set_layout, QuantLinear.to_stream) - one copy of the weights either
     way, and state_dict() / save_quant() produce the checkpoint layout.  Calls with more rows (a prompt pass) read the
-    same words with the tiled kernel, at the speed it reads the checkpoint layout; only calls of 17 to a few hundred
-    rows are faster from the 'checkpoint' layout (the kernel for that range reads nothing else), which is what a
-    model that decodes more than sixteen sequences at a time is better kept in.
+    same words with the mid-M and the tiled kernel, at the speed they read the checkpoint layout.  'checkpoint' keeps
+    the file's layout (what the functional API on raw checkpoint tensors computes on; its decode kernels for up to
+    sixteen rows are the slower ones).
 
     warmup_autotune is accepted for compatibility: launch shapes are static, there is
     nothing to tune (the reference spends 18-49 s here).  It still requires a device, as

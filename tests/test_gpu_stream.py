@@ -178,6 +178,55 @@ def test_fused_operators_with_more_rows_read_the_same_words(m):
     assert head_is_zero()
 
 
+@pytest.mark.parametrize("m", [17, 32, 33, 64, 128, 256, 300, 512])
+def test_mid_sized_calls_at_llama7b_shapes_agree_with_the_checkpoint_order_kernels(m):
+    """17 .. a few hundred rows: the K-sliced kernel (whole and paired rotary heads, 64- and 128-column strips, four and
+    eight waves, K split across workgroups) reads the streaming order too; same values as from the checkpoint order up
+    to the order of the fp32 sums, and the oracle's on sampled rows."""
+    G = gptq()
+    H, I, heads, g = 4096, 11008, 32, 128
+    rows = np.unique(np.concatenate([[0, m - 1], np.random.default_rng(m).choice(m, size=min(m, 6), replace=False)]))
+    x = O.make_x(m, H, seed=m + 7)
+    xd = torch.from_numpy(x).cuda()
+    trip = lambda d: (d["qweight"], d["qzeros"], d["scales"])
+    # gate/up
+    gate, up = O.make_layer(H, I, g, seed=1800), O.make_layer(H, I, g, seed=1801)
+    Dg, Du = to_dev(gate), to_dev(up)
+    gsw, gm = G.stream_pack(Dg["qweight"], Dg["qzeros"], Dg["scales"], g)
+    usw, um = G.stream_pack(Du["qweight"], Du["qzeros"], Du["scales"], g)
+    ys = G.llama_mlp_4_stream(g, xd, gsw, gm, usw, um)
+    yc = G.llama_mlp_4(g, xd, Dg["qweight"], Dg["scales"], Dg["qzeros"], Du["qweight"], Du["scales"], Du["qzeros"])
+    ok, max_abs, _ = O.within_tolerance(ys.cpu().numpy(), yc.float().cpu().numpy())
+    assert ok, max_abs
+    assert_close(ys[rows].cpu().numpy(), O.mlp_gateup_ref(x[rows], trip(gate), trip(up), g), f"gate/up M={m}")
+    del Dg, Du, gsw, usw
+    # down_proj (long K: 128-column strips from 256 rows on)
+    down = O.make_layer(I, H, g, seed=1802)
+    Dd = to_dev(down)
+    dsw, dm = G.stream_pack(Dd["qweight"], Dd["qzeros"], Dd["scales"], g)
+    h = O.make_x(m, I, seed=m + 8)
+    hd = torch.from_numpy(h).cuda()
+    ys = G.matmul4_stream(g, hd, dsw, dm)
+    assert_close(ys[rows].cpu().numpy(), O.quant_matmul_ref(h[rows], *trip(down), g), f"down_proj M={m}")
+    del Dd, dsw
+    # fused QKV + rotary
+    L = O.make_layer(H, 3 * H, g, seed=1803)
+    D = to_dev(L)
+    sw, meta = G.stream_pack(D["qweight"], D["qzeros"], D["scales"], g)
+    pos = (np.arange(m, dtype=np.int64)[None, :] + 5)
+    cos, sin = G.RotaryTable(128, 2048).get(torch.device("cuda"), 2048)
+    x3 = torch.from_numpy(x.reshape(1, m, H)).cuda()
+    q, kk, vv = G.qkv_rotary_stream(g, x3, sw, meta, torch.from_numpy(pos).cuda(), cos, sin, heads)
+    q2, k2, v2 = G.qkv_rotary(g, x3, D["qweight"], D["scales"], D["qzeros"], torch.from_numpy(pos).cuda(), cos, sin, heads)
+    for a, b in ((q, q2), (kk, k2), (vv, v2)):
+        ok, max_abs, _ = O.within_tolerance(a.cpu().numpy(), b.float().cpu().numpy())
+        assert ok, max_abs
+    qr, kr, vr = O.qkv_rotary_ref(x.reshape(1, m, H)[:, rows], L["qweight"], L["qzeros"], L["scales"], g, pos[:, rows], heads, max_pos=2048)
+    for got, ref, name in ((q, qr, "q"), (kk, kr, "k"), (vv, vr, "v")):
+        assert_close(got[:, :, rows].cpu().numpy(), ref, f"qkv {name} M={m}")
+    assert head_is_zero()
+
+
 @pytest.mark.parametrize("waves,depth", [(8, 1), (8, 3), (16, 1), (16, 2)])
 def test_matmul_in_every_launch_shape(waves, depth):
     G = gptq()
