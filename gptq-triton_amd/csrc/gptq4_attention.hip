@@ -20,10 +20,14 @@
 #include "../../include/gptq4.h"
 #include "gptq4_internal.h"
 
+#include <mutex>
+
 namespace {
 
 typedef float f16x_t __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+constexpr int FA_K_BUF = 64 * 17, FA_V_BUF = 128 * 9;                      // 16-byte chunks per buffer
+constexpr size_t FA_LDS_BYTES = (size_t)2 * (FA_K_BUF + FA_V_BUF) * 16;  // 71,680
 
 // (fmaxf makes the compiler quiet possible signalling NaNs first, one more instruction per operand; the scores are
 // matrix-core outputs or -inf)
@@ -41,9 +45,13 @@ __device__ __forceinline__ int key_slot(int key) {  // position of a key of a 64
 __global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t *__restrict__ q, const half_t *__restrict__ kc,
                                                                     const half_t *__restrict__ vc, half_t *__restrict__ out, int H,
                                                                     int S, int capacity, int past, float scale_log2e, int nq, int nbh) {
-    // (the LDS serves a 16-byte read of 16 lanes at a time from 64 banks: the 16 chunks must fall into different 16-byte slots of 256)
-    __shared__ uint4 k_s[2 * 64 * 16];  // two buffers of [key][16 chunks of 8 dims], chunk c of key k at c ^ (k & 15)
-    __shared__ uint4 v_s[2 * 128 * 8];  // two buffers of [dim][8 chunks of 8 key slots], chunk c of dim d at c ^ ((d >> 1) & 7)
+    // Two buffers of K [64 keys][16 chunks of 8 dims] and V^T [128 dims][8 chunks of 8 key slots], every row one chunk longer
+    // than its data (17 and 9 chunks): the LDS serves a 16-byte read of 16 lanes at a time from 64 banks, and rows 272 /
+    // 144 bytes apart put the 16 chunks into 16 different 16-byte slots of 256 - with plain strides, so that every address
+    // below is a lane constant plus an immediate.
+    extern __shared__ uint4 fa_smem[];
+    uint4 *const k_s = fa_smem;                  // 2 x 64 x 17 chunks
+    uint4 *const v_s = fa_smem + 2 * FA_K_BUF;   // 2 x 128 x 9 chunks
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -93,39 +101,33 @@ __global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t
     //      K chunk id = tid + 256 * n -> (key id / 16, chunk id % 16): whole rows per 16 lanes.
     //      V: thread (pair p = tid % 32, dc = tid / 32 + 8 * n) holds chunk dc of keys 2p and 2p + 1 - neighbours in V^T's
     //      slot order too - and writes, per dimension, one dword {key 2p, key 2p + 1}: half a wave fills 128 bytes of a row.
+    // (buffer loads: rows from kv_len on come back as zeros - they are masked.  The block's offset is part of the lane
+    // offset: the range check does not see a scalar offset)
+    const __amdgpu_buffer_rsrc_t k_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t *>(kb), 0, (int)((uint32_t)kv_len * 256u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t v_rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t *>(vb), 0, (int)((uint32_t)kv_len * 256u), 0x00020000);
+    const uint32_t k_voff = (uint32_t)(tid >> 4) * 256u + (uint32_t)(tid & 15) * 16u;  // + 16 keys per n
+    const uint32_t v_voff = (uint32_t)(2 * (tid & 31)) * 256u + (uint32_t)(tid >> 5) * 16u;  // + 1 key per kk, + 8 chunks per n
     u32x4_t kr[4], vr[2][2];
-#define FETCH_BLOCK(blk)                                                                                             \
-    _Pragma("unroll") for (int n = 0; n < 4; ++n) {                                                                  \
-        const int id = tid + 256 * n;                                                                                \
-        const int key = min((blk) * 64 + (id >> 4), kv_len - 1);                                                     \
-        kr[n] = *reinterpret_cast<const u32x4_t *>(kb + (size_t)key * 128 + 8 * (id & 15));                          \
-    }                                                                                                                \
-    _Pragma("unroll") for (int n = 0; n < 2; ++n) _Pragma("unroll") for (int kk = 0; kk < 2; ++kk) {                 \
-        const int vkey = min((blk) * 64 + 2 * (tid & 31) + kk, kv_len - 1);                                          \
-        vr[n][kk] = *reinterpret_cast<const u32x4_t *>(vb + (size_t)vkey * 128 + 8 * ((tid >> 5) + 8 * n));          \
-    }
+#define FETCH_BLOCK(blk)                                                                                                  \
+    _Pragma("unroll") for (int n = 0; n < 4; ++n)                                                                         \
+        kr[n] = __builtin_amdgcn_raw_buffer_load_b128(k_rs, k_voff + 16u * 256u * n + (uint32_t)(blk) * (64u * 256u), 0, 0);   \
+    _Pragma("unroll") for (int n = 0; n < 2; ++n) _Pragma("unroll") for (int kk = 0; kk < 2; ++kk)                        \
+        vr[n][kk] = __builtin_amdgcn_raw_buffer_load_b128(v_rs, v_voff + 256u * kk + 128u * n + (uint32_t)(blk) * (64u * 256u), 0, 0);
     const int vslot = key_slot(2 * (tid & 31));  // even: the pair's dword
+    uint4 *const k_put = k_s + (tid >> 4) * 17 + (tid & 15);                                          // + 16 rows per n
+    uint32_t *const v_put = reinterpret_cast<uint32_t *>(v_s) + (8 * (tid >> 5)) * 36 + (vslot >> 1);  // + 36 dwords per dim
     auto stage = [&](int buf) {
-        uint4 *const kd = k_s + buf * (64 * 16);
-        uint32_t *const vd = reinterpret_cast<uint32_t *>(v_s + buf * (128 * 8));
 #pragma unroll
-        for (int n = 0; n < 4; ++n) {
-            const int id = tid + 256 * n;
-            const int key = id >> 4, c = id & 15;
-            kd[key * 16 + (c ^ (key & 15))] = __builtin_bit_cast(uint4, kr[n]);
-        }
+        for (int n = 0; n < 4; ++n) k_put[buf * FA_K_BUF + n * (16 * 17)] = __builtin_bit_cast(uint4, kr[n]);
 #pragma unroll
-        for (int n = 0; n < 2; ++n) {
-            const int dc = (tid >> 5) + 8 * n;
+        for (int n = 0; n < 2; ++n)
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const int d = 8 * dc + e;
                 const uint32_t lo = vr[n][0][e >> 1], hi = vr[n][1][e >> 1];
                 // halves e of the two keys: bytes (0, 1) or (2, 3) of each word
                 const uint32_t w = (e & 1) ? __builtin_amdgcn_perm(hi, lo, 0x07060302u) : __builtin_amdgcn_perm(hi, lo, 0x05040100u);
-                vd[d * 32 + ((((vslot >> 3) ^ ((d >> 1) & 7)) << 3) + (vslot & 7)) / 2] = w;
+                v_put[buf * (FA_V_BUF * 4) + (64 * n + e) * 36] = w;
             }
-        }
     };
     FETCH_BLOCK(0)
     stage(0);
@@ -141,8 +143,8 @@ __global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t
                 FETCH_BLOCK(blk + 2)
             }
         }
-        const uint4 *const kt = k_s + buf * (64 * 16);
-        const uint4 *const vt = v_s + buf * (128 * 8);
+        const uint4 *const kt = k_s + buf * FA_K_BUF + c32 * 17 + h;         // the lane's key row of a half block, chunk h
+        const uint4 *const vt = v_s + buf * FA_V_BUF + c32 * 9 + h;          // the lane's dim row of a block of 32, chunk h
         const int key0 = blk * 64;
         if (key0 > my_last) continue;  // nothing in this block is visible to the wave (it still takes part in the staging)
 
@@ -154,14 +156,14 @@ __global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t
             for (int i = 0; i < 16; ++i) s[rb][i] = 0.f;
 #pragma unroll
             for (int ks = 0; ks < 8; ++ks) {
-                const int key = 32 * rb + c32;
-                const h8_t a = __builtin_bit_cast(h8_t, kt[key * 16 + ((2 * ks + h) ^ (key & 15))]);
+                const h8_t a = __builtin_bit_cast(h8_t, kt[rb * (32 * 17) + 2 * ks]);
                 s[rb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[ks], s[rb], 0, 0, 0);
             }
         }
         // ---- masking (only a block that reaches past the wave's first query's last key), running maximum,
         //      probabilities; the accumulators are rescaled only when some lane's maximum moved
         if (key0 + 63 > my_first) {
+            asm volatile("" ::: "memory");  // (keeps this a branch: turned into selects the masking would run for every block)
             const int limit = past + q0 + c32 - key0 - 4 * h;  // last visible key of this lane's query, in the lane's numbering
 #pragma unroll
             for (int rb = 0; rb < 2; ++rb)
@@ -176,16 +178,21 @@ __global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t
         const float m_new = fmaxf(m, mx);
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;  // (a query beyond S in a clamped row: nothing visible yet)
         float sum = 0.f;
+        const h2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
         h8_t pf[2][2];
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
             for (int u = 0; u < 2; ++u)
 #pragma unroll
-                for (int t = 0; t < 8; ++t) {
-                    const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(s[rb][8 * u + t], scale_log2e, -m_use));
-                    sum += pv;
-                    pf[rb][u][t] = (_Float16)pv;
+                for (int t = 0; t < 8; t += 2) {
+                    // (the row sum takes the probabilities as the product takes them: rounded to fp16, two per instruction)
+                    h2_t pp;
+                    pp.x = (_Float16)__builtin_amdgcn_exp2f(__builtin_fmaf(s[rb][8 * u + t], scale_log2e, -m_use));
+                    pp.y = (_Float16)__builtin_amdgcn_exp2f(__builtin_fmaf(s[rb][8 * u + t + 1], scale_log2e, -m_use));
+                    sum = __builtin_amdgcn_fdot2(pp, ones, sum, false);
+                    pf[rb][u][t] = pp.x;
+                    pf[rb][u][t + 1] = pp.y;
                 }
         if (__any(m_new != m)) {
             const float corr = __builtin_amdgcn_exp2f(m - m_use);
@@ -202,10 +209,7 @@ __global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t
         h8_t va[2][4];
         auto read_v = [&](int step, int slot) {
 #pragma unroll
-            for (int db = 0; db < 4; ++db) {
-                const int d = 32 * db + c32;
-                va[slot][db] = __builtin_bit_cast(h8_t, vt[d * 8 + ((2 * step + h) ^ ((d >> 1) & 7))]);
-            }
+            for (int db = 0; db < 4; ++db) va[slot][db] = __builtin_bit_cast(h8_t, vt[db * (32 * 9) + 2 * step]);
         };
         read_v(0, 0);
 #pragma unroll
@@ -248,7 +252,18 @@ __global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t
 int launch_attn_prefill(const half_t *q, const half_t *kc, const half_t *vc, half_t *out, int B, int H, int S, int capacity, int past,
                         float scale, hipStream_t stream) {
     const int qblocks = (S + 127) / 128;
-    hipLaunchKernelGGL(gptq4_attn_prefill_kernel, dim3((unsigned)(qblocks * B * H)), dim3(256), 0, stream, q, kc, vc, out, H, S, capacity,
-                       past, scale * 1.4426950408889634f, qblocks, B * H);
+    static bool prepared = false;
+    static std::mutex lock;
+    {
+        std::lock_guard<std::mutex> guard(lock);
+        if (!prepared) {  // more than the 64 KiB a launch may ask for unless the kernel is marked for it
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gptq4_attn_prefill_kernel),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)FA_LDS_BYTES);
+            if (e != hipSuccess) return (int)e;
+            prepared = true;
+        }
+    }
+    hipLaunchKernelGGL(gptq4_attn_prefill_kernel, dim3((unsigned)(qblocks * B * H)), dim3(256), FA_LDS_BYTES, stream, q, kc, vc, out, H, S,
+                       capacity, past, scale * 1.4426950408889634f, qblocks, B * H);
     return (int)hipGetLastError();
 }
