@@ -6,14 +6,13 @@
 // One workgroup of four waves per 128 queries of one head, a wave per 32 queries; the keys come in blocks of 64
 // through LDS, shared by the four waves.  Both products run on v_mfma_f32_32x32x16_f16 in their TRANSPOSED form, so
 // that what one produces is what the next consumes without leaving the lane:
-//   S^T = K Q^T   A = 32 keys x 16 dims out of LDS (rows 256 bytes apart, 16-byte chunks XOR-swizzled by the key),
+//   S^T = K Q^T   A = 32 keys x 16 dims out of LDS (rows of 256 bytes, 272 apart),
 //                 B = the wave's queries, in registers for the whole kernel; lane (h, q) then holds, for its query
 //                 column q, the scores of keys 8 * i + 4 * h + j of each half block (register 4 * i + j);
 //   O^T = V^T P^T A = 32 dims x 16 keys, B = 16 keys x 32 queries: the lane's own probabilities, registers 8 * u .. 8 * u + 7
 //                 of a half block for step u.  That fixes which key sits in which of the 16 contraction slots of a
 //                 step - slot 8 * h + t is key 4 * h + t (t < 4) or 8 + 4 * h + t - 4 - and V^T is written to LDS with
-//                 its keys in that order (the two middle groups of four swapped), rows of 64 keys = 128 bytes apart,
-//                 chunks swizzled by the dimension.
+//                 its keys in that order (the two middle groups of four swapped), rows of 64 keys = 128 bytes, 144 apart.
 // The softmax runs per lane on its own query column (one exchange per block with the other half-wave for the running
 // maximum; the row sums meet once, at the end), in base 2 with the scale folded in.  Blocks beyond a wave's last
 // visible key are skipped by that wave; heavy and light query blocks are paired up by workgroup id (see the kernel).
