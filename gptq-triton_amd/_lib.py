@@ -44,6 +44,7 @@ SIGNATURES = {
     "gptq4_actorder_sort_rows": (c_int, [c_void_p] * 3 + [c_int, c_int, c_void_p]),
     "gptq4_matmul": (c_int, [c_void_p] * 7 + [c_int] * 4 + [c_void_p, c_size_t, c_void_p]),
     "gptq4_matmul_static": (c_int, [c_void_p] * 6 + [c_int] * 4 + [c_void_p]),
+    "gptq4_lm_head_argmax": (c_int, [c_void_p] * 3 + [c_int] * 3 + [c_void_p, c_size_t, c_void_p]),
     "gptq4_prefill_attention": (c_int, [c_void_p] * 4 + [c_int] * 6 + [c_float, c_void_p]),
     "gptq4_static_status": (c_int, [c_void_p]),
     "gptq4_static_reset": (c_int, [c_void_p]),

@@ -730,6 +730,16 @@ int gptq4_decode_attention(const void *q, const void *k_cache, const void *v_cac
                               reinterpret_cast<hipStream_t>(stream));
 }
 
+int gptq4_lm_head_argmax(const void *x, const void *weight, int64_t *out, int B, int K, int V, void *workspace, size_t workspace_bytes,
+                         void *stream) {
+    if (!x || !weight || !out) return -GPTQ4_E_NULL;
+    if (misaligned16(x) || misaligned16(weight) || (reinterpret_cast<uintptr_t>(out) & 7)) return -GPTQ4_E_ALIGN;
+    if (workspace == nullptr || workspace_bytes < GPTQ4_WS_HEAD_BYTES + head_argmax_partial_bytes()) return -GPTQ4_E_WORKSPACE;
+    float *part = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + GPTQ4_WS_HEAD_BYTES);
+    return launch_head_argmax(reinterpret_cast<const half_t *>(x), reinterpret_cast<const half_t *>(weight), reinterpret_cast<long long *>(out),
+                              part, reinterpret_cast<int *>(workspace), B, K, V, reinterpret_cast<hipStream_t>(stream));
+}
+
 int gptq4_prefill_attention(const void *q, const void *k_cache, const void *v_cache, void *out, int B, int H, int S, int D,
                             int kv_capacity, int past, float scale, void *stream) {
     if (!q || !k_cache || !v_cache || !out) return -GPTQ4_E_NULL;

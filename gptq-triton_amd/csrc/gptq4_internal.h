@@ -232,6 +232,8 @@ int launch_rope_table(float *cos_out, float *sin_out, int max_pos, int D, float 
 int launch_rmsnorm(const half_t *x, const half_t *delta, const half_t *w, half_t *sum_out, half_t *y, const int32_t *y_index,
                    int M, int H, float eps, hipStream_t stream);
 size_t attn_decode_partial_bytes(int BH, int capacity);
+size_t head_argmax_partial_bytes();
+int launch_head_argmax(const half_t *x, const half_t *w, long long *out, float *part, int *counters, int B, int K, int V, hipStream_t stream);
 int launch_attn_prefill(const half_t *q, const half_t *kc, const half_t *vc, half_t *out, int B, int H, int S, int capacity, int past,
                         float scale, hipStream_t stream);
 int launch_attn_decode(const half_t *q, const half_t *kc, const half_t *vc, const int *positions, half_t *out,

@@ -101,6 +101,29 @@ def add_rms_norm(x: torch.Tensor, delta: torch.Tensor, weight: torch.Tensor, eps
     return s.reshape(x.shape), y.reshape(x.shape)
 
 
+HEAD_ARGMAX_K = (4096, 5120, 6656, 8192)  # row lengths gptq4_lm_head_argmax is built for
+
+
+def lm_head_argmax(x: torch.Tensor, weight: torch.Tensor, max_rows: int = 4) -> torch.Tensor:
+    """Greedy next tokens: argmax(x @ weight.T, -1) in one launch, for x fp16 [..., K] and an fp16 lm_head weight [V, K].
+    Returns int64 of x's shape without the last dimension.  The kernel takes up to 16 rows but pays up to `max_rows`
+    (one row of 4096: 52 us against 77 for the library's GEMV + argmax; eight rows: 97 against 83); more rows, and shapes
+    it is not built for, go through torch."""
+    k = x.shape[-1]
+    rows = x.numel() // max(k, 1)
+    if not (x.is_cuda and x.dtype == torch.float16 and weight.dtype == torch.float16 and weight.is_contiguous() and weight.dim() == 2
+            and weight.shape[1] == k and k in HEAD_ARGMAX_K and 0 < rows <= min(max_rows, 16) and rows * k * 2 <= 160 * 1024 - 2048
+            and weight.numel() * 2 < 0x7FFFFFF0):
+        return torch.nn.functional.linear(x, weight).argmax(-1)
+    xc = x.reshape(rows, k).contiguous()
+    out = torch.empty(rows, dtype=torch.int64, device=x.device)
+    ws = _lib.workspace(x.device, _lib.WS_HEAD_BYTES + (64 << 10))
+    rc = _lib.load().gptq4_lm_head_argmax(xc.data_ptr(), weight.data_ptr(), out.data_ptr(), rows, k, weight.shape[0], ws.data_ptr(), ws.numel(),
+                                          _lib.current_stream(x.device))
+    _lib.check(rc, "gptq4_lm_head_argmax")
+    return out.view(x.shape[:-1])
+
+
 def prefill_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, past: int = 0) -> torch.Tensor:
     """Causal attention of a prompt (or of a chunk behind `past` cached tokens): q fp16 [B, H, S, 128]; caches fp16
     [B, H, capacity, 128] holding the S new tokens in rows past .. past + S - 1 (for a plain prompt: the k and v the QKV

@@ -412,6 +412,7 @@ def _forward_with_cache(self, hidden_states, attention_mask, position_ids, cache
     if cache is not None:
         key_states, value_states = cache.update(key_states, value_states, self.layer_idx)
     kv_len = key_states.shape[-2]
+    k_all, v_all = key_states, value_states  # as the cache keeps them (a preallocated one: its whole capacity)
     if attention_mask is None and kv_len > past + q_len:
         # a preallocated cache hands back its whole capacity: without a mask only the slots written so far count
         kv_len = past + q_len
@@ -433,9 +434,10 @@ def _forward_with_cache(self, hidden_states, attention_mask, position_ids, cache
             attn_weights = attn_weights.masked_fill(~full, torch.finfo(attn_weights.dtype).min)
         attn_weights = nn.functional.softmax(attn_weights, dim=-1, dtype=torch.float32).to(query_states.dtype)
         attn_output = torch.matmul(attn_weights, value_states)
-    elif attention_mask is None and q_len > 1 and self.head_dim == 128 and key_states.is_contiguous() and value_states.is_contiguous():
+    elif attention_mask is None and q_len > 1 and self.head_dim == 128 and k_all.is_contiguous() and v_all.is_contiguous():
+        # (the kernel reads cache rows 0 .. kv_len - 1 where they lie, whatever the capacity behind them)
         from .decoder_ops import prefill_attention
-        return self.o_proj(prefill_attention(query_states, key_states, value_states, kv_len - q_len)), None
+        return self.o_proj(prefill_attention(query_states, k_all, v_all, kv_len - q_len)), None
     else:
         # as transformers' own scaled-dot-product path: a given mask is used as it is, none means causal for a prompt
         # and full attention for a single token

@@ -18,7 +18,7 @@ import torch
 import torch.nn as nn
 
 from . import _lib
-from .decoder_ops import add_rms_norm, decode_attention, rms_norm
+from .decoder_ops import add_rms_norm, decode_attention, lm_head_argmax, rms_norm
 from .fused_attention import LlamaConfigLite
 
 # up to this many rows the decoder's norms write act-order inputs in their consumer's order
@@ -217,7 +217,7 @@ class GreedyDecoder:
             oq = None if last else order_of(layers[i + 1].self_attn)
             y = layer.mlp(x, ordered=True) if om is not None else layer.mlp(x)
             h, x = add_rms_norm(h, y, norm.weight, norm.variance_epsilon, out_index=oq)
-        return self.model.lm_head(x[:, -1:, :]).argmax(-1)
+        return lm_head_argmax(x[:, -1:, :], self.model.lm_head.weight)
 
     def _layers_norm_in_matmul(self, h, position_ids, kv_offset, attend):
         """The same stack for a handful of rows: the QKV and the gate/up launch each do the residual
@@ -232,7 +232,7 @@ class GreedyDecoder:
             h, delta = layer.mlp.forward_normed(h, attn.project_out(*attend(q, kc, vc, attn)), n2.weight, n2.variance_epsilon)
         norm = self.model.model.norm
         h, x = add_rms_norm(h, delta, norm.weight, norm.variance_epsilon)
-        return self.model.lm_head(x[:, -1:, :]).argmax(-1)
+        return lm_head_argmax(x[:, -1:, :], self.model.lm_head.weight)
 
     @torch.no_grad()
     def prefill(self, input_ids: torch.Tensor) -> torch.Tensor:

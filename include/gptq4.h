@@ -222,6 +222,16 @@ int gptq4_decode_attention(const void *q, const void *k_cache, const void *v_cac
                            int kv_capacity, float scale, void *workspace,
                            size_t workspace_bytes, void *stream);
 
+/* The end of a greedy decode step in one launch: out[b] = argmax over v of fp16(x[b] . weight[v]) - the fp16 lm_head
+ * (weight fp16 [V, K], row-major as nn.Linear keeps it; no bias) and the argmax of its output, the lowest index among
+ * equal logits.  x fp16 [B, K], B <= 16; out int64 [B]; K one of 4096, 5120, 6656, 8192 (else -GPTQ4_E_SHAPE: use a
+ * dense GEMV and an argmax).  workspace: the zeroed head + 32 KiB behind it (gptq4_workspace_bytes of any operator
+ * covers it).  The sums are fp32 and rounded to fp16 once, so a logit can differ from a library GEMV's by an fp16
+ * ulp and the index with it where two logits are that close.  Replaces `model.lm_head(h).argmax(-1)` of a greedy
+ * decoding loop (the reference's generate.py leaves both to transformers). */
+int gptq4_lm_head_argmax(const void *x, const void *weight, int64_t *out, int B, int K, int V, void *workspace,
+                         size_t workspace_bytes, void *stream);
+
 /* Causal attention of S query tokens per sequence (a prompt, or a chunk of one behind `past` cached tokens): query i
  * attends to cache rows 0 .. past + i; softmax in fp32, output fp16 out [B, S, H*D] - the layout o_proj consumes, no
  * transpose.  q fp16 [B, H, S, D] (as gptq4_qkv_rotary writes it); k_cache, v_cache fp16 [B, H, kv_capacity, D] with
