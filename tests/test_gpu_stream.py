@@ -560,19 +560,26 @@ def random_quant_model(hidden, inter, heads, layers, groupsize, seed, act_order=
 
 @pytest.mark.parametrize("act_order", [False, True])
 def test_greedy_decoder_in_streaming_order_matches_the_checkpoint_layout(act_order):
-    """A small random decoder: the same greedy tokens from the streaming-order layout (one sequence and three: its
-    kernel) as from the checkpoint layout, eager and as a replayed graph; the norms fused into the projections."""
+    """A small random decoder: the same greedy tokens from the streaming-order layout (one sequence and three: the kernel
+    with the rows in LDS, the norms fused into the projections; six: the kernel that fetches the rows with every unit; twenty:
+    the mid-M kernel on the same words) as from the checkpoint layout, eager and as a replayed graph."""
     G = gptq()
     model = random_quant_model(hidden=1024, inter=2816, heads=8, layers=2, groupsize=128, seed=7, act_order=act_order)
-    for bsz in (1, 3):
+    for bsz in (1, 3, 6, 20):
         ids = torch.randint(0, model.config.vocab_size, (bsz, 12), device="cuda", generator=torch.Generator(device="cuda").manual_seed(bsz))
         G.set_layout(model, "checkpoint")
         dec = G.GreedyDecoder(model, bsz, 64, layout="keep")
         first = dec.prefill(ids)
         want = torch.cat([first, dec.decode(10)], dim=1)
-        dec = G.GreedyDecoder(model, bsz, 64)   # 'auto': streaming order for up to four sequences
+        dec = G.GreedyDecoder(model, bsz, 64)   # 'auto': streaming order
         assert model.model.layers[0].self_attn.qkv_proj._stream_meta is not None
         first = dec.prefill(ids)
         got = torch.cat([first, dec.decode(10, use_graph=True)], dim=1)
-        assert torch.equal(got, want), (bsz, got.tolist(), want.tolist())
+        if bsz <= 4:
+            assert torch.equal(got, want), (bsz, got.tolist(), want.tolist())
+        else:
+            # other kernels on both sides, other orders of the fp32 sums: a near-tie between two logits may go the other way
+            # (and the sequence then continues differently); most sequences agree to the last token
+            same = (got == want).all(dim=1).float().mean().item()
+            assert same >= 0.8 and torch.equal(got[:, 0], want[:, 0]) or same >= 0.9, (bsz, same)
     G.set_layout(model, "checkpoint")
