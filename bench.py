@@ -46,8 +46,9 @@ Also reported on the same line:
                 (gptq4_stream_probe) beside the operator itself; prints text and one JSON line
 
 Other workloads (--workload llama7b | llama13b | llama30b): a full random-init decoder of
-that shape (embedding, RMSNorm, fused QKV + rotary into a preallocated KV cache, torch
-SDPA, o_proj, fused MLP, fp16 lm_head, greedy argmax) - one timed prefill of --prompt
+that shape (embedding, RMSNorm, fused QKV + rotary into a preallocated KV cache, the
+library's prompt and decode attention, o_proj, fused MLP, fp16 lm_head + greedy argmax) - one
+timed prefill of --prompt
 tokens, then --new-tokens greedy tokens with one HIP-graph replay per token; value =
 decode tokens/s over the batch, prefill TFLOP/s and the eager (kernel-by-kernel) decode
 rate in `extra`.

@@ -27,6 +27,7 @@ typedef float f16x_t __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 constexpr int FA_K_BUF = 64 * 17, FA_V_BUF = 128 * 9;                      // 16-byte chunks per buffer
 constexpr size_t FA_LDS_BYTES = (size_t)2 * (FA_K_BUF + FA_V_BUF) * 16;  // 71,680
+constexpr int FA_GROUP = 4;  // heads of an XCD worked on together when it has many (1 MiB of keys and values each at 2048 tokens; 4 MiB of L2)
 
 // (fmaxf makes the compiler quiet possible signalling NaNs first, one more instruction per operand; the scores are
 // matrix-core outputs or -inf)
@@ -55,20 +56,40 @@ __global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int h = lane >> 5, c32 = lane & 31;
-    // Workgroup id -> (head, query block).  A query block's work grows with its index, and the grid's first half lands
-    // one workgroup per CU, the second half beside them: ids i and i + T/2 take blocks nq - 1 - j and j of the same head, so
-    // that the two a CU holds together add up to the same work everywhere (and share the head's keys in L2).
+    // Workgroup id -> (head, query block).  Consecutive ids go to the eight XCDs in turn, each with an L2 of its own:
+    // id % 8 picks the XCD and all query blocks of a head are given to one XCD (head % 8, for the heads up to the last
+    // multiple of eight; the rest are dealt as if there were one XCD), so that a head's keys and values are fetched into
+    // one L2 only.  Within an XCD the heavy halves of all its heads come first (a query block's work grows with its
+    // index), then the light halves in the matching order: when the whole grid is resident at once, a CU's two workgroups
+    // are blocks nq - 1 - j and j of one head and add up to the same work everywhere; when it is not, long work goes first.
     int qb, bh;
     {
-        const int id = blockIdx.x, half = (nq + 1) >> 1, first = nbh * half;
-        if (id < first) {
-            bh = id / half;
-            qb = nq - 1 - (id - bh * half);
+        const int nb8 = nbh & ~7, cut = nb8 * nq;
+        int y = blockIdx.x, heads = nbh, head_step = 1, head0 = 0;
+        if (y < cut) {
+            head0 = y & 7, head_step = 8, heads = nb8 >> 3, y >>= 3;
         } else {
-            const int k = id - first, low = nq - half;
-            bh = k / low;
-            qb = k - bh * low;
+            y -= cut, heads = nbh - nb8, head0 = nb8;
         }
+        // (more than eight heads to an XCD: in groups of FA_GROUP heads, each group in the order above, so that the keys and
+        // values in use stay within the L2)
+        int group0 = 0;
+        if (heads > 8) {
+            const int per = FA_GROUP * nq, g = y / per;
+            group0 = g * FA_GROUP, y -= g * per, heads = min(FA_GROUP, heads - group0);
+        }
+        const int half = (nq + 1) >> 1, first = heads * half;
+        int hl;
+        if (y < first) {
+            hl = y / half;
+            qb = nq - 1 - (y - hl * half);
+        } else {
+            const int k = y - first, low = nq - half;
+            hl = k / low;
+            qb = k - hl * low;
+        }
+        hl += group0;
+        bh = head0 + hl * head_step;
     }
     const int q0 = qb * 128 + wave * 32;  // first query of the wave
     const int kv_len = past + S;
@@ -107,17 +128,20 @@ __global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t
     const uint32_t k_voff = (uint32_t)(tid >> 4) * 256u + (uint32_t)(tid & 15) * 16u;  // + 16 keys per n
     const uint32_t v_voff = (uint32_t)(2 * (tid & 31)) * 256u + (uint32_t)(tid >> 5) * 16u;  // + 1 key per kk, + 8 chunks per n
     u32x4_t kr[4], vr[2][2];
-#define FETCH_BLOCK(blk)                                                                                                  \
+#define FETCH_K(blk)                                                                                                      \
     _Pragma("unroll") for (int n = 0; n < 4; ++n)                                                                         \
-        kr[n] = __builtin_amdgcn_raw_buffer_load_b128(k_rs, k_voff + 16u * 256u * n + (uint32_t)(blk) * (64u * 256u), 0, 0);   \
+        kr[n] = __builtin_amdgcn_raw_buffer_load_b128(k_rs, k_voff + 16u * 256u * n + (uint32_t)(blk) * (64u * 256u), 0, 0);
+#define FETCH_V(blk)                                                                                                      \
     _Pragma("unroll") for (int n = 0; n < 2; ++n) _Pragma("unroll") for (int kk = 0; kk < 2; ++kk)                        \
         vr[n][kk] = __builtin_amdgcn_raw_buffer_load_b128(v_rs, v_voff + 256u * kk + 128u * n + (uint32_t)(blk) * (64u * 256u), 0, 0);
     const int vslot = key_slot(2 * (tid & 31));  // even: the pair's dword
     uint4 *const k_put = k_s + (tid >> 4) * 17 + (tid & 15);                                          // + 16 rows per n
     uint32_t *const v_put = reinterpret_cast<uint32_t *>(v_s) + (8 * (tid >> 5)) * 36 + (vslot >> 1);  // + 36 dwords per dim
-    auto stage = [&](int buf) {
+    auto stage_k = [&](int buf) {
 #pragma unroll
         for (int n = 0; n < 4; ++n) k_put[buf * FA_K_BUF + n * (16 * 17)] = __builtin_bit_cast(uint4, kr[n]);
+    };
+    auto stage_v = [&](int buf) {
 #pragma unroll
         for (int n = 0; n < 2; ++n)
 #pragma unroll
@@ -128,27 +152,9 @@ __global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t
                 v_put[buf * (FA_V_BUF * 4) + (64 * n + e) * 36] = w;
             }
     };
-    FETCH_BLOCK(0)
-    stage(0);
-    if (nblk > 1) {
-        FETCH_BLOCK(1)
-    }
-    for (int blk = 0; blk < nblk; ++blk) {
-        const int buf = blk & 1;
-        __syncthreads();  // block blk is in its buffer; the other buffer (block blk - 1) has been read by every wave
-        if (blk + 1 < nblk) {
-            stage(buf ^ 1);
-            if (blk + 2 < nblk) {
-                FETCH_BLOCK(blk + 2)
-            }
-        }
-        const uint4 *const kt = k_s + buf * FA_K_BUF + c32 * 17 + h;         // the lane's key row of a half block, chunk h
-        const uint4 *const vt = v_s + buf * FA_V_BUF + c32 * 9 + h;          // the lane's dim row of a block of 32, chunk h
-        const int key0 = blk * 64;
-        if (key0 > my_last) continue;  // nothing in this block is visible to the wave (it still takes part in the staging)
-
-        // ---- S^T = K Q^T for the two half blocks of 32 keys
-        f16x_t s[2];
+    // ---- S^T = K Q^T for the two half blocks of 32 keys of the block in K buffer `buf`
+    auto scores = [&](int buf, f16x_t(&s)[2]) {
+        const uint4 *const kt = k_s + buf * FA_K_BUF + c32 * 17 + h;  // the lane's key row of a half block, chunk h
 #pragma unroll
         for (int rb = 0; rb < 2; ++rb) {
 #pragma unroll
@@ -159,8 +165,53 @@ __global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t
                 s[rb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[ks], s[rb], 0, 0, 0);
             }
         }
-        // ---- masking (only a block that reaches past the wave's first query's last key), running maximum,
-        //      probabilities; the accumulators are rescaled only when some lane's maximum moved
+    };
+
+    // ---- The order of work.  K is staged two blocks ahead of the block whose probabilities are being made and V one, in two
+    //      buffers each, with one barrier per block: in step i the wave takes the scores of block i, made in step i - 1,
+    //      issues the products for the scores of block i + 1, and turns block i's scores into probabilities while the matrix
+    //      cores work on those; then O^T += V^T P^T for block i.  Step i writes K block i + 2 over block i (last read in
+    //      step i - 1) and V block i + 1 over block i - 1.
+    {
+        FETCH_K(0)
+        FETCH_V(0)
+        u32x4_t k1[4];  // (block 1 of K asked for together with block 0: one round trip to memory before the first product)
+        if (nblk > 1) {
+#pragma unroll
+            for (int n = 0; n < 4; ++n) k1[n] = __builtin_amdgcn_raw_buffer_load_b128(k_rs, k_voff + 16u * 256u * n + 64u * 256u, 0, 0);
+        }
+        stage_k(0);
+        stage_v(0);
+        if (nblk > 1) {
+#pragma unroll
+            for (int n = 0; n < 4; ++n) k_put[FA_K_BUF + n * (16 * 17)] = __builtin_bit_cast(uint4, k1[n]);
+            FETCH_V(1)
+            if (nblk > 2) {
+                FETCH_K(2)
+            }
+        }
+    }
+    __syncthreads();
+    f16x_t sa[2], sb[2];
+    scores(0, sa);
+    auto step = [&](int blk, f16x_t(&s)[2], f16x_t(&sn)[2]) {
+        const int buf = blk & 1;
+        __syncthreads();  // K block blk + 1 and V block blk are in their buffers; the buffers written below have been read
+        if (blk + 1 < nblk) {
+            stage_v(buf ^ 1);
+            if (blk + 2 < nblk) {
+                FETCH_V(blk + 2)
+                stage_k(buf);
+                if (blk + 3 < nblk) {
+                    FETCH_K(blk + 3)
+                }
+            }
+        }
+        const uint4 *const vt = v_s + buf * FA_V_BUF + c32 * 9 + h;  // the lane's dim row of a block of 32, chunk h
+        const int key0 = blk * 64;
+        if (key0 > my_last) return;  // nothing in this block is visible to the wave (it still takes part in the staging)
+
+        // ---- masking (only a block that reaches past the wave's first query's last key)
         if (key0 + 63 > my_first) {
             asm volatile("" ::: "memory");  // (keeps this a branch: turned into selects the masking would run for every block)
             const int limit = past + q0 + c32 - key0 - 4 * h;  // last visible key of this lane's query, in the lane's numbering
@@ -170,6 +221,10 @@ __global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t
                 for (int i = 0; i < 16; ++i)
                     if (32 * rb + 8 * (i >> 2) + (i & 3) > limit) s[rb][i] = -INFINITY;
         }
+        // ---- the next block's scores (whatever the buffer holds after the last block: nobody reads them), then the
+        //      running maximum and the probabilities of this one; the accumulators are rescaled only when some lane's
+        //      maximum moved
+        scores(buf ^ 1, sn);
         float mx = -INFINITY;
 #pragma unroll
         for (int i = 0; i < 16; ++i) mx = max3(mx, s[0][i], s[1][i]);
@@ -206,18 +261,22 @@ __global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t
         // ---- O^T += V^T P^T: per step of 16 keys four independent products (the four blocks of 32 dims), the V^T
         //      fragments of the next step requested before this step's products are issued
         h8_t va[2][4];
-        auto read_v = [&](int step, int slot) {
+        auto read_v = [&](int st, int slot) {
 #pragma unroll
-            for (int db = 0; db < 4; ++db) va[slot][db] = __builtin_bit_cast(h8_t, vt[db * (32 * 9) + 2 * step]);
+            for (int db = 0; db < 4; ++db) va[slot][db] = __builtin_bit_cast(h8_t, vt[db * (32 * 9) + 2 * st]);
         };
         read_v(0, 0);
 #pragma unroll
-        for (int step = 0; step < 4; ++step) {
-            if (step < 3) read_v(step + 1, (step + 1) & 1);
+        for (int st = 0; st < 4; ++st) {
+            if (st < 3) read_v(st + 1, (st + 1) & 1);
 #pragma unroll
             for (int db = 0; db < 4; ++db)
-                o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[step & 1][db], pf[step >> 1][step & 1], o[db], 0, 0, 0);
+                o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[st & 1][db], pf[st >> 1][st & 1], o[db], 0, 0, 0);
         }
+    };
+    for (int blk = 0; blk < nblk; blk += 2) {
+        step(blk, sa, sb);
+        if (blk + 1 < nblk) step(blk + 1, sb, sa);
     }
 
     // ---- out[b, s, head * 128 + d] = O[s, d] / l: lane (h, q) holds dims 32 * db + 8 * i + 4 * h + j of its query
@@ -244,7 +303,8 @@ __global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t
     }
 }
 
-#undef FETCH_BLOCK
+#undef FETCH_K
+#undef FETCH_V
 
 }  // namespace
 
