@@ -743,7 +743,7 @@ int gptq4_lm_head_argmax(const void *x, const void *weight, int64_t *out, int B,
 int gptq4_prefill_attention(const void *q, const void *k_cache, const void *v_cache, void *out, int B, int H, int S, int D,
                             int kv_capacity, int past, float scale, void *stream) {
     if (!q || !k_cache || !v_cache || !out) return -GPTQ4_E_NULL;
-    if (B < 1 || H < 1 || S < 1 || D != 128 || past < 0 || kv_capacity < 1 || (long)past + S > kv_capacity || (long)B * H * ((S + 127) / 128) >= (1L << 31) ||
+    if (B < 1 || H < 1 || S < 1 || D != 128 || past < 0 || kv_capacity < 1 || kv_capacity > (1 << 23) || (long)past + S > kv_capacity || (long)B * H * ((S + 127) / 128) >= (1L << 31) ||
         (long)B * H * kv_capacity * 128 >= (1L << 40))
         return -GPTQ4_E_SHAPE;
     if (misaligned16(q) || misaligned16(k_cache) || misaligned16(v_cache) || misaligned16(out)) return -GPTQ4_E_ALIGN;

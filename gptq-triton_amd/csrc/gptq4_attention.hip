@@ -311,15 +311,17 @@ __global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t
 int launch_attn_prefill(const half_t *q, const half_t *kc, const half_t *vc, half_t *out, int B, int H, int S, int capacity, int past,
                         float scale, hipStream_t stream) {
     const int qblocks = (S + 127) / 128;
-    static bool prepared = false;
+    static bool prepared[64] = {};  // per device: the attribute belongs to the kernel as loaded on one device
     static std::mutex lock;
     {
+        int device = 0;
+        if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return (int)hipErrorInvalidDevice;
         std::lock_guard<std::mutex> guard(lock);
-        if (!prepared) {  // more than the 64 KiB a launch may ask for unless the kernel is marked for it
+        if (!prepared[device]) {  // more than the 64 KiB a launch may ask for unless the kernel is marked for it
             const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gptq4_attn_prefill_kernel),
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)FA_LDS_BYTES);
             if (e != hipSuccess) return (int)e;
-            prepared = true;
+            prepared[device] = true;
         }
     }
     hipLaunchKernelGGL(gptq4_attn_prefill_kernel, dim3((unsigned)(qblocks * B * H)), dim3(256), FA_LDS_BYTES, stream, q, kc, vc, out, H, S,

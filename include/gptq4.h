@@ -236,7 +236,7 @@ int gptq4_lm_head_argmax(const void *x, const void *weight, int64_t *out, int B,
  * attends to cache rows 0 .. past + i; softmax in fp32, output fp16 out [B, S, H*D] - the layout o_proj consumes, no
  * transpose.  q fp16 [B, H, S, D] (as gptq4_qkv_rotary writes it); k_cache, v_cache fp16 [B, H, kv_capacity, D] with
  * the S new tokens already in rows past .. past + S - 1 (gptq4_qkv_rotary with kv_offset = past puts them there; for
- * a plain prompt its k / v outputs serve as caches of capacity S).  D must be 128, past + S <= kv_capacity.  No
+ * a plain prompt its k / v outputs serve as caches of capacity S).  D must be 128, past + S <= kv_capacity <= 2^23.  No
  * workspace.  Replaces the attention core of QuantLlamaAttention.forward for a prompt (fused_attention.py:117-141:
  * scores, causal mask, fp32 softmax, weighted sum, transpose + reshape). */
 int gptq4_prefill_attention(const void *q, const void *k_cache, const void *v_cache, void *out, int B, int H, int S,
