@@ -239,10 +239,14 @@ int launch_rmsnorm(const half_t *x, const half_t *delta, const half_t *w, half_t
     return (int)hipGetLastError();
 }
 
-// Rows per split: enough workgroups to cover the chip (~2 per CU), at least 64 rows each.
+// Splits per (sequence, head): as many as fill the chip's 2 x CUs places once without spilling into a second round (40
+// heads: 12 splits = 480 workgroups, not 13 = 520), at least 64 rows each; with many heads still shares of about 256
+// rows, so that the workgroups come in several rounds and the last one is a small part (416 heads x 2048 rows: 83 us
+// with 8 splits against 88 with 2; 128 heads: 16.6 against 17.6).
 int attn_decode_splits(int BH, int capacity) {
     const int want = 2 * device_shape().cus;  // 512 workgroups on MI355X
-    int nsplit = (want + BH - 1) / BH;
+    int nsplit = want / BH;
+    if (nsplit < capacity / 256) nsplit = capacity / 256;
     const int max_split = (capacity + 63) / 64;
     if (nsplit > max_split) nsplit = max_split;
     if (nsplit < 1) nsplit = 1;
