@@ -1000,7 +1000,10 @@ int gptq4_stream_qkv_rotary(const void *x, const void *delta, const void *norm_w
 
 void gptq4_set_stream_tuning(int waves, int depth) {
     g_stream_tuning.waves = (waves == 8 || waves == 16) ? waves : 0;
-    g_stream_tuning.depth = (depth >= 1 && depth <= 3) ? depth : 0;
+    // 10 + depth: one tile per unit in the kernel for 5 .. 16 rows, 20 + depth: two wherever they can run (automatic otherwise)
+    const int single = depth >= 20 ? 20 : depth >= 10 ? 10 : 0;
+    depth -= single;
+    g_stream_tuning.depth = ((depth >= 1 && depth <= 3) ? depth : 0) + single;
 }
 
 int gptq4_stream_probe(int op, const void *x, const int32_t *sweight, const int32_t *smeta, const int32_t *up_sweight,

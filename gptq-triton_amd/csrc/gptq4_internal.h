@@ -199,8 +199,9 @@ struct StreamPlan {
     int waves, depth;  // waves per workgroup (8 or 16), units in flight per wave
     int workgroups;
     int tiles, nb;
+    int strips;  // tiles per unit (2 in the kernel for 5 .. 16 rows where the tile count is even)
     int q, r;
-    int pieces;  // most strips a workgroup's range touches
+    int pieces;  // most tiles a workgroup's range touches
     int xrow, red_off, nat_off;
     size_t lds_bytes;
     bool ok;

@@ -429,9 +429,10 @@ struct TUnit {
     u32x4_t a[4];
 };
 
-template <int EPI, int NW, int DEPTH>
+template <int EPI, int NW, int DEPTH, int NS>
 __global__ __launch_bounds__(64 * NW) void gptq4_stream_tall_kernel(STREAM_HOT_PARAMS, StreamArgs p) {
     constexpr int NV = (EPI == EPI_PLAIN) ? 1 : 2;
+    constexpr int NV2 = NV * NS;  // weight blocks per unit: NS adjacent tiles (strips; quarter-head pairs for the rotary epilogue) of NV matrices
     constexpr int NT = 64 * NW;
     constexpr int RE = (16 * 64 + NT - 1) / NT;  // (row, column of a head's half) pairs of the rotary table per thread
     extern __shared__ uint4 smem[];
@@ -486,15 +487,18 @@ __global__ __launch_bounds__(64 * NW) void gptq4_stream_tall_kernel(STREAM_HOT_P
     }
     int cp_tile = ld_tile, cp_batch = ld_batch;
     auto strip_of = [&](int tile, int v) { return (EPI == EPI_ROPE) ? ((tile >> 2) << 3) + (tile & 3) + 4 * v : tile; };
-    auto issue = [&](TUnit<NV> &U, bool live) {
+    auto issue = [&](TUnit<NV2> &U, bool live) {
         const uint32_t dead = live ? 0u : S_OFF_RANGE;
         const int g = (bpg == 1) ? ld_batch : (int)__umulhi((unsigned)ld_batch, hgroup_magic);
 #pragma unroll
-        for (int v = 0; v < NV; ++v) {
-            const int strip = strip_of(ld_tile, v);
-            U.w[v] = __builtin_amdgcn_raw_buffer_load_b128(rs_w[v], ((uint32_t)lane * 16u) | dead, (uint32_t)(strip * nb + ld_batch) * 1024u, 2);
-            U.meta[v] = __builtin_amdgcn_raw_buffer_load_b32(rs_m[v], ((uint32_t)c * 4u) | dead, (uint32_t)(strip * G + g) * 64u, 0);
-        }
+        for (int s = 0; s < NS; ++s)
+#pragma unroll
+            for (int v = 0; v < NV; ++v) {
+                const int strip = strip_of(ld_tile * NS + s, v);
+                U.w[s * NV + v] =
+                    __builtin_amdgcn_raw_buffer_load_b128(rs_w[v], ((uint32_t)lane * 16u) | dead, (uint32_t)(strip * nb + ld_batch) * 1024u, 2);
+                U.meta[s * NV + v] = __builtin_amdgcn_raw_buffer_load_b32(rs_m[v], ((uint32_t)c * 4u) | dead, (uint32_t)(strip * G + g) * 64u, 0);
+            }
 #pragma unroll
         for (int i = 0; i < 4; ++i) U.a[i] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, xoff[i] | dead, (uint32_t)ld_batch * 256u, 0);
         ld_batch -= NW;
@@ -503,7 +507,7 @@ __global__ __launch_bounds__(64 * NW) void gptq4_stream_tall_kernel(STREAM_HOT_P
             ld_tile -= 1;
         }
     };
-    TUnit<NV> ring[DEPTH];
+    TUnit<NV2> ring[DEPTH];
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) issue(ring[d], d < n);
 
@@ -523,56 +527,56 @@ __global__ __launch_bounds__(64 * NW) void gptq4_stream_tall_kernel(STREAM_HOT_P
     const bool publishes = (b0 - tile_hi * nb) != nb;
     const bool shared_lo = (a0 - tile_lo * nb) != 0;
     const int fin0 = publishes ? 1 : 0;
-    const int total = (npieces - fin0) * M * 16;
+    const int total = (npieces - fin0) * NS * M * 16;
 
-    // element e = (piece from the bottom, row, column); thread t finishes e = NT - 1 - t, + NT, ...: the bottom piece,
+    // element e = (piece from the bottom, tile of the piece's NS, row, column); thread t finishes e = NT - 1 - t, + NT, ...: the bottom piece,
     // whose other part comes from memory, falls to lanes of the last wave, which never has the most units
     const int e_mine = NT - 1 - tid;
-    const bool gets_partials = shared_lo && e_mine < min(total, M * 16);
+    const bool gets_partials = shared_lo && e_mine < min(total, NS * M * 16);
 
-    f4_t *const red = reinterpret_cast<f4_t *>(smem);  // [piece][wave][NV][lane]
+    f4_t *const red = reinterpret_cast<f4_t *>(smem);  // [piece][wave][NV2][lane]
     const float *const redf = reinterpret_cast<const float *>(red);
     for (int pc = 0; pc < npieces; ++pc)
 #pragma unroll
-        for (int v = 0; v < NV; ++v) red[((pc * NW + wave) * NV + v) * 64 + lane] = (f4_t){0.f, 0.f, 0.f, 0.f};
+        for (int v = 0; v < NV2; ++v) red[((pc * NW + wave) * NV2 + v) * 64 + lane] = (f4_t){0.f, 0.f, 0.f, 0.f};
     if (tid == 0) arrivals = 0;
     __syncthreads();
 
-    const int slot_elems = NV * 16 * M;
+    const int slot_elems = NV2 * 16 * M;
     auto arrive_top = [&]() {
         int old = 0;
         if (lane == 0) old = __hip_atomic_fetch_add(&arrivals, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_WORKGROUP);
         old = __builtin_amdgcn_readfirstlane(old);
         if (old != NW - 1) return;
         uint64_t *const mine = p.tagged + (size_t)wg * slot_elems;
-        for (int e = lane; e < slot_elems; e += 64) {  // e = (v * M + row) * 16 + column
+        for (int e = lane; e < slot_elems; e += 64) {  // e = (block * M + row) * 16 + column, block = tile of the NS * NV + matrix
             const int col = e & 15, t = e >> 4;
-            const int v = (t >= M) ? 1 : 0;
+            const int v = (t * p.m_magic) >> 16;
             const int row = t - v * M;
             float s = 0.f;
 #pragma unroll
-            for (int w = 0; w < NW; ++w) s += redf[((w * NV + v) * 64 + (row >> 2) * 16 + col) * 4 + (row & 3)];
+            for (int w = 0; w < NW; ++w) s += redf[((w * NV2 + v) * 64 + (row >> 2) * 16 + col) * 4 + (row & 3)];
             __hip_atomic_store(&mine[e], S_MARK | (uint64_t)__float_as_uint(s), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     };
-    f4_t acc[NV];
+    f4_t acc[NV2];
 #pragma unroll
-    for (int v = 0; v < NV; ++v) acc[v] = (f4_t){0.f, 0.f, 0.f, 0.f};
+    for (int v = 0; v < NV2; ++v) acc[v] = (f4_t){0.f, 0.f, 0.f, 0.f};
     auto dump = [&](int pc) {
 #pragma unroll
-        for (int v = 0; v < NV; ++v) red[((pc * NW + wave) * NV + v) * 64 + lane] = acc[v];
+        for (int v = 0; v < NV2; ++v) red[((pc * NW + wave) * NV2 + v) * 64 + lane] = acc[v];
         if (pc == 0 && publishes) arrive_top();
     };
     if (publishes && wave >= top_len) arrive_top();
 
     int cur_tile = cp_tile;
     uint4 *const turn = smem + p.nat_off + wave * (16 * 17);  // the wave's own 16 x 17 chunks
-    auto compute = [&](const TUnit<NV> &U) {
+    auto compute = [&](const TUnit<NV2> &U) {
         if (cp_tile != cur_tile) {
             dump(tile_hi - cur_tile);
             cur_tile = cp_tile;
 #pragma unroll
-            for (int v = 0; v < NV; ++v) acc[v] = (f4_t){0.f, 0.f, 0.f, 0.f};
+            for (int v = 0; v < NV2; ++v) acc[v] = (f4_t){0.f, 0.f, 0.f, 0.f};
         }
         // rows x chunks in, (row c, chunks 4 * r4 + j) out
 #pragma unroll
@@ -580,13 +584,13 @@ __global__ __launch_bounds__(64 * NW) void gptq4_stream_tall_kernel(STREAM_HOT_P
         h8_t a[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) a[j] = __builtin_bit_cast(h8_t, turn[c * 17 + 4 * r4 + j]);
-        ColDecode cd[NV];
+        ColDecode cd[NV2];
 #pragma unroll
-        for (int v = 0; v < NV; ++v) cd[v] = make_col_decode(U.meta[v] >> 16, U.meta[v]);
+        for (int v = 0; v < NV2; ++v) cd[v] = make_col_decode(U.meta[v] >> 16, U.meta[v]);
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int v = 0; v < NV; ++v)
+            for (int v = 0; v < NV2; ++v)
                 acc[v] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[j], decode_word_h8(U.w[v][j], cd[v]), acc[v], 0, 0, 0);
         cp_batch -= NW;
         if (cp_batch < 0) {
@@ -624,7 +628,7 @@ __global__ __launch_bounds__(64 * NW) void gptq4_stream_tall_kernel(STREAM_HOT_P
 #pragma unroll
     for (int v = 0; v < NV; ++v) part[v] = 0.f;
     if (gets_partials) {
-        const int e_col = e_mine & 15, e_row = e_mine >> 4;  // piece 0: e = row * 16 + column
+        const int e_col = e_mine & 15, e_s = ((e_mine >> 4) * p.m_magic) >> 16, e_row = (e_mine >> 4) - e_s * M;  // piece 0: e = (tile * M + row) * 16 + column
         const int u_first = tile_lo * nb;
         const int big = hr * (hq + 1);
         const int first = u_first < big ? sdiv_magic(u_first, hq + 1, p.q1_magic) : hr + sdiv_magic(u_first - big, hq, p.q_magic);
@@ -636,7 +640,7 @@ __global__ __launch_bounds__(64 * NW) void gptq4_stream_tall_kernel(STREAM_HOT_P
                 uint64_t all = S_MARK;
 #pragma unroll
                 for (int v = 0; v < NV; ++v) {
-                    got[v] = __hip_atomic_load(&slot[(v * M + e_row) * 16 + e_col], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    got[v] = __hip_atomic_load(&slot[((e_s * NV + v) * M + e_row) * 16 + e_col], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     all &= got[v];
                 }
                 if (p.spin_limit != 0xFFFFFFFFu && all != 0) break;
@@ -649,7 +653,7 @@ __global__ __launch_bounds__(64 * NW) void gptq4_stream_tall_kernel(STREAM_HOT_P
 #pragma unroll
             for (int v = 0; v < NV; ++v) {
                 part[v] += __uint_as_float((uint32_t)got[v]);
-                __hip_atomic_store(&slot[(v * M + e_row) * 16 + e_col], (uint64_t)0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(&slot[((e_s * NV + v) * M + e_row) * 16 + e_col], (uint64_t)0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
     }
@@ -658,16 +662,17 @@ __global__ __launch_bounds__(64 * NW) void gptq4_stream_tall_kernel(STREAM_HOT_P
     for (int e = e_mine; e < total; e += NT) {
         const int e_col = e & 15;
         const int e_t = e >> 4;
-        const int e_pb = (e_t * p.m_magic) >> 16;
-        const int e_row = e_t - e_pb * M;
-        const int e_tile = tile_lo + e_pb;
+        const int e_ps = (e_t * p.m_magic) >> 16;  // (piece, tile of the piece)
+        const int e_row = e_t - e_ps * M;
+        const int e_pb = e_ps / NS, e_s = e_ps - e_pb * NS;
+        const int e_tile = (tile_lo + e_pb) * NS + e_s;
         const int pc = npieces - 1 - e_pb;
         float s[NV];
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             s[v] = (e == e_mine) ? part[v] : 0.f;
 #pragma unroll
-            for (int w = 0; w < NW; ++w) s[v] += redf[(((pc * NW + w) * NV + v) * 64 + (e_row >> 2) * 16 + e_col) * 4 + (e_row & 3)];
+            for (int w = 0; w < NW; ++w) s[v] += redf[(((pc * NW + w) * NV2 + e_s * NV + v) * 64 + (e_row >> 2) * 16 + e_col) * 4 + (e_row & 3)];
         }
         if (EPI == EPI_PLAIN) {
             half_t o = (half_t)s[0];
@@ -828,20 +833,20 @@ int launch_shape(const StreamArgs &a, const StreamPlan &pl, bool nomath, hipStre
     return perm ? launch_kernel<EPI, NW, DEPTH, true, 0, false>(a, pl, stream) : launch_kernel<EPI, NW, DEPTH, false, 0, false>(a, pl, stream);
 }
 
-template <int EPI, int NW, int DEPTH>
+template <int EPI, int NW, int DEPTH, int NS>
 int launch_tall(const StreamArgs &a, const StreamPlan &pl, hipStream_t stream) {
     static bool prepared = false;
     static std::mutex lock;
     {
         std::lock_guard<std::mutex> guard(lock);
         if (!prepared) {
-            const void *fn = reinterpret_cast<const void *>(&gptq4_stream_tall_kernel<EPI, NW, DEPTH>);
+            const void *fn = reinterpret_cast<const void *>(&gptq4_stream_tall_kernel<EPI, NW, DEPTH, NS>);
             const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)STREAM_LDS_BUDGET);
             if (e != hipSuccess) return (int)e;
             prepared = true;
         }
     }
-    hipLaunchKernelGGL((gptq4_stream_tall_kernel<EPI, NW, DEPTH>), dim3((unsigned)pl.workgroups), dim3(64 * NW), pl.lds_bytes, stream,
+    hipLaunchKernelGGL((gptq4_stream_tall_kernel<EPI, NW, DEPTH, NS>), dim3((unsigned)pl.workgroups), dim3(64 * NW), pl.lds_bytes, stream,
                        STREAM_HOT_ARGS(a), a);
     return (int)hipGetLastError();
 }
@@ -850,11 +855,15 @@ template <int EPI>
 int launch_epi(const StreamArgs &a, const StreamPlan &pl, bool nomath, hipStream_t stream) {
     if (pl.tall) {
         if (nomath || a.perm != nullptr || a.nrm_weight != nullptr) return (int)hipErrorInvalidValue;
-        switch (pl.waves * 10 + pl.depth) {
-            case 81: return launch_tall<EPI, 8, 1>(a, pl, stream);
-            case 82: return launch_tall<EPI, 8, 2>(a, pl, stream);
-            case 161: return launch_tall<EPI, 16, 1>(a, pl, stream);
-            case 162: return launch_tall<EPI, 16, 2>(a, pl, stream);
+        switch ((pl.waves * 10 + pl.depth) * 10 + pl.strips) {
+            case 811: return launch_tall<EPI, 8, 1, 1>(a, pl, stream);
+            case 821: return launch_tall<EPI, 8, 2, 1>(a, pl, stream);
+            case 1611: return launch_tall<EPI, 16, 1, 1>(a, pl, stream);
+            case 1621: return launch_tall<EPI, 16, 2, 1>(a, pl, stream);
+            case 812: return launch_tall<EPI, 8, 1, 2>(a, pl, stream);
+            case 822: return launch_tall<EPI, 8, 2, 2>(a, pl, stream);
+            case 1612: return launch_tall<EPI, 16, 1, 2>(a, pl, stream);
+            case 1622: return launch_tall<EPI, 16, 2, 2>(a, pl, stream);
             default: return (int)hipErrorInvalidValue;
         }
     }
@@ -874,11 +883,31 @@ uint32_t smagic(int d) { return d > 1 ? (uint32_t)(0x100000000ull / (unsigned)d 
 
 StreamTuning g_stream_tuning = {0, 0};
 
+static StreamPlan stream_plan_with(int epi, int M, int N, int K, bool norm, int strips);
+
 StreamPlan stream_plan(int epi, int M, int N, int K, bool norm) {
+    // 8 .. 16 rows: a unit is the 128 input rows of TWO adjacent tiles, so that the rows' chunks - twice the bytes of a
+    // tile's weights at 16 rows - are fetched and turned once for both; only where a workgroup's range stays long (LLaMA-7B at
+    // 16 rows: gate/up 16.8 against 17.7 us, down_proj 10.7 against 11.3 with 43 units to a workgroup; QKV 13.2 against
+    // 11.4 and o_proj 7.3 against 5.9 with 24 and 16, where the ranges stop lining up with the tiles), where the tile
+    // count is even and the partial sums of two tiles fit the LDS.  (depth + 10 in the tuning call: never; + 20: wherever
+    // it can run.)
+    const int tiles = (epi == EPI_ROPE) ? N / 32 : N / 16;
+    const int mode = g_stream_tuning.depth / 10;
+    if (M > STREAM_MAX_M && (tiles % 2) == 0 && mode != 1) {
+        const StreamPlan two = stream_plan_with(epi, M, N, K, norm, 2);
+        if (two.ok && (mode == 2 || (M >= 8 && two.q >= 40))) return two;
+    }
+    return stream_plan_with(epi, M, N, K, norm, 1);
+}
+
+static StreamPlan stream_plan_with(int epi, int M, int N, int K, bool norm, int strips) {
     StreamPlan pl = {};
-    pl.depth = g_stream_tuning.depth ? g_stream_tuning.depth : 2;
+    const int tuned_depth = g_stream_tuning.depth % 10;
+    pl.depth = tuned_depth ? tuned_depth : 2;
     const int nv = (epi == EPI_PLAIN) ? 1 : 2;
-    pl.tiles = (epi == EPI_ROPE) ? N / 32 : N / 16;
+    pl.strips = strips;
+    pl.tiles = ((epi == EPI_ROPE) ? N / 32 : N / 16) / strips;
     pl.nb = K / 128;
     const long units = (long)pl.tiles * pl.nb;
     const int cus = device_shape().cus;
@@ -894,22 +923,23 @@ StreamPlan stream_plan(int epi, int M, int N, int K, bool norm) {
     if (pl.waves == 16 && pl.depth > 2) pl.depth = 2;
     pl.pieces = (pl.q + 1 + pl.nb - 1) / pl.nb + 1;
     if (M > STREAM_MAX_M) {
-        // 5 .. 16 rows: the A operand comes from memory with every unit, LDS holds the waves' partial sums (1 KiB per
-        // wave, matrix and strip) and the rotary table rows of the tokens
+        // the A operand comes from memory with every unit, LDS holds the waves' partial sums (1 KiB per wave, matrix and
+        // tile) and the rotary table rows of the tokens
         pl.tall = true;
         if (pl.depth > 2) pl.depth = 2;
         // eight waves for every shape here (LLaMA-7B down_proj at 16 rows: 11.2 us against 11.7 with sixteen)
         if (!g_stream_tuning.waves) pl.waves = 8;
         pl.xrow = 0;
-        pl.red_off = pl.pieces * pl.waves * nv * 64;
+        const int nv2 = nv * pl.strips;
+        pl.red_off = pl.pieces * pl.waves * nv2 * 64;
         pl.nat_off = pl.red_off + 2 * 16 * 64 * (int)sizeof(float) / 16;  // behind the rotary table rows: a 16 x 17 chunk slot per wave
         size_t lds = ((size_t)pl.nat_off + (size_t)pl.waves * 16 * 17) * 16;
         if (lds < (size_t)81 * 1024) lds = (size_t)81 * 1024;
         pl.lds_bytes = lds;
         pl.ok = M <= STREAM_TALL_MAX_M && !norm && lds <= STREAM_LDS_BUDGET && (long)K * N < (1L << 32) && (long)M * K < (1L << 30) &&
                 units < (1L << 24) && units * (pl.nb > pl.q + 1 ? pl.nb : pl.q + 1) < (1L << 32) &&
-                (size_t)pl.workgroups * nv * 16 * M * sizeof(uint64_t) <= GPTQ4_WS_TAGGED_BYTES && pl.nb >= pl.waves &&
-                (epi != EPI_ROPE || (N % 128) == 0);
+                (size_t)pl.workgroups * nv2 * 16 * M * sizeof(uint64_t) <= GPTQ4_WS_TAGGED_BYTES && pl.nb >= pl.waves &&
+                pl.pieces * pl.strips * M < 1024 && (epi != EPI_ROPE || (N % 128) == 0);
         return pl;
     }
     pl.xrow = K / 8 + 1;

@@ -169,7 +169,7 @@ int gptq4_column_parts(int op, int M, int K, int N, int *begin, int *cols);
 void gptq4_set_exchange_spin_limit(unsigned polls);
 
 /* Launch shape of the streaming-order decode kernel: waves per workgroup (8 or 16) and units of loads in flight per
- * wave (1..3); 0 = automatic. */
+ * wave (1..3); 0 = automatic.  depth + 10: the kernel for 5 .. 16 rows takes one tile per unit of loads everywhere, depth + 20: two wherever they can run. */
 void gptq4_set_stream_tuning(int waves, int depth);
 
 /* The streaming-order kernel's launch with the decode and the matrix-core instructions left out: the same loads,

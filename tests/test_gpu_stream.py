@@ -247,6 +247,52 @@ def test_matmul_in_every_launch_shape(waves, depth):
     assert head_is_zero()
 
 
+@pytest.mark.parametrize("mode", [10, 20])  # 5 .. 16 rows: one tile per unit of loads everywhere / two wherever they can run
+def test_rows_5_to_16_with_one_and_with_two_tiles_per_unit(mode):
+    G = gptq()
+    _lib = lib_()
+    lib = _lib.load()
+    trip = lambda d: (d["qweight"], d["qzeros"], d["scales"])
+    try:
+        lib.gptq4_set_stream_tuning(0, mode)
+        for m in (5, 8, 13, 16):
+            # plain projections, with and without a bias; ranges that cut tiles (2048 x 512: 4 units to a workgroup) and long ones
+            for (k, n, g) in ((2048, 512, 128), (4096, 4096, 128), (11008, 4096, 128), (1024, 7168, 256)):
+                L = O.make_layer(k, n, g, seed=1700 + k + n, bias=(m == 8))
+                D = to_dev(L)
+                sw, meta = G.stream_pack(D["qweight"], D["qzeros"], D["scales"], g)
+                x = O.make_x(m, k, seed=m + 7)
+                y = G.matmul4_stream(g, torch.from_numpy(x).cuda(), sw, meta, D.get("bias"))
+                ref = O.quant_matmul_ref(x, *trip(L), g, bias=L.get("bias"))
+                if L.get("bias") is None:
+                    assert_close(y.cpu().numpy(), ref, f"mode {mode} {k}x{n} M={m}")
+                else:  # (two fp16 roundings, as the reference's: the tight bound of assert_close does not apply)
+                    ok, max_abs, _ = O.within_tolerance(y.cpu().numpy(), ref)
+                    assert ok, f"mode {mode} {k}x{n} M={m} with bias: max_abs={max_abs}"
+            for (k, inter, g) in ((1024, 2816, 128), (4096, 11008, 128)):
+                gate, up = O.make_layer(k, inter, g, seed=1710 + k), O.make_layer(k, inter, g, seed=1711 + k)
+                Dg, Du = to_dev(gate), to_dev(up)
+                gsw, gm = G.stream_pack(Dg["qweight"], Dg["qzeros"], Dg["scales"], g)
+                usw, um = G.stream_pack(Du["qweight"], Du["qzeros"], Du["scales"], g)
+                x = O.make_x(m, k, seed=m + 51)
+                y = G.llama_mlp_4_stream(g, torch.from_numpy(x).cuda(), gsw, gm, usw, um)
+                assert_close(y.cpu().numpy(), O.mlp_gateup_ref(x, trip(gate), trip(up), g), f"mode {mode} gate/up {k}x{inter} M={m}")
+            for (k, heads, g) in ((1024, 8, 128), (4096, 32, 128)):
+                L = O.make_layer(k, 3 * heads * 128, g, seed=1720 + k)
+                D = to_dev(L)
+                sw, meta = G.stream_pack(D["qweight"], D["qzeros"], D["scales"], g)
+                x = O.make_x(m, k, seed=m + 61).reshape(m, 1, k)
+                pos = (np.arange(m)[:, None] * 29 + 2047 - 29 * (m - 1)).astype(np.int64)
+                cos, sin = G.RotaryTable(128, 2048).get(torch.device("cuda"), 2048)
+                q, kk, vv = G.qkv_rotary_stream(g, torch.from_numpy(x).cuda(), sw, meta, torch.from_numpy(pos).cuda(), cos, sin, heads)
+                refs = O.qkv_rotary_ref(x, *trip(L), g, pos, heads, max_pos=2048)
+                for got, ref, name in zip((q, kk, vv), refs, "qkv"):
+                    assert_close(got.cpu().numpy(), ref, f"mode {mode} qkv {name} K={k} M={m}")
+    finally:
+        lib.gptq4_set_stream_tuning(0, 0)
+    assert head_is_zero()
+
+
 def test_one_hot_rows_return_weight_rows_exactly():
     """x = e_k: the result is row k of the dequantised weight, exactly (a single term, no rounding but the weight's own)."""
     G = gptq()
