@@ -43,6 +43,15 @@ def test_against_the_oracle(b, h, s, cap, past):
     close(out.cpu().numpy(), O.prefill_attention_ref(q, k, v, past), f"B={b} H={h} S={s} past={past}")
 
 
+@pytest.mark.parametrize("b,h,s", [(1, 8, 300), (1, 13, 260), (5, 8, 140), (3, 25, 300), (8, 17, 129), (1, 80, 385)])
+def test_every_head_and_query_block_of_many_heads(b, h, s):
+    """Eight heads and more: a head's query blocks are dealt to one XCD (workgroup id % 8), the heads past the last multiple
+    of eight separately, and more than eight heads to an XCD in groups of four - every (head, query block) exactly once."""
+    q, k, v = make(b, h, s, s, seed=b * 1000 + h)
+    out = ops().prefill_attention(torch.from_numpy(q).cuda(), torch.from_numpy(k).cuda(), torch.from_numpy(v).cuda())
+    close(out.cpu().numpy(), O.prefill_attention_ref(q, k, v, 0), f"B={b} H={h} S={s}")
+
+
 def test_peaked_scores_and_long_prompts():
     """Scores with a wide range (the running maximum moves a lot) at the benchmark's size: 2048 tokens."""
     b, h, s = 1, 4, 2048
