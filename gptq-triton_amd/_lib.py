@@ -128,7 +128,13 @@ def ptr(t: torch.Tensor | None):
     return None if t is None else t.data_ptr()
 
 
+# (the raw handle without building a torch.cuda.Stream object around it: this is asked twice per launch)
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def current_stream(device: torch.device):
+    if _raw_stream is not None:
+        return _raw_stream(device.index if device.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(device).cuda_stream
 
 
@@ -143,8 +149,7 @@ _WS_BYTES = WS_HEAD_BYTES + 16 * 16 * 2 * 32768 * 4  # splitk 16, M 16, 2 matric
 
 
 def workspace(device: torch.device, need: int):
-    key = (device.index if device.index is not None else torch.cuda.current_device(),
-           torch.cuda.current_stream(device).cuda_stream)
+    key = (device.index if device.index is not None else torch.cuda.current_device(), current_stream(device))
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < need:
         if ws is not None:
