@@ -224,6 +224,9 @@ __global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t
         // ---- the next block's scores (whatever the buffer holds after the last block: nobody reads them), then the
         //      running maximum and the probabilities of this one; the accumulators are rescaled only when some lane's
         //      maximum moved
+        // (ahead of the other workgroup's wave on this SIMD while that one is staging or waiting at its barrier: 656 -> 622 us
+        // at 416 heads, 84.6 -> 80.1 at 40)
+        __builtin_amdgcn_s_setprio(1);
         scores(buf ^ 1, sn);
         float mx = -INFINITY;
 #pragma unroll
@@ -273,6 +276,7 @@ __global__ __launch_bounds__(256, 2) void gptq4_attn_prefill_kernel(const half_t
             for (int db = 0; db < 4; ++db)
                 o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(va[st & 1][db], pf[st >> 1][st & 1], o[db], 0, 0, 0);
         }
+        __builtin_amdgcn_s_setprio(0);
     };
     for (int blk = 0; blk < nblk; blk += 2) {
         step(blk, sa, sb);
